@@ -1,0 +1,8 @@
+"""MI355X-native LSTM forward + BPTT (gfx950 HIP kernels behind a C ABI).
+
+`LstmCore` drives the device-resident core (`include/flashlstm/lstm_core.h`) from torch tensors;
+the drop-in `flashlstm` Python package of the streaming surface lives in `flashlstm_poc_amd/python`.
+"""
+from .core import LstmCore, load_library, library_path, LibraryMissing, add_flashlstm_to_path
+
+__all__ = ["LstmCore", "load_library", "library_path", "LibraryMissing", "add_flashlstm_to_path"]

@@ -1,0 +1,194 @@
+"""ctypes binding of the device-resident C ABI (include/flashlstm/lstm_core.h).
+
+torch is used for device memory and streams only; every computation happens inside
+libflashlstm.so.  There is no fallback: if the library is missing, loading raises.
+"""
+from __future__ import annotations
+
+import ctypes
+import os
+import sys
+from typing import Optional, Tuple
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_LIB = None
+
+F32, F16 = 0, 1
+
+
+class LibraryMissing(RuntimeError):
+    pass
+
+
+def library_path() -> str:
+    return os.path.join(_HERE, "libflashlstm.so")
+
+
+def add_flashlstm_to_path() -> str:
+    """Puts the drop-in `flashlstm` package (StreamingLSTM & co.) on sys.path and returns its parent dir."""
+    p = os.path.join(_HERE, "python")
+    if p not in sys.path:
+        sys.path.insert(0, p)
+    return p
+
+
+def load_library() -> ctypes.CDLL:
+    global _LIB
+    if _LIB is not None:
+        return _LIB
+    path = library_path()
+    if not os.path.exists(path):
+        raise LibraryMissing(
+            f"{path} not found: build it with `make -C flashlstm_poc_amd/csrc` "
+            "(or `python -c 'import __graft_entry__ as g; g.build()'`)")
+    lib = ctypes.CDLL(path)
+    c = ctypes
+    vp, sz, i32 = c.c_void_p, c.c_size_t, c.c_int
+    lib.flstm_core_create.argtypes = [sz, sz, sz, c.POINTER(vp)]
+    lib.flstm_core_destroy.argtypes = [vp]
+    lib.flstm_core_set_option.argtypes = [vp, c.c_char_p, c.c_long]
+    lib.flstm_core_get_info.argtypes = [vp, c.c_char_p]
+    lib.flstm_core_get_info.restype = c.c_long
+    lib.flstm_core_pack_weights.argtypes = [vp, vp, vp, vp]
+    lib.flstm_core_pack_bias.argtypes = [vp, vp, vp, vp]
+    lib.flstm_core_forward.argtypes = [vp, sz, vp, i32, vp, vp, i32, vp, i32, vp, vp, i32, i32, vp]
+    lib.flstm_core_backward.argtypes = [vp, sz, vp, i32, vp, i32, vp, vp, i32, c.c_float, vp, i32,
+                                        vp, vp, vp, vp, vp, vp, vp]
+    lib.flstm_core_cache_ptr.argtypes = [vp, i32, c.POINTER(vp), c.POINTER(sz)]
+    lib.flstm_core_last_ms.argtypes = [vp, c.c_char_p]
+    lib.flstm_core_last_ms.restype = c.c_double
+    for name in ("flstm_core_create", "flstm_core_destroy", "flstm_core_set_option", "flstm_core_pack_weights",
+                 "flstm_core_pack_bias", "flstm_core_forward", "flstm_core_backward", "flstm_core_cache_ptr"):
+        getattr(lib, name).restype = i32
+    _LIB = lib
+    return lib
+
+
+def _dtype_code(t) -> int:
+    import torch
+    if t.dtype == torch.float32:
+        return F32
+    if t.dtype == torch.float16:
+        return F16
+    raise ValueError(f"unsupported dtype {t.dtype}: tensors must be float16 or float32")
+
+
+def _ptr(t) -> Optional[int]:
+    return None if t is None else t.data_ptr()
+
+
+class LstmCore:
+    """One single-layer LSTM of fixed (batch, input, hidden) on the current GPU."""
+
+    def __init__(self, batch: int, input_size: int, hidden_size: int):
+        self.lib = load_library()
+        self.B, self.I, self.H = int(batch), int(input_size), int(hidden_size)
+        h = ctypes.c_void_p()
+        rc = self.lib.flstm_core_create(self.B, self.I, self.H, ctypes.byref(h))
+        if rc != 0:
+            raise RuntimeError(f"flstm_core_create failed with status {rc}")
+        self._h = h
+
+    def close(self) -> None:
+        if getattr(self, "_h", None) is not None and self._h:
+            self.lib.flstm_core_destroy(self._h)
+            self._h = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+    @staticmethod
+    def _stream() -> int:
+        import torch
+        return torch.cuda.current_stream().cuda_stream
+
+    def set_option(self, name: str, value: int) -> None:
+        rc = self.lib.flstm_core_set_option(self._h, name.encode(), int(value))
+        if rc != 0:
+            raise ValueError(f"option {name}={value} rejected (status {rc})")
+
+    def info(self, name: str) -> int:
+        return int(self.lib.flstm_core_get_info(self._h, name.encode()))
+
+    def last_ms(self, phase: str) -> float:
+        return float(self.lib.flstm_core_last_ms(self._h, phase.encode()))
+
+    def pack(self, w_ih, w_hh, b_ih=None, b_hh=None) -> None:
+        import torch
+        for name, t, shape in (("w_ih", w_ih, (4 * self.H, self.I)), ("w_hh", w_hh, (4 * self.H, self.H))):
+            if t.dtype != torch.float32 or not t.is_cuda or not t.is_contiguous() or tuple(t.shape) != shape:
+                raise ValueError(f"{name} must be a contiguous CUDA float32 tensor of shape {shape}")
+        for name, t in (("b_ih", b_ih), ("b_hh", b_hh)):
+            if t is not None and (t.dtype != torch.float32 or not t.is_cuda or t.numel() != 4 * self.H):
+                raise ValueError(f"{name} must be a CUDA float32 tensor with 4*hidden elements")
+        rc = self.lib.flstm_core_pack_weights(self._h, w_ih.data_ptr(), w_hh.data_ptr(), self._stream())
+        if rc == 0:
+            rc = self.lib.flstm_core_pack_bias(self._h, _ptr(b_ih), _ptr(b_hh), self._stream())
+        if rc != 0:
+            raise RuntimeError(f"weight packing failed with status {rc}")
+
+    def forward(self, x, h0=None, c0=None, *, out_dtype=None, save_for_backward: bool = True,
+                want_y: bool = True) -> Tuple:
+        """x (T,B,I) fp16/fp32 on the GPU -> (y (T,B,H), hy, cy) in out_dtype (default: x.dtype)."""
+        import torch
+        if not x.is_cuda or x.dim() != 3 or x.shape[1] != self.B or x.shape[2] != self.I:
+            raise ValueError(f"x must be a CUDA tensor of shape (T, {self.B}, {self.I})")
+        x = x.contiguous()
+        T = x.shape[0]
+        out_dtype = out_dtype or x.dtype
+        st_code = F16
+        for name, t in (("h0", h0), ("c0", c0)):
+            if t is not None:
+                if not t.is_cuda or tuple(t.shape) != (self.B, self.H) or not t.is_contiguous():
+                    raise ValueError(f"{name} must be a contiguous CUDA tensor of shape ({self.B}, {self.H})")
+        if h0 is not None and c0 is not None and h0.dtype != c0.dtype:
+            raise ValueError("h0 and c0 must share a dtype")
+        if h0 is not None:
+            st_code = _dtype_code(h0)
+        elif c0 is not None:
+            st_code = _dtype_code(c0)
+        y = torch.empty((T, self.B, self.H), device=x.device, dtype=out_dtype) if want_y else None
+        hy = torch.empty((self.B, self.H), device=x.device, dtype=out_dtype)
+        cy = torch.empty_like(hy)
+        rc = self.lib.flstm_core_forward(self._h, T, x.data_ptr(), _dtype_code(x), _ptr(h0), _ptr(c0), st_code,
+                                         _ptr(y), _dtype_code(hy), hy.data_ptr(), cy.data_ptr(), _dtype_code(hy),
+                                         1 if save_for_backward else 0, self._stream())
+        if rc != 0:
+            raise RuntimeError(f"flstm_core_forward failed with status {rc}")
+        return y, hy, cy
+
+    def backward(self, x, dy, d_hn=None, d_cn=None, *, grad_scale: float = 1.0, dx_dtype=None,
+                 want_dx: bool = True):
+        """Returns (dx, dW_ih, dW_hh, db, dh0, dc0); db is the gradient of both bias vectors."""
+        import torch
+        x = x.contiguous()
+        dy = dy.contiguous()
+        T = x.shape[0]
+        if tuple(dy.shape) != (T, self.B, self.H):
+            raise ValueError(f"dy must have shape ({T}, {self.B}, {self.H})")
+        dev = x.device
+        dst_code = F16
+        if d_hn is not None and d_cn is not None and d_hn.dtype != d_cn.dtype:
+            raise ValueError("d_hn and d_cn must share a dtype")
+        if d_hn is not None:
+            d_hn = d_hn.contiguous(); dst_code = _dtype_code(d_hn)
+        if d_cn is not None:
+            d_cn = d_cn.contiguous(); dst_code = _dtype_code(d_cn)
+        dx_dtype = dx_dtype or x.dtype
+        dx = torch.empty_like(x, dtype=dx_dtype) if want_dx else None
+        dW_ih = torch.empty((4 * self.H, self.I), device=dev, dtype=torch.float32)
+        dW_hh = torch.empty((4 * self.H, self.H), device=dev, dtype=torch.float32)
+        db = torch.empty((4 * self.H,), device=dev, dtype=torch.float32)
+        dh0 = torch.empty((self.B, self.H), device=dev, dtype=torch.float32)
+        dc0 = torch.empty_like(dh0)
+        rc = self.lib.flstm_core_backward(self._h, T, x.data_ptr(), _dtype_code(x), dy.data_ptr(), _dtype_code(dy),
+                                          _ptr(d_hn), _ptr(d_cn), dst_code, float(grad_scale), _ptr(dx),
+                                          _dtype_code(dx) if dx is not None else F16, dW_ih.data_ptr(),
+                                          dW_hh.data_ptr(), db.data_ptr(), None, dh0.data_ptr(), dc0.data_ptr(),
+                                          self._stream())
+        if rc != 0:
+            raise RuntimeError(f"flstm_core_backward failed with status {rc}")
+        return dx, dW_ih, dW_hh, db, dh0, dc0

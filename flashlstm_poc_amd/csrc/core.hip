@@ -1,0 +1,470 @@
+// Plan object and orchestration of the device-resident LSTM forward / BPTT core.
+//
+// Forward  = [convert x] -> MFMA GEMM  G = X * W_ih^T  (hoisted input projection, the chunked
+//            "projchunksz" GEMM of src/lstm.cu:1204-1239) -> persistent recurrence kernel that turns G
+//            in place into the fp16 gate cache and fills the h / c state arrays -> [unpad outputs].
+// Backward = persistent BPTT kernel (reads gate cache + c states, writes dG) -> dX = dG * W_ih
+//            -> dW = dG^T * [X ; H_prev] as one split-K GEMM -> reductions into caller layout.
+#include <hip/hip_runtime.h>
+
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <new>
+
+#include "../../include/flashlstm/lstm_core.h"
+#include "gemm.h"
+#include "pack.h"
+#include "recurrent.h"
+
+using namespace flstm_hip;
+
+namespace {
+
+struct DevBuf {
+    void* p = nullptr;
+    size_t bytes = 0;
+    // grows (never shrinks); contents are lost on growth
+    hipError_t reserve(size_t need) {
+        if (need <= bytes) return hipSuccess;
+        if (p) { hipError_t e = hipFree(p); p = nullptr; bytes = 0; if (e != hipSuccess) return e; }
+        hipError_t e = hipMalloc(&p, need);
+        if (e == hipSuccess) bytes = need;
+        return e;
+    }
+    void release() { if (p) (void)hipFree(p); p = nullptr; bytes = 0; }
+    template <typename T> T* as() const { return static_cast<T*>(p); }
+};
+
+struct PhaseTimer {
+    hipEvent_t ev[8] = {};
+    bool ok = false;
+    hipError_t init() {
+        for (auto& e : ev) { hipError_t r = hipEventCreate(&e); if (r != hipSuccess) return r; }
+        ok = true;
+        return hipSuccess;
+    }
+    void destroy() { if (ok) for (auto& e : ev) (void)hipEventDestroy(e); ok = false; }
+};
+
+}  // namespace
+
+struct flstm_core_plan {
+    int num_cus = 0;
+    Dims d{};
+    RecLayout Lf{}, Lb{};
+    int ks_f = 0, ks_b = 0;
+    // options
+    int opt_stepwise = 0, opt_proj_chunk = 0, opt_spin_limit = 1 << 22, opt_dw_splits = 0;
+    bool broken_fwd = false, broken_bwd = false;  // persistent launch failed once: stay step-wise
+    long fallbacks = 0;
+    // weights
+    DevBuf wih_p, wih_t, wfrag_f, wfrag_b, bias_p;
+    bool weights_packed = false, bias_packed = false;
+    // forward state / caches
+    DevBuf X16, G, Y, C, flags_f, flags_b, status;
+    unsigned epoch_f = 0, epoch_b = 0;
+    size_t T_cache = 0;
+    bool have_cache = false;
+    // backward scratch
+    DevBuf dYp, dG, dGT, XHT, dHn, dC, dH0, db_part, dw_part;
+    PhaseTimer tm;
+    float ms_fwd[3] = {-1, -1, -1}, ms_bwd[4] = {-1, -1, -1, -1};
+};
+
+namespace {
+
+#define FL_TRY(expr)                                  \
+    do {                                              \
+        hipError_t _e = (expr);                       \
+        if (_e != hipSuccess) return int(_e);         \
+    } while (0)
+
+void replan(flstm_core_plan* p) {
+    p->Lf = plan_rec_fwd(p->d.B, p->d.Hp, p->num_cus, p->opt_stepwise || p->broken_fwd);
+    p->Lb = plan_rec_bwd(p->d.B, p->d.Hp, p->num_cus, p->opt_stepwise || p->broken_bwd);
+    p->ks_f = rec_fwd_ks(p->Lf, p->d.Hp);
+    p->ks_b = rec_bwd_ks(p->Lb, p->d.Hp);
+}
+
+int read_status(flstm_core_plan* p, hipStream_t s, int* out) {
+    FL_TRY(hipStreamSynchronize(s));
+    FL_TRY(hipMemcpy(out, p->status.p, sizeof(int), hipMemcpyDeviceToHost));
+    if (*out != 0) {
+        int zero = 0;
+        FL_TRY(hipMemcpy(p->status.p, &zero, sizeof(int), hipMemcpyHostToDevice));
+    }
+    return 0;
+}
+
+float elapsed(hipEvent_t a, hipEvent_t b) {
+    float ms = -1.f;
+    if (hipEventElapsedTime(&ms, a, b) != hipSuccess) return -1.f;
+    return ms;
+}
+
+}  // namespace
+
+extern "C" int flstm_core_create(size_t batch, size_t input_size, size_t hidden_size, flstm_core_plan** out) {
+    if (!out) return FLSTM_E_INVALID;
+    *out = nullptr;
+    if (batch == 0 || input_size == 0 || hidden_size == 0) return FLSTM_E_INVALID;
+    if (batch > (1u << 20) || input_size > (1u << 20) || hidden_size > (1u << 18)) return FLSTM_E_INVALID;
+    auto* p = new (std::nothrow) flstm_core_plan();
+    if (!p) return int(hipErrorOutOfMemory);
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e == hipSuccess) e = hipDeviceGetAttribute(&p->num_cus, hipDeviceAttributeMultiprocessorCount, dev);
+    if (e != hipSuccess) { delete p; return int(e); }
+    p->d.B = int(batch);
+    p->d.I = int(input_size);
+    p->d.H = int(hidden_size);
+    p->d.Ip = int(round_up(input_size, 64));
+    p->d.Hp = int(round_up(hidden_size, 32));
+    replan(p);
+    p->d.JF = p->Lf.jb;
+    e = p->status.reserve(64);
+    if (e == hipSuccess) e = hipMemset(p->status.p, 0, 64);
+    if (e == hipSuccess) e = p->tm.init();
+    if (e != hipSuccess) { flstm_core_destroy(p); return int(e); }
+    *out = p;
+    return 0;
+}
+
+extern "C" int flstm_core_destroy(flstm_core_plan* p) {
+    if (!p) return FLSTM_E_INVALID;
+    for (DevBuf* b : {&p->wih_p, &p->wih_t, &p->wfrag_f, &p->wfrag_b, &p->bias_p, &p->X16, &p->G, &p->Y, &p->C,
+                      &p->flags_f, &p->flags_b, &p->status, &p->dYp, &p->dG, &p->dGT, &p->XHT, &p->dHn, &p->dC,
+                      &p->dH0, &p->db_part, &p->dw_part})
+        b->release();
+    p->tm.destroy();
+    delete p;
+    return 0;
+}
+
+extern "C" int flstm_core_set_option(flstm_core_plan* p, const char* name, long value) {
+    if (!p || !name) return FLSTM_E_INVALID;
+    if (!strcmp(name, "stepwise")) { p->opt_stepwise = value != 0; replan(p); return 0; }
+    if (!strcmp(name, "proj_chunk")) { p->opt_proj_chunk = int(value); return 0; }
+    if (!strcmp(name, "spin_limit")) { if (value < 1) return FLSTM_E_INVALID; p->opt_spin_limit = int(value); return 0; }
+    if (!strcmp(name, "dw_splits")) { if (value < 0) return FLSTM_E_INVALID; p->opt_dw_splits = int(value); return 0; }
+    return FLSTM_E_INVALID;
+}
+
+extern "C" long flstm_core_get_info(const flstm_core_plan* p, const char* name) {
+    if (!p || !name) return -1;
+    if (!strcmp(name, "persistent_fwd")) return p->Lf.persistent;
+    if (!strcmp(name, "persistent_bwd")) return p->Lb.persistent;
+    if (!strcmp(name, "xcd_local_fwd")) return p->Lf.xcd_local;
+    if (!strcmp(name, "xcd_local_bwd")) return p->Lb.xcd_local;
+    if (!strcmp(name, "resident_fwd")) return p->Lf.resident;
+    if (!strcmp(name, "resident_bwd")) return p->Lb.resident;
+    if (!strcmp(name, "groups_fwd")) return p->Lf.ng;
+    if (!strcmp(name, "groups_bwd")) return p->Lb.ng;
+    if (!strcmp(name, "fallbacks")) return p->fallbacks;
+    if (!strcmp(name, "num_cus")) return p->num_cus;
+    if (!strcmp(name, "hidden_padded")) return p->d.Hp;
+    if (!strcmp(name, "input_padded")) return p->d.Ip;
+    if (!strcmp(name, "gate_slice")) return p->d.JF;
+    return -1;
+}
+
+extern "C" int flstm_core_pack_weights(flstm_core_plan* p, const float* w_ih, const float* w_hh, void* stream) {
+    if (!p || !w_ih || !w_hh) return FLSTM_E_INVALID;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const Dims& d = p->d;
+    FL_TRY(p->wih_p.reserve(size_t(4) * d.Hp * d.Ip * sizeof(half_t)));
+    FL_TRY(p->wih_t.reserve(size_t(4) * d.Hp * d.Ip * sizeof(half_t)));
+    FL_TRY(p->wfrag_f.reserve(size_t(p->Lf.nh) * 4 * p->ks_f * p->Lf.nt * kWave * sizeof(half8)));
+    FL_TRY(p->wfrag_b.reserve(size_t(p->Lb.nh) * 4 * p->ks_b * p->Lb.nt * kWave * sizeof(half8)));
+    FL_TRY(pack_weights(d, w_ih, w_hh, p->wih_p.as<half_t>(), p->wih_t.as<half_t>(), p->wfrag_f.as<half8>(),
+                        p->ks_f, p->Lf.nt, p->wfrag_b.as<half8>(), p->ks_b, p->Lb.nt, s));
+    FL_TRY(hipStreamSynchronize(s));
+    p->weights_packed = true;
+    return 0;
+}
+
+extern "C" int flstm_core_pack_bias(flstm_core_plan* p, const float* b_ih, const float* b_hh, void* stream) {
+    if (!p) return FLSTM_E_INVALID;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    FL_TRY(p->bias_p.reserve(size_t(4) * p->d.Hp * sizeof(float)));
+    if (!b_ih || !b_hh) {
+        // zeros for a missing vector: pack against a zeroed scratch vector
+        FL_TRY(p->db_part.reserve(size_t(4) * p->d.Hp * sizeof(float)));
+        FL_TRY(fill_zero(p->db_part.p, size_t(4) * p->d.Hp * sizeof(float), s));
+        const float* z = p->db_part.as<float>();
+        FL_TRY(pack_bias(p->d, b_ih ? b_ih : z, b_hh ? b_hh : z, p->bias_p.as<float>(), s));
+    } else {
+        FL_TRY(pack_bias(p->d, b_ih, b_hh, p->bias_p.as<float>(), s));
+    }
+    p->bias_packed = true;
+    return 0;
+}
+
+namespace {
+
+int forward_once(flstm_core_plan* p, size_t T, const void* x, flstm_dtype x_dtype, const void* h0,
+                 const void* c0, flstm_dtype state_dtype, hipStream_t s) {
+    const Dims& d = p->d;
+    const size_t TB = T * size_t(d.B);
+    // operand A of the projection
+    const half_t* A = nullptr;
+    size_t lda = 0;
+    if (x_dtype == FLSTM_F16 && d.I == d.Ip) {
+        A = static_cast<const half_t*>(x);
+        lda = size_t(d.I);
+    } else {
+        FL_TRY(p->X16.reserve(TB * d.Ip * sizeof(half_t)));
+        FL_TRY(convert_pad(x, x_dtype == FLSTM_F32, TB, d.I, size_t(d.I), 1.f, p->X16.as<half_t>(), TB,
+                           size_t(d.Ip), s));
+        A = p->X16.as<half_t>();
+        lda = size_t(d.Ip);
+    }
+    FL_TRY(p->G.reserve(TB * 4 * d.Hp * sizeof(half_t)));
+    FL_TRY(p->Y.reserve((TB + d.B) * d.Hp * sizeof(half_t)));
+    FL_TRY(p->C.reserve((TB + d.B) * d.Hp * sizeof(float)));
+    FL_TRY(p->flags_f.reserve(size_t(p->Lf.ng) * 256 * sizeof(unsigned)));
+    if (p->epoch_f == 0 || p->epoch_f > 0x70000000u) {
+        FL_TRY(fill_zero(p->flags_f.p, p->flags_f.bytes, s));
+        p->epoch_f = 0;
+    }
+    // initial state rows
+    if (h0) FL_TRY(convert_pad(h0, state_dtype == FLSTM_F32, size_t(d.B), d.H, size_t(d.H), 1.f, p->Y.as<half_t>(),
+                               size_t(d.B), size_t(d.Hp), s));
+    else FL_TRY(fill_zero(p->Y.p, size_t(d.B) * d.Hp * sizeof(half_t), s));
+    FL_TRY(convert_pad_f32(c0, state_dtype == FLSTM_F32, size_t(d.B), d.H, 1.f, p->C.as<float>(), size_t(d.Hp), s));
+
+    FL_TRY(hipEventRecord(p->tm.ev[0], s));
+    // hoisted input projection, optionally in chunks of time steps
+    size_t chunk_steps = (p->opt_proj_chunk <= 0 || size_t(p->opt_proj_chunk) > T) ? T : size_t(p->opt_proj_chunk);
+    for (size_t t0 = 0; t0 < T; t0 += chunk_steps) {
+        const size_t steps = (t0 + chunk_steps <= T) ? chunk_steps : T - t0;
+        GemmNT g{};
+        g.A = A + t0 * d.B * lda; g.lda = lda;
+        g.B = p->wih_p.as<half_t>(); g.ldb = size_t(d.Ip);
+        g.M = int(steps * d.B); g.N = 4 * d.Hp; g.K = d.Ip;
+        g.C16 = p->G.as<half_t>() + t0 * d.B * 4 * d.Hp; g.C32 = nullptr; g.ldc = size_t(4) * d.Hp;
+        g.alpha = 1.f; g.splits = 1; g.split_stride = 0;
+        FL_TRY(launch_gemm_nt(g, s));
+    }
+    FL_TRY(hipEventRecord(p->tm.ev[1], s));
+    RecFwdArgs a{};
+    a.wfrag = p->wfrag_f.as<half8>();
+    a.Y = p->Y.as<half_t>(); a.G = p->G.as<half_t>(); a.C = p->C.as<float>();
+    a.bias = p->bias_p.as<float>();
+    a.flags = p->flags_f.as<unsigned>(); a.status = p->status.as<int>();
+    a.seats = p->status.as<unsigned>() + 8;
+    FL_TRY(fill_zero(a.seats, 8 * sizeof(unsigned), s));
+    a.B = d.B; a.Hp = d.Hp; a.T = int(T);
+    a.epoch = p->epoch_f; a.spin_limit = p->opt_spin_limit;
+    FL_TRY(launch_rec_fwd(p->Lf, a, s));
+    p->epoch_f += unsigned(T) + 1;
+    FL_TRY(hipEventRecord(p->tm.ev[2], s));
+    return 0;
+}
+
+}  // namespace
+
+extern "C" int flstm_core_forward(flstm_core_plan* p, size_t T, const void* x, flstm_dtype x_dtype,
+                                  const void* h0, const void* c0, flstm_dtype state_dtype, void* y,
+                                  flstm_dtype y_dtype, void* hy, void* cy, flstm_dtype out_state_dtype,
+                                  int save_for_backward, void* stream) {
+    if (!p) return FLSTM_E_INVALID;
+    if (!p->weights_packed || !p->bias_packed) return FLSTM_E_NOT_PACKED;
+    if (T == 0) return 0;
+    if (!x || T > (size_t(1) << 24)) return FLSTM_E_INVALID;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const Dims& d = p->d;
+    const size_t TB = T * size_t(d.B);
+    p->have_cache = false;
+
+    int rc = forward_once(p, T, x, x_dtype, h0, c0, state_dtype, s);
+    if (rc) return rc;
+    int st = 0;
+    rc = read_status(p, s, &st);
+    if (rc) return rc;
+    if (st != 0) {
+        if (!p->Lf.persistent) return FLSTM_E_STALLED;
+        // persistent launch gave up (workgroups not co-resident or not where expected): redo step-wise
+        p->broken_fwd = true;
+        p->fallbacks++;
+        replan(p);
+        FL_TRY(fill_zero(p->flags_f.p, p->flags_f.bytes, s));
+        p->epoch_f = 0;
+        rc = forward_once(p, T, x, x_dtype, h0, c0, state_dtype, s);
+        if (rc) return rc;
+        rc = read_status(p, s, &st);
+        if (rc) return rc;
+        if (st != 0) return FLSTM_E_STALLED;
+    }
+    p->ms_fwd[0] = elapsed(p->tm.ev[0], p->tm.ev[1]);
+    p->ms_fwd[1] = elapsed(p->tm.ev[1], p->tm.ev[2]);
+    p->ms_fwd[2] = elapsed(p->tm.ev[0], p->tm.ev[2]);
+
+    FL_TRY(unpad_from_half(p->Y.as<half_t>() + size_t(d.B) * d.Hp, size_t(d.Hp), TB, d.H, y, y_dtype == FLSTM_F32, s));
+    FL_TRY(unpad_from_half(p->Y.as<half_t>() + TB * d.Hp, size_t(d.Hp), size_t(d.B), d.H, hy,
+                           out_state_dtype == FLSTM_F32, s));
+    FL_TRY(unpad_from_float(p->C.as<float>() + TB * d.Hp, size_t(d.Hp), size_t(d.B), d.H, 1.f, cy,
+                            out_state_dtype == FLSTM_F32, s));
+    FL_TRY(hipStreamSynchronize(s));
+    if (save_for_backward) { p->have_cache = true; p->T_cache = T; }
+    return 0;
+}
+
+namespace {
+
+int backward_rec_once(flstm_core_plan* p, size_t T, const void* dY, flstm_dtype dy_dtype, const void* d_hn,
+                      const void* d_cn, flstm_dtype dstate_dtype, float S, hipStream_t s) {
+    const Dims& d = p->d;
+    const size_t TB = T * size_t(d.B);
+    const half_t* dYk = nullptr;
+    float dy_scale = S;
+    if (dy_dtype == FLSTM_F16 && d.H == d.Hp) {
+        dYk = static_cast<const half_t*>(dY);
+    } else {
+        FL_TRY(p->dYp.reserve(TB * d.Hp * sizeof(half_t)));
+        FL_TRY(convert_pad(dY, dy_dtype == FLSTM_F32, TB, d.H, size_t(d.H), S, p->dYp.as<half_t>(), TB,
+                           size_t(d.Hp), s));
+        dYk = p->dYp.as<half_t>();
+        dy_scale = 1.f;
+    }
+    const size_t st_bytes = size_t(d.B) * d.Hp * sizeof(float);
+    FL_TRY(p->dHn.reserve(st_bytes));
+    FL_TRY(p->dC.reserve(st_bytes));
+    FL_TRY(p->dH0.reserve(st_bytes));
+    FL_TRY(p->dG.reserve(TB * 4 * d.Hp * sizeof(half_t)));
+    FL_TRY(p->db_part.reserve(size_t(p->Lb.ng) * 4 * d.Hp * sizeof(float)));
+    FL_TRY(p->flags_b.reserve(size_t(p->Lb.ng) * 256 * sizeof(unsigned)));
+    if (p->epoch_b == 0 || p->epoch_b > 0x70000000u) {
+        FL_TRY(fill_zero(p->flags_b.p, p->flags_b.bytes, s));
+        p->epoch_b = 0;
+    }
+    FL_TRY(convert_pad_f32(d_hn, dstate_dtype == FLSTM_F32, size_t(d.B), d.H, S, p->dHn.as<float>(), size_t(d.Hp), s));
+    FL_TRY(convert_pad_f32(d_cn, dstate_dtype == FLSTM_F32, size_t(d.B), d.H, S, p->dC.as<float>(), size_t(d.Hp), s));
+    FL_TRY(fill_zero(p->db_part.p, size_t(p->Lb.ng) * 4 * d.Hp * sizeof(float), s));
+
+    FL_TRY(hipEventRecord(p->tm.ev[3], s));
+    RecBwdArgs a{};
+    a.wfrag = p->wfrag_b.as<half8>();
+    a.G = p->G.as<half_t>(); a.C = p->C.as<float>(); a.dY = dYk; a.dG = p->dG.as<half_t>();
+    a.dHn = p->dHn.as<float>(); a.dC = p->dC.as<float>(); a.dH0 = p->dH0.as<float>();
+    a.db_part = p->db_part.as<float>();
+    a.flags = p->flags_b.as<unsigned>(); a.status = p->status.as<int>();
+    a.seats = p->status.as<unsigned>() + 8;
+    FL_TRY(fill_zero(a.seats, 8 * sizeof(unsigned), s));
+    a.B = d.B; a.Hp = d.Hp; a.T = int(T); a.jb_fwd = d.JF; a.dy_scale = dy_scale;
+    a.epoch = p->epoch_b; a.spin_limit = p->opt_spin_limit;
+    FL_TRY(launch_rec_bwd(p->Lb, a, s));
+    p->epoch_b += unsigned(T) + 2;
+    FL_TRY(hipEventRecord(p->tm.ev[4], s));
+    return 0;
+}
+
+}  // namespace
+
+extern "C" int flstm_core_backward(flstm_core_plan* p, size_t T, const void* x, flstm_dtype x_dtype,
+                                   const void* dY, flstm_dtype dy_dtype, const void* d_hn, const void* d_cn,
+                                   flstm_dtype dstate_dtype, float grad_scale, void* dx, flstm_dtype dx_dtype,
+                                   float* dW_ih, float* dW_hh, float* db_ih, float* db_hh, float* dh0,
+                                   float* dc0, void* stream) {
+    if (!p) return FLSTM_E_INVALID;
+    if (T == 0) return 0;
+    if (!p->have_cache || p->T_cache != T) return FLSTM_E_NO_CACHE;
+    if (!dY) return FLSTM_E_INVALID;
+    if ((dW_ih || dW_hh) && !x) return FLSTM_E_INVALID;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const Dims& d = p->d;
+    const size_t TB = T * size_t(d.B);
+    const float S = grad_scale > 0.f ? grad_scale : 1.f;
+    const float invS = 1.f / S;
+
+    int rc = backward_rec_once(p, T, dY, dy_dtype, d_hn, d_cn, dstate_dtype, S, s);
+    if (rc) return rc;
+    int st = 0;
+    rc = read_status(p, s, &st);
+    if (rc) return rc;
+    if (st != 0) {
+        if (!p->Lb.persistent) return FLSTM_E_STALLED;
+        p->broken_bwd = true;
+        p->fallbacks++;
+        replan(p);
+        FL_TRY(fill_zero(p->flags_b.p, p->flags_b.bytes, s));
+        p->epoch_b = 0;
+        rc = backward_rec_once(p, T, dY, dy_dtype, d_hn, d_cn, dstate_dtype, S, s);
+        if (rc) return rc;
+        rc = read_status(p, s, &st);
+        if (rc) return rc;
+        if (st != 0) return FLSTM_E_STALLED;
+    }
+
+    // dX = dG * W_ih  (contraction over the packed gate columns)
+    if (dx) {
+        GemmNT g{};
+        g.A = p->dG.as<half_t>(); g.lda = size_t(4) * d.Hp;
+        g.B = p->wih_t.as<half_t>(); g.ldb = size_t(4) * d.Hp;
+        g.M = int(TB); g.N = d.I; g.K = 4 * d.Hp;
+        if (dx_dtype == FLSTM_F32) g.C32 = static_cast<float*>(dx); else g.C16 = static_cast<half_t*>(dx);
+        g.ldc = size_t(d.I); g.alpha = invS; g.splits = 1; g.split_stride = 0;
+        FL_TRY(launch_gemm_nt(g, s));
+    }
+    FL_TRY(hipEventRecord(p->tm.ev[5], s));
+
+    if (dW_ih || dW_hh) {
+        const size_t TBp = round_up(TB, 64);
+        const int ncat = d.Ip + d.Hp;
+        FL_TRY(p->dGT.reserve(size_t(4) * d.Hp * TBp * sizeof(half_t)));
+        FL_TRY(p->XHT.reserve(size_t(ncat) * TBp * sizeof(half_t)));
+        FL_TRY(transpose_pad(p->dG.p, 0, TB, 4 * d.Hp, size_t(4) * d.Hp, p->dGT.as<half_t>(), 4 * d.Hp, TBp, s));
+        FL_TRY(transpose_pad(x, x_dtype == FLSTM_F32, TB, d.I, size_t(d.I), p->XHT.as<half_t>(), d.Ip, TBp, s));
+        // H_prev of step t is row block t of the state array (row block 0 = h0)
+        FL_TRY(transpose_pad(p->Y.p, 0, TB, d.Hp, size_t(d.Hp), p->XHT.as<half_t>() + size_t(d.Ip) * TBp, d.Hp, TBp, s));
+        const int tiles = int(ceil_div(size_t(4) * d.Hp, 256) * ceil_div(size_t(ncat), 256));
+        int want = p->opt_dw_splits > 0 ? p->opt_dw_splits : int(ceil_div(1024, size_t(tiles)));
+        if (want > 64) want = 64;
+        const int splits = gemm_effective_splits(int(TBp), want);
+        const size_t per = size_t(4) * d.Hp * ncat;
+        FL_TRY(p->dw_part.reserve(per * splits * sizeof(float)));
+        GemmNT g{};
+        g.A = p->dGT.as<half_t>(); g.lda = TBp;
+        g.B = p->XHT.as<half_t>(); g.ldb = TBp;
+        g.M = 4 * d.Hp; g.N = ncat; g.K = int(TBp);
+        g.C16 = nullptr; g.C32 = p->dw_part.as<float>(); g.ldc = size_t(ncat);
+        g.alpha = 1.f; g.splits = splits; g.split_stride = per;
+        FL_TRY(launch_gemm_nt(g, s));
+        // a null output still needs a valid address for the kernel's other half: route to scratch
+        FL_TRY(reduce_dw(d, p->dw_part.as<float>(), splits, invS, dW_ih, dW_hh, s));
+    }
+    FL_TRY(hipEventRecord(p->tm.ev[6], s));
+    if (db_ih || db_hh) FL_TRY(reduce_db(d, p->db_part.as<float>(), p->Lb.ng, invS, db_ih, db_hh, s));
+    FL_TRY(unpad_from_float(p->dH0.as<float>(), size_t(d.Hp), size_t(d.B), d.H, invS, dh0, 1, s));
+    FL_TRY(unpad_from_float(p->dC.as<float>(), size_t(d.Hp), size_t(d.B), d.H, invS, dc0, 1, s));
+    FL_TRY(hipEventRecord(p->tm.ev[7], s));
+    FL_TRY(hipStreamSynchronize(s));
+    p->ms_bwd[0] = elapsed(p->tm.ev[3], p->tm.ev[4]);
+    p->ms_bwd[1] = elapsed(p->tm.ev[4], p->tm.ev[5]);
+    p->ms_bwd[2] = elapsed(p->tm.ev[5], p->tm.ev[6]);
+    p->ms_bwd[3] = elapsed(p->tm.ev[3], p->tm.ev[7]);
+    return 0;
+}
+
+extern "C" int flstm_core_cache_ptr(const flstm_core_plan* p, int which, const void** ptr, size_t* ld) {
+    if (!p || !ptr || !ld || !p->have_cache) return FLSTM_E_INVALID;
+    switch (which) {
+        case 0: *ptr = p->Y.p; *ld = size_t(p->d.Hp); return 0;
+        case 1: *ptr = p->C.p; *ld = size_t(p->d.Hp); return 0;
+        case 2: *ptr = p->G.p; *ld = size_t(4) * p->d.Hp; return 0;
+    }
+    return FLSTM_E_INVALID;
+}
+
+extern "C" double flstm_core_last_ms(const flstm_core_plan* p, const char* phase) {
+    if (!p || !phase) return -1.0;
+    if (!strcmp(phase, "fwd_proj")) return p->ms_fwd[0];
+    if (!strcmp(phase, "fwd_rec")) return p->ms_fwd[1];
+    if (!strcmp(phase, "fwd_total")) return p->ms_fwd[2];
+    if (!strcmp(phase, "bwd_rec")) return p->ms_bwd[0];
+    if (!strcmp(phase, "bwd_dx")) return p->ms_bwd[1];
+    if (!strcmp(phase, "bwd_dw")) return p->ms_bwd[2];
+    if (!strcmp(phase, "bwd_total")) return p->ms_bwd[3];
+    return -1.0;
+}

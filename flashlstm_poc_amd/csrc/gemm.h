@@ -1,0 +1,26 @@
+// fp16 x fp16 -> fp32-accumulate MFMA GEMM for gfx950, "NT" form: both operands K-contiguous.
+#pragma once
+#include "common.h"
+
+namespace flstm_hip {
+
+struct GemmNT {
+    // C[M][N] (+)= sum_k A[m][k] * B[n][k]
+    const half_t* A; size_t lda;   // M x K, row-major, lda multiple of 8
+    const half_t* B; size_t ldb;   // N x K, row-major, ldb multiple of 8
+    int M, N, K;                   // K multiple of 32
+    // output: exactly one of C16 / C32 is non-null
+    half_t* C16; float* C32; size_t ldc;
+    float alpha;                   // C = alpha * (A * B^T)
+    // split-K: when splits > 1 partial z is written to C32 + z * split_stride (fp32 only)
+    int splits; size_t split_stride;
+};
+
+// Enqueue on `stream`. Returns hipSuccess or the launch error.
+hipError_t launch_gemm_nt(const GemmNT& g, hipStream_t stream);
+
+// Number of K slices launch_gemm_nt really produces when `wanted` are asked for (every slice gets a
+// whole number of 64-wide K slabs). Size split-K partial buffers with this.
+int gemm_effective_splits(int K, int wanted);
+
+}  // namespace flstm_hip

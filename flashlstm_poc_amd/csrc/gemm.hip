@@ -1,0 +1,185 @@
+// LDS-staged fp16 MFMA GEMM for gfx950 (CDNA4), NT form: C[M][N] = A[M][K] * B[N][K]^T.
+//
+// This is the dense contraction behind the hoisted input projection X*W_ih^T (the reference does it
+// with a CUTLASS 128x128x32 tensor-op GEMM, src/lstm.cu:1204-1239, src/lstm_internal.h:48-68), the
+// input gradient dX = dG*W_ih and the weight gradients dW = dG^T*[X;H] (reference:
+// flashlstm_v2/src/lstm_backward.cu:1112-1172 through flashlstm_v2/src/gemm.cu:222-330).
+//
+// Tiling: one 256-thread workgroup (4 wavefronts, 2x2) owns a 256x256 tile of C; every wavefront
+// owns 128x128 as a 4x4 grid of v_mfma_f32_32x32x16_f16 tiles (256 accumulator registers).  K is
+// walked in slabs of 64: global -> registers -> LDS (row pitch padded to 72 halfs so that the
+// 16-byte fragment reads of 8 consecutive lanes fall in distinct banks), double buffered, one
+// workgroup barrier per slab.  Workgroups are numbered so that the 32 that share an XCD (block id
+// mod 8) work on neighbouring tiles and reuse each other's operand slabs in that XCD's L2.
+#include "gemm.h"
+
+namespace flstm_hip {
+namespace {
+
+constexpr int BM = 256, BN = 256, BK = 64;
+constexpr int LDS_LD = 72;  // halfs per LDS row (64 + 8 pad)
+constexpr int kThreads = 256;
+constexpr size_t kLdsBytes = size_t(2) * (BM + BN) * LDS_LD * sizeof(half_t);
+
+__global__ __launch_bounds__(kThreads) void gemm_nt_256x256(GemmNT g, int tiles_m, int tiles_n,
+                                                             int k_per_split) {
+    extern __shared__ __attribute__((aligned(16))) half_t smem[];
+    half_t* As = smem;                      // [2][BM][LDS_LD]
+    half_t* Bs = smem + 2 * BM * LDS_LD;    // [2][BN][LDS_LD]
+
+    const int ntiles = tiles_m * tiles_n;
+    const int per_xcd = (ntiles + 7) / 8;
+    const int tile = (blockIdx.x % 8) * per_xcd + blockIdx.x / 8;
+    if (tile >= ntiles) return;
+    const int tm = tile / tiles_n, tn = tile % tiles_n;
+    const int m0 = tm * BM, n0 = tn * BN;
+    const int z = blockIdx.y;
+    const int k_begin = z * k_per_split;
+    const int k_end = min(g.K, k_begin + k_per_split);
+    const int nslab = (k_end - k_begin) / BK;
+
+    const int tid = threadIdx.x, wave = tid / 64, lane = tid % 64;
+    const int wm = wave / 2, wn = wave % 2;
+
+    // Global->LDS staging: 16-byte chunk c = tid + 256*i covers row c/8, halfs [8*(c%8), +8).
+    const int ld_row = tid / 8, ld_kc = (tid % 8) * 8;
+    const half_t* a_src[8];
+    const half_t* b_src[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        const int ra = min(m0 + ld_row + 32 * i, g.M - 1);
+        const int rb = min(n0 + ld_row + 32 * i, g.N - 1);
+        a_src[i] = g.A + size_t(ra) * g.lda + k_begin + ld_kc;
+        b_src[i] = g.B + size_t(rb) * g.ldb + k_begin + ld_kc;
+    }
+    const int st_off = ld_row * LDS_LD + ld_kc;
+
+    floatx16 acc[4][4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
+
+    half8 ra[8], rb[8];
+    if (nslab > 0) {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) { ra[i] = ld_half8(a_src[i]); rb[i] = ld_half8(b_src[i]); }
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            st_half8(As + st_off + 32 * i * LDS_LD, ra[i]);
+            st_half8(Bs + st_off + 32 * i * LDS_LD, rb[i]);
+        }
+    }
+    __syncthreads();
+
+    const int a_frag_off = (wm * 128 + lane % 32) * LDS_LD + 8 * (lane / 32);
+    const int b_frag_off = (wn * 128 + lane % 32) * LDS_LD + 8 * (lane / 32);
+
+    for (int s = 0; s < nslab; ++s) {
+        const int cur = s & 1;
+        const bool more = (s + 1 < nslab);
+        if (more) {
+            const int koff = (s + 1) * BK;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                ra[i] = ld_half8(a_src[i] + koff);
+                rb[i] = ld_half8(b_src[i] + koff);
+            }
+        }
+        const half_t* Ac = As + cur * BM * LDS_LD + a_frag_off;
+        const half_t* Bc = Bs + cur * BN * LDS_LD + b_frag_off;
+#pragma unroll
+        for (int kk = 0; kk < BK / 16; ++kk) {
+            half8 af[4], bf[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                af[i] = *reinterpret_cast<const half8*>(Ac + i * 32 * LDS_LD + kk * 16);
+                bf[i] = *reinterpret_cast<const half8*>(Bc + i * 32 * LDS_LD + kk * 16);
+            }
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+#pragma unroll
+                for (int j = 0; j < 4; ++j)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[i], bf[j], acc[i][j], 0, 0, 0);
+        }
+        if (more) {
+            half_t* An = As + (cur ^ 1) * BM * LDS_LD + st_off;
+            half_t* Bn = Bs + (cur ^ 1) * BN * LDS_LD + st_off;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                st_half8(An + 32 * i * LDS_LD, ra[i]);
+                st_half8(Bn + 32 * i * LDS_LD, rb[i]);
+            }
+        }
+        __syncthreads();
+    }
+
+    // Epilogue. Accumulator register r of a 32x32 tile holds row 8*(r/4) + 4*(lane/32) + r%4,
+    // column lane%32.
+    const int col_l = lane % 32;
+    const int row_l = 4 * (lane / 32);
+    float* c32 = g.C32 ? g.C32 + size_t(z) * g.split_stride : nullptr;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int col = n0 + wn * 128 + j * 32 + col_l;
+            if (col >= g.N) continue;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int row = m0 + wm * 128 + i * 32 + 8 * (r / 4) + row_l + (r % 4);
+                if (row >= g.M) continue;
+                const size_t off = size_t(row) * g.ldc + col;
+                const float v = g.alpha * acc[i][j][r];
+                if (c32) c32[off] = v;
+                else g.C16[off] = (half_t)v;
+            }
+        }
+    }
+}
+
+}  // namespace
+
+hipError_t launch_gemm_nt(const GemmNT& g, hipStream_t stream) {
+    if (g.M <= 0 || g.N <= 0 || g.K <= 0) return hipSuccess;
+    if (g.K % BK != 0 || g.lda % 8 != 0 || g.ldb % 8 != 0) return hipErrorInvalidValue;
+    if ((g.C16 == nullptr) == (g.C32 == nullptr)) return hipErrorInvalidValue;
+    int splits = g.splits < 1 ? 1 : g.splits;
+    if (splits > 1 && g.C32 == nullptr) return hipErrorInvalidValue;
+    const int nslab = g.K / BK;
+    if (splits > nslab) splits = nslab;
+    const int slabs_per_split = (nslab + splits - 1) / splits;
+    splits = (nslab + slabs_per_split - 1) / slabs_per_split;
+    if (splits != (g.splits < 1 ? 1 : g.splits) && g.splits > 1) {
+        // The caller sized its partial buffer for g.splits slices; fewer are produced, so the unused
+        // ones must read as zero.  Callers use gemm_effective_splits() to avoid this path.
+        return hipErrorInvalidValue;
+    }
+    static bool attr_set = false;
+    if (!attr_set) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_nt_256x256),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, int(kLdsBytes));
+        if (e != hipSuccess) return e;
+        attr_set = true;
+    }
+    const int tiles_m = (g.M + BM - 1) / BM, tiles_n = (g.N + BN - 1) / BN;
+    const int ntiles = tiles_m * tiles_n;
+    const int per_xcd = (ntiles + 7) / 8;
+    dim3 grid(per_xcd * 8, splits, 1);
+    hipLaunchKernelGGL(gemm_nt_256x256, grid, dim3(kThreads), kLdsBytes, stream, g, tiles_m, tiles_n,
+                       slabs_per_split * BK);
+    return hipGetLastError();
+}
+
+int gemm_effective_splits(int K, int wanted) {
+    const int nslab = K / BK;
+    if (wanted < 1) wanted = 1;
+    if (wanted > nslab) wanted = nslab;
+    if (wanted < 1) wanted = 1;
+    const int per = (nslab + wanted - 1) / wanted;
+    return (nslab + per - 1) / per;
+}
+
+}  // namespace flstm_hip

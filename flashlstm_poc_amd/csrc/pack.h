@@ -1,0 +1,60 @@
+// Layout kernels around the GEMMs and the recurrence: weight packing, dtype conversion with
+// padding, transposes, and the reductions that turn scaled/padded internals into caller tensors.
+#pragma once
+#include "common.h"
+
+namespace flstm_hip {
+
+// Packed gate order: hidden units are cut into slices of JF; slice s holds its i,f,g,o rows next to
+// each other:  q = (j / JF) * 4JF + gate * JF + j % JF.   PyTorch row of (gate, j) is gate*H + j.
+struct Dims {
+    int B, I, H;     // caller sizes
+    int Ip, Hp;      // I rounded up to 64, H rounded up to 32
+    int JF;          // slice width of the packed gate order
+};
+
+// Replaces src/kernels.cu:57-84 (pack_weights_kernel) and :45-55 (combine_bias_kernel): fp32
+// PyTorch-layout weights -> the fp16 operand layouts of the kernels in this library.
+hipError_t pack_weights(const Dims& d, const float* w_ih, const float* w_hh, half_t* wih_p /*[4Hp][Ip]*/,
+                        half_t* wih_t /*[Ip][4Hp]*/, half8* wfrag_fwd, int ks_fwd, int nt_fwd,
+                        half8* wfrag_bwd, int ks_bwd, int nt_bwd, hipStream_t s);
+hipError_t pack_bias(const Dims& d, const float* b_ih, const float* b_hh, float* bias_p, hipStream_t s);
+
+// rows x cols (ld_in, fp32 when in_f32 else fp16) -> fp16 [rows_out][ld_out], zero padded.
+// Replaces src/kernels.cu:5-43 (populate_activations_kernel).
+hipError_t convert_pad(const void* in, int in_f32, size_t rows, int cols, size_t ld_in, float scale,
+                       half_t* out, size_t rows_out, size_t ld_out, hipStream_t s);
+// fp16/fp32 (rows x cols) -> fp32 [rows][ld_out] zero padded, scaled; null input -> zeros.
+hipError_t convert_pad_f32(const void* in, int in_f32, size_t rows, int cols, float scale, float* out,
+                           size_t ld_out, hipStream_t s);
+// padded internals -> caller tensors: out[r][c] = scale * in[r][c], c < cols.
+hipError_t unpad_from_half(const half_t* in, size_t ld_in, size_t rows, int cols, void* out, int out_f32,
+                           hipStream_t s);
+hipError_t unpad_from_float(const float* in, size_t ld_in, size_t rows, int cols, float scale, void* out,
+                            int out_f32, hipStream_t s);
+
+// Row-block gather: output row r is input row (r / rows_per_block) * block_stride + r % rows_per_block.
+// Used to pull the pre-step states at every R-th step out of the state arrays (the h/c checkpoints
+// of flashlstm_v2/src/lstm_forward.cu:727-783).
+hipError_t gather_from_half(const half_t* in, size_t ld_in, size_t rows, int cols, void* out, int out_f32,
+                            size_t rows_per_block, size_t block_stride, hipStream_t s);
+hipError_t gather_from_float(const float* in, size_t ld_in, size_t rows, int cols, float scale, void* out,
+                             int out_f32, size_t rows_per_block, size_t block_stride, hipStream_t s);
+
+// out[c][r] = in[r][c] for r < rows, c < cols; out rows are ld_out long, columns [rows, ld_out) are
+// zeroed; output rows [cols, cols_out) are zeroed as well.
+hipError_t transpose_pad(const void* in, int in_f32, size_t rows, int cols, size_t ld_in, half_t* out,
+                         int cols_out, size_t ld_out, hipStream_t s);
+
+// Sums split-K partials [splits][4Hp][Ip+Hp] (packed gate rows) into dW_ih (4H x I) and
+// dW_hh (4H x H), PyTorch layout, times `scale`.  Replaces the beta=1 accumulation of
+// flashlstm_v2/src/lstm_backward.cu:1112-1142.
+hipError_t reduce_dw(const Dims& d, const float* partial, int splits, float scale, float* dw_ih,
+                     float* dw_hh, hipStream_t s);
+// db_part [ng][4Hp] packed -> db_ih == db_hh (4H), times scale (flashlstm_v2/src/lstm_backward.cu:1218-1231).
+hipError_t reduce_db(const Dims& d, const float* db_part, int ng, float scale, float* db_ih, float* db_hh,
+                     hipStream_t s);
+
+hipError_t fill_zero(void* p, size_t bytes, hipStream_t s);
+
+}  // namespace flstm_hip

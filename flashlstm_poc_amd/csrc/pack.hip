@@ -1,0 +1,307 @@
+// Layout kernels: weight packing, padded dtype conversion, transposes and output reductions.
+// All are pure HBM-bandwidth work; each thread moves a few elements with coalesced accesses.
+#include "pack.h"
+
+namespace flstm_hip {
+namespace {
+
+constexpr int kT = 256;
+
+__host__ __device__ inline int grid_for(size_t n) { return int((n + kT - 1) / kT); }
+
+// packed gate column -> PyTorch weight row, or -1 for a padding unit
+__device__ __forceinline__ int torch_row(int q, int JF, int H) {
+    const int blk = q / (4 * JF), rem = q % (4 * JF);
+    const int gate = rem / JF, j = blk * JF + rem % JF;
+    return j < H ? gate * H + j : -1;
+}
+
+__global__ void pack_wih_kernel(Dims d, const float* __restrict__ w_ih, half_t* __restrict__ wih_p,
+                                half_t* __restrict__ wih_t) {
+    const size_t idx = size_t(blockIdx.x) * kT + threadIdx.x;
+    const size_t total = size_t(4) * d.Hp * d.Ip;
+    if (idx >= total) return;
+    const int q = int(idx / d.Ip), i = int(idx % d.Ip);
+    const int row = torch_row(q, d.JF, d.H);
+    const float v = (row >= 0 && i < d.I) ? w_ih[size_t(row) * d.I + i] : 0.f;
+    wih_p[idx] = (half_t)v;
+    wih_t[size_t(i) * 4 * d.Hp + q] = (half_t)v;
+}
+
+// Forward fragments: B operand of  gates[b][q] += h[b][k] * W_hh[row(q)][k].
+// fragment (hs, wave, ks, n): lane l holds column q = hs*16*NT + n*16 + l%16,
+// k = (ks*4 + wave)*32 + 8*(l/16) + e, e = 0..7.
+__global__ void pack_wfrag_fwd_kernel(Dims d, const float* __restrict__ w_hh, half_t* __restrict__ out,
+                                      int ks_wave, int nt) {
+    const size_t idx = size_t(blockIdx.x) * kT + threadIdx.x;  // one half element
+    const int nh = d.Hp / (4 * nt);
+    const size_t total = size_t(nh) * 4 * ks_wave * nt * kWave * 8;
+    if (idx >= total) return;
+    size_t r = idx;
+    const int e = int(r % 8); r /= 8;
+    const int lane = int(r % kWave); r /= kWave;
+    const int n = int(r % nt); r /= nt;
+    const int ks = int(r % ks_wave); r /= ks_wave;
+    const int wave = int(r % 4); r /= 4;
+    const int hs = int(r);
+    const int q = hs * 16 * nt + n * 16 + lane % 16;
+    const int k = (ks * 4 + wave) * 32 + 8 * (lane / 16) + e;
+    const int row = torch_row(q, d.JF, d.H);
+    out[idx] = (half_t)((row >= 0 && k < d.H) ? w_hh[size_t(row) * d.H + k] : 0.f);
+}
+
+// Backward fragments: B operand of  dh[b][k] += dG[b][q] * W_hh[row(q)][k].
+// fragment (hs, wave, ks, n): lane l holds output column k = hs*16*NT + n*16 + l%16,
+// contraction index q = (ks*4 + wave)*32 + 8*(l/16) + e.
+__global__ void pack_wfrag_bwd_kernel(Dims d, const float* __restrict__ w_hh, half_t* __restrict__ out,
+                                      int ks_wave, int nt) {
+    const size_t idx = size_t(blockIdx.x) * kT + threadIdx.x;
+    const int nh = d.Hp / (16 * nt);
+    const size_t total = size_t(nh) * 4 * ks_wave * nt * kWave * 8;
+    if (idx >= total) return;
+    size_t r = idx;
+    const int e = int(r % 8); r /= 8;
+    const int lane = int(r % kWave); r /= kWave;
+    const int n = int(r % nt); r /= nt;
+    const int ks = int(r % ks_wave); r /= ks_wave;
+    const int wave = int(r % 4); r /= 4;
+    const int hs = int(r);
+    const int k = hs * 16 * nt + n * 16 + lane % 16;
+    const int q = (ks * 4 + wave) * 32 + 8 * (lane / 16) + e;
+    float v = 0.f;
+    if (q < 4 * d.Hp && k < d.H) {
+        const int row = torch_row(q, d.JF, d.H);
+        if (row >= 0) v = w_hh[size_t(row) * d.H + k];
+    }
+    out[idx] = (half_t)v;
+}
+
+__global__ void pack_bias_kernel(Dims d, const float* __restrict__ b_ih, const float* __restrict__ b_hh,
+                                 float* __restrict__ out) {
+    const int q = blockIdx.x * kT + threadIdx.x;
+    if (q >= 4 * d.Hp) return;
+    const int row = torch_row(q, d.JF, d.H);
+    out[q] = row >= 0 ? b_ih[row] + b_hh[row] : 0.f;
+}
+
+template <typename TIn>
+__global__ void convert_pad_kernel(const TIn* __restrict__ in, size_t rows, int cols, size_t ld_in,
+                                   float scale, half_t* __restrict__ out, size_t rows_out, size_t ld_out) {
+    const size_t idx = size_t(blockIdx.x) * kT + threadIdx.x;
+    if (idx >= rows_out * ld_out) return;
+    const size_t r = idx / ld_out;
+    const int c = int(idx % ld_out);
+    float v = 0.f;
+    if (r < rows && c < cols) v = scale * (float)in[r * ld_in + c];
+    out[idx] = (half_t)v;
+}
+
+template <typename TIn>
+__global__ void convert_pad_f32_kernel(const TIn* __restrict__ in, size_t rows, int cols, float scale,
+                                       float* __restrict__ out, size_t ld_out) {
+    const size_t idx = size_t(blockIdx.x) * kT + threadIdx.x;
+    if (idx >= rows * ld_out) return;
+    const size_t r = idx / ld_out;
+    const int c = int(idx % ld_out);
+    float v = 0.f;
+    if (in != nullptr && c < cols) v = scale * (float)in[r * cols + c];
+    out[idx] = v;
+}
+
+// Output row r comes from input row (r / rows_per_block) * block_stride + r % rows_per_block.
+template <typename TIn, typename TOut>
+__global__ void unpad_kernel(const TIn* __restrict__ in, size_t ld_in, size_t rows, int cols, float scale,
+                             TOut* __restrict__ out, size_t rows_per_block, size_t block_stride) {
+    const size_t idx = size_t(blockIdx.x) * kT + threadIdx.x;
+    if (idx >= rows * size_t(cols)) return;
+    const size_t r = idx / cols;
+    const int c = int(idx % cols);
+    const size_t rin = (r / rows_per_block) * block_stride + r % rows_per_block;
+    out[idx] = (TOut)(scale * (float)in[rin * ld_in + c]);
+}
+
+// 64x64 tile transpose through LDS.
+template <typename TIn>
+__global__ void transpose_pad_kernel(const TIn* __restrict__ in, size_t rows, int cols, size_t ld_in,
+                                     half_t* __restrict__ out, int cols_out, size_t ld_out) {
+    __shared__ half_t tile[64][66];
+    const size_t r0 = size_t(blockIdx.x) * 64;
+    const int c0 = blockIdx.y * 64;
+    const int tx = threadIdx.x % 64, ty = threadIdx.x / 64;  // 4 rows of 64 threads
+    for (int i = ty; i < 64; i += 4) {
+        const size_t r = r0 + i;
+        const int c = c0 + tx;
+        float v = 0.f;
+        if (r < rows && c < cols) v = (float)in[r * ld_in + c];
+        tile[i][tx] = (half_t)v;
+    }
+    __syncthreads();
+    for (int i = ty; i < 64; i += 4) {
+        const int c = c0 + i;       // output row
+        const size_t r = r0 + tx;   // output column
+        if (c < cols_out && r < ld_out) out[size_t(c) * ld_out + r] = tile[tx][i];
+    }
+}
+
+__global__ void reduce_dw_kernel(Dims d, const float* __restrict__ partial, int splits, float scale,
+                                 float* __restrict__ dw_ih, float* __restrict__ dw_hh) {
+    const int ncat = d.Ip + d.Hp;
+    const size_t idx = size_t(blockIdx.x) * kT + threadIdx.x;
+    const size_t per = size_t(4) * d.Hp * ncat;
+    if (idx >= per) return;
+    const int q = int(idx / ncat), n = int(idx % ncat);
+    const int row = torch_row(q, d.JF, d.H);
+    if (row < 0) return;
+    float* dst;
+    if (n < d.Ip) {
+        if (n >= d.I || dw_ih == nullptr) return;
+        dst = dw_ih + size_t(row) * d.I + n;
+    } else {
+        const int k = n - d.Ip;
+        if (k >= d.H || dw_hh == nullptr) return;
+        dst = dw_hh + size_t(row) * d.H + k;
+    }
+    float s = 0.f;
+    for (int z = 0; z < splits; ++z) s += partial[size_t(z) * per + idx];
+    *dst = scale * s;
+}
+
+__global__ void reduce_db_kernel(Dims d, const float* __restrict__ db_part, int ng, float scale,
+                                 float* __restrict__ db_ih, float* __restrict__ db_hh) {
+    const int q = blockIdx.x * kT + threadIdx.x;
+    if (q >= 4 * d.Hp) return;
+    const int row = torch_row(q, d.JF, d.H);
+    if (row < 0) return;
+    float s = 0.f;
+    for (int g = 0; g < ng; ++g) s += db_part[size_t(g) * 4 * d.Hp + q];
+    s *= scale;
+    if (db_ih) db_ih[row] = s;
+    if (db_hh) db_hh[row] = s;
+}
+
+__global__ void fill_zero_kernel(unsigned* p, size_t words) {
+    const size_t stride = size_t(gridDim.x) * kT;
+    for (size_t i = size_t(blockIdx.x) * kT + threadIdx.x; i < words; i += stride) p[i] = 0u;
+}
+
+}  // namespace
+
+hipError_t pack_weights(const Dims& d, const float* w_ih, const float* w_hh, half_t* wih_p, half_t* wih_t,
+                        half8* wfrag_fwd, int ks_fwd, int nt_fwd, half8* wfrag_bwd, int ks_bwd, int nt_bwd,
+                        hipStream_t s) {
+    const size_t n1 = size_t(4) * d.Hp * d.Ip;
+    hipLaunchKernelGGL(pack_wih_kernel, dim3(grid_for(n1)), dim3(kT), 0, s, d, w_ih, wih_p, wih_t);
+    const size_t n2 = size_t(d.Hp / (4 * nt_fwd)) * 4 * ks_fwd * nt_fwd * kWave * 8;
+    hipLaunchKernelGGL(pack_wfrag_fwd_kernel, dim3(grid_for(n2)), dim3(kT), 0, s, d, w_hh,
+                       reinterpret_cast<half_t*>(wfrag_fwd), ks_fwd, nt_fwd);
+    const size_t n3 = size_t(d.Hp / (16 * nt_bwd)) * 4 * ks_bwd * nt_bwd * kWave * 8;
+    hipLaunchKernelGGL(pack_wfrag_bwd_kernel, dim3(grid_for(n3)), dim3(kT), 0, s, d, w_hh,
+                       reinterpret_cast<half_t*>(wfrag_bwd), ks_bwd, nt_bwd);
+    return hipGetLastError();
+}
+
+hipError_t pack_bias(const Dims& d, const float* b_ih, const float* b_hh, float* bias_p, hipStream_t s) {
+    hipLaunchKernelGGL(pack_bias_kernel, dim3(grid_for(size_t(4) * d.Hp)), dim3(kT), 0, s, d, b_ih, b_hh, bias_p);
+    return hipGetLastError();
+}
+
+hipError_t convert_pad(const void* in, int in_f32, size_t rows, int cols, size_t ld_in, float scale,
+                       half_t* out, size_t rows_out, size_t ld_out, hipStream_t s) {
+    const size_t n = rows_out * ld_out;
+    if (n == 0) return hipSuccess;
+    if (in_f32)
+        hipLaunchKernelGGL(convert_pad_kernel<float>, dim3(grid_for(n)), dim3(kT), 0, s,
+                           static_cast<const float*>(in), rows, cols, ld_in, scale, out, rows_out, ld_out);
+    else
+        hipLaunchKernelGGL(convert_pad_kernel<half_t>, dim3(grid_for(n)), dim3(kT), 0, s,
+                           static_cast<const half_t*>(in), rows, cols, ld_in, scale, out, rows_out, ld_out);
+    return hipGetLastError();
+}
+
+hipError_t convert_pad_f32(const void* in, int in_f32, size_t rows, int cols, float scale, float* out,
+                           size_t ld_out, hipStream_t s) {
+    const size_t n = rows * ld_out;
+    if (n == 0) return hipSuccess;
+    if (in_f32)
+        hipLaunchKernelGGL(convert_pad_f32_kernel<float>, dim3(grid_for(n)), dim3(kT), 0, s,
+                           static_cast<const float*>(in), rows, cols, scale, out, ld_out);
+    else
+        hipLaunchKernelGGL(convert_pad_f32_kernel<half_t>, dim3(grid_for(n)), dim3(kT), 0, s,
+                           static_cast<const half_t*>(in), rows, cols, scale, out, ld_out);
+    return hipGetLastError();
+}
+
+hipError_t gather_from_half(const half_t* in, size_t ld_in, size_t rows, int cols, void* out, int out_f32,
+                            size_t rows_per_block, size_t block_stride, hipStream_t s) {
+    const size_t n = rows * size_t(cols);
+    if (n == 0 || out == nullptr) return hipSuccess;
+    if (out_f32)
+        hipLaunchKernelGGL((unpad_kernel<half_t, float>), dim3(grid_for(n)), dim3(kT), 0, s, in, ld_in, rows,
+                           cols, 1.f, static_cast<float*>(out), rows_per_block, block_stride);
+    else
+        hipLaunchKernelGGL((unpad_kernel<half_t, half_t>), dim3(grid_for(n)), dim3(kT), 0, s, in, ld_in, rows,
+                           cols, 1.f, static_cast<half_t*>(out), rows_per_block, block_stride);
+    return hipGetLastError();
+}
+
+hipError_t gather_from_float(const float* in, size_t ld_in, size_t rows, int cols, float scale, void* out,
+                             int out_f32, size_t rows_per_block, size_t block_stride, hipStream_t s) {
+    const size_t n = rows * size_t(cols);
+    if (n == 0 || out == nullptr) return hipSuccess;
+    if (out_f32)
+        hipLaunchKernelGGL((unpad_kernel<float, float>), dim3(grid_for(n)), dim3(kT), 0, s, in, ld_in, rows,
+                           cols, scale, static_cast<float*>(out), rows_per_block, block_stride);
+    else
+        hipLaunchKernelGGL((unpad_kernel<float, half_t>), dim3(grid_for(n)), dim3(kT), 0, s, in, ld_in, rows,
+                           cols, scale, static_cast<half_t*>(out), rows_per_block, block_stride);
+    return hipGetLastError();
+}
+
+hipError_t unpad_from_half(const half_t* in, size_t ld_in, size_t rows, int cols, void* out, int out_f32,
+                           hipStream_t s) {
+    return gather_from_half(in, ld_in, rows, cols, out, out_f32, rows ? rows : 1, 0, s);
+}
+
+hipError_t unpad_from_float(const float* in, size_t ld_in, size_t rows, int cols, float scale, void* out,
+                            int out_f32, hipStream_t s) {
+    return gather_from_float(in, ld_in, rows, cols, scale, out, out_f32, rows ? rows : 1, 0, s);
+}
+
+hipError_t transpose_pad(const void* in, int in_f32, size_t rows, int cols, size_t ld_in, half_t* out,
+                         int cols_out, size_t ld_out, hipStream_t s) {
+    if (cols_out == 0 || ld_out == 0) return hipSuccess;
+    dim3 grid(unsigned(ceil_div(ld_out, 64)), unsigned(ceil_div(size_t(cols_out), 64)));
+    if (in_f32)
+        hipLaunchKernelGGL(transpose_pad_kernel<float>, grid, dim3(kT), 0, s, static_cast<const float*>(in),
+                           rows, cols, ld_in, out, cols_out, ld_out);
+    else
+        hipLaunchKernelGGL(transpose_pad_kernel<half_t>, grid, dim3(kT), 0, s, static_cast<const half_t*>(in),
+                           rows, cols, ld_in, out, cols_out, ld_out);
+    return hipGetLastError();
+}
+
+hipError_t reduce_dw(const Dims& d, const float* partial, int splits, float scale, float* dw_ih, float* dw_hh,
+                     hipStream_t s) {
+    const size_t per = size_t(4) * d.Hp * (d.Ip + d.Hp);
+    hipLaunchKernelGGL(reduce_dw_kernel, dim3(grid_for(per)), dim3(kT), 0, s, d, partial, splits, scale, dw_ih,
+                       dw_hh);
+    return hipGetLastError();
+}
+
+hipError_t reduce_db(const Dims& d, const float* db_part, int ng, float scale, float* db_ih, float* db_hh,
+                     hipStream_t s) {
+    hipLaunchKernelGGL(reduce_db_kernel, dim3(grid_for(size_t(4) * d.Hp)), dim3(kT), 0, s, d, db_part, ng,
+                       scale, db_ih, db_hh);
+    return hipGetLastError();
+}
+
+hipError_t fill_zero(void* p, size_t bytes, hipStream_t s) {
+    if (bytes == 0) return hipSuccess;
+    const size_t words = bytes / 4;  // all buffers of this library are multiples of 4 bytes
+    int blocks = grid_for(words);
+    if (blocks > 4096) blocks = 4096;
+    hipLaunchKernelGGL(fill_zero_kernel, dim3(blocks), dim3(kT), 0, s, static_cast<unsigned*>(p), words);
+    return hipGetLastError();
+}
+
+}  // namespace flstm_hip

@@ -1,0 +1,69 @@
+// Persistent, W_hh-resident recurrence kernels (forward and BPTT) for gfx950.
+#pragma once
+#include "common.h"
+
+namespace flstm_hip {
+
+// How the hidden dimension is cut over workgroups, and how workgroups are tied into groups that
+// exchange h_t (forward) or dG_t (backward) every step.
+struct RecLayout {
+    int nt;          // forward: 16-wide gate-column tiles per workgroup (JB = 4*nt hidden units)
+    int jb;          // hidden units per workgroup slice
+    int nh;          // slices = Hp / jb  (workgroups per group)
+    int nrb;         // 32-row batch blocks
+    int ng;          // concurrently running groups; group g owns row blocks g, g+ng, ...
+    int gpx;         // XCD-local mode: groups per XCD
+    int xcd_local;   // 1: every group lives inside one XCD (plain stores + L2-served loads)
+    int persistent;  // 1: one launch walks all steps, 0: one launch per step
+    int resident;    // 1: weight fragments live in registers for the whole launch
+    int grid;        // workgroups per launch
+};
+
+struct RecFwdArgs {
+    const half8* wfrag;  // [nh][4 waves][ks][nt][64 lanes] MFMA B-fragments of W_hh (packed gate order)
+    half_t* Y;           // [(T+1)*B + pad][Hp]; rows [0,B) = h0, rows [(t+1)B, (t+2)B) = h_t
+    half_t* G;           // [T*B][4Hp] packed gate order; in: x-projection, out: activated i,f,g,o
+    float* C;            // [(T+1)*B][Hp]; rows [0,B) = c0, rows [(t+1)B, ..) = c_t
+    const float* bias;   // [4Hp] packed gate order, b_ih + b_hh
+    unsigned* flags;     // [ng][256]
+    unsigned* seats;     // [8] zeroed before every launch: next free workgroup slot per XCD
+    int* status;         // 0 ok, 1 spin limit hit, 2 workgroup not on the expected XCD
+    int B, Hp, T;
+    unsigned epoch;
+    int spin_limit;
+};
+
+struct RecBwdArgs {
+    const half8* wfrag;  // [nh][4 waves][ks][nt][64] B-fragments of W_hh^T (rows = hidden k, contraction = packed gate q)
+    const half_t* G;     // activated gates cache [T*B][4Hp]
+    const float* C;      // cell states [(T+1)*B][Hp]
+    const half_t* dY;    // [T*B][Hp] upstream gradient
+    half_t* dG;          // [T*B + pad][4Hp] pre-activation gradients (scaled by grad_scale)
+    float* dHn;          // [B][Hp] scaled gradient wrt final h (zeros when absent)
+    float* dC;           // [B][Hp] running scaled dc; in: gradient wrt final c, out: dc0
+    float* dH0;          // [B][Hp] out: scaled gradient wrt h0
+    float* db_part;      // [ng][4Hp] scaled bias-gradient partial sums (accumulated into)
+    unsigned* flags;     // [ng][256]
+    unsigned* seats;     // [8] zeroed before every launch
+    int* status;
+    int B, Hp, T;
+    int jb_fwd;          // hidden units per slice in the packed gate order of G / dG
+    float dy_scale;      // factor applied to dY on load (the loss scale, or 1 when dY is pre-scaled)
+    unsigned epoch;
+    int spin_limit;
+};
+
+// Picks tile shapes and the group structure for a problem size on the current device.
+RecLayout plan_rec_fwd(int B, int Hp, int num_cus, bool force_stepwise);
+RecLayout plan_rec_bwd(int B, int Hp, int num_cus, bool force_stepwise);
+
+// Number of k-steps (32 wide) every wave holds for a layout (sizes the fragment arrays).
+int rec_fwd_ks(const RecLayout& L, int Hp);
+int rec_bwd_ks(const RecLayout& L, int Hp);
+
+// Runs steps [0, T). Persistent layouts use one launch; otherwise one launch per step.
+hipError_t launch_rec_fwd(const RecLayout& L, const RecFwdArgs& a, hipStream_t stream);
+// Runs steps T-1 .. 0 and the final dh0 product.
+hipError_t launch_rec_bwd(const RecLayout& L, const RecBwdArgs& a, hipStream_t stream);
+
+}  // namespace flstm_hip

@@ -1,0 +1,546 @@
+// Persistent W_hh-resident LSTM recurrence for gfx950: forward and backward-through-time.
+//
+// What the reference does per time step with a CUTLASS GEMM launch plus a pointwise launch
+// (forward: src/lstm.cu:1241-1339 + src/kernels.cu:86-164; backward:
+// flashlstm_v2/src/lstm_backward.cu:1057-1101 + :158-227) is done here by ONE kernel launch for
+// the whole sequence:
+//
+//  * Work split.  The batch is cut into blocks of 32 rows and the hidden dimension into slices of
+//    JB units.  A workgroup (4 wavefronts, one per SIMD, up to 512 registers each) owns one slice
+//    for all row blocks of its group, i.e. all four gates of its hidden units, so the cell update
+//    is local.  Its part of W_hh (forward: 4*JB gate rows x Hp; backward: 4Hp gate rows x JB
+//    columns) is loaded once into registers as ready-made MFMA B-fragments and stays there.
+//  * K split.  The four wavefronts split the contraction dimension (interleaved 32-wide k-steps),
+//    so every element of h_{t-1} / dG_{t+1} is fetched exactly once per workgroup, straight from
+//    L2 into A-fragments; partial sums meet in LDS (fp32) and the pointwise stage reads them there.
+//  * Exchange.  h_t (forward) and dG_t (backward) are the only data that cross workgroups.  Groups
+//    are laid out so that all workgroups of a group sit on one XCD when the slice count allows
+//    (block id mod 8 is the XCD): producers use plain write-through stores, consumers fetch with
+//    device-scope relaxed atomic loads (L1 bypass, served by that XCD's L2), and a per-workgroup
+//    step flag in one cache line replaces the grid barrier -- no L2 write-back or invalidate is
+//    ever issued.  Groups that span XCDs store the exchanged values with device-scope atomic
+//    stores instead.  Every wait is bounded and reports through `status`.
+//  * Fallback.  The same kernels launched once per step (no waits, kernel boundaries order
+//    memory) serve shapes whose weights do not fit on chip, and are the safe path after a failed
+//    persistent launch.
+#include "recurrent.h"
+
+namespace flstm_hip {
+namespace {
+
+constexpr int kThreads = 256;
+constexpr int kRows = 32;  // batch rows per row block
+
+__device__ __forceinline__ unsigned xcc_id() {
+    unsigned v;
+    asm volatile("s_getreg_b32 %0, hwreg(HW_REG_XCC_ID)" : "=s"(v));
+    return v & 0xf;
+}
+
+struct Role {
+    int g, hs;
+    bool active;
+};
+
+// XCD-local mode: the hardware deals workgroups round-robin over the 8 XCDs, but where a launch
+// starts in that rotation depends on what ran before, so a workgroup takes its XCD from the
+// hardware register and claims the next free slot of that XCD.  A ninth... 33rd arrival on one XCD
+// (uneven placement) cannot be seated: it reports status 2 and the host repeats the work step-wise.
+__device__ __forceinline__ Role make_role(int nh, int ng, int gpx, int xcd_local, unsigned* seats,
+                                          int* status, int* lds_role) {
+    Role r;
+    const int w = blockIdx.x;
+    if (xcd_local) {
+        if (threadIdx.x == 0) {
+            const int xcd = int(xcc_id()) & 7;
+            const unsigned slot = __hip_atomic_fetch_add(seats + xcd, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            if (slot >= 32u) __hip_atomic_store(status, 2, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            lds_role[0] = xcd;
+            lds_role[1] = int(slot);
+        }
+        __syncthreads();
+        const int xcd = lds_role[0], slot = lds_role[1];
+        const int sub = slot / nh;
+        r.hs = slot % nh;
+        r.g = sub * 8 + xcd;
+        r.active = (slot < 32) && (sub < gpx) && (r.g < ng);
+    } else {
+        r.g = w / nh;
+        r.hs = w % nh;
+        r.active = r.g < ng;
+    }
+    return r;
+}
+
+// Waits until every workgroup of the group has published `target`. Returns false on abort.
+__device__ __forceinline__ bool wait_group(const unsigned* gflags, int nh, unsigned target,
+                                           int* status, int spin_limit, int* lds_abort) {
+    if (threadIdx.x < kWave) {
+        int spins = 0;
+        for (;;) {
+            bool ok = true;
+            for (int i = threadIdx.x; i < nh; i += kWave) {
+                const unsigned f = __hip_atomic_load(gflags + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                ok = ok && (int(f - target) >= 0);
+            }
+            if (__all(ok)) break;
+            if (++spins > spin_limit ||
+                ((spins & 1023) == 0 &&
+                 __hip_atomic_load(status, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == 1)) {
+                if (threadIdx.x == 0) {
+                    __hip_atomic_store(status, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    *lds_abort = 1;
+                }
+                break;
+            }
+        }
+    }
+    __syncthreads();
+    return *lds_abort == 0;
+}
+
+__device__ __forceinline__ void publish(unsigned* gflags, int hs, unsigned value) {
+    __builtin_amdgcn_s_waitcnt(0);  // every store of this wave has been acknowledged by L2
+    __syncthreads();
+    if (threadIdx.x == 0)
+        __hip_atomic_store(gflags + hs, value, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+// acc[mt][nt] += A(32 rows x K) * Wslice, this wave's interleaved k-steps only.
+// a0/a1 point at (row, 8*(lane/16)) of the two 16-row tiles.
+template <int NT, int KS, bool RESIDENT>
+__device__ __forceinline__ void wave_product(floatx4 (&acc)[2][NT], const half8 (&wreg)[KS][NT],
+                                             const half8* wfrag_wave, const half_t* a0,
+                                             const half_t* a1, int wave, int lane, int nks_total,
+                                             int ks_wave) {
+    if constexpr (RESIDENT) {
+        // Loads and MFMAs are unconditional: k-steps beyond the real contraction length fetch a
+        // clamped (finite) address and meet all-zero weight fragments.
+        constexpr int KC = (KS < 8) ? KS : 8;  // k-steps fetched ahead together
+        half8 fa[KC], fb[KC];
+#pragma unroll
+        for (int c = 0; c < KS / KC; ++c) {
+#pragma unroll
+            for (int k = 0; k < KC; ++k) {
+                const int kg = min((c * KC + k) * 4 + wave, nks_total - 1);
+                fa[k] = ld_half8_coherent(a0 + kg * 32);
+                fb[k] = ld_half8_coherent(a1 + kg * 32);
+            }
+#pragma unroll
+            for (int k = 0; k < KC; ++k) {
+#pragma unroll
+                for (int n = 0; n < NT; ++n) {
+                    acc[0][n] = __builtin_amdgcn_mfma_f32_16x16x32_f16(fa[k], wreg[c * KC + k][n], acc[0][n], 0, 0, 0);
+                    acc[1][n] = __builtin_amdgcn_mfma_f32_16x16x32_f16(fb[k], wreg[c * KC + k][n], acc[1][n], 0, 0, 0);
+                }
+            }
+        }
+    } else {
+        for (int k = 0; k < ks_wave; ++k) {
+            const int kg = k * 4 + wave;
+            if (kg >= nks_total) break;
+            const half8 fa = ld_half8_coherent(a0 + kg * 32);
+            const half8 fb = ld_half8_coherent(a1 + kg * 32);
+#pragma unroll
+            for (int n = 0; n < NT; ++n) {
+                const half8 w = wfrag_wave[(size_t(k) * NT + n) * kWave + lane];
+                acc[0][n] = __builtin_amdgcn_mfma_f32_16x16x32_f16(fa, w, acc[0][n], 0, 0, 0);
+                acc[1][n] = __builtin_amdgcn_mfma_f32_16x16x32_f16(fb, w, acc[1][n], 0, 0, 0);
+            }
+        }
+    }
+}
+
+template <int NT>
+__device__ __forceinline__ void spill_partials(float* part, const floatx4 (&acc)[2][NT], int wave,
+                                               int lane, int pld) {
+    float* base = part + size_t(wave) * kRows * pld;
+#pragma unroll
+    for (int m = 0; m < 2; ++m)
+#pragma unroll
+        for (int n = 0; n < NT; ++n)
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+                base[(m * 16 + 4 * (lane / 16) + i) * pld + n * 16 + lane % 16] = acc[m][n][i];
+}
+
+__device__ __forceinline__ void store_h2(half_t* dst, float a, float b, bool device_scope) {
+    union { half_t h[2]; unsigned u; } v;
+    v.h[0] = (half_t)a;
+    v.h[1] = (half_t)b;
+    if (device_scope)
+        __hip_atomic_store(reinterpret_cast<unsigned*>(dst), v.u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    else
+        *reinterpret_cast<unsigned*>(dst) = v.u;
+}
+
+__device__ __forceinline__ void load_h2(const half_t* src, float& a, float& b) {
+    union { half_t h[2]; unsigned u; } v;
+    v.u = *reinterpret_cast<const unsigned*>(src);
+    a = (float)v.h[0];
+    b = (float)v.h[1];
+}
+
+// ------------------------------------------------------------------------------------ forward
+template <int NT, int KS, bool RESIDENT>
+__global__ __launch_bounds__(kThreads) void rec_fwd_kernel(RecFwdArgs p, RecLayout L, int t_begin,
+                                                           int t_end, int ks_wave) {
+    constexpr int JB = 4 * NT;    // hidden units of this slice
+    constexpr int NC = 16 * NT;   // gate columns of this slice (i,f,g,o blocks of JB)
+    constexpr int PLD = NC + 4;
+    extern __shared__ __attribute__((aligned(16))) float part[];  // [4][32][PLD]
+    __shared__ int lds_abort;
+    __shared__ int lds_role[2];
+
+    const Role role = make_role(L.nh, L.ng, L.gpx, L.xcd_local, p.seats, p.status, lds_role);
+    if (!role.active) return;
+    const int tid = threadIdx.x, wave = tid / kWave, lane = tid % kWave;
+    if (tid == 0) lds_abort = 0;
+    const int hs = role.hs, g = role.g;
+    const int nks_total = p.Hp / 32;
+    const bool device_scope = (L.persistent != 0) && (L.xcd_local == 0);
+    unsigned* gflags = p.flags + size_t(g) * 256;
+
+    const half8* wfrag_wave = p.wfrag + (size_t(hs) * 4 + wave) * size_t(ks_wave) * NT * kWave;
+    half8 wreg[KS][NT];
+    if constexpr (RESIDENT) {
+#pragma unroll
+        for (int k = 0; k < KS; ++k)
+#pragma unroll
+            for (int n = 0; n < NT; ++n)
+                wreg[k][n] = (k < ks_wave) ? wfrag_wave[(size_t(k) * NT + n) * kWave + lane] : half8{};
+    }
+    __syncthreads();
+
+    const size_t gld = size_t(4) * p.Hp;
+    for (int t = t_begin; t < t_end; ++t) {
+        if (t > t_begin) {
+            if (!wait_group(gflags, L.nh, p.epoch + unsigned(t - t_begin), p.status, p.spin_limit, &lds_abort))
+                return;
+        }
+        for (int rb = g; rb < L.nrb; rb += L.ng) {
+            const int row0 = rb * kRows;
+            const int ra = min(row0 + lane % 16, p.B - 1);
+            const int rbw = min(row0 + 16 + lane % 16, p.B - 1);
+            const half_t* a0 = p.Y + (size_t(t) * p.B + ra) * p.Hp + 8 * (lane / 16);
+            const half_t* a1 = p.Y + (size_t(t) * p.B + rbw) * p.Hp + 8 * (lane / 16);
+            floatx4 acc[2][NT];
+#pragma unroll
+            for (int m = 0; m < 2; ++m)
+#pragma unroll
+                for (int n = 0; n < NT; ++n) acc[m][n] = floatx4{0.f, 0.f, 0.f, 0.f};
+            wave_product<NT, KS, RESIDENT>(acc, wreg, wfrag_wave, a0, a1, wave, lane, nks_total, ks_wave);
+            spill_partials<NT>(part, acc, wave, lane, PLD);
+            __syncthreads();
+
+            // Pointwise: every thread owns pairs of neighbouring hidden units of one batch row.
+            for (int pidx = tid; pidx < kRows * (JB / 2); pidx += kThreads) {
+                const int r = pidx / (JB / 2), jj = (pidx % (JB / 2)) * 2;
+                const int b = row0 + r;
+                if (b >= p.B) continue;
+                const size_t grow = (size_t(t) * p.B + b) * gld + size_t(hs) * NC;
+                float z[4][2];
+#pragma unroll
+                for (int gt = 0; gt < 4; ++gt) {
+                    const int col = gt * JB + jj;
+                    float s0 = 0.f, s1 = 0.f;
+#pragma unroll
+                    for (int w = 0; w < 4; ++w) {
+                        const float2 v = *reinterpret_cast<const float2*>(part + (size_t(w) * kRows + r) * PLD + col);
+                        s0 += v.x;
+                        s1 += v.y;
+                    }
+                    float x0, x1;
+                    load_h2(p.G + grow + col, x0, x1);
+                    const float2 bs = *reinterpret_cast<const float2*>(p.bias + size_t(hs) * NC + col);
+                    z[gt][0] = s0 + x0 + bs.x;
+                    z[gt][1] = s1 + x1 + bs.y;
+                }
+                const int j = hs * JB + jj;
+                const float2 cp = *reinterpret_cast<const float2*>(p.C + (size_t(t) * p.B + b) * p.Hp + j);
+                float cn[2], hn[2], act[4][2];
+#pragma unroll
+                for (int u = 0; u < 2; ++u) {
+                    const float ig = sigmoidf_dev(z[0][u]);
+                    const float fg = sigmoidf_dev(z[1][u]);
+                    const float gg = tanhf(z[2][u]);
+                    const float og = sigmoidf_dev(z[3][u]);
+                    const float cprev = (u == 0) ? cp.x : cp.y;
+                    cn[u] = fg * cprev + ig * gg;
+                    hn[u] = og * tanhf(cn[u]);
+                    act[0][u] = ig; act[1][u] = fg; act[2][u] = gg; act[3][u] = og;
+                }
+                *reinterpret_cast<float2*>(p.C + (size_t(t + 1) * p.B + b) * p.Hp + j) = float2{cn[0], cn[1]};
+#pragma unroll
+                for (int gt = 0; gt < 4; ++gt)
+                    store_h2(p.G + grow + gt * JB + jj, act[gt][0], act[gt][1], false);
+                store_h2(p.Y + (size_t(t + 1) * p.B + b) * p.Hp + j, hn[0], hn[1], device_scope);
+            }
+            __syncthreads();
+        }
+        publish(gflags, hs, p.epoch + unsigned(t - t_begin + 1));
+    }
+}
+
+// ----------------------------------------------------------------------------------- backward
+// Gate order and the pointwise derivative follow flashlstm_v2/src/lstm_backward.cu:199-211, except
+// that c_{t-1}, c_t come from the cell-state cache instead of being rebuilt through atanh.
+template <int NT, int KS, bool RESIDENT>
+__global__ __launch_bounds__(kThreads) void rec_bwd_kernel(RecBwdArgs p, RecLayout L, int t_first,
+                                                           int t_last, int ks_wave) {
+    constexpr int JB = 16 * NT;  // hidden units (= output columns of dG*W_hh) of this slice
+    constexpr int PLD = JB + 4;
+    extern __shared__ __attribute__((aligned(16))) float part[];  // [4][32][PLD], reused for db
+    __shared__ int lds_abort;
+    __shared__ int lds_role[2];
+
+    const Role role = make_role(L.nh, L.ng, L.gpx, L.xcd_local, p.seats, p.status, lds_role);
+    if (!role.active) return;
+    const int tid = threadIdx.x, wave = tid / kWave, lane = tid % kWave;
+    if (tid == 0) lds_abort = 0;
+    const int hs = role.hs, g = role.g;
+    const int nks_total = p.Hp / 8;  // contraction over 4Hp packed gate columns
+    const bool device_scope = (L.persistent != 0) && (L.xcd_local == 0);
+    unsigned* gflags = p.flags + size_t(g) * 256;
+    const float S = p.dy_scale;
+
+    const half8* wfrag_wave = p.wfrag + (size_t(hs) * 4 + wave) * size_t(ks_wave) * NT * kWave;
+    half8 wreg[KS][NT];
+    if constexpr (RESIDENT) {
+#pragma unroll
+        for (int k = 0; k < KS; ++k)
+#pragma unroll
+            for (int n = 0; n < NT; ++n)
+                wreg[k][n] = (k < ks_wave) ? wfrag_wave[(size_t(k) * NT + n) * kWave + lane] : half8{};
+    }
+    __syncthreads();
+
+    const size_t gld = size_t(4) * p.Hp;
+    const int JF = p.jb_fwd;
+    float dbacc[4][2] = {{0.f, 0.f}, {0.f, 0.f}, {0.f, 0.f}, {0.f, 0.f}};
+
+    for (int t = t_first; t >= t_last; --t) {
+        const bool from_product = (t < p.T - 1);
+        if (t < t_first) {
+            if (!wait_group(gflags, L.nh, p.epoch + unsigned(t_first - t), p.status, p.spin_limit, &lds_abort))
+                return;
+        }
+        for (int rb = g; rb < L.nrb; rb += L.ng) {
+            const int row0 = rb * kRows;
+            if (from_product) {
+                const int ra = min(row0 + lane % 16, p.B - 1);
+                const int rbw = min(row0 + 16 + lane % 16, p.B - 1);
+                const half_t* a0 = p.dG + (size_t(t + 1) * p.B + ra) * gld + 8 * (lane / 16);
+                const half_t* a1 = p.dG + (size_t(t + 1) * p.B + rbw) * gld + 8 * (lane / 16);
+                floatx4 acc[2][NT];
+#pragma unroll
+                for (int m = 0; m < 2; ++m)
+#pragma unroll
+                    for (int n = 0; n < NT; ++n) acc[m][n] = floatx4{0.f, 0.f, 0.f, 0.f};
+                wave_product<NT, KS, RESIDENT>(acc, wreg, wfrag_wave, a0, a1, wave, lane, nks_total, ks_wave);
+                spill_partials<NT>(part, acc, wave, lane, PLD);
+                __syncthreads();
+            }
+            for (int pidx = tid; pidx < kRows * (JB / 2); pidx += kThreads) {
+                const int r = pidx / (JB / 2), jj = (pidx % (JB / 2)) * 2;
+                const int b = row0 + r;
+                if (b >= p.B) continue;
+                const int j = hs * JB + jj;
+                const size_t sidx = size_t(b) * p.Hp + j;
+                float dh[2];
+                if (from_product) {
+                    dh[0] = 0.f; dh[1] = 0.f;
+#pragma unroll
+                    for (int w = 0; w < 4; ++w) {
+                        const float2 v = *reinterpret_cast<const float2*>(part + (size_t(w) * kRows + r) * PLD + jj);
+                        dh[0] += v.x;
+                        dh[1] += v.y;
+                    }
+                } else {
+                    const float2 v = *reinterpret_cast<const float2*>(p.dHn + sidx);
+                    dh[0] = v.x; dh[1] = v.y;
+                }
+                if (t < 0) {  // closing pass: gradient wrt h0; dc0 already sits in dC
+                    *reinterpret_cast<float2*>(p.dH0 + sidx) = float2{dh[0], dh[1]};
+                    continue;
+                }
+                float dy0, dy1;
+                load_h2(p.dY + (size_t(t) * p.B + b) * p.Hp + j, dy0, dy1);
+                dh[0] += S * dy0;
+                dh[1] += S * dy1;
+                union { u64 q; float2 f; } dcu;
+                dcu.q = __hip_atomic_load(reinterpret_cast<const u64*>(p.dC + sidx), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                const float2 cprev = *reinterpret_cast<const float2*>(p.C + (size_t(t) * p.B + b) * p.Hp + j);
+                const float2 ccur = *reinterpret_cast<const float2*>(p.C + (size_t(t + 1) * p.B + b) * p.Hp + j);
+                // packed gate column of unit j, gate gt: (j / JF) * 4JF + gt * JF + j % JF
+                const size_t grow = (size_t(t) * p.B + b) * gld + size_t(j / JF) * 4 * JF + (j % JF);
+                float gate[4][2];
+#pragma unroll
+                for (int gt = 0; gt < 4; ++gt) load_h2(p.G + grow + gt * JF, gate[gt][0], gate[gt][1]);
+                float da[4][2], dcp[2];
+#pragma unroll
+                for (int u = 0; u < 2; ++u) {
+                    const float ig = gate[0][u], fg = gate[1][u], gg = gate[2][u], og = gate[3][u];
+                    const float tc = tanhf(u == 0 ? ccur.x : ccur.y);
+                    const float cpv = (u == 0) ? cprev.x : cprev.y;
+                    const float dcn = (u == 0) ? dcu.f.x : dcu.f.y;
+                    const float dov = dh[u] * tc;
+                    const float dc = dcn + dh[u] * og * (1.f - tc * tc);
+                    da[0][u] = dc * gg * ig * (1.f - ig);
+                    da[1][u] = dc * cpv * fg * (1.f - fg);
+                    da[2][u] = dc * ig * (1.f - gg * gg);
+                    da[3][u] = dov * og * (1.f - og);
+                    dcp[u] = dc * fg;
+                }
+                *reinterpret_cast<float2*>(p.dC + sidx) = float2{dcp[0], dcp[1]};
+#pragma unroll
+                for (int gt = 0; gt < 4; ++gt) {
+                    // db sums the values the weight-gradient GEMMs will see (fp16-rounded)
+                    const half_t h0 = (half_t)da[gt][0], h1 = (half_t)da[gt][1];
+                    dbacc[gt][0] += (float)h0;
+                    dbacc[gt][1] += (float)h1;
+                    store_h2(p.dG + (size_t(t) * p.B + b) * gld + size_t(j / JF) * 4 * JF + (j % JF) + gt * JF,
+                             da[gt][0], da[gt][1], device_scope);
+                }
+            }
+            __syncthreads();
+        }
+        if (t >= 0) publish(gflags, hs, p.epoch + unsigned(t_first - t + 1));
+    }
+
+    // Bias gradient: fold this launch's sums over the threads that share a unit pair (fixed order).
+    __syncthreads();
+    float* red = part;  // [256][8]
+#pragma unroll
+    for (int gt = 0; gt < 4; ++gt) {
+        red[tid * 8 + gt * 2 + 0] = dbacc[gt][0];
+        red[tid * 8 + gt * 2 + 1] = dbacc[gt][1];
+    }
+    __syncthreads();
+    constexpr int PAIRS = JB / 2;
+    if (tid < PAIRS * 8) {
+        const int pr = tid / 8, e = tid % 8;  // pair, (gate, unit)
+        float s = 0.f;
+        for (int k = pr; k < kThreads; k += PAIRS) s += red[k * 8 + e];
+        const int gt = e / 2, u = e % 2;
+        const int j = hs * JB + pr * 2 + u;
+        const size_t q = size_t(j / JF) * 4 * JF + size_t(gt) * JF + (j % JF);
+        p.db_part[size_t(g) * gld + q] += s;
+    }
+}
+
+template <typename K>
+hipError_t raise_lds(K kernel, size_t bytes) {
+    return hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, int(bytes));
+}
+
+}  // namespace
+
+int rec_fwd_ks(const RecLayout&, int Hp) { return int(ceil_div(size_t(Hp) / 32, 4)); }
+int rec_bwd_ks(const RecLayout&, int Hp) { return int(ceil_div(size_t(Hp) / 8, 4)); }
+
+static void finish_layout(RecLayout& L, int B, int Hp, int num_cus, bool force_stepwise, bool fits) {
+    L.nh = Hp / L.jb;
+    L.nrb = int(ceil_div(size_t(B), size_t(kRows)));
+    L.resident = fits ? 1 : 0;
+    L.xcd_local = 0;
+    L.gpx = 0;
+    if (!fits || force_stepwise || L.nh > num_cus) {
+        L.persistent = 0;
+        L.ng = L.nrb;
+        L.grid = L.ng * L.nh;
+        return;
+    }
+    L.persistent = 1;
+    if (num_cus == 256 && L.nh <= 32) {
+        L.xcd_local = 1;
+        L.gpx = 32 / L.nh;
+        L.ng = L.nrb < 8 * L.gpx ? L.nrb : 8 * L.gpx;
+        L.grid = 256;
+    } else {
+        const int cap = num_cus / L.nh;
+        L.ng = L.nrb < cap ? L.nrb : cap;
+        L.grid = L.ng * L.nh;
+    }
+}
+
+RecLayout plan_rec_fwd(int B, int Hp, int num_cus, bool force_stepwise) {
+    RecLayout L{};
+    bool fits = true;
+    if (Hp <= 1024) L.nt = 8;
+    else if (Hp <= 2048) L.nt = 4;
+    else { L.nt = 8; fits = false; }
+    L.jb = 4 * L.nt;
+    finish_layout(L, B, Hp, num_cus, force_stepwise, fits);
+    return L;
+}
+
+RecLayout plan_rec_bwd(int B, int Hp, int num_cus, bool force_stepwise) {
+    RecLayout L{};
+    bool fits = true;
+    if (Hp <= 1024) L.nt = 2;
+    else if (Hp <= 2048) L.nt = 1;
+    else { L.nt = 2; fits = false; }
+    L.jb = 16 * L.nt;
+    finish_layout(L, B, Hp, num_cus, force_stepwise, fits);
+    return L;
+}
+
+template <int NT, int KS, bool RES>
+static hipError_t run_fwd(const RecLayout& L, const RecFwdArgs& a, hipStream_t stream) {
+    auto kernel = rec_fwd_kernel<NT, KS, RES>;
+    const size_t lds = size_t(4) * kRows * (16 * NT + 4) * sizeof(float);
+    hipError_t e = raise_lds(kernel, lds);
+    if (e != hipSuccess) return e;
+    const int ks_wave = rec_fwd_ks(L, a.Hp);
+    if (L.persistent) {
+        hipLaunchKernelGGL(kernel, dim3(L.grid), dim3(kThreads), lds, stream, a, L, 0, a.T, ks_wave);
+        return hipGetLastError();
+    }
+    for (int t = 0; t < a.T; ++t) {
+        hipLaunchKernelGGL(kernel, dim3(L.grid), dim3(kThreads), lds, stream, a, L, t, t + 1, ks_wave);
+        e = hipGetLastError();
+        if (e != hipSuccess) return e;
+    }
+    return hipSuccess;
+}
+
+hipError_t launch_rec_fwd(const RecLayout& L, const RecFwdArgs& a, hipStream_t stream) {
+    if (a.T <= 0 || a.B <= 0) return hipSuccess;
+    if (a.Hp % 32 != 0 || a.Hp % L.jb != 0) return hipErrorInvalidValue;
+    if (!L.resident) return run_fwd<8, 1, false>(L, a, stream);
+    if (L.nt == 8) return run_fwd<8, 8, true>(L, a, stream);
+    if (L.nt == 4) return run_fwd<4, 16, true>(L, a, stream);
+    return hipErrorInvalidValue;
+}
+
+template <int NT, int KS, bool RES>
+static hipError_t run_bwd(const RecLayout& L, const RecBwdArgs& a, hipStream_t stream) {
+    auto kernel = rec_bwd_kernel<NT, KS, RES>;
+    size_t lds = size_t(4) * kRows * (16 * NT + 4) * sizeof(float);
+    if (lds < size_t(kThreads) * 8 * sizeof(float)) lds = size_t(kThreads) * 8 * sizeof(float);
+    hipError_t e = raise_lds(kernel, lds);
+    if (e != hipSuccess) return e;
+    const int ks_wave = rec_bwd_ks(L, a.Hp);
+    if (L.persistent) {
+        hipLaunchKernelGGL(kernel, dim3(L.grid), dim3(kThreads), lds, stream, a, L, a.T - 1, -1, ks_wave);
+        return hipGetLastError();
+    }
+    for (int t = a.T - 1; t >= -1; --t) {
+        hipLaunchKernelGGL(kernel, dim3(L.grid), dim3(kThreads), lds, stream, a, L, t, t, ks_wave);
+        e = hipGetLastError();
+        if (e != hipSuccess) return e;
+    }
+    return hipSuccess;
+}
+
+hipError_t launch_rec_bwd(const RecLayout& L, const RecBwdArgs& a, hipStream_t stream) {
+    if (a.T <= 0 || a.B <= 0) return hipSuccess;
+    if (a.Hp % 32 != 0 || a.Hp % L.jb != 0) return hipErrorInvalidValue;
+    if (!L.resident) return run_bwd<2, 1, false>(L, a, stream);
+    if (L.nt == 2) return run_bwd<2, 32, true>(L, a, stream);
+    if (L.nt == 1) return run_bwd<1, 64, true>(L, a, stream);
+    return hipErrorInvalidValue;
+}
+
+}  // namespace flstm_hip

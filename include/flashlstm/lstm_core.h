@@ -1,0 +1,93 @@
+/* Device-resident LSTM forward + BPTT core for MI355X (gfx950): the C-ABI under both public
+ * surfaces of this library (lstm_api.h and lstm_v2.h).
+ *
+ * It has no single counterpart in the reference: it is the device-side work of
+ *   - lstm_forward / lstm_pack_weights               (reference src/lstm.cu:886-931, 1897-2148)
+ *   - flstm::StreamingLstmForward                    (reference flashlstm_v2/src/lstm_forward.cu:464-966)
+ *   - flstm::StreamingLstmBackward                   (reference flashlstm_v2/src/lstm_backward.cu:643-1250)
+ * with every tensor already in HBM, so that host streaming (the v2 surface) and fp32 marshalling
+ * (the v1 surface) stay outside the timed hot path.
+ *
+ * All pointers are device pointers unless noted; tensors are contiguous:
+ *   x (T,B,I)   h0,c0,hy,cy (B,H)   y,dY (T,B,H)   W_ih (4H,I)   W_hh (4H,H)   b (4H)
+ * Gate order i,f,g,o (PyTorch).  Element types are selected per argument with flstm_dtype.
+ * Every function returns 0 on success, a hipError_t value on a HIP failure, or a FLSTM_E_* code.
+ * A plan is not thread-safe; distinct plans are independent.  Calls are synchronous with respect
+ * to `stream` (they return after the enqueued work has finished and its status was checked).
+ */
+#ifndef FLASHLSTM_LSTM_CORE_H_
+#define FLASHLSTM_LSTM_CORE_H_
+
+#include <stddef.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef struct flstm_core_plan flstm_core_plan;
+
+typedef enum { FLSTM_F32 = 0, FLSTM_F16 = 1 } flstm_dtype;
+
+enum {
+    FLSTM_E_INVALID = 1,        /* same value as hipErrorInvalidValue */
+    FLSTM_E_NOT_PACKED = 2001,  /* forward before weights were packed */
+    FLSTM_E_NO_CACHE = 2002,    /* backward without a matching forward(save_for_backward=1) */
+    FLSTM_E_STALLED = 2003      /* recurrence kernels gave up waiting even in step-wise mode */
+};
+
+/* Creates a plan for fixed (batch, input, hidden); sequence length may vary per call. */
+int flstm_core_create(size_t batch, size_t input_size, size_t hidden_size, flstm_core_plan** plan);
+int flstm_core_destroy(flstm_core_plan* plan);
+
+/* Options: "stepwise" (1 = one launch per time step instead of the persistent kernels),
+ * "proj_chunk" (time steps per input-projection GEMM, <=0 = whole sequence; results do not depend
+ * on it), "spin_limit" (polls before a waiting workgroup gives up), "dw_splits" (split-K slices of
+ * the weight-gradient GEMM, 0 = automatic). */
+int flstm_core_set_option(flstm_core_plan* plan, const char* name, long value);
+/* Reads back facts about the plan: "persistent_fwd", "persistent_bwd", "xcd_local_fwd",
+ * "xcd_local_bwd", "fallbacks" (persistent launches that had to be redone step-wise). */
+long flstm_core_get_info(const flstm_core_plan* plan, const char* name);
+
+/* fp32 PyTorch-layout weights -> fp16 MFMA operand layouts held by the plan. */
+int flstm_core_pack_weights(flstm_core_plan* plan, const float* w_ih, const float* w_hh, void* stream);
+/* bias = b_ih + b_hh, kept in fp32. Either pointer may be null (treated as zeros). */
+int flstm_core_pack_bias(flstm_core_plan* plan, const float* b_ih, const float* b_hh, void* stream);
+
+/* Forward over T steps.  h0/c0 may be null (zeros).  y, hy, cy may be null (not written).
+ * With save_for_backward != 0 the plan keeps the fp16 gate cache (activated i,f,g,o), the fp32
+ * cell states and the fp16 outputs of this call for flstm_core_backward. */
+int flstm_core_forward(flstm_core_plan* plan, size_t seq_len,
+                       const void* x, flstm_dtype x_dtype,
+                       const void* h0, const void* c0, flstm_dtype state_dtype,
+                       void* y, flstm_dtype y_dtype,
+                       void* hy, void* cy, flstm_dtype out_state_dtype,
+                       int save_for_backward, void* stream);
+
+/* BPTT for the last forward of this plan.  d_hn/d_cn may be null (zeros).  Any output may be null.
+ * grad_scale (a power of two, 1 if <= 0) multiplies dY on load and is divided out of every
+ * output; use it when dY is too small for fp16 pre-activation gradients.
+ * db_ih and db_hh receive the same values. */
+int flstm_core_backward(flstm_core_plan* plan, size_t seq_len,
+                        const void* x, flstm_dtype x_dtype,
+                        const void* dY, flstm_dtype dy_dtype,
+                        const void* d_hn, const void* d_cn, flstm_dtype dstate_dtype,
+                        float grad_scale,
+                        void* dx, flstm_dtype dx_dtype,
+                        float* dW_ih, float* dW_hh, float* db_ih, float* db_hh,
+                        float* dh0, float* dc0, void* stream);
+
+/* Read access to what forward cached (device pointers, valid until the next forward/destroy):
+ *   which = 0: h states fp16 [(T+1)*B][Hp], row t*B+b = h before step t   (ld = *ld)
+ *   which = 1: c states fp32 [(T+1)*B][Hp]
+ *   which = 2: activated gates fp16 [T*B][4Hp] in the plan's packed gate order */
+int flstm_core_cache_ptr(const flstm_core_plan* plan, int which, const void** ptr, size_t* ld);
+
+/* Average device time in milliseconds of the phases of the most recent forward / backward,
+ * measured with events on the call's stream: names "fwd_proj", "fwd_rec", "fwd_total",
+ * "bwd_rec", "bwd_dx", "bwd_dw", "bwd_total".  Negative when not available. */
+double flstm_core_last_ms(const flstm_core_plan* plan, const char* phase);
+
+#ifdef __cplusplus
+}
+#endif
+#endif  /* FLASHLSTM_LSTM_CORE_H_ */
