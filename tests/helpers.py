@@ -1,0 +1,75 @@
+"""Shared helpers of the test-suite: seeded problems, torch reference, error metrics."""
+import numpy as np
+import torch
+
+# tolerances of the parity contract: max relative error (normalised by the largest reference
+# magnitude) for outputs and final states, relative L2 error for every gradient
+TOL_OUT = 1e-2
+TOL_GRAD = 1e-2
+
+
+def relmax(a, b):
+    a, b = np.asarray(a, dtype=np.float64), np.asarray(b, dtype=np.float64)
+    return float(np.abs(a - b).max() / max(np.abs(b).max(), 1e-30))
+
+
+def rell2(a, b):
+    a, b = np.asarray(a, dtype=np.float64), np.asarray(b, dtype=np.float64)
+    return float(np.linalg.norm(a - b) / max(np.linalg.norm(b), 1e-30))
+
+
+def to_np(t):
+    return t.detach().double().cpu().numpy()
+
+
+def make_problem(T, B, I, H, seed=0, device="cpu", state_scale=0.5, fp16_values=True):
+    """Seeded tensors in fp32 whose values are exactly representable in fp16 where the kernels take fp16."""
+    g = torch.Generator().manual_seed(seed)
+    k = 1.0 / max(H, 1) ** 0.5
+    u = lambda *s: (torch.rand(*s, generator=g) * 2 - 1) * k
+    n = lambda *s: torch.randn(*s, generator=g)
+    p = dict(w_ih=u(4 * H, I), w_hh=u(4 * H, H), b_ih=u(4 * H), b_hh=u(4 * H), x=n(T, B, I),
+             h0=n(B, H) * state_scale, c0=n(B, H) * state_scale, dy=n(T, B, H), d_hn=n(B, H), d_cn=n(B, H))
+    if fp16_values:
+        for name in ("x", "h0", "c0", "dy", "d_hn", "d_cn"):
+            p[name] = p[name].half().float()
+    return {k_: v.to(device) for k_, v in p.items()}
+
+
+def torch_reference(p, dtype=torch.float64, device="cpu", fp16_weights=True, with_state_grads=True):
+    """nn.LSTM forward + autograd on the (optionally fp16-rounded) weights; returns numpy arrays."""
+    T, B, I = p["x"].shape
+    H = p["w_hh"].shape[1]
+    m = torch.nn.LSTM(I, H).to(device=device, dtype=dtype)
+    rw = (lambda w: w.half().to(dtype)) if fp16_weights else (lambda w: w.to(dtype))
+    with torch.no_grad():
+        m.weight_ih_l0.copy_(rw(p["w_ih"].to(device)))
+        m.weight_hh_l0.copy_(rw(p["w_hh"].to(device)))
+        m.bias_ih_l0.copy_(p["b_ih"].to(device=device, dtype=dtype))
+        m.bias_hh_l0.copy_(p["b_hh"].to(device=device, dtype=dtype))
+    x = p["x"].to(device=device, dtype=dtype).clone().requires_grad_(True)
+    h0 = p["h0"].to(device=device, dtype=dtype).clone().requires_grad_(True)
+    c0 = p["c0"].to(device=device, dtype=dtype).clone().requires_grad_(True)
+    y, (hn, cn) = m(x, (h0[None], c0[None]))
+    loss = (y * p["dy"].to(device=device, dtype=dtype)).sum()
+    if with_state_grads:
+        loss = loss + (hn[0] * p["d_hn"].to(device=device, dtype=dtype)).sum() \
+            + (cn[0] * p["d_cn"].to(device=device, dtype=dtype)).sum()
+    loss.backward()
+    return dict(y=to_np(y), hn=to_np(hn[0]), cn=to_np(cn[0]), dx=to_np(x.grad), dw_ih=to_np(m.weight_ih_l0.grad),
+                dw_hh=to_np(m.weight_hh_l0.grad), db=to_np(m.bias_ih_l0.grad), db_hh=to_np(m.bias_hh_l0.grad),
+                dh0=to_np(h0.grad), dc0=to_np(c0.grad))
+
+
+def check_against(ref, got, label=""):
+    """got: dict with a subset of the reference keys. Asserts the parity contract and returns the errors."""
+    errs = {}
+    for k in ("y", "hn", "cn"):
+        if k in got and got[k] is not None:
+            errs[k] = relmax(got[k], ref[k])
+            assert errs[k] <= TOL_OUT, f"{label} {k}: max rel err {errs[k]:.3e} > {TOL_OUT}"
+    for k in ("dx", "dw_ih", "dw_hh", "db", "dh0", "dc0"):
+        if k in got and got[k] is not None:
+            errs[k] = rell2(got[k], ref[k])
+            assert errs[k] <= TOL_GRAD, f"{label} {k}: rel L2 err {errs[k]:.3e} > {TOL_GRAD}"
+    return errs

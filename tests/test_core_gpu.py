@@ -1,0 +1,218 @@
+"""Parity of the device-resident core (HIP kernels through the C ABI) against the CPU oracle and
+torch.nn.LSTM on the same seeded inputs.  Tolerances: max relative error <= 1e-2 on y / h_T / c_T,
+relative L2 error <= 1e-2 on every gradient (fp16 storage, fp32 accumulation, fp32 cell state)."""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from helpers import check_against, make_problem, rell2, relmax, to_np, torch_reference
+
+pytestmark = pytest.mark.gpu
+
+
+def run_core(p, *, half=True, stepwise=False, proj_chunk=0, grad_scale=1.0, state_grads=True, T=None, core=None):
+    from flashlstm_poc_amd import LstmCore
+    dev = "cuda"
+    T_full, B, I = p["x"].shape
+    H = p["w_hh"].shape[1]
+    T = T or T_full
+    cv = (lambda t: t.to(dev).half()) if half else (lambda t: t.to(dev).float())
+    own = core is None
+    if own:
+        core = LstmCore(B, I, H)
+        core.pack(p["w_ih"].to(dev), p["w_hh"].to(dev), p["b_ih"].to(dev), p["b_hh"].to(dev))
+    core.set_option("stepwise", 1 if stepwise else 0)
+    core.set_option("proj_chunk", proj_chunk)
+    x = cv(p["x"][:T])
+    y, hy, cy = core.forward(x, cv(p["h0"]), cv(p["c0"]))
+    dx, dW_ih, dW_hh, db, dh0, dc0 = core.backward(
+        x, cv(p["dy"][:T]), cv(p["d_hn"]) if state_grads else None, cv(p["d_cn"]) if state_grads else None,
+        grad_scale=grad_scale)
+    torch.cuda.synchronize()
+    out = dict(y=to_np(y), hn=to_np(hy), cn=to_np(cy), dx=to_np(dx), dw_ih=to_np(dW_ih), dw_hh=to_np(dW_hh),
+               db=to_np(db), dh0=to_np(dh0), dc0=to_np(dc0))
+    info = {k: core.info(k) for k in ("persistent_fwd", "persistent_bwd", "xcd_local_fwd", "fallbacks")}
+    if own:
+        core.close()
+    return out, info
+
+
+def oracle_reference(p, state_grads=True, T=None):
+    n = {k: to_np(v) for k, v in p.items()}
+    T = T or n["x"].shape[0]
+    f = oracle.forward(n["x"][:T], n["w_ih"], n["w_hh"], n["b_ih"], n["b_hh"], n["h0"], n["c0"],
+                       flags=oracle.FLAG_FP16_OPERANDS)
+    g = oracle.backward(n["x"][:T], n["w_ih"], n["w_hh"], f, n["dy"][:T], n["d_hn"] if state_grads else None,
+                        n["d_cn"] if state_grads else None, flags=oracle.FLAG_FP16_OPERANDS)
+    return dict(y=f["y"], hn=f["hn"], cn=f["cn"], **g), f
+
+
+# shapes of the reference's tests (python/test_lstm.py:280-302, validate_lstm_fwd.py:243-250,
+# validate_lstm_bwd.py:435-443, test_streaming_lstm.py:17-20) plus ragged / odd sizes
+SHAPES = [(4, 2, 3, 5), (7, 2, 32, 24), (32, 2, 128, 96), (16, 8, 64, 32), (32, 4, 128, 16), (64, 32, 256, 256),
+          (1, 1, 1, 1), (3, 33, 7, 9), (5, 70, 65, 33), (9, 1, 130, 257)]
+
+
+@pytest.mark.parametrize("shape", SHAPES)
+@pytest.mark.parametrize("half", [True, False])
+def test_forward_backward_match_oracle(shape, half):
+    p = make_problem(*shape, seed=hash(shape) % 1000)
+    ref, _ = oracle_reference(p)
+    got, info = run_core(p, half=half)
+    assert info["fallbacks"] == 0
+    check_against(ref, got, label=f"{shape} half={half}")
+
+
+@pytest.mark.parametrize("shape", [(4, 2, 3, 5), (16, 8, 64, 32), (64, 8, 128, 256)])
+def test_matches_torch_lstm(shape):
+    p = make_problem(*shape, seed=7)
+    ref = torch_reference(p)  # fp64 nn.LSTM on the fp16-rounded weights
+    got, _ = run_core(p)
+    check_against(ref, got, label=str(shape))
+
+
+def test_config1_through_fp32_io():
+    # BASELINE config 1: I=128, H=256, B=8, T=64, h0 = c0 = 0, loss = sum(y^2)
+    torch.manual_seed(0)
+    m = torch.nn.LSTM(128, 256)
+    x = torch.randn(64, 8, 128)
+    from flashlstm_poc_amd import LstmCore
+    core = LstmCore(8, 128, 256)
+    core.pack(*(t.detach().cuda() for t in (m.weight_ih_l0, m.weight_hh_l0, m.bias_ih_l0, m.bias_hh_l0)))
+    y, hy, cy = core.forward(x.cuda())
+    dx, dW_ih, dW_hh, db, dh0, dc0 = core.backward(x.cuda(), 2.0 * y)
+    xr = x.clone().requires_grad_(True)
+    yr, (hr, cr) = m(xr)
+    (yr ** 2).sum().backward()
+    assert relmax(to_np(y), to_np(yr)) <= 1e-2 and relmax(to_np(cy), to_np(cr[0])) <= 1e-2
+    for got, ref in ((dx, xr.grad), (dW_ih, m.weight_ih_l0.grad), (dW_hh, m.weight_hh_l0.grad), (db, m.bias_ih_l0.grad)):
+        assert rell2(to_np(got), to_np(ref)) <= 1e-2
+    core.close()
+
+
+@pytest.mark.parametrize("shape", [(12, 40, 32, 64), (20, 16, 64, 1024)])
+def test_persistent_and_stepwise_agree(shape):
+    p = make_problem(*shape, seed=3)
+    a, ia = run_core(p, stepwise=False)
+    b, ib = run_core(p, stepwise=True)
+    assert ia["persistent_fwd"] == 1 and ib["persistent_fwd"] == 0
+    for k in ("y", "hn", "cn"):
+        np.testing.assert_array_equal(a[k], b[k])       # same arithmetic, same order
+    for k in ("dx", "dh0", "dc0", "dw_hh", "db"):
+        assert rell2(a[k], b[k]) < 1e-5, k
+
+
+def test_projection_chunk_size_does_not_change_results():
+    p = make_problem(17, 6, 48, 40, seed=9)
+    base, _ = run_core(p, proj_chunk=0)
+    for chunk in (-1, 1, 2, 5, 17, 64):
+        got, _ = run_core(p, proj_chunk=chunk)
+        for k in ("y", "cn", "dx", "dw_ih"):
+            np.testing.assert_array_equal(got[k], base[k], err_msg=f"chunk {chunk} {k}")
+
+
+def test_handle_reuse_with_shorter_and_longer_sequences():
+    # the reference re-runs one handle with T/2 and T+1 (python/test_lstm.py:186-271)
+    from flashlstm_poc_amd import LstmCore
+    T, B, I, H = 12, 3, 20, 24
+    p = make_problem(T + 1, B, I, H, seed=21)
+    core = LstmCore(B, I, H)
+    core.pack(*(p[k].cuda() for k in ("w_ih", "w_hh", "b_ih", "b_hh")))
+    for t in (T, T // 2, T + 1, 1):
+        ref, _ = oracle_reference(p, T=t)
+        got, _ = run_core(p, T=t, core=core)
+        check_against(ref, got, label=f"T={t}")
+    core.close()
+
+
+def test_missing_state_gradients_equal_zero_state_gradients():
+    p = make_problem(6, 4, 10, 12, seed=4)
+    a, _ = run_core(p, state_grads=False)
+    q = dict(p); q["d_hn"] = torch.zeros_like(p["d_hn"]); q["d_cn"] = torch.zeros_like(p["d_cn"])
+    b, _ = run_core(q, state_grads=True)
+    for k in a:
+        np.testing.assert_array_equal(a[k], b[k], err_msg=k)
+    ref, _ = oracle_reference(p, state_grads=False)
+    check_against(ref, a)
+
+
+def test_grad_scale_rescues_tiny_upstream_gradients():
+    # dY ~ 1e-7 underflows fp16 pre-activation gradients unless scaled (power of two => exact otherwise)
+    p = make_problem(8, 4, 16, 32, seed=5, fp16_values=False)
+    p["dy"] = p["dy"] * 1e-7; p["d_hn"] = p["d_hn"] * 0; p["d_cn"] = p["d_cn"] * 0
+    ref, _ = oracle_reference(p)
+    got, _ = run_core(p, half=False, grad_scale=2.0 ** 20)
+    check_against(ref, got, label="scaled")
+    unscaled, _ = run_core(p, half=False, grad_scale=1.0)
+    assert rell2(unscaled["dx"], ref["dx"]) > 1e-2   # the unscaled run really loses the gradient
+
+
+def test_zero_recurrent_weights_and_zero_input_special_cases():
+    p = make_problem(5, 3, 8, 16, seed=6)
+    p["w_hh"] = torch.zeros_like(p["w_hh"])
+    ref, _ = oracle_reference(p)
+    got, _ = run_core(p)
+    check_against(ref, got, label="W_hh=0")
+    assert np.abs(got["dw_hh"] - ref["dw_hh"]).max() <= 1e-2 * np.abs(ref["dw_hh"]).max()
+    q = make_problem(5, 3, 8, 16, seed=6)
+    for k in ("x", "h0", "c0", "b_ih", "b_hh"):
+        q[k] = torch.zeros_like(q[k])
+    got, _ = run_core(q)
+    assert np.all(got["y"] == 0) and np.all(got["cn"] == 0)
+
+
+def test_gate_cache_and_state_arrays_hold_what_the_oracle_computes():
+    import ctypes
+    from flashlstm_poc_amd import LstmCore
+    T, B, I, H = 6, 5, 12, 40
+    p = make_problem(T, B, I, H, seed=8)
+    _, f = oracle_reference(p)
+    core = LstmCore(B, I, H)
+    core.pack(*(p[k].cuda() for k in ("w_ih", "w_hh", "b_ih", "b_hh")))
+    core.forward(p["x"].cuda().half(), p["h0"].cuda().half(), p["c0"].cuda().half())
+    Hp, JF = core.info("hidden_padded"), core.info("gate_slice")
+
+    def view(which, rows, cols, dtype):
+        ptr, ld = ctypes.c_void_p(), ctypes.c_size_t()
+        assert core.lib.flstm_core_cache_ptr(core._h, which, ctypes.byref(ptr), ctypes.byref(ld)) == 0
+        t = torch.empty((rows, ld.value), dtype=dtype, device="cuda")
+        nbytes = t.numel() * t.element_size()
+        assert ctypes.CDLL("libamdhip64.so").hipMemcpy(ctypes.c_void_p(t.data_ptr()), ptr, ctypes.c_size_t(nbytes), 3) == 0
+        return to_np(t)[:, :cols]
+
+    h_all = view(0, (T + 1) * B, Hp, torch.float16).reshape(T + 1, B, Hp)[..., :H]
+    c_all = view(1, (T + 1) * B, Hp, torch.float32).reshape(T + 1, B, Hp)[..., :H]
+    gates = view(2, T * B, 4 * Hp, torch.float16).reshape(T, B, 4 * Hp)
+    assert relmax(h_all, f["h_all"]) <= 1e-2 and relmax(c_all, f["c_all"]) <= 1e-2
+    np.testing.assert_array_equal(h_all[0], to_np(p["h0"]))          # entry 0 is the initial state
+    # packed gate order: unit j, gate g sits at (j // JF) * 4JF + g * JF + j % JF
+    j = np.arange(H)
+    for g in range(4):
+        cols = (j // JF) * 4 * JF + g * JF + j % JF
+        assert relmax(gates[..., cols], f["gates"][..., g * H:(g + 1) * H]) <= 1e-2
+    assert gates.min() >= -1.0 and gates.max() <= 1.0
+    core.close()
+
+
+def test_error_codes():
+    from flashlstm_poc_amd import LstmCore
+    core = LstmCore(2, 3, 5)
+    x = torch.zeros(4, 2, 3, device="cuda", dtype=torch.float16)
+    with pytest.raises(RuntimeError, match="2001"):     # forward before packing
+        core.forward(x)
+    w = make_problem(4, 2, 3, 5)
+    core.pack(*(w[k].cuda() for k in ("w_ih", "w_hh", "b_ih", "b_hh")))
+    with pytest.raises(RuntimeError, match="2002"):     # backward without forward
+        core.backward(x, torch.zeros(4, 2, 5, device="cuda", dtype=torch.float16))
+    core.forward(x, save_for_backward=False)
+    with pytest.raises(RuntimeError, match="2002"):
+        core.backward(x, torch.zeros(4, 2, 5, device="cuda", dtype=torch.float16))
+    core.forward(x)
+    with pytest.raises(RuntimeError, match="2002"):     # sequence length differs from the cached forward
+        core.backward(x[:3], torch.zeros(3, 2, 5, device="cuda", dtype=torch.float16))
+    with pytest.raises(ValueError):
+        core.set_option("no_such_option", 1)
+    with pytest.raises(ValueError):
+        core.forward(torch.zeros(4, 3, 3, device="cuda", dtype=torch.float16))
+    core.close()

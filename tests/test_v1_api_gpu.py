@@ -1,0 +1,127 @@
+"""The fp32 C API (include/flashlstm/lstm_api.h) called through ctypes exactly like the reference's
+python/test_lstm.py:44-84 binds it: presets, random shapes, handle reuse with T/2 and T+1, error codes."""
+import ctypes
+import random
+
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from helpers import TOL_OUT, make_problem, rell2, relmax, to_np
+
+pytestmark = pytest.mark.gpu
+
+ACC32, ACC16 = 0, 1
+
+
+class Buffers(ctypes.Structure):
+    _fields_ = [("impl", ctypes.c_void_p)]
+
+
+def bind():
+    from flashlstm_poc_amd import library_path
+    lib = ctypes.CDLL(library_path())
+    sz, vp, i32 = ctypes.c_size_t, ctypes.c_void_p, ctypes.c_int
+    lib.lstm_create_buffers.argtypes = [i32, sz, sz, sz, sz, i32, ctypes.POINTER(Buffers)]
+    lib.lstm_destroy_buffers.argtypes = [ctypes.POINTER(Buffers)]
+    lib.lstm_set_execution_mode.argtypes = [ctypes.POINTER(Buffers), i32]
+    lib.lstm_pack_weights.argtypes = [i32, vp, vp, sz, sz, ctypes.POINTER(Buffers)]
+    lib.lstm_forward.argtypes = [vp] * 8 + [sz] * 4 + [ctypes.POINTER(Buffers), i32]
+    lib.lstm_backward.argtypes = [vp] * 10 + [sz] * 4 + [ctypes.POINTER(Buffers)]
+    return lib
+
+
+def forward(lib, buf, p, T, precision):
+    B, I = p["x"].shape[1:]
+    H = p["w_hh"].shape[1]
+    d = {k: p[k].cuda().float().contiguous() for k in ("b_ih", "b_hh", "h0", "c0")}
+    x = p["x"][:T].cuda().float().contiguous()
+    out = torch.empty(T, B, H, device="cuda"); hn = torch.empty(B, H, device="cuda"); cn = torch.empty(B, H, device="cuda")
+    rc = lib.lstm_forward(x.data_ptr(), d["b_ih"].data_ptr(), d["b_hh"].data_ptr(), d["h0"].data_ptr(),
+                          d["c0"].data_ptr(), out.data_ptr(), hn.data_ptr(), cn.data_ptr(), T, B, I, H,
+                          ctypes.byref(buf), precision)
+    return rc, out, hn, cn
+
+
+def oracle_fwd(p, T):
+    n = {k: to_np(v) for k, v in p.items()}
+    return oracle.forward(n["x"][:T], n["w_ih"], n["w_hh"], n["b_ih"], n["b_hh"], n["h0"], n["c0"],
+                          flags=oracle.FLAG_FP16_OPERANDS)
+
+
+PRESET = [(7, 2, 32, 24), (5, 3, 48, 32), (32, 2, 128, 96), (16, 4, 64, 64), (24, 8, 96, 128)]
+rng = random.Random(1234)
+RANDOM = [(rng.randint(1, 24), rng.randint(1, 8), rng.randint(1, 64), rng.randint(1, 64)) for _ in range(4)]
+
+
+@pytest.mark.parametrize("shape", PRESET + RANDOM)
+@pytest.mark.parametrize("mode", [0, 1])
+def test_forward_presets_with_sequence_shrink_and_grow(shape, mode):
+    lib = bind()
+    T, B, I, H = shape
+    p = make_problem(T + 1, B, I, H, seed=1234 + T, state_scale=1.0, fp16_values=False)   # h0, c0 ~ N(0,1)
+    buf = Buffers()
+    assert lib.lstm_create_buffers(ACC16, T, B, I, H, 64, ctypes.byref(buf)) == 0
+    assert lib.lstm_set_execution_mode(ctypes.byref(buf), mode) == 0
+    w_ih, w_hh = p["w_ih"].cuda().contiguous(), p["w_hh"].cuda().contiguous()
+    assert lib.lstm_pack_weights(ACC16, w_ih.data_ptr(), w_hh.data_ptr(), I, H, ctypes.byref(buf)) == 0
+    for t in (T, max(1, T // 2), T + 1):
+        rc, out, hn, cn = forward(lib, buf, p, t, ACC16)
+        assert rc == 0
+        f = oracle_fwd(p, t)
+        assert relmax(to_np(out), f["y"]) <= TOL_OUT
+        assert relmax(to_np(hn), f["hn"]) <= TOL_OUT
+        assert relmax(to_np(cn), f["cn"]) <= TOL_OUT
+        # the reference's own acceptance band (python/test_lstm.py:370-381)
+        np.testing.assert_allclose(to_np(out), f["y"], atol=1e-3 + 2e-3, rtol=5e-2)
+    assert lib.lstm_destroy_buffers(ctypes.byref(buf)) == 0
+    assert buf.impl is None
+
+
+def test_backward_addition_matches_oracle():
+    lib = bind()
+    T, B, I, H = 9, 4, 24, 40
+    p = make_problem(T, B, I, H, seed=77, fp16_values=False)
+    buf = Buffers()
+    assert lib.lstm_create_buffers(ACC32, T, B, I, H, 0, ctypes.byref(buf)) == 0
+    w_ih, w_hh = p["w_ih"].cuda().contiguous(), p["w_hh"].cuda().contiguous()
+    assert lib.lstm_pack_weights(ACC32, w_ih.data_ptr(), w_hh.data_ptr(), I, H, ctypes.byref(buf)) == 0
+    rc, out, hn, cn = forward(lib, buf, p, T, ACC32)
+    assert rc == 0
+    x = p["x"].cuda().contiguous(); dy = p["dy"].cuda().contiguous()
+    d_hn = p["d_hn"].cuda().contiguous(); d_cn = p["d_cn"].cuda().contiguous()
+    dx = torch.empty_like(x); dW_ih = torch.empty_like(w_ih); dW_hh = torch.empty_like(w_hh)
+    db = torch.empty(4 * H, device="cuda"); dh0 = torch.empty(B, H, device="cuda"); dc0 = torch.empty(B, H, device="cuda")
+    rc = lib.lstm_backward(x.data_ptr(), dy.data_ptr(), d_hn.data_ptr(), d_cn.data_ptr(), dx.data_ptr(),
+                           dW_ih.data_ptr(), dW_hh.data_ptr(), db.data_ptr(), dh0.data_ptr(), dc0.data_ptr(),
+                           T, B, I, H, ctypes.byref(buf))
+    assert rc == 0
+    n = {k: to_np(v) for k, v in p.items()}
+    f = oracle_fwd(p, T)
+    g = oracle.backward(n["x"], n["w_ih"], n["w_hh"], f, n["dy"], n["d_hn"], n["d_cn"], flags=oracle.FLAG_FP16_OPERANDS)
+    for got, k in ((dx, "dx"), (dW_ih, "dw_ih"), (dW_hh, "dw_hh"), (db, "db"), (dh0, "dh0"), (dc0, "dc0")):
+        assert rell2(to_np(got), g[k]) <= 1e-2, k
+    lib.lstm_destroy_buffers(ctypes.byref(buf))
+
+
+def test_error_codes_follow_the_reference():
+    # reference src/lstm.cu:861-904,1912-1920: everything invalid returns 1
+    lib = bind()
+    T, B, I, H = 4, 2, 8, 8
+    p = make_problem(T, B, I, H)
+    buf = Buffers()
+    assert lib.lstm_create_buffers(ACC32, T, B, I, H, 0, ctypes.byref(buf)) == 0
+    rc, *_ = forward(lib, buf, p, T, ACC32)
+    assert rc == 1                                           # weights not packed yet
+    w_ih, w_hh = p["w_ih"].cuda().contiguous(), p["w_hh"].cuda().contiguous()
+    assert lib.lstm_pack_weights(ACC16, w_ih.data_ptr(), w_hh.data_ptr(), I, H, ctypes.byref(buf)) == 1   # precision
+    assert lib.lstm_pack_weights(ACC32, w_ih.data_ptr(), w_hh.data_ptr(), I + 1, H, ctypes.byref(buf)) == 1  # dims
+    assert lib.lstm_pack_weights(ACC32, w_ih.data_ptr(), w_hh.data_ptr(), I, H, ctypes.byref(buf)) == 0
+    assert forward(lib, buf, p, T, ACC16)[0] == 1            # precision differs from create
+    q = make_problem(T, B + 1, I, H)
+    assert forward(lib, buf, q, T, ACC32)[0] == 1            # batch differs from create
+    assert lib.lstm_set_execution_mode(ctypes.byref(buf), 5) == 1
+    assert forward(lib, buf, p, T, ACC32)[0] == 0
+    assert lib.lstm_destroy_buffers(ctypes.byref(buf)) == 0
+    assert forward(lib, buf, p, T, ACC32)[0] == 1            # destroyed handle

@@ -1,0 +1,161 @@
+"""The streaming C entry points (include/flashlstm_v2/lstm.hpp) through ctypes, as the reference's
+flashlstm_v2/scripts/validate_lstm_fwd.py:71-95 and validate_lstm_bwd.py:71-133 bind them: pinned host
+sequences, fp16 device states, fp32 device weights, host h/c checkpoints with mixed dtypes."""
+import ctypes
+import os
+import subprocess
+import sys
+
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from helpers import make_problem, rell2, relmax, to_np
+
+pytestmark = pytest.mark.gpu
+
+
+class GateCacheHost(ctypes.Structure):
+    _fields_ = [("h_ptr", ctypes.c_void_p), ("c_ptr", ctypes.c_void_p)]
+
+
+class Options(ctypes.Structure):
+    _fields_ = [("h_dtype", ctypes.c_int), ("c_dtype", ctypes.c_int)]
+
+
+def bind():
+    from flashlstm_poc_amd import library_path
+    lib = ctypes.CDLL(library_path())
+    sz, vp = ctypes.c_size_t, ctypes.c_void_p
+    lib.flstm_StreamingLstmForward.argtypes = [sz] * 5 + [vp] * 8 + [GateCacheHost, ctypes.POINTER(Options)] + [vp] * 5
+    lib.flstm_StreamingLstmForward.restype = None
+    lib.flstm_StreamingLstmBackward.argtypes = [sz] * 5 + [vp, vp, GateCacheHost] + [vp] * 19 + [ctypes.POINTER(Options)]
+    lib.flstm_StreamingLstmBackward.restype = None
+    return lib
+
+
+def pinned(t, dtype=torch.float16):
+    out = torch.empty(t.shape, dtype=dtype, pin_memory=True)
+    out.copy_(t)
+    return out
+
+
+def run_v2(p, R=1, h_dtype=torch.float32, c_dtype=torch.float32, pin=True, state_grads=True, fresh_backward=False):
+    lib = bind()
+    T, B, I = p["x"].shape
+    H = p["w_hh"].shape[1]
+    n_ck = (T + R - 1) // R
+    mk = pinned if pin else (lambda t, dtype=torch.float16: t.to(dtype).contiguous())
+    x_host = mk(p["x"]); dy_host = mk(p["dy"])
+    y_host = torch.empty(T, B, H, dtype=torch.float16, pin_memory=pin)
+    ck_h = torch.empty(n_ck, B, H, dtype=h_dtype, pin_memory=pin); ck_c = torch.empty(n_ck, B, H, dtype=c_dtype, pin_memory=pin)
+    dx_host = torch.empty(T, B, I, dtype=torch.float16, pin_memory=pin)
+    dev = {k: p[k].cuda().float().contiguous() for k in ("w_ih", "w_hh", "b_ih", "b_hh")}
+    h0 = p["h0"].cuda().half(); c0 = p["c0"].cuda().half()
+    d_hn = p["d_hn"].cuda().half(); d_cn = p["d_cn"].cuda().half()
+    hy = torch.empty(B, H, device="cuda", dtype=torch.float16); cy = torch.empty_like(hy)
+    dW_ih = torch.full_like(dev["w_ih"], 7.0); dW_hh = torch.full_like(dev["w_hh"], 7.0)   # must be overwritten
+    db_ih = torch.full_like(dev["b_ih"], 7.0); db_hh = torch.full_like(dev["b_hh"], 7.0)
+    dh0 = torch.empty(B, H, device="cuda"); dc0 = torch.empty(B, H, device="cuda")
+    streams = [torch.cuda.Stream() for _ in range(3)]
+    torch.cuda.synchronize()
+    cache = GateCacheHost(ck_h.data_ptr(), ck_c.data_ptr())
+    opt = Options(0 if h_dtype == torch.float32 else 1, 0 if c_dtype == torch.float32 else 1)
+    s = [st.cuda_stream for st in streams]
+    lib.flstm_StreamingLstmForward(T, B, I, H, R, x_host.data_ptr(), h0.data_ptr(), c0.data_ptr(),
+                                   dev["w_ih"].data_ptr(), dev["w_hh"].data_ptr(), dev["b_ih"].data_ptr(),
+                                   dev["b_hh"].data_ptr(), y_host.data_ptr(), cache, ctypes.byref(opt), hy.data_ptr(),
+                                   cy.data_ptr(), s[0], s[1], s[2])
+    if fresh_backward:   # forget the device-side caches: backward must rebuild them from x, h0, c0
+        lib.flstm_ReleaseStreamingCaches()
+    lib.flstm_StreamingLstmBackward(T, B, I, H, R, x_host.data_ptr(), y_host.data_ptr(), cache, dy_host.data_ptr(),
+                                    d_hn.data_ptr() if state_grads else None, d_cn.data_ptr() if state_grads else None,
+                                    h0.data_ptr(), c0.data_ptr(), dev["w_ih"].data_ptr(), dev["w_hh"].data_ptr(),
+                                    dev["b_ih"].data_ptr(), dev["b_hh"].data_ptr(), dx_host.data_ptr(),
+                                    dW_ih.data_ptr(), dW_hh.data_ptr(), db_ih.data_ptr(), db_hh.data_ptr(),
+                                    dh0.data_ptr(), dc0.data_ptr(), s[0], s[1], s[2], ctypes.byref(opt))
+    torch.cuda.synchronize()
+    return dict(y=to_np(y_host), hn=to_np(hy), cn=to_np(cy), ck_h=to_np(ck_h), ck_c=to_np(ck_c), dx=to_np(dx_host),
+                dw_ih=to_np(dW_ih), dw_hh=to_np(dW_hh), db=to_np(db_ih), db_hh=to_np(db_hh), dh0=to_np(dh0), dc0=to_np(dc0))
+
+
+def reference(p, state_grads=True):
+    n = {k: to_np(v) for k, v in p.items()}
+    f = oracle.forward(n["x"], n["w_ih"], n["w_hh"], n["b_ih"], n["b_hh"], n["h0"], n["c0"], flags=oracle.FLAG_FP16_OPERANDS)
+    g = oracle.backward(n["x"], n["w_ih"], n["w_hh"], f, n["dy"], n["d_hn"] if state_grads else None,
+                        n["d_cn"] if state_grads else None, flags=oracle.FLAG_FP16_OPERANDS)
+    return f, g
+
+
+def compare(out, f, g, R):
+    assert relmax(out["y"], f["y"]) <= 1e-2 and relmax(out["hn"], f["hn"]) <= 1e-2 and relmax(out["cn"], f["cn"]) <= 1e-2
+    for k in ("dx", "dw_ih", "dw_hh", "db", "dh0", "dc0"):
+        assert rell2(out[k], g[k]) <= 1e-2, k
+    np.testing.assert_array_equal(out["db"], out["db_hh"])
+    # checkpoint k = state BEFORE step k*R (reference lstm_forward.cu:370-375,727-783)
+    assert relmax(out["ck_h"], oracle.checkpoints(f["h_all"], R)) <= 1e-2
+    assert relmax(out["ck_c"], oracle.checkpoints(f["c_all"], R)) <= 1e-2
+
+
+# validate_lstm_fwd.py:243-250 / validate_lstm_bwd.py:435-443 shapes, R = 4, h cache fp16 + c cache fp32
+@pytest.mark.parametrize("shape", [(4, 2, 3, 5), (16, 8, 64, 32), (32, 4, 128, 16), (64, 32, 256, 256)])
+def test_validator_shapes_mixed_cache_dtypes(shape):
+    p = make_problem(*shape, seed=42)
+    f, g = reference(p)
+    out = run_v2(p, R=4, h_dtype=torch.float16, c_dtype=torch.float32)
+    compare(out, f, g, 4)
+    np.testing.assert_array_equal(out["ck_h"][0], to_np(p["h0"]))   # entry 0 is exactly (h0, c0)
+    np.testing.assert_array_equal(out["ck_c"][0], to_np(p["c0"]))
+
+
+@pytest.mark.parametrize("R", [1, 3, 7, 50])
+def test_recompute_interval_only_changes_the_checkpoints(R):
+    p = make_problem(10, 3, 12, 20, seed=1)
+    f, g = reference(p)
+    out = run_v2(p, R=R)
+    compare(out, f, g, R)
+    assert out["ck_h"].shape[0] == (10 + R - 1) // R
+
+
+def test_backward_without_device_cache_recomputes_the_forward_pass():
+    p = make_problem(12, 5, 16, 24, seed=2)
+    f, g = reference(p)
+    a = run_v2(p, R=4, fresh_backward=False)
+    b = run_v2(p, R=4, fresh_backward=True)
+    compare(b, f, g, 4)
+    for k in ("dx", "dw_ih", "dw_hh", "db", "dh0", "dc0"):
+        np.testing.assert_array_equal(a[k], b[k], err_msg=k)
+
+
+def test_null_state_gradients_and_pageable_host_memory():
+    p = make_problem(6, 4, 8, 16, seed=3)
+    f, g = reference(p, state_grads=False)
+    out = run_v2(p, R=2, pin=False, state_grads=False)
+    compare(out, f, g, 2)
+
+
+def test_invalid_arguments_abort_like_the_reference():
+    # R = 0 and non-distinct streams make the C entry points print and abort() (lstm_forward.cu:497-502,1029-1037)
+    code = r'''
+import ctypes, sys, torch
+sys.path.insert(0, %r)
+from test_v2_api_gpu import bind, GateCacheHost, Options
+lib = bind()
+x = torch.zeros(2, 1, 4, dtype=torch.float16, pin_memory=True); y = torch.zeros(2, 1, 4, dtype=torch.float16, pin_memory=True)
+ck = torch.zeros(2, 1, 4, pin_memory=True); w = torch.zeros(16, 4, device="cuda"); b = torch.zeros(16, device="cuda")
+h = torch.zeros(1, 4, device="cuda", dtype=torch.float16)
+s = [torch.cuda.Stream() for _ in range(3)]
+mode = sys.argv[1]
+R = 0 if mode == "r0" else 1
+st = [s[0].cuda_stream, s[0].cuda_stream if mode == "streams" else s[1].cuda_stream, s[2].cuda_stream]
+lib.flstm_StreamingLstmForward(2, 1, 4, 4, R, x.data_ptr(), h.data_ptr(), h.data_ptr(), w.data_ptr(), w.data_ptr(), b.data_ptr(),
+    b.data_ptr(), y.data_ptr(), GateCacheHost(ck.data_ptr(), ck.data_ptr()), None, h.data_ptr(), h.data_ptr(), *st)
+print("survived")
+''' % os.path.dirname(os.path.abspath(__file__))
+    for mode, expect_abort in (("r0", True), ("streams", True), ("ok", False)):
+        r = subprocess.run([sys.executable, "-c", code, mode], capture_output=True, text=True, timeout=300)
+        if expect_abort:
+            assert r.returncode != 0 and "flstm_StreamingLstmForward failed" in r.stderr, (mode, r.returncode, r.stderr[-300:])
+        else:
+            assert r.returncode == 0 and "survived" in r.stdout, r.stderr[-300:]
