@@ -1,0 +1,194 @@
+#!/usr/bin/env python3
+"""Headline benchmark: single-layer LSTM forward + backward (BPTT) with the fp16 gate cache on one MI355X.
+
+A "step" is one forward + backward pass of the hot path over one synthetic batch with every tensor
+already resident in HBM (fp16 x / dY, packed fp16 weights); weight packing and plan creation happen
+before the timed region.  Prints ONE JSON line.
+
+  python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload config3|config2|config4]
+                  [--no-cpu-baseline] [--no-parity]
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+PEAK_FP16_TFLOPS = 2500.0   # MI355X dense fp16 MFMA peak (2.5 PFLOP/s)
+PEAK_HBM_GBS = 8000.0
+
+WORKLOADS = {
+    # name: (T, B, I, H, backward?)
+    "config2": (512, 64, 1024, 1024, False),
+    "config3": (1024, 256, 1024, 1024, True),
+    "config4": (2048, 16, 2048, 2048, True),
+}
+
+
+def make_inputs(T, B, I, H, seed=0):
+    import torch
+    g = torch.Generator(device="cuda").manual_seed(seed)
+    k = 1.0 / H ** 0.5
+    u = lambda *s: (torch.rand(*s, generator=g, device="cuda") * 2 - 1) * k
+    n = lambda *s: torch.randn(*s, generator=g, device="cuda")
+    return dict(w_ih=u(4 * H, I), w_hh=u(4 * H, H), b_ih=u(4 * H), b_hh=u(4 * H), x=n(T, B, I).half(),
+                h0=(n(B, H) * 0.1).half(), c0=(n(B, H) * 0.1).half(), dy=n(T, B, H).half())
+
+
+def parity_check(B, I, H, T=32):
+    """Same kernels at a short length against fp32 torch.nn.LSTM on the fp16-rounded operands."""
+    import torch
+    from flashlstm_poc_amd import LstmCore
+    p = make_inputs(T, B, I, H, seed=1)
+    core = LstmCore(B, I, H)
+    core.pack(p["w_ih"], p["w_hh"], p["b_ih"], p["b_hh"])
+    y, hy, cy = core.forward(p["x"], p["h0"], p["c0"])
+    dx, dW_ih, dW_hh, db, dh0, dc0 = core.backward(p["x"], p["dy"])
+    m = torch.nn.LSTM(I, H, device="cuda")
+    with torch.no_grad():
+        m.weight_ih_l0.copy_(p["w_ih"].half().float()); m.weight_hh_l0.copy_(p["w_hh"].half().float())
+        m.bias_ih_l0.copy_(p["b_ih"]); m.bias_hh_l0.copy_(p["b_hh"])
+    xr = p["x"].float().requires_grad_(True)
+    hr = p["h0"].float().requires_grad_(True); cr = p["c0"].float().requires_grad_(True)
+    yr, (hn, cn) = m(xr, (hr[None], cr[None]))
+    (yr * p["dy"].float()).sum().backward()
+    relmax = lambda a, b: ((a.float() - b.float()).abs().max() / b.float().abs().max()).item()
+    rell2 = lambda a, b: ((a.float() - b.float()).norm() / b.float().norm()).item()
+    errs = {"y": relmax(y, yr), "h_T": relmax(hy, hn[0]), "c_T": relmax(cy, cn[0]), "dx": rell2(dx, xr.grad),
+            "dW_ih": rell2(dW_ih, m.weight_ih_l0.grad), "dW_hh": rell2(dW_hh, m.weight_hh_l0.grad),
+            "db": rell2(db, m.bias_ih_l0.grad), "dh0": rell2(dh0, hr.grad), "dc0": rell2(dc0, cr.grad)}
+    core.close()
+    worst = max(errs.values())
+    return {"T": T, "max_err": round(worst, 6), "tolerance": 1e-2, "ok": bool(worst <= 1e-2)}
+
+
+def cpu_baseline(B, I, H, backward, budget_s=20.0):
+    """torch.nn.LSTM (fp32, CPU) on this host's cores, on a time-bounded sample of the same workload:
+    same B, I, H and seeded inputs, reduced T (LSTM cost is linear in T)."""
+    import torch
+    threads = torch.get_num_threads()
+    T = 8
+    torch.manual_seed(0)
+    m = torch.nn.LSTM(I, H)
+    x = torch.randn(T, B, I, requires_grad=backward)
+    dy = torch.randn(T, B, H)
+
+    def once():
+        y, _ = m(x)
+        if backward:
+            m.zero_grad(set_to_none=True)
+            x.grad = None
+            (y * dy).sum().backward()
+
+    once()  # warm-up
+    t0 = time.perf_counter(); once(); probe = time.perf_counter() - t0
+    reps = max(1, min(20, int(budget_s / max(probe, 1e-3))))
+    t0 = time.perf_counter()
+    for _ in range(reps):
+        once()
+    dt = (time.perf_counter() - t0) / reps
+    return {"value": round(B * T / dt, 1), "unit": "batch*timesteps/s", "cores": threads, "kind": "port",
+            "impl": "torch.nn.LSTM fp32 on CPU (the oracle named for this path)",
+            "sample": f"same B={B}, I={I}, H={H}, {'fwd+bwd' if backward else 'fwd'}, T reduced to {T}, "
+                      f"{reps} repeats after 1 warm-up, {dt * 1e3:.1f} ms each; os.cpu_count()={os.cpu_count()}"}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=10)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--workload", default="config3", choices=sorted(WORKLOADS))
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-parity", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py: this build runs on ONE GPU (the recurrence shards over batch; no multi-GPU path is "
+              "built) -- rerun with --gpus 1", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    from flashlstm_poc_amd import LstmCore
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        sys.exit(1)
+    torch.cuda.set_device(0)
+    T, B, I, H, backward = WORKLOADS[args.workload]
+    p = make_inputs(T, B, I, H)
+    core = LstmCore(B, I, H)
+    core.pack(p["w_ih"], p["w_hh"], p["b_ih"], p["b_hh"])
+
+    def step():
+        core.forward(p["x"], p["h0"], p["c0"], save_for_backward=backward)
+        if backward:
+            core.backward(p["x"], p["dy"])
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    phases = ["fwd_proj", "fwd_rec"] + (["bwd_rec", "bwd_dx", "bwd_dw"] if backward else [])
+    acc = {k: 0.0 for k in phases}
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    e0.record()
+    for _ in range(args.steps):
+        step()
+        for k in phases:   # device time of each phase of this step (hipEvents on the launch stream)
+            acc[k] += core.last_ms(k)
+    e1.record()
+    torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3 / args.steps
+    ms = e0.elapsed_time(e1) / args.steps
+    phase_ms = {k: v / args.steps for k, v in acc.items()}
+
+    flops_fwd = 8.0 * T * B * H * (I + H)
+    flops = flops_fwd * (3.0 if backward else 1.0)
+    # algorithmic FLOPs per launch of each kernel (2*m*n*k per contraction)
+    kflops = {"fwd_proj": 2.0 * T * B * 4 * H * I, "fwd_rec": 2.0 * T * B * 4 * H * H,
+              "bwd_rec": 2.0 * T * B * 4 * H * H, "bwd_dx": 2.0 * T * B * 4 * H * I,
+              "bwd_dw": 2.0 * T * B * 4 * H * (I + H)}
+    kname = {"fwd_proj": "gemm_nt_256x256 (X*W_ih^T)", "fwd_rec": "rec_fwd_kernel (persistent recurrence)",
+             "bwd_rec": "rec_bwd_kernel (persistent BPTT)", "bwd_dx": "gemm_nt_256x256 (dG*W_ih)",
+             "bwd_dw": "transpose_pad x3 + gemm_nt_256x256 split-K (dG^T*[X;H]) + reduce_dw"}
+    kernels = []
+    for k in phases:
+        tf = kflops[k] / (phase_ms[k] * 1e-3) / 1e12 if phase_ms[k] > 0 else 0.0
+        kernels.append({"phase": k, "kernel": kname[k], "ms": round(phase_ms[k], 4), "tflops": round(tf, 1),
+                        "frac_of_peak": round(tf / PEAK_FP16_TFLOPS, 4)})
+    dom = max(kernels, key=lambda d: d["ms"])
+    roofline = {"kernel": dom["kernel"], "bound": "mfma", "achieved": dom["tflops"], "peak": PEAK_FP16_TFLOPS,
+                "unit": "TFLOP/s", "frac": dom["frac_of_peak"], "traffic": None,
+                "launch_ms": dom["ms"], "flops_per_launch": kflops[dom["phase"]]}
+    if dom["phase"] in ("fwd_rec", "bwd_rec"):
+        roofline["us_per_timestep"] = round(dom["ms"] * 1e3 / T, 3)
+
+    out = {
+        "metric": "fwd+bwd batch*timesteps/sec" if backward else "fwd batch*timesteps/sec",
+        "value": round(B * T / (ms * 1e-3), 1),
+        "unit": "batch*timesteps/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms, 4), "wall_ms_per_step": round(wall_ms, 4),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "fp16 storage, fp32 accumulate, fp32 cell state", "data": "synthetic",
+        "config": {"workload": f"{args.workload}: single-layer LSTM {'fwd+bwd with fp16 gate cache' if backward else 'forward'}"
+                               f", I={I}, H={H}, B={B}, T={T}", "T": T, "B": B, "I": I, "H": H},
+        "mfu": round(flops / (ms * 1e-3) / (PEAK_FP16_TFLOPS * 1e12), 4),
+        "mfu_target": 0.40, "tflops": round(flops / (ms * 1e-3) / 1e12, 1), "flops_per_step": flops,
+        "persistent": {"fwd": core.info("persistent_fwd"), "bwd": core.info("persistent_bwd"),
+                       "xcd_local_fwd": core.info("xcd_local_fwd"), "xcd_local_bwd": core.info("xcd_local_bwd"),
+                       "fallbacks": core.info("fallbacks")},
+        "roofline": roofline, "kernels": kernels,
+    }
+    core.close()
+    if not args.no_parity:
+        out["parity"] = parity_check(B, I, H)
+    if not args.no_cpu_baseline:
+        out["cpu_baseline"] = cpu_baseline(B, I, H, backward)
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

@@ -62,12 +62,14 @@ struct flstm_core_plan {
     DevBuf wih_p, wih_t, wfrag_f, wfrag_b, bias_p;
     bool weights_packed = false, bias_packed = false;
     // forward state / caches
-    DevBuf X16, G, Y, C, flags_f, flags_b, status;
+    DevBuf X16, G, Y, C, flags_f, flags_b, status, xch_f, xch_b;
     unsigned epoch_f = 0, epoch_b = 0;
     size_t T_cache = 0;
     bool have_cache = false;
     // backward scratch
-    DevBuf dYp, dG, dGT, XHT, dHn, dC, dH0, db_part, dw_part;
+    DevBuf dYp, dG, dGT, XHT, dHn, dC, dH0, db_part, dw_part, prof;
+    int opt_profile = 0, wall_khz = 100000;
+    long long prof_f[8] = {}, prof_b[8] = {};
     PhaseTimer tm;
     float ms_fwd[3] = {-1, -1, -1}, ms_bwd[4] = {-1, -1, -1, -1};
 };
@@ -134,8 +136,8 @@ extern "C" int flstm_core_create(size_t batch, size_t input_size, size_t hidden_
 extern "C" int flstm_core_destroy(flstm_core_plan* p) {
     if (!p) return FLSTM_E_INVALID;
     for (DevBuf* b : {&p->wih_p, &p->wih_t, &p->wfrag_f, &p->wfrag_b, &p->bias_p, &p->X16, &p->G, &p->Y, &p->C,
-                      &p->flags_f, &p->flags_b, &p->status, &p->dYp, &p->dG, &p->dGT, &p->XHT, &p->dHn, &p->dC,
-                      &p->dH0, &p->db_part, &p->dw_part})
+                      &p->flags_f, &p->flags_b, &p->status, &p->xch_f, &p->xch_b, &p->dYp, &p->dG, &p->dGT, &p->XHT, &p->dHn, &p->dC,
+                      &p->dH0, &p->db_part, &p->dw_part, &p->prof})
         b->release();
     p->tm.destroy();
     delete p;
@@ -147,6 +149,17 @@ extern "C" int flstm_core_set_option(flstm_core_plan* p, const char* name, long 
     if (!strcmp(name, "stepwise")) { p->opt_stepwise = value != 0; replan(p); return 0; }
     if (!strcmp(name, "proj_chunk")) { p->opt_proj_chunk = int(value); return 0; }
     if (!strcmp(name, "spin_limit")) { if (value < 1) return FLSTM_E_INVALID; p->opt_spin_limit = int(value); return 0; }
+    if (!strcmp(name, "profile")) {
+        p->opt_profile = value != 0;
+        if (p->opt_profile) {
+            FL_TRY(p->prof.reserve(16 * sizeof(long long)));
+            int dev = 0;
+            FL_TRY(hipGetDevice(&dev));
+            (void)hipDeviceGetAttribute(&p->wall_khz, hipDeviceAttributeWallClockRate, dev);
+            if (p->wall_khz <= 0) p->wall_khz = 100000;
+        }
+        return 0;
+    }
     if (!strcmp(name, "dw_splits")) { if (value < 0) return FLSTM_E_INVALID; p->opt_dw_splits = int(value); return 0; }
     return FLSTM_E_INVALID;
 }
@@ -233,6 +246,9 @@ int forward_once(flstm_core_plan* p, size_t T, const void* x, flstm_dtype x_dtyp
                                size_t(d.B), size_t(d.Hp), s));
     else FL_TRY(fill_zero(p->Y.p, size_t(d.B) * d.Hp * sizeof(half_t), s));
     FL_TRY(convert_pad_f32(c0, state_dtype == FLSTM_F32, size_t(d.B), d.H, 1.f, p->C.as<float>(), size_t(d.Hp), s));
+    const size_t xslot = exchange_slot_halfs(d.B, d.Hp);
+    FL_TRY(p->xch_f.reserve(2 * xslot * sizeof(half_t)));
+    FL_TRY(to_exchange_layout(p->Y.as<half_t>(), d.B, d.Hp, size_t(d.Hp), p->xch_f.as<half_t>(), s));
 
     FL_TRY(hipEventRecord(p->tm.ev[0], s));
     // hoisted input projection, optionally in chunks of time steps
@@ -251,12 +267,18 @@ int forward_once(flstm_core_plan* p, size_t T, const void* x, flstm_dtype x_dtyp
     RecFwdArgs a{};
     a.wfrag = p->wfrag_f.as<half8>();
     a.Y = p->Y.as<half_t>(); a.G = p->G.as<half_t>(); a.C = p->C.as<float>();
+    a.X = p->xch_f.as<half_t>(); a.x_slot = xslot;
     a.bias = p->bias_p.as<float>();
     a.flags = p->flags_f.as<unsigned>(); a.status = p->status.as<int>();
     a.seats = p->status.as<unsigned>() + 8;
     FL_TRY(fill_zero(a.seats, 8 * sizeof(unsigned), s));
     a.B = d.B; a.Hp = d.Hp; a.T = int(T);
     a.epoch = p->epoch_f; a.spin_limit = p->opt_spin_limit;
+    a.prof = nullptr;
+    if (p->opt_profile) {
+        FL_TRY(fill_zero(p->prof.p, 16 * sizeof(long long), s));
+        a.prof = p->prof.as<long long>();
+    }
     FL_TRY(launch_rec_fwd(p->Lf, a, s));
     p->epoch_f += unsigned(T) + 1;
     FL_TRY(hipEventRecord(p->tm.ev[2], s));
@@ -297,6 +319,7 @@ extern "C" int flstm_core_forward(flstm_core_plan* p, size_t T, const void* x, f
         if (rc) return rc;
         if (st != 0) return FLSTM_E_STALLED;
     }
+    if (p->opt_profile) FL_TRY(hipMemcpy(p->prof_f, p->prof.p, sizeof(p->prof_f), hipMemcpyDeviceToHost));
     p->ms_fwd[0] = elapsed(p->tm.ev[0], p->tm.ev[1]);
     p->ms_fwd[1] = elapsed(p->tm.ev[1], p->tm.ev[2]);
     p->ms_fwd[2] = elapsed(p->tm.ev[0], p->tm.ev[2]);
@@ -335,6 +358,8 @@ int backward_rec_once(flstm_core_plan* p, size_t T, const void* dY, flstm_dtype 
     FL_TRY(p->dG.reserve(TB * 4 * d.Hp * sizeof(half_t)));
     FL_TRY(p->db_part.reserve(size_t(p->Lb.ng) * 4 * d.Hp * sizeof(float)));
     FL_TRY(p->flags_b.reserve(size_t(p->Lb.ng) * 256 * sizeof(unsigned)));
+    const size_t xslot = exchange_slot_halfs(d.B, 4 * d.Hp);
+    FL_TRY(p->xch_b.reserve(2 * xslot * sizeof(half_t)));
     if (p->epoch_b == 0 || p->epoch_b > 0x70000000u) {
         FL_TRY(fill_zero(p->flags_b.p, p->flags_b.bytes, s));
         p->epoch_b = 0;
@@ -348,12 +373,18 @@ int backward_rec_once(flstm_core_plan* p, size_t T, const void* dY, flstm_dtype 
     a.wfrag = p->wfrag_b.as<half8>();
     a.G = p->G.as<half_t>(); a.C = p->C.as<float>(); a.dY = dYk; a.dG = p->dG.as<half_t>();
     a.dHn = p->dHn.as<float>(); a.dC = p->dC.as<float>(); a.dH0 = p->dH0.as<float>();
+    a.X = p->xch_b.as<half_t>(); a.x_slot = xslot;
     a.db_part = p->db_part.as<float>();
     a.flags = p->flags_b.as<unsigned>(); a.status = p->status.as<int>();
     a.seats = p->status.as<unsigned>() + 8;
     FL_TRY(fill_zero(a.seats, 8 * sizeof(unsigned), s));
     a.B = d.B; a.Hp = d.Hp; a.T = int(T); a.jb_fwd = d.JF; a.dy_scale = dy_scale;
     a.epoch = p->epoch_b; a.spin_limit = p->opt_spin_limit;
+    a.prof = nullptr;
+    if (p->opt_profile) {
+        FL_TRY(fill_zero(p->prof.p, 16 * sizeof(long long), s));
+        a.prof = p->prof.as<long long>() + 8;
+    }
     FL_TRY(launch_rec_bwd(p->Lb, a, s));
     p->epoch_b += unsigned(T) + 2;
     FL_TRY(hipEventRecord(p->tm.ev[4], s));
@@ -440,6 +471,8 @@ extern "C" int flstm_core_backward(flstm_core_plan* p, size_t T, const void* x, 
     FL_TRY(unpad_from_float(p->dC.as<float>(), size_t(d.Hp), size_t(d.B), d.H, invS, dc0, 1, s));
     FL_TRY(hipEventRecord(p->tm.ev[7], s));
     FL_TRY(hipStreamSynchronize(s));
+    if (p->opt_profile)
+        FL_TRY(hipMemcpy(p->prof_b, p->prof.as<long long>() + 8, sizeof(p->prof_b), hipMemcpyDeviceToHost));
     p->ms_bwd[0] = elapsed(p->tm.ev[3], p->tm.ev[4]);
     p->ms_bwd[1] = elapsed(p->tm.ev[4], p->tm.ev[5]);
     p->ms_bwd[2] = elapsed(p->tm.ev[5], p->tm.ev[6]);
@@ -466,5 +499,10 @@ extern "C" double flstm_core_last_ms(const flstm_core_plan* p, const char* phase
     if (!strcmp(phase, "bwd_dx")) return p->ms_bwd[1];
     if (!strcmp(phase, "bwd_dw")) return p->ms_bwd[2];
     if (!strcmp(phase, "bwd_total")) return p->ms_bwd[3];
+    // cycle counters of workgroup 0 (option "profile"): wait, product, partials, pointwise, publish
+    if (!strncmp(phase, "fwd_clk", 7) && phase[7] >= '0' && phase[7] <= '7')
+        return double(p->prof_f[phase[7] - '0']) / p->wall_khz;
+    if (!strncmp(phase, "bwd_clk", 7) && phase[7] >= '0' && phase[7] <= '7')
+        return double(p->prof_b[phase[7] - '0']) / p->wall_khz;
     return -1.0;
 }

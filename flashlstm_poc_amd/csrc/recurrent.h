@@ -21,7 +21,9 @@ struct RecLayout {
 
 struct RecFwdArgs {
     const half8* wfrag;  // [nh][4 waves][ks][nt][64 lanes] MFMA B-fragments of W_hh (packed gate order)
-    half_t* Y;           // [(T+1)*B + pad][Hp]; rows [0,B) = h0, rows [(t+1)B, (t+2)B) = h_t
+    half_t* Y;           // [(T+1)*B][Hp]; rows [0,B) = h0, rows [(t+1)B, (t+2)B) = h_t (row-major, for later kernels)
+    half_t* X;           // exchange ring, 2 slots of x_slot halfs, fragment-major; step t reads slot t&1 (h_{t-1})
+    size_t x_slot;
     half_t* G;           // [T*B][4Hp] packed gate order; in: x-projection, out: activated i,f,g,o
     float* C;            // [(T+1)*B][Hp]; rows [0,B) = c0, rows [(t+1)B, ..) = c_t
     const float* bias;   // [4Hp] packed gate order, b_ih + b_hh
@@ -31,6 +33,7 @@ struct RecFwdArgs {
     int B, Hp, T;
     unsigned epoch;
     int spin_limit;
+    long long* prof;     // optional [8] cycle counters of workgroup 0 per phase (null = off)
 };
 
 struct RecBwdArgs {
@@ -38,7 +41,9 @@ struct RecBwdArgs {
     const half_t* G;     // activated gates cache [T*B][4Hp]
     const float* C;      // cell states [(T+1)*B][Hp]
     const half_t* dY;    // [T*B][Hp] upstream gradient
-    half_t* dG;          // [T*B + pad][4Hp] pre-activation gradients (scaled by grad_scale)
+    half_t* dG;          // [T*B][4Hp] pre-activation gradients (scaled), row-major, for the GEMMs
+    half_t* X;           // exchange ring, 2 slots of x_slot halfs, fragment-major; step t writes slot t&1 (dG_t)
+    size_t x_slot;
     float* dHn;          // [B][Hp] scaled gradient wrt final h (zeros when absent)
     float* dC;           // [B][Hp] running scaled dc; in: gradient wrt final c, out: dc0
     float* dH0;          // [B][Hp] out: scaled gradient wrt h0
@@ -51,11 +56,17 @@ struct RecBwdArgs {
     float dy_scale;      // factor applied to dY on load (the loss scale, or 1 when dY is pre-scaled)
     unsigned epoch;
     int spin_limit;
+    long long* prof;     // optional [8] cycle counters of workgroup 0 per phase (null = off)
 };
 
 // Picks tile shapes and the group structure for a problem size on the current device.
 RecLayout plan_rec_fwd(int B, int Hp, int num_cus, bool force_stepwise);
 RecLayout plan_rec_bwd(int B, int Hp, int num_cus, bool force_stepwise);
+
+// Halfs in one slot of an exchange ring for a [rows][cols] operand (rows padded to 32).
+size_t exchange_slot_halfs(int rows, int cols);
+// Row-major [rows][cols] (cols % 32 == 0) -> fragment-major exchange layout.
+hipError_t to_exchange_layout(const half_t* in, int rows, int cols, size_t ld, half_t* out, hipStream_t s);
 
 // Number of k-steps (32 wide) every wave holds for a layout (sizes the fragment arrays).
 int rec_fwd_ks(const RecLayout& L, int Hp);

@@ -106,8 +106,26 @@ __device__ __forceinline__ void publish(unsigned* gflags, int hs, unsigned value
         __hip_atomic_store(gflags + hs, value, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
+// Exchange layout ("fragment-major").  The operand a step fetches from its peers -- h_{t-1} in the
+// forward pass, dG_{t+1} in the backward pass -- is stored as ready-made MFMA A-fragments so that
+// every load instruction of a wave covers one contiguous 512-byte run:
+//   element (row r, column k) of a [rows][K] matrix, nks = K / 32, sits at (in halfs)
+//   ((((r/16)*nks + k/32)*2 + (k%8)/4)*64 + r%16 + 16*((k%32)/8))*4 + k%4
+// i.e. [16-row tile][32-wide k-step][low / high half of the lane's 8 values][lane][4 halfs].
+__device__ __forceinline__ size_t xch_offset(int r, int k, int nks) {
+    return ((((size_t(r / 16) * nks + k / 32) * 2 + (k % 8) / 4) * 64) + (r % 16) + 16 * ((k % 32) / 8)) * 4 + (k % 4);
+}
+
+// One A-fragment: two coalesced 8-byte device-scope loads (L1 bypass, served by the XCD's L2).
+__device__ __forceinline__ half8 ld_frag(const half_t* frag_lane) {
+    union { u64 q[2]; half8 h; } u;
+    u.q[0] = __hip_atomic_load(reinterpret_cast<const u64*>(frag_lane), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    u.q[1] = __hip_atomic_load(reinterpret_cast<const u64*>(frag_lane + 256), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    return u.h;
+}
+
 // acc[mt][nt] += A(32 rows x K) * Wslice, this wave's interleaved k-steps only.
-// a0/a1 point at (row, 8*(lane/16)) of the two 16-row tiles.
+// a0/a1: fragment (row tile, k-step 0) of the two 16-row tiles, already offset by lane*4 halfs.
 template <int NT, int KS, bool RESIDENT>
 __device__ __forceinline__ void wave_product(floatx4 (&acc)[2][NT], const half8 (&wreg)[KS][NT],
                                              const half8* wfrag_wave, const half_t* a0,
@@ -123,8 +141,8 @@ __device__ __forceinline__ void wave_product(floatx4 (&acc)[2][NT], const half8 
 #pragma unroll
             for (int k = 0; k < KC; ++k) {
                 const int kg = min((c * KC + k) * 4 + wave, nks_total - 1);
-                fa[k] = ld_half8_coherent(a0 + kg * 32);
-                fb[k] = ld_half8_coherent(a1 + kg * 32);
+                fa[k] = ld_frag(a0 + size_t(kg) * 512);
+                fb[k] = ld_frag(a1 + size_t(kg) * 512);
             }
 #pragma unroll
             for (int k = 0; k < KC; ++k) {
@@ -139,8 +157,8 @@ __device__ __forceinline__ void wave_product(floatx4 (&acc)[2][NT], const half8 
         for (int k = 0; k < ks_wave; ++k) {
             const int kg = k * 4 + wave;
             if (kg >= nks_total) break;
-            const half8 fa = ld_half8_coherent(a0 + kg * 32);
-            const half8 fb = ld_half8_coherent(a1 + kg * 32);
+            const half8 fa = ld_frag(a0 + size_t(kg) * 512);
+            const half8 fb = ld_frag(a1 + size_t(kg) * 512);
 #pragma unroll
             for (int n = 0; n < NT; ++n) {
                 const half8 w = wfrag_wave[(size_t(k) * NT + n) * kWave + lane];
@@ -181,13 +199,55 @@ __device__ __forceinline__ void load_h2(const half_t* src, float& a, float& b) {
     b = (float)v.h[1];
 }
 
+__device__ __forceinline__ void unpack_h2(unsigned u, float& a, float& b) {
+    union { half_t h[2]; unsigned u; } v;
+    v.u = u;
+    a = (float)v.h[0];
+    b = (float)v.h[1];
+}
+
+__device__ __forceinline__ unsigned pack_h2(float a, float b) {
+    union { half_t h[2]; unsigned u; } v;
+    v.h[0] = (half_t)a;
+    v.h[1] = (half_t)b;
+    return v.u;
+}
+
+__device__ __forceinline__ void store_u32(half_t* dst, unsigned u, bool device_scope) {
+    if (device_scope)
+        __hip_atomic_store(reinterpret_cast<unsigned*>(dst), u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    else
+        *reinterpret_cast<unsigned*>(dst) = u;
+}
+
+// Cycle counters of workgroup 0 per phase (only when the host passes a buffer): wait, product,
+// partial exchange, pointwise, publish.
+struct PhaseClock {
+    long long* out;
+    long long last;
+    __device__ __forceinline__ void start() { if (out) last = wall_clock64(); }
+    __device__ __forceinline__ void lap(int slot) {
+        if (out && threadIdx.x == 0) {
+            const long long now = wall_clock64();
+            out[slot] += now - last;
+            last = now;
+        }
+    }
+};
+
 // ------------------------------------------------------------------------------------ forward
+// Per step and row block: [wait for h_{t-1}] -> K-split MFMA product -> partial sums through LDS ->
+// pointwise cell update -> store h_t, publish -> store c_t and the activated gates -> prefetch the
+// next step's x-projection.  Only the h_t store and the flag sit between this step and the next one
+// of the other workgroups; everything HBM-bound (x-projection fetch, cache stores) is off that path.
 template <int NT, int KS, bool RESIDENT>
 __global__ __launch_bounds__(kThreads) void rec_fwd_kernel(RecFwdArgs p, RecLayout L, int t_begin,
                                                            int t_end, int ks_wave) {
     constexpr int JB = 4 * NT;    // hidden units of this slice
     constexpr int NC = 16 * NT;   // gate columns of this slice (i,f,g,o blocks of JB)
     constexpr int PLD = NC + 4;
+    constexpr int NPAIR = kRows * (JB / 2);                 // unit pairs per row block
+    constexpr int NP = (NPAIR + kThreads - 1) / kThreads;   // pairs per thread
     extern __shared__ __attribute__((aligned(16))) float part[];  // [4][32][PLD]
     __shared__ int lds_abort;
     __shared__ int lds_role[2];
@@ -200,6 +260,7 @@ __global__ __launch_bounds__(kThreads) void rec_fwd_kernel(RecFwdArgs p, RecLayo
     const int nks_total = p.Hp / 32;
     const bool device_scope = (L.persistent != 0) && (L.xcd_local == 0);
     unsigned* gflags = p.flags + size_t(g) * 256;
+    PhaseClock clk{(blockIdx.x == 0) ? p.prof : nullptr, 0};
 
     const half8* wfrag_wave = p.wfrag + (size_t(hs) * 4 + wave) * size_t(ks_wave) * NT * kWave;
     half8 wreg[KS][NT];
@@ -210,75 +271,139 @@ __global__ __launch_bounds__(kThreads) void rec_fwd_kernel(RecFwdArgs p, RecLayo
             for (int n = 0; n < NT; ++n)
                 wreg[k][n] = (k < ks_wave) ? wfrag_wave[(size_t(k) * NT + n) * kWave + lane] : half8{};
     }
-    __syncthreads();
 
     const size_t gld = size_t(4) * p.Hp;
+    // this thread's unit pairs: row r, units jj, jj+1 of the slice
+    int pr[NP], pj[NP];
+    bool pv[NP];
+    float2 bs[NP][4];
+#pragma unroll
+    for (int q = 0; q < NP; ++q) {
+        const int pidx = tid + q * kThreads;
+        pv[q] = pidx < NPAIR;
+        pr[q] = pv[q] ? pidx / (JB / 2) : 0;
+        pj[q] = pv[q] ? (pidx % (JB / 2)) * 2 : 0;
+#pragma unroll
+        for (int gt = 0; gt < 4; ++gt)
+            bs[q][gt] = *reinterpret_cast<const float2*>(p.bias + size_t(hs) * NC + gt * JB + pj[q]);
+    }
+    const int rb_count = (L.nrb - g + L.ng - 1) / L.ng;
+    const bool c_in_regs = (rb_count == 1) && (t_end - t_begin > 1);
+    float2 creg[NP];
+    unsigned xp[NP][4];
+    auto prefetch = [&](int t, int rb) {
+#pragma unroll
+        for (int q = 0; q < NP; ++q) {
+            const int b = rb * kRows + pr[q];
+            if (pv[q] && b < p.B) {
+                const half_t* src = p.G + (size_t(t) * p.B + b) * gld + size_t(hs) * NC + pj[q];
+#pragma unroll
+                for (int gt = 0; gt < 4; ++gt) xp[q][gt] = *reinterpret_cast<const unsigned*>(src + gt * JB);
+            }
+        }
+    };
+    if (c_in_regs) {
+#pragma unroll
+        for (int q = 0; q < NP; ++q) {
+            const int b = g * kRows + pr[q];
+            creg[q] = (pv[q] && b < p.B)
+                          ? *reinterpret_cast<const float2*>(p.C + (size_t(t_begin) * p.B + b) * p.Hp + hs * JB + pj[q])
+                          : float2{0.f, 0.f};
+        }
+    }
+    prefetch(t_begin, g);
+    __syncthreads();
+    clk.start();
+
     for (int t = t_begin; t < t_end; ++t) {
         if (t > t_begin) {
             if (!wait_group(gflags, L.nh, p.epoch + unsigned(t - t_begin), p.status, p.spin_limit, &lds_abort))
                 return;
         }
+        clk.lap(0);
         for (int rb = g; rb < L.nrb; rb += L.ng) {
             const int row0 = rb * kRows;
-            const int ra = min(row0 + lane % 16, p.B - 1);
-            const int rbw = min(row0 + 16 + lane % 16, p.B - 1);
-            const half_t* a0 = p.Y + (size_t(t) * p.B + ra) * p.Hp + 8 * (lane / 16);
-            const half_t* a1 = p.Y + (size_t(t) * p.B + rbw) * p.Hp + 8 * (lane / 16);
+            const half_t* xin = p.X + size_t(t & 1) * p.x_slot;        // h_{t-1}, fragment-major
+            half_t* xout = p.X + size_t((t + 1) & 1) * p.x_slot;       // h_t
+            const half_t* a0 = xin + size_t(2 * rb) * nks_total * 512 + lane * 4;
+            const half_t* a1 = a0 + size_t(nks_total) * 512;
             floatx4 acc[2][NT];
 #pragma unroll
             for (int m = 0; m < 2; ++m)
 #pragma unroll
                 for (int n = 0; n < NT; ++n) acc[m][n] = floatx4{0.f, 0.f, 0.f, 0.f};
             wave_product<NT, KS, RESIDENT>(acc, wreg, wfrag_wave, a0, a1, wave, lane, nks_total, ks_wave);
+            clk.lap(1);
             spill_partials<NT>(part, acc, wave, lane, PLD);
             __syncthreads();
+            clk.lap(2);
 
-            // Pointwise: every thread owns pairs of neighbouring hidden units of one batch row.
-            for (int pidx = tid; pidx < kRows * (JB / 2); pidx += kThreads) {
-                const int r = pidx / (JB / 2), jj = (pidx % (JB / 2)) * 2;
-                const int b = row0 + r;
-                if (b >= p.B) continue;
-                const size_t grow = (size_t(t) * p.B + b) * gld + size_t(hs) * NC;
+            unsigned act[NP][4], hnew[NP];
+            float2 cnew[NP];
+#pragma unroll
+            for (int q = 0; q < NP; ++q) {
+                const int b = row0 + pr[q];
+                if (!(pv[q] && b < p.B)) continue;
                 float z[4][2];
 #pragma unroll
                 for (int gt = 0; gt < 4; ++gt) {
-                    const int col = gt * JB + jj;
+                    const int col = gt * JB + pj[q];
                     float s0 = 0.f, s1 = 0.f;
 #pragma unroll
                     for (int w = 0; w < 4; ++w) {
-                        const float2 v = *reinterpret_cast<const float2*>(part + (size_t(w) * kRows + r) * PLD + col);
+                        const float2 v = *reinterpret_cast<const float2*>(part + (size_t(w) * kRows + pr[q]) * PLD + col);
                         s0 += v.x;
                         s1 += v.y;
                     }
                     float x0, x1;
-                    load_h2(p.G + grow + col, x0, x1);
-                    const float2 bs = *reinterpret_cast<const float2*>(p.bias + size_t(hs) * NC + col);
-                    z[gt][0] = s0 + x0 + bs.x;
-                    z[gt][1] = s1 + x1 + bs.y;
+                    unpack_h2(xp[q][gt], x0, x1);
+                    z[gt][0] = s0 + x0 + bs[q][gt].x;
+                    z[gt][1] = s1 + x1 + bs[q][gt].y;
                 }
-                const int j = hs * JB + jj;
-                const float2 cp = *reinterpret_cast<const float2*>(p.C + (size_t(t) * p.B + b) * p.Hp + j);
-                float cn[2], hn[2], act[4][2];
+                const int j = hs * JB + pj[q];
+                const float2 cp = c_in_regs ? creg[q]
+                                            : *reinterpret_cast<const float2*>(p.C + (size_t(t) * p.B + b) * p.Hp + j);
+                float cn[2], hn[2], a4[4][2];
 #pragma unroll
                 for (int u = 0; u < 2; ++u) {
                     const float ig = sigmoidf_dev(z[0][u]);
                     const float fg = sigmoidf_dev(z[1][u]);
-                    const float gg = tanhf(z[2][u]);
+                    const float gg = tanhf_dev(z[2][u]);
                     const float og = sigmoidf_dev(z[3][u]);
-                    const float cprev = (u == 0) ? cp.x : cp.y;
-                    cn[u] = fg * cprev + ig * gg;
-                    hn[u] = og * tanhf(cn[u]);
-                    act[0][u] = ig; act[1][u] = fg; act[2][u] = gg; act[3][u] = og;
+                    cn[u] = fg * (u == 0 ? cp.x : cp.y) + ig * gg;
+                    hn[u] = og * tanhf_dev(cn[u]);
+                    a4[0][u] = ig; a4[1][u] = fg; a4[2][u] = gg; a4[3][u] = og;
                 }
-                *reinterpret_cast<float2*>(p.C + (size_t(t + 1) * p.B + b) * p.Hp + j) = float2{cn[0], cn[1]};
+                // the exchanged value goes out first
+                hnew[q] = pack_h2(hn[0], hn[1]);
+                store_u32(xout + xch_offset(b, j, nks_total), hnew[q], device_scope);
+                cnew[q] = float2{cn[0], cn[1]};
+                creg[q] = cnew[q];
 #pragma unroll
-                for (int gt = 0; gt < 4; ++gt)
-                    store_h2(p.G + grow + gt * JB + jj, act[gt][0], act[gt][1], false);
-                store_h2(p.Y + (size_t(t + 1) * p.B + b) * p.Hp + j, hn[0], hn[1], device_scope);
+                for (int gt = 0; gt < 4; ++gt) act[q][gt] = pack_h2(a4[gt][0], a4[gt][1]);
             }
-            __syncthreads();
+            clk.lap(3);
+            const bool last_rb = (rb + L.ng >= L.nrb);
+            if (last_rb) publish(gflags, hs, p.epoch + unsigned(t - t_begin + 1));
+            else __syncthreads();
+            clk.lap(4);
+            // caches for the backward pass: off the critical path
+#pragma unroll
+            for (int q = 0; q < NP; ++q) {
+                const int b = row0 + pr[q];
+                if (!(pv[q] && b < p.B)) continue;
+                const int j = hs * JB + pj[q];
+                *reinterpret_cast<float2*>(p.C + (size_t(t + 1) * p.B + b) * p.Hp + j) = cnew[q];
+                *reinterpret_cast<unsigned*>(p.Y + (size_t(t + 1) * p.B + b) * p.Hp + j) = hnew[q];
+                half_t* dst = p.G + (size_t(t) * p.B + b) * gld + size_t(hs) * NC + pj[q];
+#pragma unroll
+                for (int gt = 0; gt < 4; ++gt) *reinterpret_cast<unsigned*>(dst + gt * JB) = act[q][gt];
+            }
+            // x-projection of the next work item
+            int nt_ = t, nrb_ = rb + L.ng;
+            if (nrb_ >= L.nrb) { nt_ = t + 1; nrb_ = g; }
+            if (nt_ < t_end) prefetch(nt_, nrb_);
         }
-        publish(gflags, hs, p.epoch + unsigned(t - t_begin + 1));
     }
 }
 
@@ -290,6 +415,8 @@ __global__ __launch_bounds__(kThreads) void rec_bwd_kernel(RecBwdArgs p, RecLayo
                                                            int t_last, int ks_wave) {
     constexpr int JB = 16 * NT;  // hidden units (= output columns of dG*W_hh) of this slice
     constexpr int PLD = JB + 4;
+    constexpr int NPAIR = kRows * (JB / 2);
+    constexpr int NP = (NPAIR + kThreads - 1) / kThreads;
     extern __shared__ __attribute__((aligned(16))) float part[];  // [4][32][PLD], reused for db
     __shared__ int lds_abort;
     __shared__ int lds_role[2];
@@ -303,6 +430,7 @@ __global__ __launch_bounds__(kThreads) void rec_bwd_kernel(RecBwdArgs p, RecLayo
     const bool device_scope = (L.persistent != 0) && (L.xcd_local == 0);
     unsigned* gflags = p.flags + size_t(g) * 256;
     const float S = p.dy_scale;
+    PhaseClock clk{(blockIdx.x == 0) ? p.prof : nullptr, 0};
 
     const half8* wfrag_wave = p.wfrag + (size_t(hs) * 4 + wave) * size_t(ks_wave) * NT * kWave;
     half8 wreg[KS][NT];
@@ -313,11 +441,54 @@ __global__ __launch_bounds__(kThreads) void rec_bwd_kernel(RecBwdArgs p, RecLayo
             for (int n = 0; n < NT; ++n)
                 wreg[k][n] = (k < ks_wave) ? wfrag_wave[(size_t(k) * NT + n) * kWave + lane] : half8{};
     }
-    __syncthreads();
 
     const size_t gld = size_t(4) * p.Hp;
     const int JF = p.jb_fwd;
+    int pr[NP], pj[NP];
+    bool pv[NP];
+    size_t pq[NP];  // packed gate column of (unit j, gate 0)
+#pragma unroll
+    for (int q = 0; q < NP; ++q) {
+        const int pidx = tid + q * kThreads;
+        pv[q] = pidx < NPAIR;
+        pr[q] = pv[q] ? pidx / (JB / 2) : 0;
+        pj[q] = pv[q] ? (pidx % (JB / 2)) * 2 : 0;
+        const int j = hs * JB + pj[q];
+        pq[q] = size_t(j / JF) * 4 * JF + (j % JF);
+    }
+    const int rb_count = (L.nrb - g + L.ng - 1) / L.ng;
+    const bool dc_in_regs = (rb_count == 1) && (t_first - t_last > 0);
+    float2 dcreg[NP];
+    if (dc_in_regs) {
+#pragma unroll
+        for (int q = 0; q < NP; ++q) {
+            const int b = g * kRows + pr[q];
+            dcreg[q] = (pv[q] && b < p.B) ? *reinterpret_cast<const float2*>(p.dC + size_t(b) * p.Hp + hs * JB + pj[q])
+                                          : float2{0.f, 0.f};
+        }
+    }
+    // prefetched per work item: activated gates, c_{t-1}, c_t, dY_t
+    unsigned pg[NP][4], pdy[NP];
+    float2 pcp[NP], pcc[NP];
+    auto prefetch = [&](int t, int rb) {
+#pragma unroll
+        for (int q = 0; q < NP; ++q) {
+            const int b = rb * kRows + pr[q];
+            if (pv[q] && b < p.B) {
+                const int j = hs * JB + pj[q];
+                const half_t* gsrc = p.G + (size_t(t) * p.B + b) * gld + pq[q];
+#pragma unroll
+                for (int gt = 0; gt < 4; ++gt) pg[q][gt] = *reinterpret_cast<const unsigned*>(gsrc + gt * JF);
+                pcp[q] = *reinterpret_cast<const float2*>(p.C + (size_t(t) * p.B + b) * p.Hp + j);
+                pcc[q] = *reinterpret_cast<const float2*>(p.C + (size_t(t + 1) * p.B + b) * p.Hp + j);
+                pdy[q] = *reinterpret_cast<const unsigned*>(p.dY + (size_t(t) * p.B + b) * p.Hp + j);
+            }
+        }
+    };
+    if (t_first >= 0) prefetch(t_first, g);
+    __syncthreads();
     float dbacc[4][2] = {{0.f, 0.f}, {0.f, 0.f}, {0.f, 0.f}, {0.f, 0.f}};
+    clk.start();
 
     for (int t = t_first; t >= t_last; --t) {
         const bool from_product = (t < p.T - 1);
@@ -325,34 +496,39 @@ __global__ __launch_bounds__(kThreads) void rec_bwd_kernel(RecBwdArgs p, RecLayo
             if (!wait_group(gflags, L.nh, p.epoch + unsigned(t_first - t), p.status, p.spin_limit, &lds_abort))
                 return;
         }
+        clk.lap(0);
         for (int rb = g; rb < L.nrb; rb += L.ng) {
             const int row0 = rb * kRows;
             if (from_product) {
-                const int ra = min(row0 + lane % 16, p.B - 1);
-                const int rbw = min(row0 + 16 + lane % 16, p.B - 1);
-                const half_t* a0 = p.dG + (size_t(t + 1) * p.B + ra) * gld + 8 * (lane / 16);
-                const half_t* a1 = p.dG + (size_t(t + 1) * p.B + rbw) * gld + 8 * (lane / 16);
+                const half_t* xin = p.X + size_t((t + 1) & 1) * p.x_slot;   // dG_{t+1}, fragment-major
+                const half_t* a0 = xin + size_t(2 * rb) * nks_total * 512 + lane * 4;
+                const half_t* a1 = a0 + size_t(nks_total) * 512;
                 floatx4 acc[2][NT];
 #pragma unroll
                 for (int m = 0; m < 2; ++m)
 #pragma unroll
                     for (int n = 0; n < NT; ++n) acc[m][n] = floatx4{0.f, 0.f, 0.f, 0.f};
                 wave_product<NT, KS, RESIDENT>(acc, wreg, wfrag_wave, a0, a1, wave, lane, nks_total, ks_wave);
+                clk.lap(1);
                 spill_partials<NT>(part, acc, wave, lane, PLD);
                 __syncthreads();
+                clk.lap(2);
             }
-            for (int pidx = tid; pidx < kRows * (JB / 2); pidx += kThreads) {
-                const int r = pidx / (JB / 2), jj = (pidx % (JB / 2)) * 2;
-                const int b = row0 + r;
-                if (b >= p.B) continue;
-                const int j = hs * JB + jj;
+            float2 dcnew[NP];
+            unsigned dgnew[NP][4];
+            half_t* xout = p.X + size_t(t & 1) * p.x_slot;   // dG_t for the peers
+#pragma unroll
+            for (int q = 0; q < NP; ++q) {
+                const int b = row0 + pr[q];
+                if (!(pv[q] && b < p.B)) continue;
+                const int j = hs * JB + pj[q];
                 const size_t sidx = size_t(b) * p.Hp + j;
                 float dh[2];
                 if (from_product) {
                     dh[0] = 0.f; dh[1] = 0.f;
 #pragma unroll
                     for (int w = 0; w < 4; ++w) {
-                        const float2 v = *reinterpret_cast<const float2*>(part + (size_t(w) * kRows + r) * PLD + jj);
+                        const float2 v = *reinterpret_cast<const float2*>(part + (size_t(w) * kRows + pr[q]) * PLD + pj[q]);
                         dh[0] += v.x;
                         dh[1] += v.y;
                     }
@@ -360,30 +536,33 @@ __global__ __launch_bounds__(kThreads) void rec_bwd_kernel(RecBwdArgs p, RecLayo
                     const float2 v = *reinterpret_cast<const float2*>(p.dHn + sidx);
                     dh[0] = v.x; dh[1] = v.y;
                 }
-                if (t < 0) {  // closing pass: gradient wrt h0; dc0 already sits in dC
+                if (t < 0) {  // closing pass: gradient wrt h0; dc0 is the running dc
                     *reinterpret_cast<float2*>(p.dH0 + sidx) = float2{dh[0], dh[1]};
+                    if (dc_in_regs) *reinterpret_cast<float2*>(p.dC + sidx) = dcreg[q];
                     continue;
                 }
                 float dy0, dy1;
-                load_h2(p.dY + (size_t(t) * p.B + b) * p.Hp + j, dy0, dy1);
+                unpack_h2(pdy[q], dy0, dy1);
                 dh[0] += S * dy0;
                 dh[1] += S * dy1;
-                union { u64 q; float2 f; } dcu;
-                dcu.q = __hip_atomic_load(reinterpret_cast<const u64*>(p.dC + sidx), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                const float2 cprev = *reinterpret_cast<const float2*>(p.C + (size_t(t) * p.B + b) * p.Hp + j);
-                const float2 ccur = *reinterpret_cast<const float2*>(p.C + (size_t(t + 1) * p.B + b) * p.Hp + j);
-                // packed gate column of unit j, gate gt: (j / JF) * 4JF + gt * JF + j % JF
-                const size_t grow = (size_t(t) * p.B + b) * gld + size_t(j / JF) * 4 * JF + (j % JF);
+                float2 dcin;
+                if (dc_in_regs) {
+                    dcin = dcreg[q];
+                } else {
+                    union { u64 q64; float2 f; } dcu;
+                    dcu.q64 = __hip_atomic_load(reinterpret_cast<const u64*>(p.dC + sidx), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    dcin = dcu.f;
+                }
                 float gate[4][2];
 #pragma unroll
-                for (int gt = 0; gt < 4; ++gt) load_h2(p.G + grow + gt * JF, gate[gt][0], gate[gt][1]);
+                for (int gt = 0; gt < 4; ++gt) unpack_h2(pg[q][gt], gate[gt][0], gate[gt][1]);
                 float da[4][2], dcp[2];
 #pragma unroll
                 for (int u = 0; u < 2; ++u) {
                     const float ig = gate[0][u], fg = gate[1][u], gg = gate[2][u], og = gate[3][u];
-                    const float tc = tanhf(u == 0 ? ccur.x : ccur.y);
-                    const float cpv = (u == 0) ? cprev.x : cprev.y;
-                    const float dcn = (u == 0) ? dcu.f.x : dcu.f.y;
+                    const float tc = tanhf_dev(u == 0 ? pcc[q].x : pcc[q].y);
+                    const float cpv = (u == 0) ? pcp[q].x : pcp[q].y;
+                    const float dcn = (u == 0) ? dcin.x : dcin.y;
                     const float dov = dh[u] * tc;
                     const float dc = dcn + dh[u] * og * (1.f - tc * tc);
                     da[0][u] = dc * gg * ig * (1.f - ig);
@@ -392,20 +571,48 @@ __global__ __launch_bounds__(kThreads) void rec_bwd_kernel(RecBwdArgs p, RecLayo
                     da[3][u] = dov * og * (1.f - og);
                     dcp[u] = dc * fg;
                 }
-                *reinterpret_cast<float2*>(p.dC + sidx) = float2{dcp[0], dcp[1]};
 #pragma unroll
                 for (int gt = 0; gt < 4; ++gt) {
                     // db sums the values the weight-gradient GEMMs will see (fp16-rounded)
-                    const half_t h0 = (half_t)da[gt][0], h1 = (half_t)da[gt][1];
-                    dbacc[gt][0] += (float)h0;
-                    dbacc[gt][1] += (float)h1;
-                    store_h2(p.dG + (size_t(t) * p.B + b) * gld + size_t(j / JF) * 4 * JF + (j % JF) + gt * JF,
-                             da[gt][0], da[gt][1], device_scope);
+                    const unsigned u32 = pack_h2(da[gt][0], da[gt][1]);
+                    float r0, r1;
+                    unpack_h2(u32, r0, r1);
+                    dbacc[gt][0] += r0;
+                    dbacc[gt][1] += r1;
+                    dgnew[q][gt] = u32;
+                    store_u32(xout + xch_offset(b, int(pq[q]) + gt * JF, nks_total), u32, device_scope);
+                }
+                dcnew[q] = float2{dcp[0], dcp[1]};
+                dcreg[q] = dcnew[q];
+            }
+            clk.lap(3);
+            const bool last_rb = (rb + L.ng >= L.nrb);
+            if (last_rb && t >= 0) publish(gflags, hs, p.epoch + unsigned(t_first - t + 1));
+            else __syncthreads();
+            clk.lap(4);
+            if (t >= 0) {   // row-major dG for the GEMMs that follow; running dc when it lives in memory
+#pragma unroll
+                for (int q = 0; q < NP; ++q) {
+                    const int b = row0 + pr[q];
+                    if (!(pv[q] && b < p.B)) continue;
+                    half_t* gdst = p.dG + (size_t(t) * p.B + b) * gld + pq[q];
+#pragma unroll
+                    for (int gt = 0; gt < 4; ++gt) *reinterpret_cast<unsigned*>(gdst + gt * JF) = dgnew[q][gt];
+                    if (!dc_in_regs) *reinterpret_cast<float2*>(p.dC + size_t(b) * p.Hp + hs * JB + pj[q]) = dcnew[q];
                 }
             }
-            __syncthreads();
+            int nt_ = t, nrb_ = rb + L.ng;
+            if (nrb_ >= L.nrb) { nt_ = t - 1; nrb_ = g; }
+            if (nt_ >= t_last && nt_ >= 0) prefetch(nt_, nrb_);
         }
-        if (t >= 0) publish(gflags, hs, p.epoch + unsigned(t_first - t + 1));
+    }
+    // single-step launches leave dc in memory for the next launch
+    if (dc_in_regs && t_last >= 0) {
+#pragma unroll
+        for (int q = 0; q < NP; ++q) {
+            const int b = g * kRows + pr[q];
+            if (pv[q] && b < p.B) *reinterpret_cast<float2*>(p.dC + size_t(b) * p.Hp + hs * JB + pj[q]) = dcreg[q];
+        }
     }
 
     // Bias gradient: fold this launch's sums over the threads that share a unit pair (fixed order).
@@ -419,14 +626,24 @@ __global__ __launch_bounds__(kThreads) void rec_bwd_kernel(RecBwdArgs p, RecLayo
     __syncthreads();
     constexpr int PAIRS = JB / 2;
     if (tid < PAIRS * 8) {
-        const int pr = tid / 8, e = tid % 8;  // pair, (gate, unit)
-        float s = 0.f;
-        for (int k = pr; k < kThreads; k += PAIRS) s += red[k * 8 + e];
+        const int prr = tid / 8, e = tid % 8;  // pair, (gate, unit)
+        float sum = 0.f;
+        for (int k = prr; k < kThreads; k += PAIRS) sum += red[k * 8 + e];
         const int gt = e / 2, u = e % 2;
-        const int j = hs * JB + pr * 2 + u;
+        const int j = hs * JB + prr * 2 + u;
         const size_t q = size_t(j / JF) * 4 * JF + size_t(gt) * JF + (j % JF);
-        p.db_part[size_t(g) * gld + q] += s;
+        p.db_part[size_t(g) * gld + q] += sum;
     }
+}
+
+// rows x cols row-major (ld) -> fragment-major exchange layout (one thread per pair of halfs)
+__global__ void to_exchange_layout_kernel(const half_t* __restrict__ in, int rows, int cols, size_t ld,
+                                          half_t* __restrict__ out, int nks) {
+    const size_t idx = size_t(blockIdx.x) * blockDim.x + threadIdx.x;
+    const size_t pairs = size_t(rows) * (cols / 2);
+    if (idx >= pairs) return;
+    const int r = int(idx / (cols / 2)), k = int(idx % (cols / 2)) * 2;
+    *reinterpret_cast<unsigned*>(out + xch_offset(r, k, nks)) = *reinterpret_cast<const unsigned*>(in + size_t(r) * ld + k);
 }
 
 template <typename K>
@@ -435,6 +652,17 @@ hipError_t raise_lds(K kernel, size_t bytes) {
 }
 
 }  // namespace
+
+hipError_t to_exchange_layout(const half_t* in, int rows, int cols, size_t ld, half_t* out, hipStream_t s) {
+    if (rows <= 0 || cols <= 0) return hipSuccess;
+    if (cols % 32 != 0) return hipErrorInvalidValue;
+    const size_t pairs = size_t(rows) * (cols / 2);
+    hipLaunchKernelGGL(to_exchange_layout_kernel, dim3(unsigned((pairs + 255) / 256)), dim3(256), 0, s, in, rows, cols,
+                       ld, out, cols / 32);
+    return hipGetLastError();
+}
+
+size_t exchange_slot_halfs(int rows, int cols) { return round_up(size_t(rows), 32) * size_t(cols); }
 
 int rec_fwd_ks(const RecLayout&, int Hp) { return int(ceil_div(size_t(Hp) / 32, 4)); }
 int rec_bwd_ks(const RecLayout&, int Hp) { return int(ceil_div(size_t(Hp) / 8, 4)); }
