@@ -5,12 +5,14 @@
 // input gradient dX = dG*W_ih and the weight gradients dW = dG^T*[X;H] (reference:
 // flashlstm_v2/src/lstm_backward.cu:1112-1172 through flashlstm_v2/src/gemm.cu:222-330).
 //
-// Tiling: one 256-thread workgroup (4 wavefronts, 2x2) owns a 256x256 tile of C; every wavefront
-// owns 128x128 as a 4x4 grid of v_mfma_f32_32x32x16_f16 tiles (256 accumulator registers).  K is
-// walked in slabs of 64: global -> registers -> LDS (row pitch padded to 72 halfs so that the
+// Tiling: one 256-thread workgroup (4 wavefronts, 2x2, one per SIMD) owns a 256x256 tile of C; every
+// wavefront owns 128x128 as a 4x4 grid of v_mfma_f32_32x32x16_f16 tiles (256 accumulator registers).
+// K is walked in slabs of 64: global -> registers -> LDS (row pitch padded to 72 halfs so that the
 // 16-byte fragment reads of 8 consecutive lanes fall in distinct banks), double buffered, one
-// workgroup barrier per slab.  Workgroups are numbered so that the 32 that share an XCD (block id
-// mod 8) work on neighbouring tiles and reuse each other's operand slabs in that XCD's L2.
+// workgroup barrier per slab.  The MFMA operands are swapped (D = B_tile * A_tile^T) so that a lane ends
+// up with four consecutive columns of one row of C and stores them as one 8- or 16-byte access.
+// Workgroups are numbered so that the 32 that share an XCD (block id mod 8) work on neighbouring tiles
+// and reuse each other's operand slabs in that XCD's L2.
 #include "gemm.h"
 
 namespace flstm_hip {
@@ -102,7 +104,7 @@ __global__ __launch_bounds__(kThreads) void gemm_nt_256x256(GemmNT g, int tiles_
             for (int i = 0; i < 4; ++i)
 #pragma unroll
                 for (int j = 0; j < 4; ++j)
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[i], bf[j], acc[i][j], 0, 0, 0);
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(bf[j], af[i], acc[i][j], 0, 0, 0);
         }
         if (more) {
             half_t* An = As + (cur ^ 1) * BM * LDS_LD + st_off;
@@ -116,25 +118,54 @@ __global__ __launch_bounds__(kThreads) void gemm_nt_256x256(GemmNT g, int tiles_
         __syncthreads();
     }
 
-    // Epilogue. Accumulator register r of a 32x32 tile holds row 8*(r/4) + 4*(lane/32) + r%4,
-    // column lane%32.
-    const int col_l = lane % 32;
-    const int row_l = 4 * (lane / 32);
+    // Epilogue.  With swapped operands register r of tile (i, j) holds row (i*32 + lane%32) of the
+    // wave's 128x128 block and column j*32 + 8*(r/4) + 4*(lane/32) + r%4: four consecutive columns per
+    // group of four registers.
+    const int row = m0 + wm * 128 + lane % 32;
+    const int colb = n0 + wn * 128 + 4 * (lane / 32);
     float* c32 = g.C32 ? g.C32 + size_t(z) * g.split_stride : nullptr;
+    const bool full = (m0 + BM <= g.M) && (n0 + BN <= g.N) && (g.ldc % 4 == 0);
+    if (full) {
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
+        for (int i = 0; i < 4; ++i) {
+            const size_t rowoff = size_t(row + i * 32) * g.ldc + colb;
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            const int col = n0 + wn * 128 + j * 32 + col_l;
-            if (col >= g.N) continue;
+            for (int j = 0; j < 4; ++j) {
 #pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                const int row = m0 + wm * 128 + i * 32 + 8 * (r / 4) + row_l + (r % 4);
-                if (row >= g.M) continue;
-                const size_t off = size_t(row) * g.ldc + col;
-                const float v = g.alpha * acc[i][j][r];
-                if (c32) c32[off] = v;
-                else g.C16[off] = (half_t)v;
+                for (int q = 0; q < 4; ++q) {
+                    const size_t off = rowoff + j * 32 + 8 * q;
+                    if (c32) {
+                        floatx4 v;
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) v[e] = g.alpha * acc[i][j][4 * q + e];
+                        *reinterpret_cast<floatx4*>(c32 + off) = v;
+                    } else {
+                        half4 v;
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) v[e] = (half_t)(g.alpha * acc[i][j][4 * q + e]);
+                        *reinterpret_cast<half4*>(g.C16 + off) = v;
+                    }
+                }
+                __builtin_amdgcn_sched_barrier(0);   // one 32x32 tile at a time: keeps register use flat
+            }
+        }
+    } else {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int r_ = row + i * 32;
+            if (r_ >= g.M) continue;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const int col = colb + j * 32 + 8 * (r / 4) + (r % 4);
+                    if (col >= g.N) continue;
+                    const size_t off = size_t(r_) * g.ldc + col;
+                    const float v = g.alpha * acc[i][j][r];
+                    if (c32) c32[off] = v;
+                    else g.C16[off] = (half_t)v;
+                }
+                __builtin_amdgcn_sched_barrier(0);
             }
         }
     }
@@ -146,6 +177,9 @@ hipError_t launch_gemm_nt(const GemmNT& g, hipStream_t stream) {
     if (g.M <= 0 || g.N <= 0 || g.K <= 0) return hipSuccess;
     if (g.K % BK != 0 || g.lda % 8 != 0 || g.ldb % 8 != 0) return hipErrorInvalidValue;
     if ((g.C16 == nullptr) == (g.C32 == nullptr)) return hipErrorInvalidValue;
+    // the vector stores of full tiles need an aligned base (rows are covered by the ldc % 4 test in the kernel)
+    if (g.C32 && (reinterpret_cast<uintptr_t>(g.C32) % 16 != 0 || g.split_stride % 4 != 0)) return hipErrorInvalidValue;
+    if (g.C16 && (reinterpret_cast<uintptr_t>(g.C16) % 8 != 0)) return hipErrorInvalidValue;
     int splits = g.splits < 1 ? 1 : g.splits;
     if (splits > 1 && g.C32 == nullptr) return hipErrorInvalidValue;
     const int nslab = g.K / BK;
