@@ -67,7 +67,7 @@ struct flstm_core_plan {
     size_t T_cache = 0;
     bool have_cache = false;
     // backward scratch
-    DevBuf dYp, dG, dGT, XHT, dHn, dC, dH0, db_part, dw_part, prof;
+    DevBuf dYp, dG, dHn, dC, dH0, db_part, dw_part, prof;
     int opt_profile = 0, wall_khz = 100000;
     long long prof_f[8] = {}, prof_b[8] = {};
     PhaseTimer tm;
@@ -136,7 +136,7 @@ extern "C" int flstm_core_create(size_t batch, size_t input_size, size_t hidden_
 extern "C" int flstm_core_destroy(flstm_core_plan* p) {
     if (!p) return FLSTM_E_INVALID;
     for (DevBuf* b : {&p->wih_p, &p->wih_t, &p->wfrag_f, &p->wfrag_b, &p->bias_p, &p->X16, &p->G, &p->Y, &p->C,
-                      &p->flags_f, &p->flags_b, &p->status, &p->xch_f, &p->xch_b, &p->dYp, &p->dG, &p->dGT, &p->XHT, &p->dHn, &p->dC,
+                      &p->flags_f, &p->flags_b, &p->status, &p->xch_f, &p->xch_b, &p->dYp, &p->dG, &p->dHn, &p->dC,
                       &p->dH0, &p->db_part, &p->dw_part, &p->prof})
         b->release();
     p->tm.destroy();
@@ -402,7 +402,7 @@ extern "C" int flstm_core_backward(flstm_core_plan* p, size_t T, const void* x, 
     if (T == 0) return 0;
     if (!p->have_cache || p->T_cache != T) return FLSTM_E_NO_CACHE;
     if (!dY) return FLSTM_E_INVALID;
-    if ((dW_ih || dW_hh) && !x) return FLSTM_E_INVALID;
+    if (dW_ih && !x) return FLSTM_E_INVALID;
     hipStream_t s = static_cast<hipStream_t>(stream);
     const Dims& d = p->d;
     const size_t TB = T * size_t(d.B);
@@ -440,30 +440,36 @@ extern "C" int flstm_core_backward(flstm_core_plan* p, size_t T, const void* x, 
     }
     FL_TRY(hipEventRecord(p->tm.ev[5], s));
 
-    if (dW_ih || dW_hh) {
-        const size_t TBp = round_up(TB, 64);
-        const int ncat = d.Ip + d.Hp;
-        FL_TRY(p->dGT.reserve(size_t(4) * d.Hp * TBp * sizeof(half_t)));
-        FL_TRY(p->XHT.reserve(size_t(ncat) * TBp * sizeof(half_t)));
-        FL_TRY(transpose_pad(p->dG.p, 0, TB, 4 * d.Hp, size_t(4) * d.Hp, p->dGT.as<half_t>(), 4 * d.Hp, TBp, s));
-        FL_TRY(transpose_pad(x, x_dtype == FLSTM_F32, TB, d.I, size_t(d.I), p->XHT.as<half_t>(), d.Ip, TBp, s));
-        // H_prev of step t is row block t of the state array (row block 0 = h0)
-        FL_TRY(transpose_pad(p->Y.p, 0, TB, d.Hp, size_t(d.Hp), p->XHT.as<half_t>() + size_t(d.Ip) * TBp, d.Hp, TBp, s));
-        const int tiles = int(ceil_div(size_t(4) * d.Hp, 256) * ceil_div(size_t(ncat), 256));
+    // dW_ih = dG^T * X and dW_hh = dG^T * H_prev: k-major operands exactly as the recurrence left them
+    // (H_prev of step t is row block t of the state array, row block 0 = h0), split over K, fp32 partials.
+    for (int which = 0; which < 2; ++which) {
+        float* dst = which == 0 ? dW_ih : dW_hh;
+        if (!dst) continue;
+        const half_t* Bop;
+        int ncols, out_cols;
+        size_t ldb;
+        if (which == 0) {
+            const bool direct = (x_dtype == FLSTM_F16 && d.I == d.Ip);
+            Bop = direct ? static_cast<const half_t*>(x) : p->X16.as<half_t>();
+            ncols = d.Ip; ldb = size_t(d.Ip); out_cols = d.I;
+        } else {
+            Bop = p->Y.as<half_t>();
+            ncols = d.Hp; ldb = size_t(d.Hp); out_cols = d.H;
+        }
+        const int tiles = int(ceil_div(size_t(4) * d.Hp, 256) * ceil_div(size_t(ncols), 256));
         int want = p->opt_dw_splits > 0 ? p->opt_dw_splits : int(ceil_div(1024, size_t(tiles)));
         if (want > 64) want = 64;
-        const int splits = gemm_effective_splits(int(TBp), want);
-        const size_t per = size_t(4) * d.Hp * ncat;
+        const int splits = gemm_effective_splits(int(TB), want);
+        const size_t per = size_t(4) * d.Hp * ncols;
         FL_TRY(p->dw_part.reserve(per * splits * sizeof(float)));
         GemmNT g{};
-        g.A = p->dGT.as<half_t>(); g.lda = TBp;
-        g.B = p->XHT.as<half_t>(); g.ldb = TBp;
-        g.M = 4 * d.Hp; g.N = ncat; g.K = int(TBp);
-        g.C16 = nullptr; g.C32 = p->dw_part.as<float>(); g.ldc = size_t(ncat);
+        g.A = p->dG.as<half_t>(); g.lda = size_t(4) * d.Hp;
+        g.B = Bop; g.ldb = ldb;
+        g.M = 4 * d.Hp; g.N = ncols; g.K = int(TB);
+        g.C16 = nullptr; g.C32 = p->dw_part.as<float>(); g.ldc = size_t(ncols);
         g.alpha = 1.f; g.splits = splits; g.split_stride = per;
-        FL_TRY(launch_gemm_nt(g, s));
-        // a null output still needs a valid address for the kernel's other half: route to scratch
-        FL_TRY(reduce_dw(d, p->dw_part.as<float>(), splits, invS, dW_ih, dW_hh, s));
+        FL_TRY(launch_gemm_tn(g, s));
+        FL_TRY(reduce_dw(d, p->dw_part.as<float>(), splits, ncols, out_cols, invS, dst, s));
     }
     FL_TRY(hipEventRecord(p->tm.ev[6], s));
     if (db_ih || db_hh) FL_TRY(reduce_db(d, p->db_part.as<float>(), p->Lb.ng, invS, db_ih, db_hh, s));

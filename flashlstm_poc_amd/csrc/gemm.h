@@ -19,7 +19,11 @@ struct GemmNT {
 // Enqueue on `stream`. Returns hipSuccess or the launch error.
 hipError_t launch_gemm_nt(const GemmNT& g, hipStream_t stream);
 
-// Number of K slices launch_gemm_nt really produces when `wanted` are asked for (every slice gets a
+// Same contraction with k-major operands: A is [K][M] (lda = row pitch, M % 8 == 0), B is [K][N]
+// (N % 8 == 0); K is arbitrary.  C[M][N] as above.
+hipError_t launch_gemm_tn(const GemmNT& g, hipStream_t stream);
+
+// Number of K slices the launchers really produce when `wanted` are asked for (every slice gets a
 // whole number of 64-wide K slabs). Size split-K partial buffers with this.
 int gemm_effective_splits(int K, int wanted);
 

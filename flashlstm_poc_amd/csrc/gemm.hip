@@ -20,109 +20,19 @@ namespace {
 
 constexpr int BM = 256, BN = 256, BK = 64;
 constexpr int LDS_LD = 72;  // halfs per LDS row (64 + 8 pad)
-constexpr int kThreads = 256;
+constexpr int kWavesN = 4;                 // wavefronts along N (2 along M): wave tile 128 x (256 / kWavesN)
+constexpr int kThreads = 128 * kWavesN;
+constexpr int kTN = 8 / kWavesN;            // 32-wide MFMA tiles per wave along N
+constexpr int kLd = 2048 / kThreads;        // 16-byte chunks per thread, operand and slab
 constexpr size_t kLdsBytes = size_t(2) * (BM + BN) * LDS_LD * sizeof(half_t);
 
-__global__ __launch_bounds__(kThreads) void gemm_nt_256x256(GemmNT g, int tiles_m, int tiles_n,
-                                                             int k_per_split) {
-    extern __shared__ __attribute__((aligned(16))) half_t smem[];
-    half_t* As = smem;                      // [2][BM][LDS_LD]
-    half_t* Bs = smem + 2 * BM * LDS_LD;    // [2][BN][LDS_LD]
-
-    const int ntiles = tiles_m * tiles_n;
-    const int per_xcd = (ntiles + 7) / 8;
-    const int tile = (blockIdx.x % 8) * per_xcd + blockIdx.x / 8;
-    if (tile >= ntiles) return;
-    const int tm = tile / tiles_n, tn = tile % tiles_n;
-    const int m0 = tm * BM, n0 = tn * BN;
-    const int z = blockIdx.y;
-    const int k_begin = z * k_per_split;
-    const int k_end = min(g.K, k_begin + k_per_split);
-    const int nslab = (k_end - k_begin) / BK;
-
-    const int tid = threadIdx.x, wave = tid / 64, lane = tid % 64;
-    const int wm = wave / 2, wn = wave % 2;
-
-    // Global->LDS staging: 16-byte chunk c = tid + 256*i covers row c/8, halfs [8*(c%8), +8).
-    const int ld_row = tid / 8, ld_kc = (tid % 8) * 8;
-    const half_t* a_src[8];
-    const half_t* b_src[8];
-#pragma unroll
-    for (int i = 0; i < 8; ++i) {
-        const int ra = min(m0 + ld_row + 32 * i, g.M - 1);
-        const int rb = min(n0 + ld_row + 32 * i, g.N - 1);
-        a_src[i] = g.A + size_t(ra) * g.lda + k_begin + ld_kc;
-        b_src[i] = g.B + size_t(rb) * g.ldb + k_begin + ld_kc;
-    }
-    const int st_off = ld_row * LDS_LD + ld_kc;
-
-    floatx16 acc[4][4];
-#pragma unroll
-    for (int i = 0; i < 4; ++i)
-#pragma unroll
-        for (int j = 0; j < 4; ++j)
-#pragma unroll
-            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
-
-    half8 ra[8], rb[8];
-    if (nslab > 0) {
-#pragma unroll
-        for (int i = 0; i < 8; ++i) { ra[i] = ld_half8(a_src[i]); rb[i] = ld_half8(b_src[i]); }
-#pragma unroll
-        for (int i = 0; i < 8; ++i) {
-            st_half8(As + st_off + 32 * i * LDS_LD, ra[i]);
-            st_half8(Bs + st_off + 32 * i * LDS_LD, rb[i]);
-        }
-    }
-    __syncthreads();
-
-    const int a_frag_off = (wm * 128 + lane % 32) * LDS_LD + 8 * (lane / 32);
-    const int b_frag_off = (wn * 128 + lane % 32) * LDS_LD + 8 * (lane / 32);
-
-    for (int s = 0; s < nslab; ++s) {
-        const int cur = s & 1;
-        const bool more = (s + 1 < nslab);
-        if (more) {
-            const int koff = (s + 1) * BK;
-#pragma unroll
-            for (int i = 0; i < 8; ++i) {
-                ra[i] = ld_half8(a_src[i] + koff);
-                rb[i] = ld_half8(b_src[i] + koff);
-            }
-        }
-        const half_t* Ac = As + cur * BM * LDS_LD + a_frag_off;
-        const half_t* Bc = Bs + cur * BN * LDS_LD + b_frag_off;
-#pragma unroll
-        for (int kk = 0; kk < BK / 16; ++kk) {
-            half8 af[4], bf[4];
-#pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                af[i] = *reinterpret_cast<const half8*>(Ac + i * 32 * LDS_LD + kk * 16);
-                bf[i] = *reinterpret_cast<const half8*>(Bc + i * 32 * LDS_LD + kk * 16);
-            }
-#pragma unroll
-            for (int i = 0; i < 4; ++i)
-#pragma unroll
-                for (int j = 0; j < 4; ++j)
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(bf[j], af[i], acc[i][j], 0, 0, 0);
-        }
-        if (more) {
-            half_t* An = As + (cur ^ 1) * BM * LDS_LD + st_off;
-            half_t* Bn = Bs + (cur ^ 1) * BN * LDS_LD + st_off;
-#pragma unroll
-            for (int i = 0; i < 8; ++i) {
-                st_half8(An + 32 * i * LDS_LD, ra[i]);
-                st_half8(Bn + 32 * i * LDS_LD, rb[i]);
-            }
-        }
-        __syncthreads();
-    }
-
-    // Epilogue.  With swapped operands register r of tile (i, j) holds row (i*32 + lane%32) of the
-    // wave's 128x128 block and column j*32 + 8*(r/4) + 4*(lane/32) + r%4: four consecutive columns per
-    // group of four registers.
+// Epilogue shared by both kernels.  With swapped MFMA operands register r of tile (i, j) holds row
+// (i*32 + lane%32) of the wave's 128 x 64 block and column j*32 + 8*(r/4) + 4*(lane/32) + r%4: four
+// consecutive columns per group of four registers, stored as one 8-byte (fp16) or 16-byte (fp32) access.
+__device__ __forceinline__ void store_tile(const GemmNT& g, floatx16 (&acc)[4][kTN], int m0, int n0, int wm,
+                                           int wn, int lane, int z) {
     const int row = m0 + wm * 128 + lane % 32;
-    const int colb = n0 + wn * 128 + 4 * (lane / 32);
+    const int colb = n0 + wn * 32 * kTN + 4 * (lane / 32);
     float* c32 = g.C32 ? g.C32 + size_t(z) * g.split_stride : nullptr;
     const bool full = (m0 + BM <= g.M) && (n0 + BN <= g.N) && (g.ldc % 4 == 0);
     if (full) {
@@ -130,7 +40,7 @@ __global__ __launch_bounds__(kThreads) void gemm_nt_256x256(GemmNT g, int tiles_
         for (int i = 0; i < 4; ++i) {
             const size_t rowoff = size_t(row + i * 32) * g.ldc + colb;
 #pragma unroll
-            for (int j = 0; j < 4; ++j) {
+            for (int j = 0; j < kTN; ++j) {
 #pragma unroll
                 for (int q = 0; q < 4; ++q) {
                     const size_t off = rowoff + j * 32 + 8 * q;
@@ -155,7 +65,7 @@ __global__ __launch_bounds__(kThreads) void gemm_nt_256x256(GemmNT g, int tiles_
             const int r_ = row + i * 32;
             if (r_ >= g.M) continue;
 #pragma unroll
-            for (int j = 0; j < 4; ++j) {
+            for (int j = 0; j < kTN; ++j) {
 #pragma unroll
                 for (int r = 0; r < 16; ++r) {
                     const int col = colb + j * 32 + 8 * (r / 4) + (r % 4);
@@ -169,6 +79,218 @@ __global__ __launch_bounds__(kThreads) void gemm_nt_256x256(GemmNT g, int tiles_
             }
         }
     }
+}
+
+
+__global__ __launch_bounds__(kThreads) void gemm_nt_256x256(GemmNT g, int tiles_m, int tiles_n,
+                                                             int k_per_split) {
+    extern __shared__ __attribute__((aligned(16))) half_t smem[];
+    half_t* As = smem;                      // [2][BM][LDS_LD]
+    half_t* Bs = smem + 2 * BM * LDS_LD;    // [2][BN][LDS_LD]
+
+    const int ntiles = tiles_m * tiles_n;
+    const int per_xcd = (ntiles + 7) / 8;
+    const int tile = (blockIdx.x % 8) * per_xcd + blockIdx.x / 8;
+    if (tile >= ntiles) return;
+    const int tm = tile / tiles_n, tn = tile % tiles_n;
+    const int m0 = tm * BM, n0 = tn * BN;
+    const int z = blockIdx.y;
+    const int k_begin = z * k_per_split;
+    const int k_end = min(g.K, k_begin + k_per_split);
+    const int nslab = (k_end - k_begin) / BK;
+
+    const int tid = threadIdx.x, wave = tid / 64, lane = tid % 64;
+    const int wm = wave / kWavesN, wn = wave % kWavesN;
+
+    // Global->LDS staging: 16-byte chunk c = tid + 256*i covers row c/8, halfs [8*(c%8), +8).
+    const int ld_row = tid / 8, ld_kc = (tid % 8) * 8;
+    const half_t* a_src[kLd];
+    const half_t* b_src[kLd];
+    constexpr int kRowStep = kThreads / 8;
+#pragma unroll
+    for (int i = 0; i < kLd; ++i) {
+        const int ra = min(m0 + ld_row + kRowStep * i, g.M - 1);
+        const int rb = min(n0 + ld_row + kRowStep * i, g.N - 1);
+        a_src[i] = g.A + size_t(ra) * g.lda + k_begin + ld_kc;
+        b_src[i] = g.B + size_t(rb) * g.ldb + k_begin + ld_kc;
+    }
+    const int st_off = ld_row * LDS_LD + ld_kc;
+
+    floatx16 acc[4][kTN];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < kTN; ++j)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
+
+    half8 ra[kLd], rb[kLd];
+    if (nslab > 0) {
+#pragma unroll
+        for (int i = 0; i < kLd; ++i) { ra[i] = ld_half8(a_src[i]); rb[i] = ld_half8(b_src[i]); }
+#pragma unroll
+        for (int i = 0; i < kLd; ++i) {
+            st_half8(As + st_off + kRowStep * i * LDS_LD, ra[i]);
+            st_half8(Bs + st_off + kRowStep * i * LDS_LD, rb[i]);
+        }
+    }
+    __syncthreads();
+
+    const int a_frag_off = (wm * 128 + lane % 32) * LDS_LD + 8 * (lane / 32);
+    const int b_frag_off = (wn * 32 * kTN + lane % 32) * LDS_LD + 8 * (lane / 32);
+
+    for (int s = 0; s < nslab; ++s) {
+        const int cur = s & 1;
+        const bool more = (s + 1 < nslab);
+        if (more) {
+            const int koff = (s + 1) * BK;
+#pragma unroll
+            for (int i = 0; i < kLd; ++i) {
+                ra[i] = ld_half8(a_src[i] + koff);
+                rb[i] = ld_half8(b_src[i] + koff);
+            }
+        }
+        const half_t* Ac = As + cur * BM * LDS_LD + a_frag_off;
+        const half_t* Bc = Bs + cur * BN * LDS_LD + b_frag_off;
+#pragma unroll
+        for (int kk = 0; kk < BK / 16; ++kk) {
+            half8 af[4], bf[kTN];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) af[i] = *reinterpret_cast<const half8*>(Ac + i * 32 * LDS_LD + kk * 16);
+#pragma unroll
+            for (int j = 0; j < kTN; ++j) bf[j] = *reinterpret_cast<const half8*>(Bc + j * 32 * LDS_LD + kk * 16);
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+#pragma unroll
+                for (int j = 0; j < kTN; ++j)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(bf[j], af[i], acc[i][j], 0, 0, 0);
+        }
+        if (more) {
+            half_t* An = As + (cur ^ 1) * BM * LDS_LD + st_off;
+            half_t* Bn = Bs + (cur ^ 1) * BN * LDS_LD + st_off;
+#pragma unroll
+            for (int i = 0; i < kLd; ++i) {
+                st_half8(An + kRowStep * i * LDS_LD, ra[i]);
+                st_half8(Bn + kRowStep * i * LDS_LD, rb[i]);
+            }
+        }
+        __syncthreads();
+    }
+
+    store_tile(g, acc, m0, n0, wm, wn, lane, z);
+}
+
+// TN form: C[M][N] = alpha * sum_k A[k][m] * B[k][n] with both operands stored k-major ([K][M] and
+// [K][N], m / n contiguous) -- the shape of the weight gradients dW = dG^T * X, whose operands come out
+// of the recurrence as [time*batch][features].  Slabs are staged in LDS exactly as they sit in memory
+// (coalesced 16-byte rows along m / n) and the MFMA fragments, which need 8 consecutive k per lane,
+// are read with the gfx950 transposing LDS load ds_read_b64_tr_b16: in every group of 16 lanes, lane j
+// supplies 4 halfs of row j/4 and receives the k-column for its own m, so no transposed copy of the
+// operands ever exists in HBM.  Rows k >= K read as zero.
+constexpr int kPitchT = 256 + 16;   // halfs per LDS row: 4 consecutive k rows fall in distinct banks
+constexpr size_t kLdsBytesTN = size_t(2) * 2 * BK * kPitchT * sizeof(half_t);
+
+typedef short short4v __attribute__((ext_vector_type(4)));
+typedef __attribute__((address_space(3))) short4v lds_short4;
+
+__device__ __forceinline__ half8 read_frag_tr(const half_t* lds_lane) {
+    union { short4v s[2]; half8 h; } u;
+    u.s[0] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_short4*)(lds_lane));
+    u.s[1] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_short4*)(lds_lane + 4 * kPitchT));
+    return u.h;
+}
+
+__global__ __launch_bounds__(kThreads) void gemm_tn_256x256(GemmNT g, int tiles_m, int tiles_n,
+                                                             int slabs_per_split) {
+    extern __shared__ __attribute__((aligned(16))) half_t smem[];
+    half_t* As = smem;                        // [2][BK][kPitchT]
+    half_t* Bs = smem + 2 * BK * kPitchT;     // [2][BK][kPitchT]
+
+    const int ntiles = tiles_m * tiles_n;
+    const int per_xcd = (ntiles + 7) / 8;
+    const int tile = (blockIdx.x % 8) * per_xcd + blockIdx.x / 8;
+    if (tile >= ntiles) return;
+    const int tm = tile / tiles_n, tn = tile % tiles_n;
+    const int m0 = tm * BM, n0 = tn * BN;
+    const int z = blockIdx.y;
+    const int nslab_total = (g.K + BK - 1) / BK;
+    const int slab_begin = z * slabs_per_split;
+    const int nslab = min(nslab_total - slab_begin, slabs_per_split);
+    const int k_begin = slab_begin * BK;
+
+    const int tid = threadIdx.x, wave = tid / 64, lane = tid % 64;
+    const int wm = wave / kWavesN, wn = wave % kWavesN;
+
+    // Global->LDS staging: 16-byte chunk c = tid + kThreads*i is k-row c/32, columns [8*(c%32), +8).
+    const int ld_k = tid / 32, ld_c = (tid % 32) * 8;
+    constexpr int kRowStep = kThreads / 32;
+    const bool a_ok = (m0 + ld_c) < g.M, b_ok = (n0 + ld_c) < g.N;
+    const half_t* a_src = g.A + min(m0 + ld_c, g.M - 8);
+    const half_t* b_src = g.B + min(n0 + ld_c, g.N - 8);
+    const int st_off = ld_k * kPitchT + ld_c;
+    half8 ra[kLd], rb[kLd];
+    auto fetch = [&](int slab) {
+#pragma unroll
+        for (int i = 0; i < kLd; ++i) {
+            const int k = k_begin + slab * BK + ld_k + kRowStep * i;
+            const int kc = min(k, g.K - 1);
+            ra[i] = ld_half8(a_src + size_t(kc) * g.lda);
+            rb[i] = ld_half8(b_src + size_t(kc) * g.ldb);
+            if (!(a_ok && k < g.K)) ra[i] = half8{};
+            if (!(b_ok && k < g.K)) rb[i] = half8{};
+        }
+    };
+    auto stage = [&](int buf) {
+#pragma unroll
+        for (int i = 0; i < kLd; ++i) {
+            st_half8(As + buf * BK * kPitchT + st_off + kRowStep * i * kPitchT, ra[i]);
+            st_half8(Bs + buf * BK * kPitchT + st_off + kRowStep * i * kPitchT, rb[i]);
+        }
+    };
+    // transposing fragment read: lane (group gq = lane/16, j = lane%16) addresses k-row 8*(gq/2) + j/4,
+    // column 16*(gq%2) + 4*(j%4) of a 32-wide tile; it receives k = 8*(lane/32) .. +7 for column lane%32.
+    const int gq = lane / 16, jq = lane % 16;
+    const int frag_off = (8 * (gq / 2) + jq / 4) * kPitchT + 16 * (gq % 2) + 4 * (jq % 4);
+    const int a_frag_off = frag_off + wm * 128;
+    const int b_frag_off = frag_off + wn * 32 * kTN;
+
+    floatx16 acc[4][kTN];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < kTN; ++j)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
+
+    if (nslab > 0) {
+        fetch(0);
+        stage(0);
+    }
+    __syncthreads();
+
+    for (int s = 0; s < nslab; ++s) {
+        const int cur = s & 1;
+        const bool more = (s + 1 < nslab);
+        if (more) fetch(s + 1);
+        const half_t* Ac = As + cur * BK * kPitchT + a_frag_off;
+        const half_t* Bc = Bs + cur * BK * kPitchT + b_frag_off;
+#pragma unroll
+        for (int kk = 0; kk < BK / 16; ++kk) {
+            half8 af[4], bf[kTN];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) af[i] = read_frag_tr(Ac + kk * 16 * kPitchT + i * 32);
+#pragma unroll
+            for (int j = 0; j < kTN; ++j) bf[j] = read_frag_tr(Bc + kk * 16 * kPitchT + j * 32);
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+#pragma unroll
+                for (int j = 0; j < kTN; ++j)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(bf[j], af[i], acc[i][j], 0, 0, 0);
+        }
+        if (more) stage(cur ^ 1);
+        __syncthreads();
+    }
+    store_tile(g, acc, m0, n0, wm, wn, lane, z);
 }
 
 }  // namespace
@@ -207,8 +329,34 @@ hipError_t launch_gemm_nt(const GemmNT& g, hipStream_t stream) {
     return hipGetLastError();
 }
 
+hipError_t launch_gemm_tn(const GemmNT& g, hipStream_t stream) {
+    if (g.M <= 0 || g.N <= 0 || g.K <= 0) return hipSuccess;
+    if (g.M % 8 != 0 || g.N % 8 != 0 || g.lda % 8 != 0 || g.ldb % 8 != 0) return hipErrorInvalidValue;
+    if ((g.C16 == nullptr) == (g.C32 == nullptr)) return hipErrorInvalidValue;
+    if (g.C32 && (reinterpret_cast<uintptr_t>(g.C32) % 16 != 0 || g.split_stride % 4 != 0)) return hipErrorInvalidValue;
+    if (g.C16 && (reinterpret_cast<uintptr_t>(g.C16) % 8 != 0)) return hipErrorInvalidValue;
+    const int splits = g.splits < 1 ? 1 : g.splits;
+    if (splits > 1 && g.C32 == nullptr) return hipErrorInvalidValue;
+    if (gemm_effective_splits(g.K, splits) != splits) return hipErrorInvalidValue;
+    static bool attr_set = false;
+    if (!attr_set) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_tn_256x256),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, int(kLdsBytesTN));
+        if (e != hipSuccess) return e;
+        attr_set = true;
+    }
+    const int nslab = (g.K + BK - 1) / BK;
+    const int slabs_per_split = (nslab + splits - 1) / splits;
+    const int tiles_m = (g.M + BM - 1) / BM, tiles_n = (g.N + BN - 1) / BN;
+    const int per_xcd = (tiles_m * tiles_n + 7) / 8;
+    dim3 grid(per_xcd * 8, splits, 1);
+    hipLaunchKernelGGL(gemm_tn_256x256, grid, dim3(kThreads), kLdsBytesTN, stream, g, tiles_m, tiles_n,
+                       slabs_per_split);
+    return hipGetLastError();
+}
+
 int gemm_effective_splits(int K, int wanted) {
-    const int nslab = K / BK;
+    const int nslab = (K + BK - 1) / BK;
     if (wanted < 1) wanted = 1;
     if (wanted > nslab) wanted = nslab;
     if (wanted < 1) wanted = 1;

@@ -143,27 +143,18 @@ __global__ void transpose_pad_kernel(const TIn* __restrict__ in, size_t rows, in
     }
 }
 
-__global__ void reduce_dw_kernel(Dims d, const float* __restrict__ partial, int splits, float scale,
-                                 float* __restrict__ dw_ih, float* __restrict__ dw_hh) {
-    const int ncat = d.Ip + d.Hp;
+// partial [splits][4Hp][ncols] with packed gate rows -> dst [4H][out_cols] in PyTorch row order
+__global__ void reduce_dw_kernel(Dims d, const float* __restrict__ partial, int splits, int ncols, int out_cols,
+                                 float scale, float* __restrict__ dst) {
     const size_t idx = size_t(blockIdx.x) * kT + threadIdx.x;
-    const size_t per = size_t(4) * d.Hp * ncat;
+    const size_t per = size_t(4) * d.Hp * ncols;
     if (idx >= per) return;
-    const int q = int(idx / ncat), n = int(idx % ncat);
+    const int q = int(idx / ncols), n = int(idx % ncols);
     const int row = torch_row(q, d.JF, d.H);
-    if (row < 0) return;
-    float* dst;
-    if (n < d.Ip) {
-        if (n >= d.I || dw_ih == nullptr) return;
-        dst = dw_ih + size_t(row) * d.I + n;
-    } else {
-        const int k = n - d.Ip;
-        if (k >= d.H || dw_hh == nullptr) return;
-        dst = dw_hh + size_t(row) * d.H + k;
-    }
+    if (row < 0 || n >= out_cols) return;
     float s = 0.f;
     for (int z = 0; z < splits; ++z) s += partial[size_t(z) * per + idx];
-    *dst = scale * s;
+    dst[size_t(row) * out_cols + n] = scale * s;
 }
 
 __global__ void reduce_db_kernel(Dims d, const float* __restrict__ db_part, int ng, float scale,
@@ -280,11 +271,12 @@ hipError_t transpose_pad(const void* in, int in_f32, size_t rows, int cols, size
     return hipGetLastError();
 }
 
-hipError_t reduce_dw(const Dims& d, const float* partial, int splits, float scale, float* dw_ih, float* dw_hh,
-                     hipStream_t s) {
-    const size_t per = size_t(4) * d.Hp * (d.Ip + d.Hp);
-    hipLaunchKernelGGL(reduce_dw_kernel, dim3(grid_for(per)), dim3(kT), 0, s, d, partial, splits, scale, dw_ih,
-                       dw_hh);
+hipError_t reduce_dw(const Dims& d, const float* partial, int splits, int ncols, int out_cols, float scale,
+                     float* dst, hipStream_t s) {
+    if (dst == nullptr) return hipSuccess;
+    const size_t per = size_t(4) * d.Hp * ncols;
+    hipLaunchKernelGGL(reduce_dw_kernel, dim3(grid_for(per)), dim3(kT), 0, s, d, partial, splits, ncols, out_cols,
+                       scale, dst);
     return hipGetLastError();
 }
 
