@@ -229,16 +229,32 @@ __global__ __launch_bounds__(kThreads) void gemm_tn_256x256(GemmNT g, int tiles_
     const half_t* b_src = g.B + min(n0 + ld_c, g.N - 8);
     const int st_off = ld_k * kPitchT + ld_c;
     half8 ra[kLd], rb[kLd];
+    // per-thread row pointers advance by one slab per fetch; only the slab that crosses K (always the
+    // last one of the matrix) needs per-row masking
+    const half_t* a_ptr = a_src + size_t(k_begin + ld_k) * g.lda;
+    const half_t* b_ptr = b_src + size_t(k_begin + ld_k) * g.ldb;
+    const size_t a_step = size_t(kRowStep) * g.lda, b_step = size_t(kRowStep) * g.ldb;
     auto fetch = [&](int slab) {
+        const int k0 = k_begin + slab * BK;
+        if (a_ok && b_ok && k0 + BK <= g.K) {
 #pragma unroll
-        for (int i = 0; i < kLd; ++i) {
-            const int k = k_begin + slab * BK + ld_k + kRowStep * i;
-            const int kc = min(k, g.K - 1);
-            ra[i] = ld_half8(a_src + size_t(kc) * g.lda);
-            rb[i] = ld_half8(b_src + size_t(kc) * g.ldb);
-            if (!(a_ok && k < g.K)) ra[i] = half8{};
-            if (!(b_ok && k < g.K)) rb[i] = half8{};
+            for (int i = 0; i < kLd; ++i) {
+                ra[i] = ld_half8(a_ptr + i * a_step);
+                rb[i] = ld_half8(b_ptr + i * b_step);
+            }
+        } else {
+#pragma unroll
+            for (int i = 0; i < kLd; ++i) {
+                const int k = k0 + ld_k + kRowStep * i;
+                const int kc = min(k, g.K - 1);
+                ra[i] = ld_half8(a_src + size_t(kc) * g.lda);
+                rb[i] = ld_half8(b_src + size_t(kc) * g.ldb);
+                if (!(a_ok && k < g.K)) ra[i] = half8{};
+                if (!(b_ok && k < g.K)) rb[i] = half8{};
+            }
         }
+        a_ptr += size_t(BK) * g.lda;
+        b_ptr += size_t(BK) * g.ldb;
     };
     auto stage = [&](int buf) {
 #pragma unroll
