@@ -26,6 +26,24 @@ constexpr int kTN = 8 / kWavesN;            // 32-wide MFMA tiles per wave along
 constexpr int kLd = 2048 / kThreads;        // 16-byte chunks per thread, operand and slab
 constexpr size_t kLdsBytes = size_t(2) * (BM + BN) * LDS_LD * sizeof(half_t);
 
+// Work list: items are (K-split z, tile) pairs ordered z-major, tiles row-major.  The hardware deals
+// workgroups round-robin over the 8 XCDs in dispatch order (x fastest), so the 32 workgroups that run
+// together on one XCD are given 32 CONSECUTIVE items: one K range and a compact block of tiles, whose
+// operand slabs they then share through that XCD's L2.
+__device__ __forceinline__ bool work_item(int tiles_m, int tiles_n, int splits, int& tm, int& tn, int& z) {
+    const int ntiles = tiles_m * tiles_n;
+    const int items = ntiles * splits;
+    const int lin = blockIdx.y * gridDim.x + blockIdx.x;   // dispatch order
+    const int xcd = lin % 8, s = lin / 8;
+    const int item = ((s / 32) * 8 + xcd) * 32 + s % 32;
+    if (item >= items) return false;
+    z = item / ntiles;
+    const int tile = item % ntiles;
+    tm = tile / tiles_n;
+    tn = tile % tiles_n;
+    return true;
+}
+
 // Epilogue shared by both kernels.  With swapped MFMA operands register r of tile (i, j) holds row
 // (i*32 + lane%32) of the wave's 128 x 64 block and column j*32 + 8*(r/4) + 4*(lane/32) + r%4: four
 // consecutive columns per group of four registers, stored as one 8-byte (fp16) or 16-byte (fp32) access.
@@ -88,13 +106,9 @@ __global__ __launch_bounds__(kThreads) void gemm_nt_256x256(GemmNT g, int tiles_
     half_t* As = smem;                      // [2][BM][LDS_LD]
     half_t* Bs = smem + 2 * BM * LDS_LD;    // [2][BN][LDS_LD]
 
-    const int ntiles = tiles_m * tiles_n;
-    const int per_xcd = (ntiles + 7) / 8;
-    const int tile = (blockIdx.x % 8) * per_xcd + blockIdx.x / 8;
-    if (tile >= ntiles) return;
-    const int tm = tile / tiles_n, tn = tile % tiles_n;
+    int tm, tn, z;
+    if (!work_item(tiles_m, tiles_n, gridDim.y, tm, tn, z)) return;
     const int m0 = tm * BM, n0 = tn * BN;
-    const int z = blockIdx.y;
     const int k_begin = z * k_per_split;
     const int k_end = min(g.K, k_begin + k_per_split);
     const int nslab = (k_end - k_begin) / BK;
@@ -206,13 +220,9 @@ __global__ __launch_bounds__(kThreads) void gemm_tn_256x256(GemmNT g, int tiles_
     half_t* As = smem;                        // [2][BK][kPitchT]
     half_t* Bs = smem + 2 * BK * kPitchT;     // [2][BK][kPitchT]
 
-    const int ntiles = tiles_m * tiles_n;
-    const int per_xcd = (ntiles + 7) / 8;
-    const int tile = (blockIdx.x % 8) * per_xcd + blockIdx.x / 8;
-    if (tile >= ntiles) return;
-    const int tm = tile / tiles_n, tn = tile % tiles_n;
+    int tm, tn, z;
+    if (!work_item(tiles_m, tiles_n, gridDim.y, tm, tn, z)) return;
     const int m0 = tm * BM, n0 = tn * BN;
-    const int z = blockIdx.y;
     const int nslab_total = (g.K + BK - 1) / BK;
     const int slab_begin = z * slabs_per_split;
     const int nslab = min(nslab_total - slab_begin, slabs_per_split);
@@ -337,9 +347,10 @@ hipError_t launch_gemm_nt(const GemmNT& g, hipStream_t stream) {
         attr_set = true;
     }
     const int tiles_m = (g.M + BM - 1) / BM, tiles_n = (g.N + BN - 1) / BN;
-    const int ntiles = tiles_m * tiles_n;
-    const int per_xcd = (ntiles + 7) / 8;
-    dim3 grid(per_xcd * 8, splits, 1);
+    // gridDim.y carries the split count; x is padded so that x*y is a whole number of 256-workgroup rounds
+    const int items = tiles_m * tiles_n * splits;
+    const int rounded = (items + 255) / 256 * 256;
+    dim3 grid((rounded + splits - 1) / splits, splits, 1);
     hipLaunchKernelGGL(gemm_nt_256x256, grid, dim3(kThreads), kLdsBytes, stream, g, tiles_m, tiles_n,
                        slabs_per_split * BK);
     return hipGetLastError();
@@ -364,8 +375,9 @@ hipError_t launch_gemm_tn(const GemmNT& g, hipStream_t stream) {
     const int nslab = (g.K + BK - 1) / BK;
     const int slabs_per_split = (nslab + splits - 1) / splits;
     const int tiles_m = (g.M + BM - 1) / BM, tiles_n = (g.N + BN - 1) / BN;
-    const int per_xcd = (tiles_m * tiles_n + 7) / 8;
-    dim3 grid(per_xcd * 8, splits, 1);
+    const int items = tiles_m * tiles_n * splits;
+    const int rounded = (items + 255) / 256 * 256;
+    dim3 grid((rounded + splits - 1) / splits, splits, 1);
     hipLaunchKernelGGL(gemm_tn_256x256, grid, dim3(kThreads), kLdsBytesTN, stream, g, tiles_m, tiles_n,
                        slabs_per_split);
     return hipGetLastError();

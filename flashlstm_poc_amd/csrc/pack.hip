@@ -170,6 +170,12 @@ __global__ void reduce_db_kernel(Dims d, const float* __restrict__ db_part, int 
     if (db_hh) db_hh[row] = s;
 }
 
+// flat 16-byte copy (both ends 16-byte aligned, n16 chunks)
+__global__ void copy16_kernel(const uint4* __restrict__ in, uint4* __restrict__ out, size_t n16) {
+    const size_t stride = size_t(gridDim.x) * kT;
+    for (size_t i = size_t(blockIdx.x) * kT + threadIdx.x; i < n16; i += stride) out[i] = in[i];
+}
+
 __global__ void fill_zero_kernel(unsigned* p, size_t words) {
     const size_t stride = size_t(gridDim.x) * kT;
     for (size_t i = size_t(blockIdx.x) * kT + threadIdx.x; i < words; i += stride) p[i] = 0u;
@@ -226,6 +232,16 @@ hipError_t gather_from_half(const half_t* in, size_t ld_in, size_t rows, int col
                             size_t rows_per_block, size_t block_stride, hipStream_t s) {
     const size_t n = rows * size_t(cols);
     if (n == 0 || out == nullptr) return hipSuccess;
+    // unpadded fp16 rows that are contiguous on both sides: a flat vector copy
+    if (!out_f32 && size_t(cols) == ld_in && rows_per_block >= rows && (n * sizeof(half_t)) % 16 == 0 &&
+        reinterpret_cast<uintptr_t>(in) % 16 == 0 && reinterpret_cast<uintptr_t>(out) % 16 == 0) {
+        const size_t n16 = n * sizeof(half_t) / 16;
+        size_t blocks = (n16 + kT - 1) / kT;
+        if (blocks > 8192) blocks = 8192;
+        hipLaunchKernelGGL(copy16_kernel, dim3(unsigned(blocks)), dim3(kT), 0, s, reinterpret_cast<const uint4*>(in),
+                           static_cast<uint4*>(out), n16);
+        return hipGetLastError();
+    }
     if (out_f32)
         hipLaunchKernelGGL((unpad_kernel<half_t, float>), dim3(grid_for(n)), dim3(kT), 0, s, in, ld_in, rows,
                            cols, 1.f, static_cast<float*>(out), rows_per_block, block_stride);
