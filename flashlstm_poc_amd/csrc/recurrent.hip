@@ -108,48 +108,88 @@ __device__ __forceinline__ void publish(unsigned* gflags, int hs, unsigned value
 
 // Exchange layout ("fragment-major").  The operand a step fetches from its peers -- h_{t-1} in the
 // forward pass, dG_{t+1} in the backward pass -- is stored as ready-made MFMA A-fragments so that
-// every load instruction of a wave covers one contiguous 512-byte run:
+// every load instruction of a wave covers one contiguous kilobyte:
 //   element (row r, column k) of a [rows][K] matrix, nks = K / 32, sits at (in halfs)
-//   ((((r/16)*nks + k/32)*2 + (k%8)/4)*64 + r%16 + 16*((k%32)/8))*4 + k%4
-// i.e. [16-row tile][32-wide k-step][low / high half of the lane's 8 values][lane][4 halfs].
+//   ((r/16)*nks + k/32)*512 + (r%16 + 16*((k%32)/8))*8 + k%8
+// i.e. [16-row tile][32-wide k-step][lane][8 halfs].
 __device__ __forceinline__ size_t xch_offset(int r, int k, int nks) {
-    return ((((size_t(r / 16) * nks + k / 32) * 2 + (k % 8) / 4) * 64) + (r % 16) + 16 * ((k % 32) / 8)) * 4 + (k % 4);
+    return (size_t(r / 16) * nks + k / 32) * 512 + ((r % 16) + 16 * ((k % 32) / 8)) * 8 + (k % 8);
 }
 
-// One A-fragment: two coalesced 8-byte device-scope loads (L1 bypass, served by the XCD's L2).
+// One A-fragment through compiler-visible loads: two 8-byte device-scope relaxed atomic loads
+// (L1 bypass, served by the XCD's L2).  Used by the step-wise / non-resident path.
 __device__ __forceinline__ half8 ld_frag(const half_t* frag_lane) {
     union { u64 q[2]; half8 h; } u;
     u.q[0] = __hip_atomic_load(reinterpret_cast<const u64*>(frag_lane), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    u.q[1] = __hip_atomic_load(reinterpret_cast<const u64*>(frag_lane + 256), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    u.q[1] = __hip_atomic_load(reinterpret_cast<const u64*>(frag_lane) + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     return u.h;
 }
 
+// The persistent kernels fetch fragments with ONE 16-byte load per lane carrying the device-scope bit
+// (sc1: bypass the per-CU L1, hit the L2).  A CU's vector-memory path costs the same per instruction
+// whether a lane moves 8 or 16 bytes: 8-byte loads top out at ~24 B/clk per CU, 16-byte loads at
+// ~54 B/clk (measured), and the backward step is bound by exactly this fetch.  The compiler offers no
+// 16-byte load with that scope, hence the two small asm helpers.  Loads return in issue order, so
+// waiting until at most N younger loads are outstanding guarantees that everything issued before
+// them has landed; the registers are listed as operands of the wait so that no consumer can be
+// scheduled above it.
+__device__ __forceinline__ void ld_frag_async(half8& dst, const half_t* frag_lane) {
+    asm volatile("global_load_dwordx4 %0, %1, off sc1" : "=v"(dst) : "v"(frag_lane) : "memory");
+}
+template <int N>
+__device__ __forceinline__ void wait_frags(half8 (&a)[4], half8 (&b)[4]) {
+    asm volatile("s_waitcnt vmcnt(%8)"
+                 : "+v"(a[0]), "+v"(a[1]), "+v"(a[2]), "+v"(a[3]), "+v"(b[0]), "+v"(b[1]), "+v"(b[2]), "+v"(b[3])
+                 : "n"(N)
+                 : "memory");
+}
+
 // acc[mt][nt] += A(32 rows x K) * Wslice, this wave's interleaved k-steps only.
-// a0/a1: fragment (row tile, k-step 0) of the two 16-row tiles, already offset by lane*4 halfs.
-template <int NT, int KS, bool RESIDENT>
-__device__ __forceinline__ void wave_product(floatx4 (&acc)[2][NT], const half8 (&wreg)[KS][NT],
-                                             const half8* wfrag_wave, const half_t* a0,
+// a0/a1: fragment (row tile, k-step 0) of the two 16-row tiles, already offset by lane*8 halfs.
+// The last KL of a wave's KS k-steps keep their weight fragments in LDS instead of registers (wlds:
+// this wave's [KL][NT][64 lanes] block); reading them back costs a few ds_read_b128 per step and frees
+// 4*KL*NT registers for fragments in flight.
+template <int NT, int KS, bool RESIDENT, int KL = 0>
+__device__ __forceinline__ void wave_product(floatx4 (&acc)[2][NT], const half8 (&wreg)[KS - KL][NT],
+                                             const half8* wlds, const half8* wfrag_wave, const half_t* a0,
                                              const half_t* a1, int wave, int lane, int nks_total,
                                              int ks_wave) {
-    if constexpr (RESIDENT) {
+    if constexpr (RESIDENT && (KS % 8 == 0)) {
         // Loads and MFMAs are unconditional: k-steps beyond the real contraction length fetch a
-        // clamped (finite) address and meet all-zero weight fragments.
-        constexpr int KC = (KS < 8) ? KS : 8;  // k-steps fetched ahead together
-        half8 fa[KC], fb[KC];
+        // clamped (finite) address and meet all-zero weight fragments.  Chunks of 4 k-steps (8
+        // fragments) alternate between two register sets: one is in flight while the other feeds the
+        // MFMAs.
+        constexpr int NCH = KS / 4;
+        half8 fa[2][4], fb[2][4];
+        auto issue = [&](int c, int buf) {
 #pragma unroll
-        for (int c = 0; c < KS / KC; ++c) {
+            for (int k = 0; k < 4; ++k) {
+                const int kg = min((c * 4 + k) * 4 + wave, nks_total - 1);
+                ld_frag_async(fa[buf][k], a0 + size_t(kg) * 512);
+                ld_frag_async(fb[buf][k], a1 + size_t(kg) * 512);
+            }
+        };
+        issue(0, 0);
 #pragma unroll
-            for (int k = 0; k < KC; ++k) {
-                const int kg = min((c * KC + k) * 4 + wave, nks_total - 1);
-                fa[k] = ld_frag(a0 + size_t(kg) * 512);
-                fb[k] = ld_frag(a1 + size_t(kg) * 512);
+        for (int c = 0; c < NCH; ++c) {
+            const int buf = c & 1;
+            if (c + 1 < NCH) {
+                issue(c + 1, buf ^ 1);
+                wait_frags<8>(fa[buf], fb[buf]);
+            } else {
+                wait_frags<0>(fa[buf], fb[buf]);
             }
 #pragma unroll
-            for (int k = 0; k < KC; ++k) {
+            for (int k = 0; k < 4; ++k) {
+                constexpr int KR = KS - KL;
+                const int ks = c * 4 + k;
 #pragma unroll
                 for (int n = 0; n < NT; ++n) {
-                    acc[0][n] = __builtin_amdgcn_mfma_f32_16x16x32_f16(fa[k], wreg[c * KC + k][n], acc[0][n], 0, 0, 0);
-                    acc[1][n] = __builtin_amdgcn_mfma_f32_16x16x32_f16(fb[k], wreg[c * KC + k][n], acc[1][n], 0, 0, 0);
+                    half8 w;
+                    if (ks < KR) w = wreg[ks < KR ? ks : 0][n];
+                    else w = wlds[((ks - KR) * NT + n) * kWave + lane];
+                    acc[0][n] = __builtin_amdgcn_mfma_f32_16x16x32_f16(fa[buf][k], w, acc[0][n], 0, 0, 0);
+                    acc[1][n] = __builtin_amdgcn_mfma_f32_16x16x32_f16(fb[buf][k], w, acc[1][n], 0, 0, 0);
                 }
             }
         }
@@ -325,14 +365,14 @@ __global__ __launch_bounds__(kThreads) void rec_fwd_kernel(RecFwdArgs p, RecLayo
             const int row0 = rb * kRows;
             const half_t* xin = p.X + size_t(t & 1) * p.x_slot;        // h_{t-1}, fragment-major
             half_t* xout = p.X + size_t((t + 1) & 1) * p.x_slot;       // h_t
-            const half_t* a0 = xin + size_t(2 * rb) * nks_total * 512 + lane * 4;
+            const half_t* a0 = xin + size_t(2 * rb) * nks_total * 512 + lane * 8;
             const half_t* a1 = a0 + size_t(nks_total) * 512;
             floatx4 acc[2][NT];
 #pragma unroll
             for (int m = 0; m < 2; ++m)
 #pragma unroll
                 for (int n = 0; n < NT; ++n) acc[m][n] = floatx4{0.f, 0.f, 0.f, 0.f};
-            wave_product<NT, KS, RESIDENT>(acc, wreg, wfrag_wave, a0, a1, wave, lane, nks_total, ks_wave);
+            wave_product<NT, KS, RESIDENT>(acc, wreg, nullptr, wfrag_wave, a0, a1, wave, lane, nks_total, ks_wave);
             clk.lap(1);
             spill_partials<NT>(part, acc, wave, lane, PLD);
             __syncthreads();
@@ -410,11 +450,12 @@ __global__ __launch_bounds__(kThreads) void rec_fwd_kernel(RecFwdArgs p, RecLayo
 // ----------------------------------------------------------------------------------- backward
 // Gate order and the pointwise derivative follow flashlstm_v2/src/lstm_backward.cu:199-211, except
 // that c_{t-1}, c_t come from the cell-state cache instead of being rebuilt through atanh.
-template <int NT, int KS, bool RESIDENT>
+template <int NT, int KS, bool RESIDENT, int KL>
 __global__ __launch_bounds__(kThreads) void rec_bwd_kernel(RecBwdArgs p, RecLayout L, int t_first,
                                                            int t_last, int ks_wave) {
     constexpr int JB = 16 * NT;  // hidden units (= output columns of dG*W_hh) of this slice
     constexpr int PLD = JB + 4;
+    constexpr int KR = KS - KL;  // k-steps whose weight fragments stay in registers
     constexpr int NPAIR = kRows * (JB / 2);
     constexpr int NP = (NPAIR + kThreads - 1) / kThreads;
     extern __shared__ __attribute__((aligned(16))) float part[];  // [4][32][PLD], reused for db
@@ -433,13 +474,21 @@ __global__ __launch_bounds__(kThreads) void rec_bwd_kernel(RecBwdArgs p, RecLayo
     PhaseClock clk{(blockIdx.x == 0) ? p.prof : nullptr, 0};
 
     const half8* wfrag_wave = p.wfrag + (size_t(hs) * 4 + wave) * size_t(ks_wave) * NT * kWave;
-    half8 wreg[KS][NT];
+    half8 wreg[KR][NT];
+    // LDS: [partials 4*32*PLD floats | weight fragments of the last KL k-steps, one block per wave]
+    half8* wlds = reinterpret_cast<half8*>(part + 4 * kRows * PLD) + size_t(wave) * KL * NT * kWave;
     if constexpr (RESIDENT) {
 #pragma unroll
-        for (int k = 0; k < KS; ++k)
+        for (int k = 0; k < KR; ++k)
 #pragma unroll
             for (int n = 0; n < NT; ++n)
                 wreg[k][n] = (k < ks_wave) ? wfrag_wave[(size_t(k) * NT + n) * kWave + lane] : half8{};
+#pragma unroll
+        for (int k = 0; k < KL; ++k)
+#pragma unroll
+            for (int n = 0; n < NT; ++n)
+                wlds[(k * NT + n) * kWave + lane] =
+                    (KR + k < ks_wave) ? wfrag_wave[(size_t(KR + k) * NT + n) * kWave + lane] : half8{};
     }
 
     const size_t gld = size_t(4) * p.Hp;
@@ -501,14 +550,14 @@ __global__ __launch_bounds__(kThreads) void rec_bwd_kernel(RecBwdArgs p, RecLayo
             const int row0 = rb * kRows;
             if (from_product) {
                 const half_t* xin = p.X + size_t((t + 1) & 1) * p.x_slot;   // dG_{t+1}, fragment-major
-                const half_t* a0 = xin + size_t(2 * rb) * nks_total * 512 + lane * 4;
+                const half_t* a0 = xin + size_t(2 * rb) * nks_total * 512 + lane * 8;
                 const half_t* a1 = a0 + size_t(nks_total) * 512;
                 floatx4 acc[2][NT];
 #pragma unroll
                 for (int m = 0; m < 2; ++m)
 #pragma unroll
                     for (int n = 0; n < NT; ++n) acc[m][n] = floatx4{0.f, 0.f, 0.f, 0.f};
-                wave_product<NT, KS, RESIDENT>(acc, wreg, wfrag_wave, a0, a1, wave, lane, nks_total, ks_wave);
+                wave_product<NT, KS, RESIDENT, KL>(acc, wreg, wlds, wfrag_wave, a0, a1, wave, lane, nks_total, ks_wave);
                 clk.lap(1);
                 spill_partials<NT>(part, acc, wave, lane, PLD);
                 __syncthreads();
@@ -742,11 +791,11 @@ hipError_t launch_rec_fwd(const RecLayout& L, const RecFwdArgs& a, hipStream_t s
     return hipErrorInvalidValue;
 }
 
-template <int NT, int KS, bool RES>
+template <int NT, int KS, bool RES, int KL>
 static hipError_t run_bwd(const RecLayout& L, const RecBwdArgs& a, hipStream_t stream) {
-    auto kernel = rec_bwd_kernel<NT, KS, RES>;
-    size_t lds = size_t(4) * kRows * (16 * NT + 4) * sizeof(float);
-    if (lds < size_t(kThreads) * 8 * sizeof(float)) lds = size_t(kThreads) * 8 * sizeof(float);
+    auto kernel = rec_bwd_kernel<NT, KS, RES, KL>;
+    static_assert(size_t(4) * kRows * (16 * NT + 4) >= size_t(kThreads) * 8, "db reduction reuses the partial-sum area");
+    const size_t lds = size_t(4) * kRows * (16 * NT + 4) * sizeof(float) + size_t(4) * KL * NT * kWave * sizeof(half8);
     hipError_t e = raise_lds(kernel, lds);
     if (e != hipSuccess) return e;
     const int ks_wave = rec_bwd_ks(L, a.Hp);
@@ -765,9 +814,9 @@ static hipError_t run_bwd(const RecLayout& L, const RecBwdArgs& a, hipStream_t s
 hipError_t launch_rec_bwd(const RecLayout& L, const RecBwdArgs& a, hipStream_t stream) {
     if (a.T <= 0 || a.B <= 0) return hipSuccess;
     if (a.Hp % 32 != 0 || a.Hp % L.jb != 0) return hipErrorInvalidValue;
-    if (!L.resident) return run_bwd<2, 1, false>(L, a, stream);
-    if (L.nt == 2) return run_bwd<2, 32, true>(L, a, stream);
-    if (L.nt == 1) return run_bwd<1, 64, true>(L, a, stream);
+    if (!L.resident) return run_bwd<2, 1, false, 0>(L, a, stream);
+    if (L.nt == 2) return run_bwd<2, 32, true, 8>(L, a, stream);
+    if (L.nt == 1) return run_bwd<1, 64, true, 16>(L, a, stream);
     return hipErrorInvalidValue;
 }
 
