@@ -14,7 +14,11 @@
 // Workgroups are numbered so that the 32 that share an XCD (block id mod 8) work on neighbouring tiles
 // and reuse each other's operand slabs in that XCD's L2.
 #include "gemm.h"
+#include <cstdlib>
 
+#ifdef GEMM_PROF
+__device__ long long g_gemm_prof[8];
+#endif
 namespace flstm_hip {
 namespace {
 
@@ -26,22 +30,30 @@ constexpr int kTN = 8 / kWavesN;            // 32-wide MFMA tiles per wave along
 constexpr int kLd = 2048 / kThreads;        // 16-byte chunks per thread, operand and slab
 constexpr size_t kLdsBytes = size_t(2) * (BM + BN) * LDS_LD * sizeof(half_t);
 
-// Work list: items are (K-split z, tile) pairs ordered z-major, tiles row-major.  The hardware deals
-// workgroups round-robin over the 8 XCDs in dispatch order (x fastest), so the 32 workgroups that run
-// together on one XCD are given 32 CONSECUTIVE items: one K range and a compact block of tiles, whose
-// operand slabs they then share through that XCD's L2.
-__device__ __forceinline__ bool work_item(int tiles_m, int tiles_n, int splits, int& tm, int& tn, int& z) {
-    const int ntiles = tiles_m * tiles_n;
-    const int items = ntiles * splits;
-    const int lin = blockIdx.y * gridDim.x + blockIdx.x;   // dispatch order
+// Work order.  The hardware deals workgroups round-robin over the 8 XCDs in dispatch order, so the 32
+// workgroups with the same (dispatch index mod 8) that run together share one XCD and its 4 MiB L2.  They
+// are given one SUPER-TILE: a compact sm x sn block of tiles (sm * sn = 32, normally 8 x 4, i.e.
+// 2048 x 1024 of C) of one K split, for which they fetch sm + sn operand panels instead of up to 33.
+// Consecutive super-tiles of an XCD walk down M inside one column group, so the B panels of that group
+// stay in its L2 from one round to the next.
+struct TileOrder {
+    int tiles_m, tiles_n, splits;
+    int sm, sn;        // super-tile shape in tiles
+    int nsm, nsn;      // super-tiles along M and N
+    int per_xcd;       // super-tiles (= rounds) per XCD
+};
+
+__device__ __forceinline__ bool work_item(const TileOrder& o, int lin, int& tm, int& tn, int& z) {
     const int xcd = lin % 8, s = lin / 8;
-    const int item = ((s / 32) * 8 + xcd) * 32 + s % 32;
-    if (item >= items) return false;
-    z = item / ntiles;
-    const int tile = item % ntiles;
-    tm = tile / tiles_n;
-    tn = tile % tiles_n;
-    return true;
+    const int slot = s % 32, round = s / 32;
+    const int nst = o.nsm * o.nsn * o.splits;
+    const int st = xcd * o.per_xcd + round;
+    if (round >= o.per_xcd || st >= nst) return false;
+    z = st / (o.nsm * o.nsn);
+    const int r = st % (o.nsm * o.nsn);
+    tm = (r % o.nsm) * o.sm + slot / o.sn;
+    tn = (r / o.nsm) * o.sn + slot % o.sn;
+    return tm < o.tiles_m && tn < o.tiles_n;
 }
 
 // Epilogue shared by both kernels.  With swapped MFMA operands register r of tile (i, j) holds row
@@ -100,14 +112,13 @@ __device__ __forceinline__ void store_tile(const GemmNT& g, floatx16 (&acc)[4][k
 }
 
 
-__global__ __launch_bounds__(kThreads) void gemm_nt_256x256(GemmNT g, int tiles_m, int tiles_n,
-                                                             int k_per_split) {
+__global__ __launch_bounds__(kThreads) void gemm_nt_256x256(GemmNT g, TileOrder order, int k_per_split) {
     extern __shared__ __attribute__((aligned(16))) half_t smem[];
     half_t* As = smem;                      // [2][BM][LDS_LD]
     half_t* Bs = smem + 2 * BM * LDS_LD;    // [2][BN][LDS_LD]
 
     int tm, tn, z;
-    if (!work_item(tiles_m, tiles_n, gridDim.y, tm, tn, z)) return;
+    if (!work_item(order, blockIdx.x, tm, tn, z)) return;
     const int m0 = tm * BM, n0 = tn * BN;
     const int k_begin = z * k_per_split;
     const int k_end = min(g.K, k_begin + k_per_split);
@@ -194,6 +205,267 @@ __global__ __launch_bounds__(kThreads) void gemm_nt_256x256(GemmNT g, int tiles_
     store_tile(g, acc, m0, n0, wm, wn, lane, z);
 }
 
+// ------------------------------------------------------------------------------ streaming NT kernel
+// Same contraction and wave layout, different data path.  Operand slabs go from global memory straight
+// into LDS (global_load_lds_dwordx4: no staging registers, no LDS store instructions), double buffered
+// in slabs of 64 k.  Wavefronts 4..7 are the copiers: each issues the 16 one-KiB copies of its quarter of
+// the next slab between its first MFMAs of the current one.  A copy instruction holds its wave until the
+// texture-address unit takes it (about 16 clocks each, 64 per slab and workgroup); the copier's partner
+// on the same SIMD (wavefront - 4) issues no copies, so it keeps the matrix pipeline fed meanwhile.
+// The kernel is persistent: each workgroup walks its list of work items and the copies keep running
+// across item boundaries, so the first slab of the next tile arrives during the last MFMAs and the
+// output stores of this one.
+//
+// LDS rows are 128 bytes (8 chunks of 16).  The LDS has 64 banks of 4 bytes and serves a 16-byte read
+// for 16 lanes per clock, so the 16 rows read together must land in 16 different 16-byte bank groups of
+// the 256-byte bank row; two rows share a bank row, hence chunk c of row r sits at position c ^ (r/2)%8.
+#ifndef GEMM_COPY_MODE
+#define GEMM_COPY_MODE 2
+#endif
+constexpr int kSlabBytes = (BM + BN) * BK * 2;               // 64 KiB: A rows then B rows
+constexpr int kEpiBytesPerWave = 32 * 64 * 2;                 // one 32 x 64 fp16 block of the wave's output
+constexpr size_t kLdsBytesStream = size_t(2) * kSlabBytes + 8 * kEpiBytesPerWave;   // 160 KiB
+constexpr int kCopiesPerWave = 8;                            // 8 waves x 8 KiB = one slab
+
+typedef __attribute__((address_space(3))) void lds_void;
+typedef __attribute__((address_space(1))) const void global_void;
+
+__device__ __forceinline__ void copy_1k_to_lds(const char* src_lane, char* lds_block) {
+    __builtin_amdgcn_global_load_lds((global_void*)(src_lane), (lds_void*)(lds_block), 16, 0, 0);
+}
+
+template <int N>
+__device__ __forceinline__ void wait_vm() {
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
+}
+
+// fp16 epilogue of a full tile with whole-line stores.  In the accumulators one row of the wave's 128 x 64
+// block is spread over two lanes in 8-byte pieces, which makes 32 partial-line writes per store instruction.
+// Each 32 x 64 block is therefore turned through a private 4 KiB of LDS (16-byte chunks XOR-swizzled by
+// row / 2, so the 16-byte reads are conflict free): 8 lanes then hold one 128-byte row segment and a store
+// instruction writes 8 complete lines.  16 stores per wave instead of 32.
+__device__ __forceinline__ void store_tile_lines(const GemmNT& g, floatx16 (&acc)[4][kTN], int m0, int n0, int wm,
+                                                 int wn, int lane, char* stage) {
+    static_assert(kTN == 2, "the staging block is 64 columns wide");
+    const int wr = lane % 32;                              // row written by this lane
+    const int wsw = (wr >> 1) & 7;
+    const int rr = lane / 8, rc = lane % 8;                // row (+ 8p) and 16-byte chunk read by this lane
+    half_t* cbase = g.C16 + size_t(m0 + wm * 128) * g.ldc + n0 + wn * 64 + rc * 8;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+#pragma unroll
+        for (int j = 0; j < kTN; ++j)
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                half4 v;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) v[e] = (half_t)(g.alpha * acc[i][j][4 * q + e]);
+                const int chunk = 4 * j + q;
+                *reinterpret_cast<half4*>(stage + wr * 128 + ((chunk ^ wsw) * 16) + 8 * (lane / 32)) = v;
+            }
+#pragma unroll
+        for (int p = 0; p < 4; ++p) {
+            const int row = rr + 8 * p;
+            const half8 v = *reinterpret_cast<const half8*>(stage + row * 128 + ((rc ^ ((row >> 1) & 7)) * 16));
+            *reinterpret_cast<half8*>(cbase + size_t(i * 32 + row) * g.ldc) = v;
+        }
+        __builtin_amdgcn_sched_barrier(0);
+    }
+}
+
+__global__ __launch_bounds__(kThreads) void gemm_nt_stream(GemmNT g, TileOrder order, int k_per_split) {
+    extern __shared__ __attribute__((aligned(1024))) char lds[];
+
+    const int tid = threadIdx.x, lane = tid % 64;
+    const int wave = __builtin_amdgcn_readfirstlane(tid / 64);
+    const int wm = wave / kWavesN, wn = wave % kWavesN;
+    // Wave w issues copy c after its MFMA number 4c + phase.  The two waves of a SIMD (w and w + 4) are two
+    // MFMAs apart and at most two waves of the workgroup issue in the same slot, so a copy instruction,
+    // which holds its wave until the texture-address unit accepts it, rarely finds the unit busy and never
+    // stalls both waves of a SIMD at once.
+    const int phase = (wave + 2 * (wave / 4)) % 4;
+    const int rounds = order.per_xcd;
+
+    // ordinal n of this workgroup -> (tile, split) in the order of work_item().  Ordinals that fall on a
+    // tile outside the matrix are skipped, by the copy sequence and the consumer alike.
+    auto decode = [&](int n, int& m0, int& n0, int& z, int& kb, int& nk) -> bool {
+        int tm, tn;
+        if (!work_item(order, n * int(gridDim.x) + blockIdx.x, tm, tn, z)) return false;
+        m0 = tm * BM;
+        n0 = tn * BN;
+        kb = z * k_per_split;
+        nk = (min(g.K, kb + k_per_split) - kb) / BK;
+        return nk > 0;
+    };
+
+    // ---- copier state: the slab copied next is slab ld_k of item ordinal ld_n.  Copy c of a slab
+    // (operand c % 2, row block i = c / 2) fills rows [64q + 8i, +8) of the tile, q = wave % 4; lane l
+    // lands at row l / 8, chunk position l % 8 and therefore fetches chunk (l % 8) ^ swizzle(row).
+    int ld_n = 0, ld_k = 0, ld_nk = 0, ld_m0 = 0, ld_n0 = 0, ld_kb = 0;
+    bool ld_valid = false;
+    auto loader_open = [&]() {
+        int z;
+        ld_valid = false;
+        while (ld_n < rounds && !(ld_valid = decode(ld_n, ld_m0, ld_n0, z, ld_kb, ld_nk))) ++ld_n;
+        ld_k = 0;
+    };
+    const int cp_row = wave * 32 + lane / 8;
+    auto issue_copy = [&](int slot, int c) {
+        if (!ld_valid) return;
+        const int i = c / 2;
+        const int rt = cp_row + 8 * i;
+#ifdef GEMM_SAMETILE
+        ld_m0 = 0; ld_n0 = 0;
+#endif
+        const int chunk = (lane % 8) ^ ((rt >> 1) & 7);
+        const int koff = ld_kb + ld_k * BK + chunk * 8;
+        char* dst = lds + slot * kSlabBytes + wave * 4096 + i * 1024;
+        if (c % 2 == 0) {
+            const int row = min(ld_m0 + rt, g.M - 1);
+            copy_1k_to_lds(reinterpret_cast<const char*>(g.A + size_t(row) * g.lda + koff), dst);
+        } else {
+            const int row = min(ld_n0 + rt, g.N - 1);
+            copy_1k_to_lds(reinterpret_cast<const char*>(g.B + size_t(row) * g.ldb + koff), dst + BM * BK * 2);
+        }
+    };
+    auto loader_advance = [&]() {
+        if (!ld_valid) return;
+        if (++ld_k == ld_nk) {
+            ++ld_n;
+            loader_open();
+        }
+    };
+
+    // ---- consumer: fragment addresses inside a slab (tile rows of one lane are multiples of 32 apart,
+    // so the swizzle depends on the lane only)
+    const int a_frag = (wm * 128 + lane % 32) * (BK * 2);
+    const int b_frag = BM * BK * 2 + (wn * 32 * kTN + lane % 32) * (BK * 2);
+    int pos[BK / 16];
+#pragma unroll
+    for (int kk = 0; kk < BK / 16; ++kk) pos[kk] = ((2 * kk + lane / 32) ^ ((lane % 32) >> 1 & 7)) * 16;
+
+    bool copied = false;   // this wave has copies in flight for the slab consumed next
+    loader_open();
+    copied = ld_valid;
+#pragma unroll
+    for (int c = 0; c < kCopiesPerWave; ++c) issue_copy(0, c);
+    loader_advance();
+
+    int slot = 0;            // LDS buffer of the slab consumed next
+    int stores_young = 0;    // 16 / 32: that many output stores of a full tile were issued after the copies in flight
+    for (int n = 0; n < rounds; ++n) {
+        int m0, n0, z, kb, nk;
+        if (!decode(n, m0, n0, z, kb, nk)) continue;
+        floatx16 acc[4][kTN];
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+#pragma unroll
+            for (int j = 0; j < kTN; ++j)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
+
+        for (int ks = 0; ks < nk; ++ks) {
+#ifdef GEMM_PROF
+            long long t0 = clock64();
+#endif
+            // Memory operations complete in issue order: a copier waits until nothing but the output stores
+            // issued after its copies (if any) is outstanding.
+            if (copied) {
+                if (stores_young == 32) wait_vm<32>();
+                else if (stores_young == 16) wait_vm<16>();
+                else wait_vm<0>();
+            }
+            stores_young = 0;
+#ifdef GEMM_PROF
+            long long t1 = clock64();
+#endif
+            // a bare barrier: every copier has waited for its own copies above, and a fence here would
+            // make the compiler drain memory operations that are meant to stay in flight
+            __builtin_amdgcn_s_barrier();   // slab complete in LDS; the other buffer is no longer read
+#ifdef GEMM_PROF
+            long long t2 = clock64();
+#endif
+            const int fill = slot ^ 1;
+            const char* st = lds + slot * kSlabBytes;
+            slot ^= 1;
+            // Source order below is the schedule (pinned by sched_barrier): fragments of the next 16-wide
+            // k-step are read while this one is multiplied; a copier issues one copy after each of its
+            // first 16 MFMAs.
+            constexpr int KK = BK / 16;
+            constexpr int kPerStep = 4 * kTN;   // MFMAs per k-step
+            half8 af[2][4], bf[2][kTN];
+            auto read_frags = [&](int kk, int set) {
+#pragma unroll
+                for (int i = 0; i < 4; ++i)
+                    af[set][i] = *reinterpret_cast<const half8*>(st + a_frag + i * 32 * BK * 2 + pos[kk]);
+#pragma unroll
+                for (int j = 0; j < kTN; ++j)
+                    bf[set][j] = *reinterpret_cast<const half8*>(st + b_frag + j * 32 * BK * 2 + pos[kk]);
+            };
+#if GEMM_COPY_MODE == 0   // all copies first
+#pragma unroll
+            for (int c = 0; c < kCopiesPerWave; ++c) issue_copy(fill, c);
+            __builtin_amdgcn_sched_barrier(0);
+#endif
+            read_frags(0, 0);
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int kk = 0; kk < KK; ++kk) {
+                const int cur = kk & 1;
+                if (kk + 1 < KK) read_frags(kk + 1, cur ^ 1);
+                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int m = 0; m < kPerStep; ++m) {
+                    const int i = m / kTN, j = m % kTN;
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(bf[cur][j], af[cur][i], acc[i][j], 0, 0, 0);
+                    const int done = kk * kPerStep + m;
+                    (void)done;
+#if GEMM_COPY_MODE == 1   // staggered over the whole slab
+                    __builtin_amdgcn_sched_barrier(0);
+                    if (done % 4 == phase) issue_copy(fill, done / 4);
+                    __builtin_amdgcn_sched_barrier(0);
+#elif GEMM_COPY_MODE == 2   // one copy after every second MFMA of the first half
+                    if (done < 16 && done % 2 == 1) {
+                        __builtin_amdgcn_sched_barrier(0);
+                        issue_copy(fill, done / 2);
+                        __builtin_amdgcn_sched_barrier(0);
+                    }
+#elif GEMM_COPY_MODE == 3   // one copy after each of the first 8 MFMAs
+                    if (done < 8) {
+                        __builtin_amdgcn_sched_barrier(0);
+                        issue_copy(fill, done);
+                        __builtin_amdgcn_sched_barrier(0);
+                    }
+#endif
+                }
+            }
+            copied = ld_valid;
+            loader_advance();
+#ifdef GEMM_PROF
+            if (blockIdx.x == 0 && tid == GEMM_PROF) {
+                long long t4 = clock64();
+                g_gemm_prof[0] += t1 - t0; g_gemm_prof[1] += t2 - t1; g_gemm_prof[3] += t4 - t2; g_gemm_prof[4] += 1;
+            }
+#endif
+        }
+        const bool full = (m0 + BM <= g.M) && (n0 + BN <= g.N) && (g.ldc % 4 == 0);
+#ifdef GEMM_NOSTORE
+        { float t = 0; for (int i = 0; i < 4; ++i) for (int j = 0; j < kTN; ++j) for (int r = 0; r < 16; ++r) t += acc[i][j][r];
+          if (t == 1234.5f) g.C16[0] = (half_t)t; }
+        stores_young = 0;
+#else
+        if (full && g.C16 && g.ldc % 8 == 0 && reinterpret_cast<uintptr_t>(g.C16) % 16 == 0) {
+            store_tile_lines(g, acc, m0, n0, wm, wn, lane, lds + 2 * kSlabBytes + wave * kEpiBytesPerWave);
+            stores_young = 16;
+        } else {
+            store_tile(g, acc, m0, n0, wm, wn, lane, z);
+            stores_young = full ? 32 : -1;
+        }
+#endif
+    }
+    wait_vm<0>();   // no copy may still be heading for LDS when the workgroup retires
+}
+
 // TN form: C[M][N] = alpha * sum_k A[k][m] * B[k][n] with both operands stored k-major ([K][M] and
 // [K][N], m / n contiguous) -- the shape of the weight gradients dW = dG^T * X, whose operands come out
 // of the recurrence as [time*batch][features].  Slabs are staged in LDS exactly as they sit in memory
@@ -201,7 +473,8 @@ __global__ __launch_bounds__(kThreads) void gemm_nt_256x256(GemmNT g, int tiles_
 // are read with the gfx950 transposing LDS load ds_read_b64_tr_b16: in every group of 16 lanes, lane j
 // supplies 4 halfs of row j/4 and receives the k-column for its own m, so no transposed copy of the
 // operands ever exists in HBM.  Rows k >= K read as zero.
-constexpr int kPitchT = 256 + 16;   // halfs per LDS row: 4 consecutive k rows fall in distinct banks
+constexpr int kPitchT = 256 + 32;   // halfs per LDS row: 576 bytes = 64 mod 256, so the four k rows that 32 lanes
+                                    // read together (64 bytes each) cover the 64 banks exactly once
 constexpr size_t kLdsBytesTN = size_t(2) * 2 * BK * kPitchT * sizeof(half_t);
 
 typedef short short4v __attribute__((ext_vector_type(4)));
@@ -214,14 +487,45 @@ __device__ __forceinline__ half8 read_frag_tr(const half_t* lds_lane) {
     return u.h;
 }
 
-__global__ __launch_bounds__(kThreads) void gemm_tn_256x256(GemmNT g, int tiles_m, int tiles_n,
-                                                             int slabs_per_split) {
+// fp32 epilogue of a full tile with whole-line stores (split-K partials): every 32 x 32 accumulator tile
+// is one 128-byte line per row; it is turned through a private 4 KiB of LDS so that 8 lanes hold one row
+// and a store instruction writes 8 complete lines instead of 32 quarter lines.
+__device__ __forceinline__ void store_tile_lines_f32(const GemmNT& g, floatx16 (&acc)[4][kTN], int m0, int n0,
+                                                     int wm, int wn, int lane, int z, char* stage) {
+    const int wr = lane % 32;
+    const int wsw = (wr >> 1) & 7;
+    const int rr = lane / 8, rc = lane % 8;
+    float* cbase = g.C32 + size_t(z) * g.split_stride + size_t(m0 + wm * 128) * g.ldc + n0 + wn * 32 * kTN + rc * 4;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+#pragma unroll
+        for (int j = 0; j < kTN; ++j) {
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                floatx4 v;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) v[e] = g.alpha * acc[i][j][4 * q + e];
+                const int chunk = 2 * q + lane / 32;
+                *reinterpret_cast<floatx4*>(stage + wr * 128 + ((chunk ^ wsw) * 16)) = v;
+            }
+#pragma unroll
+            for (int p = 0; p < 4; ++p) {
+                const int row = rr + 8 * p;
+                const floatx4 v = *reinterpret_cast<const floatx4*>(stage + row * 128 + ((rc ^ ((row >> 1) & 7)) * 16));
+                *reinterpret_cast<floatx4*>(cbase + size_t(i * 32 + row) * g.ldc + j * 32) = v;
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    }
+}
+
+__global__ __launch_bounds__(kThreads) void gemm_tn_256x256(GemmNT g, TileOrder order, int slabs_per_split) {
     extern __shared__ __attribute__((aligned(16))) half_t smem[];
     half_t* As = smem;                        // [2][BK][kPitchT]
     half_t* Bs = smem + 2 * BK * kPitchT;     // [2][BK][kPitchT]
 
     int tm, tn, z;
-    if (!work_item(tiles_m, tiles_n, gridDim.y, tm, tn, z)) return;
+    if (!work_item(order, blockIdx.x, tm, tn, z)) return;
     const int m0 = tm * BM, n0 = tn * BN;
     const int nslab_total = (g.K + BK - 1) / BK;
     const int slab_begin = z * slabs_per_split;
@@ -316,10 +620,32 @@ __global__ __launch_bounds__(kThreads) void gemm_tn_256x256(GemmNT g, int tiles_
         if (more) stage(cur ^ 1);
         __syncthreads();
     }
+    const bool full = (m0 + BM <= g.M) && (n0 + BN <= g.N) && (g.ldc % 4 == 0);
+    if (full && g.C32) {
+        // the slab buffers are free once every wave has left the main loop (the barrier that ends it)
+        store_tile_lines_f32(g, acc, m0, n0, wm, wn, lane, z, reinterpret_cast<char*>(smem) + wave * 4096);
+        return;
+    }
     store_tile(g, acc, m0, n0, wm, wn, lane, z);
 }
 
 }  // namespace
+
+static TileOrder make_order(int tiles_m, int tiles_n, int splits) {
+    TileOrder o{};
+    o.tiles_m = tiles_m; o.tiles_n = tiles_n; o.splits = splits;
+    long best = -1;
+    const int shapes[6] = {8, 4, 16, 2, 32, 1};   // sm candidates, preferred first
+    for (int sm : shapes) {
+        const int sn = 32 / sm;
+        const long n = long((tiles_m + sm - 1) / sm) * ((tiles_n + sn - 1) / sn);
+        if (best < 0 || n < best) { best = n; o.sm = sm; o.sn = sn; }
+    }
+    o.nsm = (tiles_m + o.sm - 1) / o.sm;
+    o.nsn = (tiles_n + o.sn - 1) / o.sn;
+    o.per_xcd = (o.nsm * o.nsn * splits + 7) / 8;
+    return o;
+}
 
 hipError_t launch_gemm_nt(const GemmNT& g, hipStream_t stream) {
     if (g.M <= 0 || g.N <= 0 || g.K <= 0) return hipSuccess;
@@ -347,11 +673,21 @@ hipError_t launch_gemm_nt(const GemmNT& g, hipStream_t stream) {
         attr_set = true;
     }
     const int tiles_m = (g.M + BM - 1) / BM, tiles_n = (g.N + BN - 1) / BN;
-    // gridDim.y carries the split count; x is padded so that x*y is a whole number of 256-workgroup rounds
-    const int items = tiles_m * tiles_n * splits;
-    const int rounded = (items + 255) / 256 * 256;
-    dim3 grid((rounded + splits - 1) / splits, splits, 1);
-    hipLaunchKernelGGL(gemm_nt_256x256, grid, dim3(kThreads), kLdsBytes, stream, g, tiles_m, tiles_n,
+    const TileOrder order = make_order(tiles_m, tiles_n, splits);
+    static const bool staged = getenv("FLASHLSTM_GEMM_STAGED") != nullptr;
+    if (!staged) {
+        static bool attr2 = false;
+        if (!attr2) {
+            hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_nt_stream),
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, int(kLdsBytesStream));
+            if (e != hipSuccess) return e;
+            attr2 = true;
+        }
+        hipLaunchKernelGGL(gemm_nt_stream, dim3(256), dim3(kThreads), kLdsBytesStream, stream, g, order,
+                           slabs_per_split * BK);
+        return hipGetLastError();
+    }
+    hipLaunchKernelGGL(gemm_nt_256x256, dim3(order.per_xcd * 256), dim3(kThreads), kLdsBytes, stream, g, order,
                        slabs_per_split * BK);
     return hipGetLastError();
 }
@@ -375,10 +711,8 @@ hipError_t launch_gemm_tn(const GemmNT& g, hipStream_t stream) {
     const int nslab = (g.K + BK - 1) / BK;
     const int slabs_per_split = (nslab + splits - 1) / splits;
     const int tiles_m = (g.M + BM - 1) / BM, tiles_n = (g.N + BN - 1) / BN;
-    const int items = tiles_m * tiles_n * splits;
-    const int rounded = (items + 255) / 256 * 256;
-    dim3 grid((rounded + splits - 1) / splits, splits, 1);
-    hipLaunchKernelGGL(gemm_tn_256x256, grid, dim3(kThreads), kLdsBytesTN, stream, g, tiles_m, tiles_n,
+    const TileOrder order = make_order(tiles_m, tiles_n, splits);
+    hipLaunchKernelGGL(gemm_tn_256x256, dim3(order.per_xcd * 256), dim3(kThreads), kLdsBytesTN, stream, g, order,
                        slabs_per_split);
     return hipGetLastError();
 }
