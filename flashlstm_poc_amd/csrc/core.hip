@@ -62,8 +62,7 @@ struct flstm_core_plan {
     DevBuf wih_p, wih_t, wfrag_f, wfrag_b, bias_p;
     bool weights_packed = false, bias_packed = false;
     // forward state / caches
-    DevBuf X16, G, Y, C, flags_f, flags_b, status, xch_f, xch_b;
-    unsigned epoch_f = 0, epoch_b = 0;
+    DevBuf X16, G, Y, C, status, xch_f, xch_b;
     size_t T_cache = 0;
     bool have_cache = false;
     // backward scratch
@@ -136,7 +135,7 @@ extern "C" int flstm_core_create(size_t batch, size_t input_size, size_t hidden_
 extern "C" int flstm_core_destroy(flstm_core_plan* p) {
     if (!p) return FLSTM_E_INVALID;
     for (DevBuf* b : {&p->wih_p, &p->wih_t, &p->wfrag_f, &p->wfrag_b, &p->bias_p, &p->X16, &p->G, &p->Y, &p->C,
-                      &p->flags_f, &p->flags_b, &p->status, &p->xch_f, &p->xch_b, &p->dYp, &p->dG, &p->dHn, &p->dC,
+                      &p->status, &p->xch_f, &p->xch_b, &p->dYp, &p->dG, &p->dHn, &p->dC,
                       &p->dH0, &p->db_part, &p->dw_part, &p->prof})
         b->release();
     p->tm.destroy();
@@ -236,18 +235,16 @@ int forward_once(flstm_core_plan* p, size_t T, const void* x, flstm_dtype x_dtyp
     FL_TRY(p->G.reserve(TB * 4 * d.Hp * sizeof(half_t)));
     FL_TRY(p->Y.reserve((TB + d.B) * d.Hp * sizeof(half_t)));
     FL_TRY(p->C.reserve((TB + d.B) * d.Hp * sizeof(float)));
-    FL_TRY(p->flags_f.reserve(size_t(p->Lf.ng) * 256 * sizeof(unsigned)));
-    if (p->epoch_f == 0 || p->epoch_f > 0x70000000u) {
-        FL_TRY(fill_zero(p->flags_f.p, p->flags_f.bytes, s));
-        p->epoch_f = 0;
-    }
     // initial state rows
     if (h0) FL_TRY(convert_pad(h0, state_dtype == FLSTM_F32, size_t(d.B), d.H, size_t(d.H), 1.f, p->Y.as<half_t>(),
                                size_t(d.B), size_t(d.Hp), s));
     else FL_TRY(fill_zero(p->Y.p, size_t(d.B) * d.Hp * sizeof(half_t), s));
     FL_TRY(convert_pad_f32(c0, state_dtype == FLSTM_F32, size_t(d.B), d.H, 1.f, p->C.as<float>(), size_t(d.Hp), s));
     const size_t xslot = exchange_slot_halfs(d.B, d.Hp);
-    FL_TRY(p->xch_f.reserve(2 * xslot * sizeof(half_t)));
+    // exchange ring: slot 0 = h0 (rows past B zero), slots 1 and 2 = the 'unwritten' pattern
+    FL_TRY(p->xch_f.reserve(3 * xslot * sizeof(half_t)));
+    FL_TRY(fill_zero(p->xch_f.p, xslot * sizeof(half_t), s));
+    FL_TRY(fill_words(p->xch_f.as<half_t>() + xslot, 2 * xslot * sizeof(half_t), 0xFFFFFFFFu, s));
     FL_TRY(to_exchange_layout(p->Y.as<half_t>(), d.B, d.Hp, size_t(d.Hp), p->xch_f.as<half_t>(), s));
 
     FL_TRY(hipEventRecord(p->tm.ev[0], s));
@@ -269,18 +266,17 @@ int forward_once(flstm_core_plan* p, size_t T, const void* x, flstm_dtype x_dtyp
     a.Y = p->Y.as<half_t>(); a.G = p->G.as<half_t>(); a.C = p->C.as<float>();
     a.X = p->xch_f.as<half_t>(); a.x_slot = xslot;
     a.bias = p->bias_p.as<float>();
-    a.flags = p->flags_f.as<unsigned>(); a.status = p->status.as<int>();
+    a.status = p->status.as<int>();
     a.seats = p->status.as<unsigned>() + 8;
     FL_TRY(fill_zero(a.seats, 8 * sizeof(unsigned), s));
     a.B = d.B; a.Hp = d.Hp; a.T = int(T);
-    a.epoch = p->epoch_f; a.spin_limit = p->opt_spin_limit;
+    a.spin_limit = p->opt_spin_limit;
     a.prof = nullptr;
     if (p->opt_profile) {
         FL_TRY(fill_zero(p->prof.p, 16 * sizeof(long long), s));
         a.prof = p->prof.as<long long>();
     }
     FL_TRY(launch_rec_fwd(p->Lf, a, s));
-    p->epoch_f += unsigned(T) + 1;
     FL_TRY(hipEventRecord(p->tm.ev[2], s));
     return 0;
 }
@@ -311,8 +307,6 @@ extern "C" int flstm_core_forward(flstm_core_plan* p, size_t T, const void* x, f
         p->broken_fwd = true;
         p->fallbacks++;
         replan(p);
-        FL_TRY(fill_zero(p->flags_f.p, p->flags_f.bytes, s));
-        p->epoch_f = 0;
         rc = forward_once(p, T, x, x_dtype, h0, c0, state_dtype, s);
         if (rc) return rc;
         rc = read_status(p, s, &st);
@@ -357,13 +351,9 @@ int backward_rec_once(flstm_core_plan* p, size_t T, const void* dY, flstm_dtype 
     FL_TRY(p->dH0.reserve(st_bytes));
     FL_TRY(p->dG.reserve(TB * 4 * d.Hp * sizeof(half_t)));
     FL_TRY(p->db_part.reserve(size_t(p->Lb.ng) * 4 * d.Hp * sizeof(float)));
-    FL_TRY(p->flags_b.reserve(size_t(p->Lb.ng) * 256 * sizeof(unsigned)));
     const size_t xslot = exchange_slot_halfs(d.B, 4 * d.Hp);
-    FL_TRY(p->xch_b.reserve(2 * xslot * sizeof(half_t)));
-    if (p->epoch_b == 0 || p->epoch_b > 0x70000000u) {
-        FL_TRY(fill_zero(p->flags_b.p, p->flags_b.bytes, s));
-        p->epoch_b = 0;
-    }
+    FL_TRY(p->xch_b.reserve(3 * xslot * sizeof(half_t)));
+    FL_TRY(fill_words(p->xch_b.p, 3 * xslot * sizeof(half_t), 0xFFFFFFFFu, s));
     FL_TRY(convert_pad_f32(d_hn, dstate_dtype == FLSTM_F32, size_t(d.B), d.H, S, p->dHn.as<float>(), size_t(d.Hp), s));
     FL_TRY(convert_pad_f32(d_cn, dstate_dtype == FLSTM_F32, size_t(d.B), d.H, S, p->dC.as<float>(), size_t(d.Hp), s));
     FL_TRY(fill_zero(p->db_part.p, size_t(p->Lb.ng) * 4 * d.Hp * sizeof(float), s));
@@ -375,18 +365,17 @@ int backward_rec_once(flstm_core_plan* p, size_t T, const void* dY, flstm_dtype 
     a.dHn = p->dHn.as<float>(); a.dC = p->dC.as<float>(); a.dH0 = p->dH0.as<float>();
     a.X = p->xch_b.as<half_t>(); a.x_slot = xslot;
     a.db_part = p->db_part.as<float>();
-    a.flags = p->flags_b.as<unsigned>(); a.status = p->status.as<int>();
+    a.status = p->status.as<int>();
     a.seats = p->status.as<unsigned>() + 8;
     FL_TRY(fill_zero(a.seats, 8 * sizeof(unsigned), s));
     a.B = d.B; a.Hp = d.Hp; a.T = int(T); a.jb_fwd = d.JF; a.dy_scale = dy_scale;
-    a.epoch = p->epoch_b; a.spin_limit = p->opt_spin_limit;
+    a.spin_limit = p->opt_spin_limit;
     a.prof = nullptr;
     if (p->opt_profile) {
         FL_TRY(fill_zero(p->prof.p, 16 * sizeof(long long), s));
         a.prof = p->prof.as<long long>() + 8;
     }
     FL_TRY(launch_rec_bwd(p->Lb, a, s));
-    p->epoch_b += unsigned(T) + 2;
     FL_TRY(hipEventRecord(p->tm.ev[4], s));
     return 0;
 }
@@ -419,8 +408,6 @@ extern "C" int flstm_core_backward(flstm_core_plan* p, size_t T, const void* x, 
         p->broken_bwd = true;
         p->fallbacks++;
         replan(p);
-        FL_TRY(fill_zero(p->flags_b.p, p->flags_b.bytes, s));
-        p->epoch_b = 0;
         rc = backward_rec_once(p, T, dY, dy_dtype, d_hn, d_cn, dstate_dtype, S, s);
         if (rc) return rc;
         rc = read_status(p, s, &st);

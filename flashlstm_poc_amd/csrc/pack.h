@@ -56,5 +56,7 @@ hipError_t reduce_db(const Dims& d, const float* db_part, int ng, float scale, f
                      hipStream_t s);
 
 hipError_t fill_zero(void* p, size_t bytes, hipStream_t s);
+// Fills a buffer (multiple of 4 bytes) with one 32-bit pattern; a kernel, so it may be captured in a graph.
+hipError_t fill_words(void* p, size_t bytes, unsigned value, hipStream_t s);
 
 }  // namespace flstm_hip

@@ -176,9 +176,9 @@ __global__ void copy16_kernel(const uint4* __restrict__ in, uint4* __restrict__ 
     for (size_t i = size_t(blockIdx.x) * kT + threadIdx.x; i < n16; i += stride) out[i] = in[i];
 }
 
-__global__ void fill_zero_kernel(unsigned* p, size_t words) {
+__global__ void fill_words_kernel(unsigned* p, size_t words, unsigned value) {
     const size_t stride = size_t(gridDim.x) * kT;
-    for (size_t i = size_t(blockIdx.x) * kT + threadIdx.x; i < words; i += stride) p[i] = 0u;
+    for (size_t i = size_t(blockIdx.x) * kT + threadIdx.x; i < words; i += stride) p[i] = value;
 }
 
 }  // namespace
@@ -303,13 +303,15 @@ hipError_t reduce_db(const Dims& d, const float* db_part, int ng, float scale, f
     return hipGetLastError();
 }
 
-hipError_t fill_zero(void* p, size_t bytes, hipStream_t s) {
+hipError_t fill_words(void* p, size_t bytes, unsigned value, hipStream_t s) {
     if (bytes == 0) return hipSuccess;
     const size_t words = bytes / 4;  // all buffers of this library are multiples of 4 bytes
     int blocks = grid_for(words);
     if (blocks > 4096) blocks = 4096;
-    hipLaunchKernelGGL(fill_zero_kernel, dim3(blocks), dim3(kT), 0, s, static_cast<unsigned*>(p), words);
+    hipLaunchKernelGGL(fill_words_kernel, dim3(blocks), dim3(kT), 0, s, static_cast<unsigned*>(p), words, value);
     return hipGetLastError();
 }
+
+hipError_t fill_zero(void* p, size_t bytes, hipStream_t s) { return fill_words(p, bytes, 0u, s); }
 
 }  // namespace flstm_hip

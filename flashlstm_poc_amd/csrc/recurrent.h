@@ -22,17 +22,17 @@ struct RecLayout {
 struct RecFwdArgs {
     const half8* wfrag;  // [nh][4 waves][ks][nt][64 lanes] MFMA B-fragments of W_hh (packed gate order)
     half_t* Y;           // [(T+1)*B][Hp]; rows [0,B) = h0, rows [(t+1)B, (t+2)B) = h_t (row-major, for later kernels)
-    half_t* X;           // exchange ring, 2 slots of x_slot halfs, fragment-major; step t reads slot t&1 (h_{t-1})
+    half_t* X;           // exchange ring, 3 slots of x_slot halfs, fragment-major; step t reads slot t%3 (h_{t-1}),
+                         // writes slot (t+1)%3; before a launch slot 0 holds h0 (padding rows zero) and the
+                         // other two hold the 0xFFFF 'unwritten' pattern
     size_t x_slot;
     half_t* G;           // [T*B][4Hp] packed gate order; in: x-projection, out: activated i,f,g,o
     float* C;            // [(T+1)*B][Hp]; rows [0,B) = c0, rows [(t+1)B, ..) = c_t
     const float* bias;   // [4Hp] packed gate order, b_ih + b_hh
-    unsigned* flags;     // [ng][256]
     unsigned* seats;     // [8] zeroed before every launch: next free workgroup slot per XCD
     int* status;         // 0 ok, 1 spin limit hit, 2 workgroup not on the expected XCD
     int B, Hp, T;
-    unsigned epoch;
-    int spin_limit;
+    int spin_limit;      // reloads of a fragment chunk that still shows the 'unwritten' pattern before giving up
     long long* prof;     // optional [8] cycle counters of workgroup 0 per phase (null = off)
 };
 
@@ -42,19 +42,18 @@ struct RecBwdArgs {
     const float* C;      // cell states [(T+1)*B][Hp]
     const half_t* dY;    // [T*B][Hp] upstream gradient
     half_t* dG;          // [T*B][4Hp] pre-activation gradients (scaled), row-major, for the GEMMs
-    half_t* X;           // exchange ring, 2 slots of x_slot halfs, fragment-major; step t writes slot t&1 (dG_t)
+    half_t* X;           // exchange ring, 3 slots of x_slot halfs, fragment-major; step t writes slot t%3 (dG_t);
+                         // before a launch all three hold the 0xFFFF 'unwritten' pattern
     size_t x_slot;
     float* dHn;          // [B][Hp] scaled gradient wrt final h (zeros when absent)
     float* dC;           // [B][Hp] running scaled dc; in: gradient wrt final c, out: dc0
     float* dH0;          // [B][Hp] out: scaled gradient wrt h0
     float* db_part;      // [ng][4Hp] scaled bias-gradient partial sums (accumulated into)
-    unsigned* flags;     // [ng][256]
     unsigned* seats;     // [8] zeroed before every launch
     int* status;
     int B, Hp, T;
     int jb_fwd;          // hidden units per slice in the packed gate order of G / dG
     float dy_scale;      // factor applied to dY on load (the loss scale, or 1 when dY is pre-scaled)
-    unsigned epoch;
     int spin_limit;
     long long* prof;     // optional [8] cycle counters of workgroup 0 per phase (null = off)
 };

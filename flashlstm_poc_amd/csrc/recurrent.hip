@@ -14,12 +14,17 @@
 //    so every element of h_{t-1} / dG_{t+1} is fetched exactly once per workgroup, straight from
 //    L2 into A-fragments; partial sums meet in LDS (fp32) and the pointwise stage reads them there.
 //  * Exchange.  h_t (forward) and dG_t (backward) are the only data that cross workgroups.  Groups
-//    are laid out so that all workgroups of a group sit on one XCD when the slice count allows
-//    (block id mod 8 is the XCD): producers use plain write-through stores, consumers fetch with
-//    device-scope relaxed atomic loads (L1 bypass, served by that XCD's L2), and a per-workgroup
-//    step flag in one cache line replaces the grid barrier -- no L2 write-back or invalidate is
-//    ever issued.  Groups that span XCDs store the exchanged values with device-scope atomic
-//    stores instead.  Every wait is bounded and reports through `status`.
+//    are laid out so that all workgroups of a group sit on one XCD when the slice count allows:
+//    producers use plain write-through stores, consumers fetch with device-scope loads (L1 bypass,
+//    served by that XCD's L2); no L2 write-back or invalidate is ever issued.  Groups that span XCDs
+//    store the exchanged values with device-scope atomic stores instead.
+//    There are no flags and no barrier between workgroups: the data validates itself.  The
+//    exchange ring has three slots; while a workgroup writes step t into one slot it refills its own
+//    region of the slot that step t+1 will use with a pattern no fp16 result can produce (0xFFFF pairs,
+//    a NaN payload the arithmetic never generates).  A consumer simply loads its MFMA fragments and,
+//    as long as a fragment still shows the pattern, loads it again.  Compared with a flag per
+//    workgroup this takes two L2 round trips (store acknowledgement, flag poll) off the path between
+//    one step and the next.  Every retry loop is bounded and reports through `status`.
 //  * Fallback.  The same kernels launched once per step (no waits, kernel boundaries order
 //    memory) serve shapes whose weights do not fit on chip, and are the safe path after a failed
 //    persistent launch.
@@ -72,39 +77,17 @@ __device__ __forceinline__ Role make_role(int nh, int ng, int gpx, int xcd_local
     return r;
 }
 
-// Waits until every workgroup of the group has published `target`. Returns false on abort.
-__device__ __forceinline__ bool wait_group(const unsigned* gflags, int nh, unsigned target,
-                                           int* status, int spin_limit, int* lds_abort) {
-    if (threadIdx.x < kWave) {
-        int spins = 0;
-        for (;;) {
-            bool ok = true;
-            for (int i = threadIdx.x; i < nh; i += kWave) {
-                const unsigned f = __hip_atomic_load(gflags + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                ok = ok && (int(f - target) >= 0);
-            }
-            if (__all(ok)) break;
-            if (++spins > spin_limit ||
-                ((spins & 1023) == 0 &&
-                 __hip_atomic_load(status, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == 1)) {
-                if (threadIdx.x == 0) {
-                    __hip_atomic_store(status, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                    *lds_abort = 1;
-                }
-                break;
-            }
-        }
-    }
-    __syncthreads();
-    return *lds_abort == 0;
-}
+// Pattern that marks a not-yet-written pair of halfs in the exchange ring.
+constexpr unsigned kUnwritten = 0xFFFFFFFFu;
 
-__device__ __forceinline__ void publish(unsigned* gflags, int hs, unsigned value) {
-    __builtin_amdgcn_s_waitcnt(0);  // every store of this wave has been acknowledged by L2
-    __syncthreads();
-    if (threadIdx.x == 0)
-        __hip_atomic_store(gflags + hs, value, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-}
+// How a persistent launch validates what it fetches (off for step-wise launches, where the kernel
+// boundary orders memory).
+struct Poll {
+    bool on;
+    int limit;        // reloads of one fragment chunk before the launch gives up
+    int* status;      // global: 1 = gave up
+    int* lds_abort;   // workgroup: some wave gave up
+};
 
 // Exchange layout ("fragment-major").  The operand a step fetches from its peers -- h_{t-1} in the
 // forward pass, dG_{t+1} in the backward pass -- is stored as ready-made MFMA A-fragments so that
@@ -153,7 +136,7 @@ template <int NT, int KS, bool RESIDENT, int KL = 0>
 __device__ __forceinline__ void wave_product(floatx4 (&acc)[2][NT], const half8 (&wreg)[KS - KL][NT],
                                              const half8* wlds, const half8* wfrag_wave, const half_t* a0,
                                              const half_t* a1, int wave, int lane, int nks_total,
-                                             int ks_wave) {
+                                             int ks_wave, const Poll& poll) {
     if constexpr (RESIDENT && (KS % 8 == 0)) {
         // Loads and MFMAs are unconditional: k-steps beyond the real contraction length fetch a
         // clamped (finite) address and meet all-zero weight fragments.  Chunks of 4 k-steps (8
@@ -178,6 +161,35 @@ __device__ __forceinline__ void wave_product(floatx4 (&acc)[2][NT], const half8 
                 wait_frags<8>(fa[buf], fb[buf]);
             } else {
                 wait_frags<0>(fa[buf], fb[buf]);
+            }
+            if (poll.on) {
+                // A pair of halfs that still holds the pattern has not been written yet by its producer:
+                // fetch the chunk again (the chunk in flight behind it has to land first, loads return
+                // in order).  The decision is wave-uniform.
+                int spins = 0;
+                for (;;) {
+                    unsigned m = 0u;
+#pragma unroll
+                    for (int k = 0; k < 4; ++k) {
+                        const uint4 ua = __builtin_bit_cast(uint4, fa[buf][k]);
+                        const uint4 ub = __builtin_bit_cast(uint4, fb[buf][k]);
+                        m = max(m, max(max(ua.x, ua.y), max(ua.z, ua.w)));
+                        m = max(m, max(max(ub.x, ub.y), max(ub.z, ub.w)));
+                    }
+                    if (!__any(m == kUnwritten)) break;
+                    ++spins;
+                    if (spins > poll.limit || *reinterpret_cast<volatile int*>(poll.lds_abort) != 0 ||
+                        ((spins & 255) == 0 &&
+                         __hip_atomic_load(poll.status, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0)) {
+                        if (lane == 0) {
+                            __hip_atomic_store(poll.status, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                            *reinterpret_cast<volatile int*>(poll.lds_abort) = 1;
+                        }
+                        break;   // results are garbage from here on; the workgroup leaves at its next barrier
+                    }
+                    issue(c, buf);
+                    wait_frags<0>(fa[buf], fb[buf]);
+                }
             }
 #pragma unroll
             for (int k = 0; k < 4; ++k) {
@@ -222,23 +234,6 @@ __device__ __forceinline__ void spill_partials(float* part, const floatx4 (&acc)
                 base[(m * 16 + 4 * (lane / 16) + i) * pld + n * 16 + lane % 16] = acc[m][n][i];
 }
 
-__device__ __forceinline__ void store_h2(half_t* dst, float a, float b, bool device_scope) {
-    union { half_t h[2]; unsigned u; } v;
-    v.h[0] = (half_t)a;
-    v.h[1] = (half_t)b;
-    if (device_scope)
-        __hip_atomic_store(reinterpret_cast<unsigned*>(dst), v.u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    else
-        *reinterpret_cast<unsigned*>(dst) = v.u;
-}
-
-__device__ __forceinline__ void load_h2(const half_t* src, float& a, float& b) {
-    union { half_t h[2]; unsigned u; } v;
-    v.u = *reinterpret_cast<const unsigned*>(src);
-    a = (float)v.h[0];
-    b = (float)v.h[1];
-}
-
 __device__ __forceinline__ void unpack_h2(unsigned u, float& a, float& b) {
     union { half_t h[2]; unsigned u; } v;
     v.u = u;
@@ -253,54 +248,137 @@ __device__ __forceinline__ unsigned pack_h2(float a, float b) {
     return v.u;
 }
 
-__device__ __forceinline__ void store_u32(half_t* dst, unsigned u, bool device_scope) {
+// The pointwise stage gives every thread one GROUP of N consecutive hidden units of one batch row
+// (N = 4 for 32-unit slices, 2 for 16-unit slices: 8 groups per row, 256 groups per row block), so
+// that its global accesses are as wide as the work split allows: a vector-memory instruction costs
+// the same 16+ clocks of address processing whatever its width, and the steps are short enough for
+// that to show.  Pack<N> is N halfs as raw bits.
+template <int N> struct Pack;
+template <> struct Pack<2> { unsigned v; };
+template <> struct Pack<4> { uint2 v; };
+
+__device__ __forceinline__ Pack<2> ld_pack(const half_t* p, Pack<2>*) { return Pack<2>{*reinterpret_cast<const unsigned*>(p)}; }
+__device__ __forceinline__ Pack<4> ld_pack(const half_t* p, Pack<4>*) { return Pack<4>{*reinterpret_cast<const uint2*>(p)}; }
+__device__ __forceinline__ void st_pack(half_t* p, Pack<2> v) { *reinterpret_cast<unsigned*>(p) = v.v; }
+__device__ __forceinline__ void st_pack(half_t* p, Pack<4> v) { *reinterpret_cast<uint2*>(p) = v.v; }
+__device__ __forceinline__ void unpack(Pack<2> v, float (&f)[2]) { unpack_h2(v.v, f[0], f[1]); }
+__device__ __forceinline__ void unpack(Pack<4> v, float (&f)[4]) {
+    unpack_h2(v.v.x, f[0], f[1]);
+    unpack_h2(v.v.y, f[2], f[3]);
+}
+__device__ __forceinline__ Pack<2> pack(const float (&f)[2]) { return Pack<2>{pack_h2(f[0], f[1])}; }
+__device__ __forceinline__ Pack<4> pack(const float (&f)[4]) {
+    return Pack<4>{uint2{pack_h2(f[0], f[1]), pack_h2(f[2], f[3])}};
+}
+__device__ __forceinline__ Pack<2> pack_fill(unsigned w, Pack<2>*) { return Pack<2>{w}; }
+__device__ __forceinline__ Pack<4> pack_fill(unsigned w, Pack<4>*) { return Pack<4>{uint2{w, w}}; }
+
+// One group into the exchange ring.  Consumers validate every 32-bit word on its own, so the two words
+// of an 8-byte group need not become visible together.
+__device__ __forceinline__ void store_xch(half_t* dst, Pack<2> v, bool device_scope) {
     if (device_scope)
-        __hip_atomic_store(reinterpret_cast<unsigned*>(dst), u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __hip_atomic_store(reinterpret_cast<unsigned*>(dst), v.v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     else
-        *reinterpret_cast<unsigned*>(dst) = u;
+        *reinterpret_cast<unsigned*>(dst) = v.v;
+}
+__device__ __forceinline__ void store_xch(half_t* dst, Pack<4> v, bool device_scope) {
+    if (device_scope) {
+        const u64 w = (u64(v.v.y) << 32) | v.v.x;
+        __hip_atomic_store(reinterpret_cast<u64*>(dst), w, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    } else {
+        *reinterpret_cast<uint2*>(dst) = v.v;
+    }
 }
 
-// Cycle counters of workgroup 0 per phase (only when the host passes a buffer): wait, product,
-// partial exchange, pointwise, publish.
+__device__ __forceinline__ void ld_f32(const float* p, float (&f)[2]) {
+    const float2 v = *reinterpret_cast<const float2*>(p);
+    f[0] = v.x; f[1] = v.y;
+}
+__device__ __forceinline__ void ld_f32(const float* p, float (&f)[4]) {
+    const float4 v = *reinterpret_cast<const float4*>(p);
+    f[0] = v.x; f[1] = v.y; f[2] = v.z; f[3] = v.w;
+}
+__device__ __forceinline__ void st_f32(float* p, const float (&f)[2]) { *reinterpret_cast<float2*>(p) = float2{f[0], f[1]}; }
+__device__ __forceinline__ void st_f32(float* p, const float (&f)[4]) {
+    *reinterpret_cast<float4*>(p) = float4{f[0], f[1], f[2], f[3]};
+}
+// the same, past the L1 (the value was written by this thread through a plain store earlier on)
+__device__ __forceinline__ void ld_f32_coherent(const float* p, float (&f)[2]) {
+    union { u64 q; float v[2]; } u;
+    u.q = __hip_atomic_load(reinterpret_cast<const u64*>(p), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    f[0] = u.v[0]; f[1] = u.v[1];
+}
+__device__ __forceinline__ void ld_f32_coherent(const float* p, float (&f)[4]) {
+    union { u64 q[2]; float v[4]; } u;
+    u.q[0] = __hip_atomic_load(reinterpret_cast<const u64*>(p), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    u.q[1] = __hip_atomic_load(reinterpret_cast<const u64*>(p) + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) f[i] = u.v[i];
+}
+
+// Thread -> (row, group): the 8 groups of a row go to consecutive lanes, and the rows are taken in the
+// order 0, 8, 1, 9, ...: the 16 lanes that the LDS serves together then read the partial sums of rows
+// r and r + 8, which are 32 banks apart for every row pitch in use (132, 68, 36, 20 floats).
+__device__ __forceinline__ int group_row(int idx) { return (idx % 2) * 8 + (idx / 2) % 8 + (idx / 16) * 16; }
+
+// Cycle counters of workgroup 0 per phase (only when the host passes a buffer): product (including the
+// wait for the operand), partial exchange, pointwise, cache stores + prefetch.  Thread 0 accumulates in
+// LDS and writes the totals once at the end, so the measurement adds no memory round trips to a step.
 struct PhaseClock {
     long long* out;
     long long last;
-    __device__ __forceinline__ void start() { if (out) last = wall_clock64(); }
+    __device__ __forceinline__ long long* acc() {
+        __shared__ long long lds_acc[4];
+        return lds_acc;
+    }
+    __device__ __forceinline__ void start() {
+        if (out && threadIdx.x == 0) {
+            for (int i = 0; i < 4; ++i) acc()[i] = 0;
+            last = wall_clock64();
+        }
+    }
     __device__ __forceinline__ void lap(int slot) {
         if (out && threadIdx.x == 0) {
             const long long now = wall_clock64();
-            out[slot] += now - last;
+            acc()[slot] += now - last;
             last = now;
         }
+    }
+    __device__ __forceinline__ void flush() {
+        if (out && threadIdx.x == 0)
+            for (int i = 0; i < 4; ++i) out[i] += acc()[i];
     }
 };
 
 // ------------------------------------------------------------------------------------ forward
-// Per step and row block: [wait for h_{t-1}] -> K-split MFMA product -> partial sums through LDS ->
-// pointwise cell update -> store h_t, publish -> store c_t and the activated gates -> prefetch the
-// next step's x-projection.  Only the h_t store and the flag sit between this step and the next one
-// of the other workgroups; everything HBM-bound (x-projection fetch, cache stores) is off that path.
+// Per step and row block: K-split MFMA product on h_{t-1} as it arrives -> partial sums through LDS
+// (two buffers, one barrier per step) -> pointwise cell update -> store h_t -> store c_t and the
+// activated gates -> prefetch the next step's x-projection.  Only the h_t store sits between this step
+// and the next one of the other workgroups; everything HBM-bound (x-projection fetch, cache stores) is
+// off that path.
 template <int NT, int KS, bool RESIDENT>
 __global__ __launch_bounds__(kThreads) void rec_fwd_kernel(RecFwdArgs p, RecLayout L, int t_begin,
                                                            int t_end, int ks_wave) {
     constexpr int JB = 4 * NT;    // hidden units of this slice
     constexpr int NC = 16 * NT;   // gate columns of this slice (i,f,g,o blocks of JB)
     constexpr int PLD = NC + 4;
-    constexpr int NPAIR = kRows * (JB / 2);                 // unit pairs per row block
-    constexpr int NP = (NPAIR + kThreads - 1) / kThreads;   // pairs per thread
-    extern __shared__ __attribute__((aligned(16))) float part[];  // [4][32][PLD]
+    constexpr int UPT = JB / 8;               // hidden units per thread: 8 groups per batch row
+    static_assert(UPT == 2 || UPT == 4, "slices of 16 or 32 hidden units");
+    typedef Pack<UPT> PackT;
+    extern __shared__ __attribute__((aligned(16))) float part_all[];  // [2][4][32][PLD]
     __shared__ int lds_abort;
     __shared__ int lds_role[2];
 
+    if (threadIdx.x == 0) lds_abort = 0;
     const Role role = make_role(L.nh, L.ng, L.gpx, L.xcd_local, p.seats, p.status, lds_role);
     if (!role.active) return;
     const int tid = threadIdx.x, wave = tid / kWave, lane = tid % kWave;
-    if (tid == 0) lds_abort = 0;
     const int hs = role.hs, g = role.g;
     const int nks_total = p.Hp / 32;
     const bool device_scope = (L.persistent != 0) && (L.xcd_local == 0);
-    unsigned* gflags = p.flags + size_t(g) * 256;
+    const Poll poll{L.persistent != 0, p.spin_limit, p.status, &lds_abort};
     PhaseClock clk{(blockIdx.x == 0) ? p.prof : nullptr, 0};
+    int item = 0;   // work items done: selects the partial-sum buffer
 
     const half8* wfrag_wave = p.wfrag + (size_t(hs) * 4 + wave) * size_t(ks_wave) * NT * kWave;
     half8 wreg[KS][NT];
@@ -313,58 +391,40 @@ __global__ __launch_bounds__(kThreads) void rec_fwd_kernel(RecFwdArgs p, RecLayo
     }
 
     const size_t gld = size_t(4) * p.Hp;
-    // this thread's unit pairs: row r, units jj, jj+1 of the slice
-    int pr[NP], pj[NP];
-    bool pv[NP];
-    float2 bs[NP][4];
+    // this thread's group: row pr of the row block, units pj .. pj+UPT-1 of the slice
+    const int pr = group_row(tid / 8);
+    const int pj = (tid % 8) * UPT;
+    const int j = hs * JB + pj;   // first hidden unit of the group
+    float bs[4][UPT];
 #pragma unroll
-    for (int q = 0; q < NP; ++q) {
-        const int pidx = tid + q * kThreads;
-        pv[q] = pidx < NPAIR;
-        pr[q] = pv[q] ? pidx / (JB / 2) : 0;
-        pj[q] = pv[q] ? (pidx % (JB / 2)) * 2 : 0;
-#pragma unroll
-        for (int gt = 0; gt < 4; ++gt)
-            bs[q][gt] = *reinterpret_cast<const float2*>(p.bias + size_t(hs) * NC + gt * JB + pj[q]);
-    }
+    for (int gt = 0; gt < 4; ++gt) ld_f32(p.bias + size_t(hs) * NC + gt * JB + pj, bs[gt]);
     const int rb_count = (L.nrb - g + L.ng - 1) / L.ng;
     const bool c_in_regs = (rb_count == 1) && (t_end - t_begin > 1);
-    float2 creg[NP];
-    unsigned xp[NP][4];
+    float creg[UPT] = {};
+    PackT xp[4];
     auto prefetch = [&](int t, int rb) {
+        const int b = rb * kRows + pr;
+        if (b < p.B) {
+            const half_t* src = p.G + (size_t(t) * p.B + b) * gld + size_t(hs) * NC + pj;
 #pragma unroll
-        for (int q = 0; q < NP; ++q) {
-            const int b = rb * kRows + pr[q];
-            if (pv[q] && b < p.B) {
-                const half_t* src = p.G + (size_t(t) * p.B + b) * gld + size_t(hs) * NC + pj[q];
-#pragma unroll
-                for (int gt = 0; gt < 4; ++gt) xp[q][gt] = *reinterpret_cast<const unsigned*>(src + gt * JB);
-            }
+            for (int gt = 0; gt < 4; ++gt) xp[gt] = ld_pack(src + gt * JB, (PackT*)nullptr);
         }
     };
     if (c_in_regs) {
-#pragma unroll
-        for (int q = 0; q < NP; ++q) {
-            const int b = g * kRows + pr[q];
-            creg[q] = (pv[q] && b < p.B)
-                          ? *reinterpret_cast<const float2*>(p.C + (size_t(t_begin) * p.B + b) * p.Hp + hs * JB + pj[q])
-                          : float2{0.f, 0.f};
-        }
+        const int b = g * kRows + pr;
+        if (b < p.B) ld_f32(p.C + (size_t(t_begin) * p.B + b) * p.Hp + j, creg);
     }
     prefetch(t_begin, g);
     __syncthreads();
     clk.start();
 
     for (int t = t_begin; t < t_end; ++t) {
-        if (t > t_begin) {
-            if (!wait_group(gflags, L.nh, p.epoch + unsigned(t - t_begin), p.status, p.spin_limit, &lds_abort))
-                return;
-        }
-        clk.lap(0);
-        for (int rb = g; rb < L.nrb; rb += L.ng) {
+        for (int rb = g; rb < L.nrb; rb += L.ng, ++item) {
             const int row0 = rb * kRows;
-            const half_t* xin = p.X + size_t(t & 1) * p.x_slot;        // h_{t-1}, fragment-major
-            half_t* xout = p.X + size_t((t + 1) & 1) * p.x_slot;       // h_t
+            float* part = part_all + size_t(item & 1) * 4 * kRows * PLD;
+            const half_t* xin = p.X + size_t(t % 3) * p.x_slot;          // h_{t-1}, fragment-major
+            half_t* xout = p.X + size_t((t + 1) % 3) * p.x_slot;         // h_t
+            half_t* xnext = p.X + size_t((t + 2) % 3) * p.x_slot;        // will take h_{t+1}: marked unwritten
             const half_t* a0 = xin + size_t(2 * rb) * nks_total * 512 + lane * 8;
             const half_t* a1 = a0 + size_t(nks_total) * 512;
             floatx4 acc[2][NT];
@@ -372,79 +432,79 @@ __global__ __launch_bounds__(kThreads) void rec_fwd_kernel(RecFwdArgs p, RecLayo
             for (int m = 0; m < 2; ++m)
 #pragma unroll
                 for (int n = 0; n < NT; ++n) acc[m][n] = floatx4{0.f, 0.f, 0.f, 0.f};
-            wave_product<NT, KS, RESIDENT>(acc, wreg, nullptr, wfrag_wave, a0, a1, wave, lane, nks_total, ks_wave);
-            clk.lap(1);
+            wave_product<NT, KS, RESIDENT>(acc, wreg, nullptr, wfrag_wave, a0, a1, wave, lane, nks_total, ks_wave, poll);
+            clk.lap(0);
             spill_partials<NT>(part, acc, wave, lane, PLD);
             __syncthreads();
-            clk.lap(2);
+            if (lds_abort != 0) return;
+            clk.lap(1);
 
-            unsigned act[NP][4], hnew[NP];
-            float2 cnew[NP];
-#pragma unroll
-            for (int q = 0; q < NP; ++q) {
-                const int b = row0 + pr[q];
-                if (!(pv[q] && b < p.B)) continue;
-                float z[4][2];
+            // Every peer of this group has delivered h_{t-1}, so all of them are done reading h_{t-2}:
+            // its slot can be marked for reuse.  The mark is acknowledged long before the wait that
+            // precedes the h_t store below, so whoever sees this step's h_t also sees the mark.
+            const int b = row0 + pr;
+            const size_t xoff = xch_offset(b, j, nks_total);
+            store_xch(xnext + xoff, pack_fill(kUnwritten, (PackT*)nullptr), device_scope);
+            PackT act[4], hnew = pack_fill(0u, (PackT*)nullptr);   // batch rows past B travel as zeros
+            const bool live = b < p.B;
+            if (live) {
+                float z[4][UPT];
 #pragma unroll
                 for (int gt = 0; gt < 4; ++gt) {
-                    const int col = gt * JB + pj[q];
-                    float s0 = 0.f, s1 = 0.f;
+                    float x[UPT];
+                    unpack(xp[gt], x);
+#pragma unroll
+                    for (int u = 0; u < UPT; ++u) z[gt][u] = bs[gt][u] + x[u];
 #pragma unroll
                     for (int w = 0; w < 4; ++w) {
-                        const float2 v = *reinterpret_cast<const float2*>(part + (size_t(w) * kRows + pr[q]) * PLD + col);
-                        s0 += v.x;
-                        s1 += v.y;
-                    }
-                    float x0, x1;
-                    unpack_h2(xp[q][gt], x0, x1);
-                    z[gt][0] = s0 + x0 + bs[q][gt].x;
-                    z[gt][1] = s1 + x1 + bs[q][gt].y;
-                }
-                const int j = hs * JB + pj[q];
-                const float2 cp = c_in_regs ? creg[q]
-                                            : *reinterpret_cast<const float2*>(p.C + (size_t(t) * p.B + b) * p.Hp + j);
-                float cn[2], hn[2], a4[4][2];
+                        float v[UPT];
+                        ld_f32(part + (size_t(w) * kRows + pr) * PLD + gt * JB + pj, v);
 #pragma unroll
-                for (int u = 0; u < 2; ++u) {
+                        for (int u = 0; u < UPT; ++u) z[gt][u] += v[u];
+                    }
+                }
+                float cp[UPT];
+                if (c_in_regs) {
+#pragma unroll
+                    for (int u = 0; u < UPT; ++u) cp[u] = creg[u];
+                } else {
+                    ld_f32_coherent(p.C + (size_t(t) * p.B + b) * p.Hp + j, cp);
+                }
+                float hn[UPT], a4[4][UPT];
+#pragma unroll
+                for (int u = 0; u < UPT; ++u) {
                     const float ig = sigmoidf_dev(z[0][u]);
                     const float fg = sigmoidf_dev(z[1][u]);
                     const float gg = tanhf_dev(z[2][u]);
                     const float og = sigmoidf_dev(z[3][u]);
-                    cn[u] = fg * (u == 0 ? cp.x : cp.y) + ig * gg;
-                    hn[u] = og * tanhf_dev(cn[u]);
+                    creg[u] = fg * cp[u] + ig * gg;
+                    hn[u] = og * tanhf_dev(creg[u]);
                     a4[0][u] = ig; a4[1][u] = fg; a4[2][u] = gg; a4[3][u] = og;
                 }
-                // the exchanged value goes out first
-                hnew[q] = pack_h2(hn[0], hn[1]);
-                store_u32(xout + xch_offset(b, j, nks_total), hnew[q], device_scope);
-                cnew[q] = float2{cn[0], cn[1]};
-                creg[q] = cnew[q];
+                hnew = pack(hn);
 #pragma unroll
-                for (int gt = 0; gt < 4; ++gt) act[q][gt] = pack_h2(a4[gt][0], a4[gt][1]);
+                for (int gt = 0; gt < 4; ++gt) act[gt] = pack(a4[gt]);
             }
-            clk.lap(3);
-            const bool last_rb = (rb + L.ng >= L.nrb);
-            if (last_rb) publish(gflags, hs, p.epoch + unsigned(t - t_begin + 1));
-            else __syncthreads();
-            clk.lap(4);
+            // the exchanged value goes out first, after the mark above has been acknowledged
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+            store_xch(xout + xoff, hnew, device_scope);
+            clk.lap(2);
             // caches for the backward pass: off the critical path
+            if (live) {
+                st_f32(p.C + (size_t(t + 1) * p.B + b) * p.Hp + j, creg);
+                st_pack(p.Y + (size_t(t + 1) * p.B + b) * p.Hp + j, hnew);
+                half_t* dst = p.G + (size_t(t) * p.B + b) * gld + size_t(hs) * NC + pj;
 #pragma unroll
-            for (int q = 0; q < NP; ++q) {
-                const int b = row0 + pr[q];
-                if (!(pv[q] && b < p.B)) continue;
-                const int j = hs * JB + pj[q];
-                *reinterpret_cast<float2*>(p.C + (size_t(t + 1) * p.B + b) * p.Hp + j) = cnew[q];
-                *reinterpret_cast<unsigned*>(p.Y + (size_t(t + 1) * p.B + b) * p.Hp + j) = hnew[q];
-                half_t* dst = p.G + (size_t(t) * p.B + b) * gld + size_t(hs) * NC + pj[q];
-#pragma unroll
-                for (int gt = 0; gt < 4; ++gt) *reinterpret_cast<unsigned*>(dst + gt * JB) = act[q][gt];
+                for (int gt = 0; gt < 4; ++gt) st_pack(dst + gt * JB, act[gt]);
             }
             // x-projection of the next work item
             int nt_ = t, nrb_ = rb + L.ng;
             if (nrb_ >= L.nrb) { nt_ = t + 1; nrb_ = g; }
             if (nt_ < t_end) prefetch(nt_, nrb_);
+            clk.lap(3);
         }
     }
+    clk.flush();
 }
 
 // ----------------------------------------------------------------------------------- backward
@@ -456,27 +516,29 @@ __global__ __launch_bounds__(kThreads) void rec_bwd_kernel(RecBwdArgs p, RecLayo
     constexpr int JB = 16 * NT;  // hidden units (= output columns of dG*W_hh) of this slice
     constexpr int PLD = JB + 4;
     constexpr int KR = KS - KL;  // k-steps whose weight fragments stay in registers
-    constexpr int NPAIR = kRows * (JB / 2);
-    constexpr int NP = (NPAIR + kThreads - 1) / kThreads;
-    extern __shared__ __attribute__((aligned(16))) float part[];  // [4][32][PLD], reused for db
+    constexpr int UPT = JB / 8;               // hidden units per thread: 8 groups per batch row
+    static_assert(UPT == 2 || UPT == 4, "slices of 16 or 32 hidden units");
+    typedef Pack<UPT> PackT;
+    extern __shared__ __attribute__((aligned(16))) float part_all[];  // [2][4][32][PLD], reused for db
     __shared__ int lds_abort;
     __shared__ int lds_role[2];
 
+    if (threadIdx.x == 0) lds_abort = 0;
     const Role role = make_role(L.nh, L.ng, L.gpx, L.xcd_local, p.seats, p.status, lds_role);
     if (!role.active) return;
     const int tid = threadIdx.x, wave = tid / kWave, lane = tid % kWave;
-    if (tid == 0) lds_abort = 0;
     const int hs = role.hs, g = role.g;
     const int nks_total = p.Hp / 8;  // contraction over 4Hp packed gate columns
     const bool device_scope = (L.persistent != 0) && (L.xcd_local == 0);
-    unsigned* gflags = p.flags + size_t(g) * 256;
+    const Poll poll{L.persistent != 0, p.spin_limit, p.status, &lds_abort};
     const float S = p.dy_scale;
     PhaseClock clk{(blockIdx.x == 0) ? p.prof : nullptr, 0};
+    int item = 0;   // work items done: selects the partial-sum buffer
 
     const half8* wfrag_wave = p.wfrag + (size_t(hs) * 4 + wave) * size_t(ks_wave) * NT * kWave;
     half8 wreg[KR][NT];
-    // LDS: [partials 4*32*PLD floats | weight fragments of the last KL k-steps, one block per wave]
-    half8* wlds = reinterpret_cast<half8*>(part + 4 * kRows * PLD) + size_t(wave) * KL * NT * kWave;
+    // LDS: [partials 2*4*32*PLD floats | weight fragments of the last KL k-steps, one block per wave]
+    half8* wlds = reinterpret_cast<half8*>(part_all + 2 * 4 * kRows * PLD) + size_t(wave) * KL * NT * kWave;
     if constexpr (RESIDENT) {
 #pragma unroll
         for (int k = 0; k < KR; ++k)
@@ -492,64 +554,47 @@ __global__ __launch_bounds__(kThreads) void rec_bwd_kernel(RecBwdArgs p, RecLayo
     }
 
     const size_t gld = size_t(4) * p.Hp;
-    const int JF = p.jb_fwd;
-    int pr[NP], pj[NP];
-    bool pv[NP];
-    size_t pq[NP];  // packed gate column of (unit j, gate 0)
-#pragma unroll
-    for (int q = 0; q < NP; ++q) {
-        const int pidx = tid + q * kThreads;
-        pv[q] = pidx < NPAIR;
-        pr[q] = pv[q] ? pidx / (JB / 2) : 0;
-        pj[q] = pv[q] ? (pidx % (JB / 2)) * 2 : 0;
-        const int j = hs * JB + pj[q];
-        pq[q] = size_t(j / JF) * 4 * JF + (j % JF);
-    }
+    const int JF = p.jb_fwd;   // a multiple of 4: a group never straddles two blocks of the packed gate order
+    // this thread's group: row pr of the row block, units pj .. pj+UPT-1 of the slice
+    const int pr = group_row(tid / 8);
+    const int pj = (tid % 8) * UPT;
+    const int j = hs * JB + pj;
+    const size_t pq = size_t(j / JF) * 4 * JF + (j % JF);   // packed gate column of (unit j, gate 0)
     const int rb_count = (L.nrb - g + L.ng - 1) / L.ng;
     const bool dc_in_regs = (rb_count == 1) && (t_first - t_last > 0);
-    float2 dcreg[NP];
+    float dcreg[UPT] = {};
     if (dc_in_regs) {
-#pragma unroll
-        for (int q = 0; q < NP; ++q) {
-            const int b = g * kRows + pr[q];
-            dcreg[q] = (pv[q] && b < p.B) ? *reinterpret_cast<const float2*>(p.dC + size_t(b) * p.Hp + hs * JB + pj[q])
-                                          : float2{0.f, 0.f};
-        }
+        const int b = g * kRows + pr;
+        if (b < p.B) ld_f32(p.dC + size_t(b) * p.Hp + j, dcreg);
     }
     // prefetched per work item: activated gates, c_{t-1}, c_t, dY_t
-    unsigned pg[NP][4], pdy[NP];
-    float2 pcp[NP], pcc[NP];
+    PackT pg[4], pdy;
+    float pcp[UPT], pcc[UPT];
     auto prefetch = [&](int t, int rb) {
+        const int b = rb * kRows + pr;
+        if (b < p.B) {
+            const half_t* gsrc = p.G + (size_t(t) * p.B + b) * gld + pq;
 #pragma unroll
-        for (int q = 0; q < NP; ++q) {
-            const int b = rb * kRows + pr[q];
-            if (pv[q] && b < p.B) {
-                const int j = hs * JB + pj[q];
-                const half_t* gsrc = p.G + (size_t(t) * p.B + b) * gld + pq[q];
-#pragma unroll
-                for (int gt = 0; gt < 4; ++gt) pg[q][gt] = *reinterpret_cast<const unsigned*>(gsrc + gt * JF);
-                pcp[q] = *reinterpret_cast<const float2*>(p.C + (size_t(t) * p.B + b) * p.Hp + j);
-                pcc[q] = *reinterpret_cast<const float2*>(p.C + (size_t(t + 1) * p.B + b) * p.Hp + j);
-                pdy[q] = *reinterpret_cast<const unsigned*>(p.dY + (size_t(t) * p.B + b) * p.Hp + j);
-            }
+            for (int gt = 0; gt < 4; ++gt) pg[gt] = ld_pack(gsrc + gt * JF, (PackT*)nullptr);
+            ld_f32(p.C + (size_t(t) * p.B + b) * p.Hp + j, pcp);
+            ld_f32(p.C + (size_t(t + 1) * p.B + b) * p.Hp + j, pcc);
+            pdy = ld_pack(p.dY + (size_t(t) * p.B + b) * p.Hp + j, (PackT*)nullptr);
         }
     };
     if (t_first >= 0) prefetch(t_first, g);
     __syncthreads();
-    float dbacc[4][2] = {{0.f, 0.f}, {0.f, 0.f}, {0.f, 0.f}, {0.f, 0.f}};
+    float dbacc[4][UPT] = {};
     clk.start();
 
     for (int t = t_first; t >= t_last; --t) {
         const bool from_product = (t < p.T - 1);
-        if (t < t_first) {
-            if (!wait_group(gflags, L.nh, p.epoch + unsigned(t_first - t), p.status, p.spin_limit, &lds_abort))
-                return;
-        }
-        clk.lap(0);
-        for (int rb = g; rb < L.nrb; rb += L.ng) {
+        for (int rb = g; rb < L.nrb; rb += L.ng, ++item) {
             const int row0 = rb * kRows;
+            float* part = part_all + size_t(item & 1) * 4 * kRows * PLD;
+            // ring slot of step u is (u + 3) % 3: this step reads dG_{t+1}, writes dG_t and marks the
+            // slot of dG_{t-1} unwritten
             if (from_product) {
-                const half_t* xin = p.X + size_t((t + 1) & 1) * p.x_slot;   // dG_{t+1}, fragment-major
+                const half_t* xin = p.X + size_t((t + 4) % 3) * p.x_slot;   // dG_{t+1}, fragment-major
                 const half_t* a0 = xin + size_t(2 * rb) * nks_total * 512 + lane * 8;
                 const half_t* a1 = a0 + size_t(nks_total) * 512;
                 floatx4 acc[2][NT];
@@ -557,130 +602,125 @@ __global__ __launch_bounds__(kThreads) void rec_bwd_kernel(RecBwdArgs p, RecLayo
                 for (int m = 0; m < 2; ++m)
 #pragma unroll
                     for (int n = 0; n < NT; ++n) acc[m][n] = floatx4{0.f, 0.f, 0.f, 0.f};
-                wave_product<NT, KS, RESIDENT, KL>(acc, wreg, wlds, wfrag_wave, a0, a1, wave, lane, nks_total, ks_wave);
-                clk.lap(1);
+                wave_product<NT, KS, RESIDENT, KL>(acc, wreg, wlds, wfrag_wave, a0, a1, wave, lane, nks_total, ks_wave, poll);
+                clk.lap(0);
                 spill_partials<NT>(part, acc, wave, lane, PLD);
                 __syncthreads();
-                clk.lap(2);
+                if (lds_abort != 0) return;
+                clk.lap(1);
             }
-            float2 dcnew[NP];
-            unsigned dgnew[NP][4];
-            half_t* xout = p.X + size_t(t & 1) * p.x_slot;   // dG_t for the peers
-#pragma unroll
-            for (int q = 0; q < NP; ++q) {
-                const int b = row0 + pr[q];
-                if (!(pv[q] && b < p.B)) continue;
-                const int j = hs * JB + pj[q];
-                const size_t sidx = size_t(b) * p.Hp + j;
-                float dh[2];
-                if (from_product) {
-                    dh[0] = 0.f; dh[1] = 0.f;
-#pragma unroll
-                    for (int w = 0; w < 4; ++w) {
-                        const float2 v = *reinterpret_cast<const float2*>(part + (size_t(w) * kRows + pr[q]) * PLD + pj[q]);
-                        dh[0] += v.x;
-                        dh[1] += v.y;
-                    }
-                } else {
-                    const float2 v = *reinterpret_cast<const float2*>(p.dHn + sidx);
-                    dh[0] = v.x; dh[1] = v.y;
-                }
-                if (t < 0) {  // closing pass: gradient wrt h0; dc0 is the running dc
-                    *reinterpret_cast<float2*>(p.dH0 + sidx) = float2{dh[0], dh[1]};
-                    if (dc_in_regs) *reinterpret_cast<float2*>(p.dC + sidx) = dcreg[q];
-                    continue;
-                }
-                float dy0, dy1;
-                unpack_h2(pdy[q], dy0, dy1);
-                dh[0] += S * dy0;
-                dh[1] += S * dy1;
-                float2 dcin;
-                if (dc_in_regs) {
-                    dcin = dcreg[q];
-                } else {
-                    union { u64 q64; float2 f; } dcu;
-                    dcu.q64 = __hip_atomic_load(reinterpret_cast<const u64*>(p.dC + sidx), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                    dcin = dcu.f;
-                }
-                float gate[4][2];
-#pragma unroll
-                for (int gt = 0; gt < 4; ++gt) unpack_h2(pg[q][gt], gate[gt][0], gate[gt][1]);
-                float da[4][2], dcp[2];
-#pragma unroll
-                for (int u = 0; u < 2; ++u) {
-                    const float ig = gate[0][u], fg = gate[1][u], gg = gate[2][u], og = gate[3][u];
-                    const float tc = tanhf_dev(u == 0 ? pcc[q].x : pcc[q].y);
-                    const float cpv = (u == 0) ? pcp[q].x : pcp[q].y;
-                    const float dcn = (u == 0) ? dcin.x : dcin.y;
-                    const float dov = dh[u] * tc;
-                    const float dc = dcn + dh[u] * og * (1.f - tc * tc);
-                    da[0][u] = dc * gg * ig * (1.f - ig);
-                    da[1][u] = dc * cpv * fg * (1.f - fg);
-                    da[2][u] = dc * ig * (1.f - gg * gg);
-                    da[3][u] = dov * og * (1.f - og);
-                    dcp[u] = dc * fg;
-                }
+            const int b = row0 + pr;
+            const bool live = b < p.B;
+            const size_t sidx = size_t(b) * p.Hp + j;
+            half_t* xout = p.X + size_t((t + 3) % 3) * p.x_slot;    // dG_t for the peers
+            half_t* xnext = p.X + size_t((t + 2) % 3) * p.x_slot;   // will take dG_{t-1}
+            unsigned xoff[4];   // 32 bits: a slot is far below 4G halfs
+            PackT dgnew[4];
+            if (t >= 0) {
+                // every peer has delivered dG_{t+1}, so all of them are done reading dG_{t+2}: mark its slot
 #pragma unroll
                 for (int gt = 0; gt < 4; ++gt) {
-                    // db sums the values the weight-gradient GEMMs will see (fp16-rounded)
-                    const unsigned u32 = pack_h2(da[gt][0], da[gt][1]);
-                    float r0, r1;
-                    unpack_h2(u32, r0, r1);
-                    dbacc[gt][0] += r0;
-                    dbacc[gt][1] += r1;
-                    dgnew[q][gt] = u32;
-                    store_u32(xout + xch_offset(b, int(pq[q]) + gt * JF, nks_total), u32, device_scope);
+                    xoff[gt] = unsigned(xch_offset(b, int(pq) + gt * JF, nks_total));
+                    dgnew[gt] = pack_fill(0u, (PackT*)nullptr);   // batch rows past B travel as zeros
+                    store_xch(xnext + xoff[gt], pack_fill(kUnwritten, (PackT*)nullptr), device_scope);
                 }
-                dcnew[q] = float2{dcp[0], dcp[1]};
-                dcreg[q] = dcnew[q];
             }
-            clk.lap(3);
-            const bool last_rb = (rb + L.ng >= L.nrb);
-            if (last_rb && t >= 0) publish(gflags, hs, p.epoch + unsigned(t_first - t + 1));
-            else __syncthreads();
-            clk.lap(4);
-            if (t >= 0) {   // row-major dG for the GEMMs that follow; running dc when it lives in memory
+            if (live) {
+                float dh[UPT];
+                if (from_product) {
 #pragma unroll
-                for (int q = 0; q < NP; ++q) {
-                    const int b = row0 + pr[q];
-                    if (!(pv[q] && b < p.B)) continue;
-                    half_t* gdst = p.dG + (size_t(t) * p.B + b) * gld + pq[q];
+                    for (int u = 0; u < UPT; ++u) dh[u] = 0.f;
 #pragma unroll
-                    for (int gt = 0; gt < 4; ++gt) *reinterpret_cast<unsigned*>(gdst + gt * JF) = dgnew[q][gt];
-                    if (!dc_in_regs) *reinterpret_cast<float2*>(p.dC + size_t(b) * p.Hp + hs * JB + pj[q]) = dcnew[q];
+                    for (int w = 0; w < 4; ++w) {
+                        float v[UPT];
+                        ld_f32(part + (size_t(w) * kRows + pr) * PLD + pj, v);
+#pragma unroll
+                        for (int u = 0; u < UPT; ++u) dh[u] += v[u];
+                    }
+                } else {
+                    ld_f32(p.dHn + sidx, dh);
                 }
+                if (t < 0) {  // closing pass: gradient wrt h0; dc0 is the running dc
+                    st_f32(p.dH0 + sidx, dh);
+                    if (dc_in_regs) st_f32(p.dC + sidx, dcreg);
+                } else {
+                    float dy[UPT], dcin[UPT];
+                    unpack(pdy, dy);
+                    if (dc_in_regs) {
+#pragma unroll
+                        for (int u = 0; u < UPT; ++u) dcin[u] = dcreg[u];
+                    } else {
+                        ld_f32_coherent(p.dC + sidx, dcin);
+                    }
+                    float gate[4][UPT];
+#pragma unroll
+                    for (int gt = 0; gt < 4; ++gt) unpack(pg[gt], gate[gt]);
+                    float da[4][UPT];
+#pragma unroll
+                    for (int u = 0; u < UPT; ++u) {
+                        const float ig = gate[0][u], fg = gate[1][u], gg = gate[2][u], og = gate[3][u];
+                        const float dhu = dh[u] + S * dy[u];
+                        const float tc = tanhf_dev(pcc[u]);
+                        const float dov = dhu * tc;
+                        const float dc = dcin[u] + dhu * og * (1.f - tc * tc);
+                        da[0][u] = dc * gg * ig * (1.f - ig);
+                        da[1][u] = dc * pcp[u] * fg * (1.f - fg);
+                        da[2][u] = dc * ig * (1.f - gg * gg);
+                        da[3][u] = dov * og * (1.f - og);
+                        dcreg[u] = dc * fg;
+                    }
+#pragma unroll
+                    for (int gt = 0; gt < 4; ++gt) {
+                        // db sums the values the weight-gradient GEMMs will see (fp16-rounded)
+                        dgnew[gt] = pack(da[gt]);
+                        float r[UPT];
+                        unpack(dgnew[gt], r);
+#pragma unroll
+                        for (int u = 0; u < UPT; ++u) dbacc[gt][u] += r[u];
+                    }
+                }
+            }
+            if (t >= 0) {
+                // the exchanged values go out first, after the marks above have been acknowledged
+                asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+#pragma unroll
+                for (int gt = 0; gt < 4; ++gt) store_xch(xout + xoff[gt], dgnew[gt], device_scope);
+            }
+            clk.lap(2);
+            if (t >= 0 && live) {   // row-major dG for the GEMMs that follow; running dc when it lives in memory
+                half_t* gdst = p.dG + (size_t(t) * p.B + b) * gld + pq;
+#pragma unroll
+                for (int gt = 0; gt < 4; ++gt) st_pack(gdst + gt * JF, dgnew[gt]);
+                if (!dc_in_regs) st_f32(p.dC + sidx, dcreg);
             }
             int nt_ = t, nrb_ = rb + L.ng;
             if (nrb_ >= L.nrb) { nt_ = t - 1; nrb_ = g; }
             if (nt_ >= t_last && nt_ >= 0) prefetch(nt_, nrb_);
+            clk.lap(3);
         }
     }
+    clk.flush();
     // single-step launches leave dc in memory for the next launch
     if (dc_in_regs && t_last >= 0) {
-#pragma unroll
-        for (int q = 0; q < NP; ++q) {
-            const int b = g * kRows + pr[q];
-            if (pv[q] && b < p.B) *reinterpret_cast<float2*>(p.dC + size_t(b) * p.Hp + hs * JB + pj[q]) = dcreg[q];
-        }
+        const int b = g * kRows + pr;
+        if (b < p.B) st_f32(p.dC + size_t(b) * p.Hp + j, dcreg);
     }
 
-    // Bias gradient: fold this launch's sums over the threads that share a unit pair (fixed order).
+    // Bias gradient: fold this launch's sums over the threads that share a group column (fixed order).
     __syncthreads();
-    float* red = part;  // [256][8]
+    float* red = part_all;  // [256][4 * UPT]
 #pragma unroll
-    for (int gt = 0; gt < 4; ++gt) {
-        red[tid * 8 + gt * 2 + 0] = dbacc[gt][0];
-        red[tid * 8 + gt * 2 + 1] = dbacc[gt][1];
-    }
+    for (int gt = 0; gt < 4; ++gt)
+#pragma unroll
+        for (int u = 0; u < UPT; ++u) red[tid * (4 * UPT) + gt * UPT + u] = dbacc[gt][u];
     __syncthreads();
-    constexpr int PAIRS = JB / 2;
-    if (tid < PAIRS * 8) {
-        const int prr = tid / 8, e = tid % 8;  // pair, (gate, unit)
+    if (tid < 8 * 4 * UPT) {
+        const int gc = tid / (4 * UPT), e = tid % (4 * UPT);  // group column, (gate, unit)
         float sum = 0.f;
-        for (int k = prr; k < kThreads; k += PAIRS) sum += red[k * 8 + e];
-        const int gt = e / 2, u = e % 2;
-        const int j = hs * JB + prr * 2 + u;
-        const size_t q = size_t(j / JF) * 4 * JF + size_t(gt) * JF + (j % JF);
+        for (int k = gc; k < kThreads; k += 8) sum += red[k * (4 * UPT) + e];
+        const int gt = e / UPT, u = e % UPT;
+        const int ju = hs * JB + gc * UPT + u;
+        const size_t q = size_t(ju / JF) * 4 * JF + size_t(gt) * JF + (ju % JF);
         p.db_part[size_t(g) * gld + q] += sum;
     }
 }
@@ -766,7 +806,7 @@ RecLayout plan_rec_bwd(int B, int Hp, int num_cus, bool force_stepwise) {
 template <int NT, int KS, bool RES>
 static hipError_t run_fwd(const RecLayout& L, const RecFwdArgs& a, hipStream_t stream) {
     auto kernel = rec_fwd_kernel<NT, KS, RES>;
-    const size_t lds = size_t(4) * kRows * (16 * NT + 4) * sizeof(float);
+    const size_t lds = size_t(2) * 4 * kRows * (16 * NT + 4) * sizeof(float);
     hipError_t e = raise_lds(kernel, lds);
     if (e != hipSuccess) return e;
     const int ks_wave = rec_fwd_ks(L, a.Hp);
@@ -794,8 +834,8 @@ hipError_t launch_rec_fwd(const RecLayout& L, const RecFwdArgs& a, hipStream_t s
 template <int NT, int KS, bool RES, int KL>
 static hipError_t run_bwd(const RecLayout& L, const RecBwdArgs& a, hipStream_t stream) {
     auto kernel = rec_bwd_kernel<NT, KS, RES, KL>;
-    static_assert(size_t(4) * kRows * (16 * NT + 4) >= size_t(kThreads) * 8, "db reduction reuses the partial-sum area");
-    const size_t lds = size_t(4) * kRows * (16 * NT + 4) * sizeof(float) + size_t(4) * KL * NT * kWave * sizeof(half8);
+    static_assert(size_t(2) * 4 * kRows * (16 * NT + 4) >= size_t(kThreads) * 8 * NT, "db reduction reuses the partial-sum area");
+    const size_t lds = size_t(2) * 4 * kRows * (16 * NT + 4) * sizeof(float) + size_t(4) * KL * NT * kWave * sizeof(half8);
     hipError_t e = raise_lds(kernel, lds);
     if (e != hipSuccess) return e;
     const int ks_wave = rec_bwd_ks(L, a.Hp);
@@ -816,7 +856,7 @@ hipError_t launch_rec_bwd(const RecLayout& L, const RecBwdArgs& a, hipStream_t s
     if (a.Hp % 32 != 0 || a.Hp % L.jb != 0) return hipErrorInvalidValue;
     if (!L.resident) return run_bwd<2, 1, false, 0>(L, a, stream);
     if (L.nt == 2) return run_bwd<2, 32, true, 8>(L, a, stream);
-    if (L.nt == 1) return run_bwd<1, 64, true, 16>(L, a, stream);
+    if (L.nt == 1) return run_bwd<1, 64, true, 24>(L, a, stream);
     return hipErrorInvalidValue;
 }
 
