@@ -258,6 +258,7 @@ int forward_once(flstm_core_plan* p, size_t T, const void* x, flstm_dtype x_dtyp
         g.M = int(steps * d.B); g.N = 4 * d.Hp; g.K = d.Ip;
         g.C16 = p->G.as<half_t>() + t0 * d.B * 4 * d.Hp; g.C32 = nullptr; g.ldc = size_t(4) * d.Hp;
         g.alpha = 1.f; g.splits = 1; g.split_stride = 0;
+        g.bias = p->bias_p.as<float>();   // b_ih + b_hh, packed gate order: the recurrence reads x-projection + bias
         FL_TRY(launch_gemm_nt(g, s));
     }
     FL_TRY(hipEventRecord(p->tm.ev[1], s));
@@ -265,7 +266,6 @@ int forward_once(flstm_core_plan* p, size_t T, const void* x, flstm_dtype x_dtyp
     a.wfrag = p->wfrag_f.as<half8>();
     a.Y = p->Y.as<half_t>(); a.G = p->G.as<half_t>(); a.C = p->C.as<float>();
     a.X = p->xch_f.as<half_t>(); a.x_slot = xslot;
-    a.bias = p->bias_p.as<float>();
     a.status = p->status.as<int>();
     a.seats = p->status.as<unsigned>() + 8;
     FL_TRY(fill_zero(a.seats, 8 * sizeof(unsigned), s));

@@ -14,6 +14,8 @@ struct GemmNT {
     float alpha;                   // C = alpha * (A * B^T)
     // split-K: when splits > 1 partial z is written to C32 + z * split_stride (fp32 only)
     int splits; size_t split_stride;
+    // optional per-column term: C = alpha * (A * B^T) + bias[n]  (NT form only)
+    const float* bias;
 };
 
 // Enqueue on `stream`. Returns hipSuccess or the launch error.

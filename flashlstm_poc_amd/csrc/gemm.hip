@@ -1,34 +1,27 @@
-// LDS-staged fp16 MFMA GEMM for gfx950 (CDNA4), NT form: C[M][N] = A[M][K] * B[N][K]^T.
+// fp16 MFMA GEMMs for gfx950 (CDNA4), fp32 accumulation.
 //
-// This is the dense contraction behind the hoisted input projection X*W_ih^T (the reference does it
-// with a CUTLASS 128x128x32 tensor-op GEMM, src/lstm.cu:1204-1239, src/lstm_internal.h:48-68), the
-// input gradient dX = dG*W_ih and the weight gradients dW = dG^T*[X;H] (reference:
+// These are the dense contractions around the recurrence: the hoisted input projection X*W_ih^T (the
+// reference does it with a CUTLASS 128x128x32 tensor-op GEMM, src/lstm.cu:1204-1239,
+// src/lstm_internal.h:48-68), the input gradient dX = dG*W_ih (both "NT": operands K-contiguous) and the
+// weight gradients dW = dG^T*[X;H] ("TN": operands k-major; reference:
 // flashlstm_v2/src/lstm_backward.cu:1112-1172 through flashlstm_v2/src/gemm.cu:222-330).
 //
-// Tiling: one 256-thread workgroup (4 wavefronts, 2x2, one per SIMD) owns a 256x256 tile of C; every
-// wavefront owns 128x128 as a 4x4 grid of v_mfma_f32_32x32x16_f16 tiles (256 accumulator registers).
-// K is walked in slabs of 64: global -> registers -> LDS (row pitch padded to 72 halfs so that the
-// 16-byte fragment reads of 8 consecutive lanes fall in distinct banks), double buffered, one
-// workgroup barrier per slab.  The MFMA operands are swapped (D = B_tile * A_tile^T) so that a lane ends
-// up with four consecutive columns of one row of C and stores them as one 8- or 16-byte access.
-// Workgroups are numbered so that the 32 that share an XCD (block id mod 8) work on neighbouring tiles
-// and reuse each other's operand slabs in that XCD's L2.
+// Common tiling: one 512-thread workgroup (8 wavefronts, 2 along M x 4 along N, two per SIMD) owns a
+// 256x256 tile of C; every wavefront owns 128x64 as a 4x2 grid of v_mfma_f32_32x32x16_f16 tiles (128
+// accumulator registers).  K is walked in slabs of 64 through double-buffered LDS.  The MFMA operands are
+// swapped (D = B_tile * A_tile^T) so that a lane ends up with four consecutive columns of one row of C;
+// full tiles are then turned through a little LDS so that every store instruction writes whole 128-byte
+// lines.  The work order gives the 32 workgroups that share an XCD one compact block of tiles.
 #include "gemm.h"
-#include <cstdlib>
 
-#ifdef GEMM_PROF
-__device__ long long g_gemm_prof[8];
-#endif
 namespace flstm_hip {
 namespace {
 
 constexpr int BM = 256, BN = 256, BK = 64;
-constexpr int LDS_LD = 72;  // halfs per LDS row (64 + 8 pad)
 constexpr int kWavesN = 4;                 // wavefronts along N (2 along M): wave tile 128 x (256 / kWavesN)
 constexpr int kThreads = 128 * kWavesN;
 constexpr int kTN = 8 / kWavesN;            // 32-wide MFMA tiles per wave along N
 constexpr int kLd = 2048 / kThreads;        // 16-byte chunks per thread, operand and slab
-constexpr size_t kLdsBytes = size_t(2) * (BM + BN) * LDS_LD * sizeof(half_t);
 
 // Work order.  The hardware deals workgroups round-robin over the 8 XCDs in dispatch order, so the 32
 // workgroups with the same (dispatch index mod 8) that run together share one XCD and its 4 MiB L2.  They
@@ -59,6 +52,11 @@ __device__ __forceinline__ bool work_item(const TileOrder& o, int lin, int& tm, 
 // Epilogue shared by both kernels.  With swapped MFMA operands register r of tile (i, j) holds row
 // (i*32 + lane%32) of the wave's 128 x 64 block and column j*32 + 8*(r/4) + 4*(lane/32) + r%4: four
 // consecutive columns per group of four registers, stored as one 8-byte (fp16) or 16-byte (fp32) access.
+// bias[col .. col+3] of a full tile (col % 4 == 0), zeros when the GEMM has no bias
+__device__ __forceinline__ floatx4 bias4(const GemmNT& g, int col) {
+    return g.bias ? *reinterpret_cast<const floatx4*>(g.bias + col) : floatx4{0.f, 0.f, 0.f, 0.f};
+}
+
 __device__ __forceinline__ void store_tile(const GemmNT& g, floatx16 (&acc)[4][kTN], int m0, int n0, int wm,
                                            int wn, int lane, int z) {
     const int row = m0 + wm * 128 + lane % 32;
@@ -77,12 +75,13 @@ __device__ __forceinline__ void store_tile(const GemmNT& g, floatx16 (&acc)[4][k
                     if (c32) {
                         floatx4 v;
 #pragma unroll
-                        for (int e = 0; e < 4; ++e) v[e] = g.alpha * acc[i][j][4 * q + e];
+                        for (int e = 0; e < 4; ++e) v[e] = g.alpha * acc[i][j][4 * q + e] + bias4(g, colb + j * 32 + 8 * q)[e];
                         *reinterpret_cast<floatx4*>(c32 + off) = v;
                     } else {
                         half4 v;
 #pragma unroll
-                        for (int e = 0; e < 4; ++e) v[e] = (half_t)(g.alpha * acc[i][j][4 * q + e]);
+                        for (int e = 0; e < 4; ++e)
+                            v[e] = (half_t)(g.alpha * acc[i][j][4 * q + e] + bias4(g, colb + j * 32 + 8 * q)[e]);
                         *reinterpret_cast<half4*>(g.C16 + off) = v;
                     }
                 }
@@ -101,7 +100,7 @@ __device__ __forceinline__ void store_tile(const GemmNT& g, floatx16 (&acc)[4][k
                     const int col = colb + j * 32 + 8 * (r / 4) + (r % 4);
                     if (col >= g.N) continue;
                     const size_t off = size_t(r_) * g.ldc + col;
-                    const float v = g.alpha * acc[i][j][r];
+                    const float v = g.alpha * acc[i][j][r] + (g.bias ? g.bias[col] : 0.f);
                     if (c32) c32[off] = v;
                     else g.C16[off] = (half_t)v;
                 }
@@ -112,106 +111,12 @@ __device__ __forceinline__ void store_tile(const GemmNT& g, floatx16 (&acc)[4][k
 }
 
 
-__global__ __launch_bounds__(kThreads) void gemm_nt_256x256(GemmNT g, TileOrder order, int k_per_split) {
-    extern __shared__ __attribute__((aligned(16))) half_t smem[];
-    half_t* As = smem;                      // [2][BM][LDS_LD]
-    half_t* Bs = smem + 2 * BM * LDS_LD;    // [2][BN][LDS_LD]
-
-    int tm, tn, z;
-    if (!work_item(order, blockIdx.x, tm, tn, z)) return;
-    const int m0 = tm * BM, n0 = tn * BN;
-    const int k_begin = z * k_per_split;
-    const int k_end = min(g.K, k_begin + k_per_split);
-    const int nslab = (k_end - k_begin) / BK;
-
-    const int tid = threadIdx.x, wave = tid / 64, lane = tid % 64;
-    const int wm = wave / kWavesN, wn = wave % kWavesN;
-
-    // Global->LDS staging: 16-byte chunk c = tid + 256*i covers row c/8, halfs [8*(c%8), +8).
-    const int ld_row = tid / 8, ld_kc = (tid % 8) * 8;
-    const half_t* a_src[kLd];
-    const half_t* b_src[kLd];
-    constexpr int kRowStep = kThreads / 8;
-#pragma unroll
-    for (int i = 0; i < kLd; ++i) {
-        const int ra = min(m0 + ld_row + kRowStep * i, g.M - 1);
-        const int rb = min(n0 + ld_row + kRowStep * i, g.N - 1);
-        a_src[i] = g.A + size_t(ra) * g.lda + k_begin + ld_kc;
-        b_src[i] = g.B + size_t(rb) * g.ldb + k_begin + ld_kc;
-    }
-    const int st_off = ld_row * LDS_LD + ld_kc;
-
-    floatx16 acc[4][kTN];
-#pragma unroll
-    for (int i = 0; i < 4; ++i)
-#pragma unroll
-        for (int j = 0; j < kTN; ++j)
-#pragma unroll
-            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
-
-    half8 ra[kLd], rb[kLd];
-    if (nslab > 0) {
-#pragma unroll
-        for (int i = 0; i < kLd; ++i) { ra[i] = ld_half8(a_src[i]); rb[i] = ld_half8(b_src[i]); }
-#pragma unroll
-        for (int i = 0; i < kLd; ++i) {
-            st_half8(As + st_off + kRowStep * i * LDS_LD, ra[i]);
-            st_half8(Bs + st_off + kRowStep * i * LDS_LD, rb[i]);
-        }
-    }
-    __syncthreads();
-
-    const int a_frag_off = (wm * 128 + lane % 32) * LDS_LD + 8 * (lane / 32);
-    const int b_frag_off = (wn * 32 * kTN + lane % 32) * LDS_LD + 8 * (lane / 32);
-
-    for (int s = 0; s < nslab; ++s) {
-        const int cur = s & 1;
-        const bool more = (s + 1 < nslab);
-        if (more) {
-            const int koff = (s + 1) * BK;
-#pragma unroll
-            for (int i = 0; i < kLd; ++i) {
-                ra[i] = ld_half8(a_src[i] + koff);
-                rb[i] = ld_half8(b_src[i] + koff);
-            }
-        }
-        const half_t* Ac = As + cur * BM * LDS_LD + a_frag_off;
-        const half_t* Bc = Bs + cur * BN * LDS_LD + b_frag_off;
-#pragma unroll
-        for (int kk = 0; kk < BK / 16; ++kk) {
-            half8 af[4], bf[kTN];
-#pragma unroll
-            for (int i = 0; i < 4; ++i) af[i] = *reinterpret_cast<const half8*>(Ac + i * 32 * LDS_LD + kk * 16);
-#pragma unroll
-            for (int j = 0; j < kTN; ++j) bf[j] = *reinterpret_cast<const half8*>(Bc + j * 32 * LDS_LD + kk * 16);
-#pragma unroll
-            for (int i = 0; i < 4; ++i)
-#pragma unroll
-                for (int j = 0; j < kTN; ++j)
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(bf[j], af[i], acc[i][j], 0, 0, 0);
-        }
-        if (more) {
-            half_t* An = As + (cur ^ 1) * BM * LDS_LD + st_off;
-            half_t* Bn = Bs + (cur ^ 1) * BN * LDS_LD + st_off;
-#pragma unroll
-            for (int i = 0; i < kLd; ++i) {
-                st_half8(An + kRowStep * i * LDS_LD, ra[i]);
-                st_half8(Bn + kRowStep * i * LDS_LD, rb[i]);
-            }
-        }
-        __syncthreads();
-    }
-
-    store_tile(g, acc, m0, n0, wm, wn, lane, z);
-}
-
-// ------------------------------------------------------------------------------ streaming NT kernel
-// Same contraction and wave layout, different data path.  Operand slabs go from global memory straight
-// into LDS (global_load_lds_dwordx4: no staging registers, no LDS store instructions), double buffered
-// in slabs of 64 k.  Wavefronts 4..7 are the copiers: each issues the 16 one-KiB copies of its quarter of
-// the next slab between its first MFMAs of the current one.  A copy instruction holds its wave until the
-// texture-address unit takes it (about 16 clocks each, 64 per slab and workgroup); the copier's partner
-// on the same SIMD (wavefront - 4) issues no copies, so it keeps the matrix pipeline fed meanwhile.
+// ------------------------------------------------------------------------------------- NT kernel
+// C[M][N] = alpha * A[M][K] * B[N][K]^T (+ bias[n]).  Operand slabs go from global memory straight into
+// LDS (global_load_lds_dwordx4: no staging registers, no LDS store instructions), double buffered in
+// slabs of 64 k.  Every wave copies 8 KiB of the next slab, one 1 KiB copy after every second MFMA of the
+// first half of the current slab: a copy instruction holds its wave until the texture-address unit takes
+// it (16+ clocks each, 64 per slab and workgroup), so they are spread out rather than issued in a burst.
 // The kernel is persistent: each workgroup walks its list of work items and the copies keep running
 // across item boundaries, so the first slab of the next tile arrives during the last MFMAs and the
 // output stores of this one.
@@ -219,9 +124,6 @@ __global__ __launch_bounds__(kThreads) void gemm_nt_256x256(GemmNT g, TileOrder 
 // LDS rows are 128 bytes (8 chunks of 16).  The LDS has 64 banks of 4 bytes and serves a 16-byte read
 // for 16 lanes per clock, so the 16 rows read together must land in 16 different 16-byte bank groups of
 // the 256-byte bank row; two rows share a bank row, hence chunk c of row r sits at position c ^ (r/2)%8.
-#ifndef GEMM_COPY_MODE
-#define GEMM_COPY_MODE 2
-#endif
 constexpr int kSlabBytes = (BM + BN) * BK * 2;               // 64 KiB: A rows then B rows
 constexpr int kEpiBytesPerWave = 32 * 64 * 2;                 // one 32 x 64 fp16 block of the wave's output
 constexpr size_t kLdsBytesStream = size_t(2) * kSlabBytes + 8 * kEpiBytesPerWave;   // 160 KiB
@@ -251,6 +153,11 @@ __device__ __forceinline__ void store_tile_lines(const GemmNT& g, floatx16 (&acc
     const int wsw = (wr >> 1) & 7;
     const int rr = lane / 8, rc = lane % 8;                // row (+ 8p) and 16-byte chunk read by this lane
     half_t* cbase = g.C16 + size_t(m0 + wm * 128) * g.ldc + n0 + wn * 64 + rc * 8;
+    floatx4 bv[kTN][4];   // bias of this lane's 32 columns
+#pragma unroll
+    for (int j = 0; j < kTN; ++j)
+#pragma unroll
+        for (int q = 0; q < 4; ++q) bv[j][q] = bias4(g, n0 + wn * 64 + j * 32 + 8 * q + 4 * (lane / 32));
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
 #pragma unroll
@@ -259,7 +166,7 @@ __device__ __forceinline__ void store_tile_lines(const GemmNT& g, floatx16 (&acc
             for (int q = 0; q < 4; ++q) {
                 half4 v;
 #pragma unroll
-                for (int e = 0; e < 4; ++e) v[e] = (half_t)(g.alpha * acc[i][j][4 * q + e]);
+                for (int e = 0; e < 4; ++e) v[e] = (half_t)(g.alpha * acc[i][j][4 * q + e] + bv[j][q][e]);
                 const int chunk = 4 * j + q;
                 *reinterpret_cast<half4*>(stage + wr * 128 + ((chunk ^ wsw) * 16) + 8 * (lane / 32)) = v;
             }
@@ -279,11 +186,6 @@ __global__ __launch_bounds__(kThreads) void gemm_nt_stream(GemmNT g, TileOrder o
     const int tid = threadIdx.x, lane = tid % 64;
     const int wave = __builtin_amdgcn_readfirstlane(tid / 64);
     const int wm = wave / kWavesN, wn = wave % kWavesN;
-    // Wave w issues copy c after its MFMA number 4c + phase.  The two waves of a SIMD (w and w + 4) are two
-    // MFMAs apart and at most two waves of the workgroup issue in the same slot, so a copy instruction,
-    // which holds its wave until the texture-address unit accepts it, rarely finds the unit busy and never
-    // stalls both waves of a SIMD at once.
-    const int phase = (wave + 2 * (wave / 4)) % 4;
     const int rounds = order.per_xcd;
 
     // ordinal n of this workgroup -> (tile, split) in the order of work_item().  Ordinals that fall on a
@@ -314,9 +216,6 @@ __global__ __launch_bounds__(kThreads) void gemm_nt_stream(GemmNT g, TileOrder o
         if (!ld_valid) return;
         const int i = c / 2;
         const int rt = cp_row + 8 * i;
-#ifdef GEMM_SAMETILE
-        ld_m0 = 0; ld_n0 = 0;
-#endif
         const int chunk = (lane % 8) ^ ((rt >> 1) & 7);
         const int koff = ld_kb + ld_k * BK + chunk * 8;
         char* dst = lds + slot * kSlabBytes + wave * 4096 + i * 1024;
@@ -365,9 +264,6 @@ __global__ __launch_bounds__(kThreads) void gemm_nt_stream(GemmNT g, TileOrder o
                 for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
 
         for (int ks = 0; ks < nk; ++ks) {
-#ifdef GEMM_PROF
-            long long t0 = clock64();
-#endif
             // Memory operations complete in issue order: a copier waits until nothing but the output stores
             // issued after its copies (if any) is outstanding.
             if (copied) {
@@ -376,15 +272,9 @@ __global__ __launch_bounds__(kThreads) void gemm_nt_stream(GemmNT g, TileOrder o
                 else wait_vm<0>();
             }
             stores_young = 0;
-#ifdef GEMM_PROF
-            long long t1 = clock64();
-#endif
             // a bare barrier: every copier has waited for its own copies above, and a fence here would
             // make the compiler drain memory operations that are meant to stay in flight
             __builtin_amdgcn_s_barrier();   // slab complete in LDS; the other buffer is no longer read
-#ifdef GEMM_PROF
-            long long t2 = clock64();
-#endif
             const int fill = slot ^ 1;
             const char* st = lds + slot * kSlabBytes;
             slot ^= 1;
@@ -402,11 +292,6 @@ __global__ __launch_bounds__(kThreads) void gemm_nt_stream(GemmNT g, TileOrder o
                 for (int j = 0; j < kTN; ++j)
                     bf[set][j] = *reinterpret_cast<const half8*>(st + b_frag + j * 32 * BK * 2 + pos[kk]);
             };
-#if GEMM_COPY_MODE == 0   // all copies first
-#pragma unroll
-            for (int c = 0; c < kCopiesPerWave; ++c) issue_copy(fill, c);
-            __builtin_amdgcn_sched_barrier(0);
-#endif
             read_frags(0, 0);
             __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
@@ -419,41 +304,17 @@ __global__ __launch_bounds__(kThreads) void gemm_nt_stream(GemmNT g, TileOrder o
                     const int i = m / kTN, j = m % kTN;
                     acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(bf[cur][j], af[cur][i], acc[i][j], 0, 0, 0);
                     const int done = kk * kPerStep + m;
-                    (void)done;
-#if GEMM_COPY_MODE == 1   // staggered over the whole slab
-                    __builtin_amdgcn_sched_barrier(0);
-                    if (done % 4 == phase) issue_copy(fill, done / 4);
-                    __builtin_amdgcn_sched_barrier(0);
-#elif GEMM_COPY_MODE == 2   // one copy after every second MFMA of the first half
-                    if (done < 16 && done % 2 == 1) {
+                    if (done < 2 * kCopiesPerWave && done % 2 == 1) {
                         __builtin_amdgcn_sched_barrier(0);
                         issue_copy(fill, done / 2);
                         __builtin_amdgcn_sched_barrier(0);
                     }
-#elif GEMM_COPY_MODE == 3   // one copy after each of the first 8 MFMAs
-                    if (done < 8) {
-                        __builtin_amdgcn_sched_barrier(0);
-                        issue_copy(fill, done);
-                        __builtin_amdgcn_sched_barrier(0);
-                    }
-#endif
                 }
             }
             copied = ld_valid;
             loader_advance();
-#ifdef GEMM_PROF
-            if (blockIdx.x == 0 && tid == GEMM_PROF) {
-                long long t4 = clock64();
-                g_gemm_prof[0] += t1 - t0; g_gemm_prof[1] += t2 - t1; g_gemm_prof[3] += t4 - t2; g_gemm_prof[4] += 1;
-            }
-#endif
         }
         const bool full = (m0 + BM <= g.M) && (n0 + BN <= g.N) && (g.ldc % 4 == 0);
-#ifdef GEMM_NOSTORE
-        { float t = 0; for (int i = 0; i < 4; ++i) for (int j = 0; j < kTN; ++j) for (int r = 0; r < 16; ++r) t += acc[i][j][r];
-          if (t == 1234.5f) g.C16[0] = (half_t)t; }
-        stores_young = 0;
-#else
         if (full && g.C16 && g.ldc % 8 == 0 && reinterpret_cast<uintptr_t>(g.C16) % 16 == 0) {
             store_tile_lines(g, acc, m0, n0, wm, wn, lane, lds + 2 * kSlabBytes + wave * kEpiBytesPerWave);
             stores_young = 16;
@@ -461,7 +322,6 @@ __global__ __launch_bounds__(kThreads) void gemm_nt_stream(GemmNT g, TileOrder o
             store_tile(g, acc, m0, n0, wm, wn, lane, z);
             stores_young = full ? 32 : -1;
         }
-#endif
     }
     wait_vm<0>();   // no copy may still be heading for LDS when the workgroup retires
 }
@@ -654,6 +514,7 @@ hipError_t launch_gemm_nt(const GemmNT& g, hipStream_t stream) {
     // the vector stores of full tiles need an aligned base (rows are covered by the ldc % 4 test in the kernel)
     if (g.C32 && (reinterpret_cast<uintptr_t>(g.C32) % 16 != 0 || g.split_stride % 4 != 0)) return hipErrorInvalidValue;
     if (g.C16 && (reinterpret_cast<uintptr_t>(g.C16) % 8 != 0)) return hipErrorInvalidValue;
+    if (g.bias && (reinterpret_cast<uintptr_t>(g.bias) % 16 != 0 || g.splits > 1)) return hipErrorInvalidValue;
     int splits = g.splits < 1 ? 1 : g.splits;
     if (splits > 1 && g.C32 == nullptr) return hipErrorInvalidValue;
     const int nslab = g.K / BK;
@@ -665,36 +526,23 @@ hipError_t launch_gemm_nt(const GemmNT& g, hipStream_t stream) {
         // ones must read as zero.  Callers use gemm_effective_splits() to avoid this path.
         return hipErrorInvalidValue;
     }
+    const int tiles_m = (g.M + BM - 1) / BM, tiles_n = (g.N + BN - 1) / BN;
+    const TileOrder order = make_order(tiles_m, tiles_n, splits);
     static bool attr_set = false;
     if (!attr_set) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_nt_256x256),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, int(kLdsBytes));
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_nt_stream),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, int(kLdsBytesStream));
         if (e != hipSuccess) return e;
         attr_set = true;
     }
-    const int tiles_m = (g.M + BM - 1) / BM, tiles_n = (g.N + BN - 1) / BN;
-    const TileOrder order = make_order(tiles_m, tiles_n, splits);
-    static const bool staged = getenv("FLASHLSTM_GEMM_STAGED") != nullptr;
-    if (!staged) {
-        static bool attr2 = false;
-        if (!attr2) {
-            hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_nt_stream),
-                                               hipFuncAttributeMaxDynamicSharedMemorySize, int(kLdsBytesStream));
-            if (e != hipSuccess) return e;
-            attr2 = true;
-        }
-        hipLaunchKernelGGL(gemm_nt_stream, dim3(256), dim3(kThreads), kLdsBytesStream, stream, g, order,
-                           slabs_per_split * BK);
-        return hipGetLastError();
-    }
-    hipLaunchKernelGGL(gemm_nt_256x256, dim3(order.per_xcd * 256), dim3(kThreads), kLdsBytes, stream, g, order,
+    hipLaunchKernelGGL(gemm_nt_stream, dim3(256), dim3(kThreads), kLdsBytesStream, stream, g, order,
                        slabs_per_split * BK);
     return hipGetLastError();
 }
 
 hipError_t launch_gemm_tn(const GemmNT& g, hipStream_t stream) {
     if (g.M <= 0 || g.N <= 0 || g.K <= 0) return hipSuccess;
-    if (g.M % 8 != 0 || g.N % 8 != 0 || g.lda % 8 != 0 || g.ldb % 8 != 0) return hipErrorInvalidValue;
+    if (g.M % 8 != 0 || g.N % 8 != 0 || g.lda % 8 != 0 || g.ldb % 8 != 0 || g.bias) return hipErrorInvalidValue;
     if ((g.C16 == nullptr) == (g.C32 == nullptr)) return hipErrorInvalidValue;
     if (g.C32 && (reinterpret_cast<uintptr_t>(g.C32) % 16 != 0 || g.split_stride % 4 != 0)) return hipErrorInvalidValue;
     if (g.C16 && (reinterpret_cast<uintptr_t>(g.C16) % 8 != 0)) return hipErrorInvalidValue;

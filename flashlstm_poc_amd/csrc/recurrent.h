@@ -26,9 +26,8 @@ struct RecFwdArgs {
                          // writes slot (t+1)%3; before a launch slot 0 holds h0 (padding rows zero) and the
                          // other two hold the 0xFFFF 'unwritten' pattern
     size_t x_slot;
-    half_t* G;           // [T*B][4Hp] packed gate order; in: x-projection, out: activated i,f,g,o
+    half_t* G;           // [T*B][4Hp] packed gate order; in: x-projection + bias, out: activated i,f,g,o
     float* C;            // [(T+1)*B][Hp]; rows [0,B) = c0, rows [(t+1)B, ..) = c_t
-    const float* bias;   // [4Hp] packed gate order, b_ih + b_hh
     unsigned* seats;     // [8] zeroed before every launch: next free workgroup slot per XCD
     int* status;         // 0 ok, 1 spin limit hit, 2 workgroup not on the expected XCD
     int B, Hp, T;

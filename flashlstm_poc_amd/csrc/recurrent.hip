@@ -127,7 +127,7 @@ __device__ __forceinline__ void wait_frags(half8 (&a)[4], half8 (&b)[4]) {
                  : "memory");
 }
 
-// acc[mt][nt] += A(32 rows x K) * Wslice, this wave's interleaved k-steps only.
+// acc[mt][nt] += (A(32 rows x K) * Wslice)^T, this wave's interleaved k-steps only.
 // a0/a1: fragment (row tile, k-step 0) of the two 16-row tiles, already offset by lane*8 halfs.
 // The last KL of a wave's KS k-steps keep their weight fragments in LDS instead of registers (wlds:
 // this wave's [KL][NT][64 lanes] block); reading them back costs a few ds_read_b128 per step and frees
@@ -200,8 +200,8 @@ __device__ __forceinline__ void wave_product(floatx4 (&acc)[2][NT], const half8 
                     half8 w;
                     if (ks < KR) w = wreg[ks < KR ? ks : 0][n];
                     else w = wlds[((ks - KR) * NT + n) * kWave + lane];
-                    acc[0][n] = __builtin_amdgcn_mfma_f32_16x16x32_f16(fa[buf][k], w, acc[0][n], 0, 0, 0);
-                    acc[1][n] = __builtin_amdgcn_mfma_f32_16x16x32_f16(fb[buf][k], w, acc[1][n], 0, 0, 0);
+                    acc[0][n] = __builtin_amdgcn_mfma_f32_16x16x32_f16(w, fa[buf][k], acc[0][n], 0, 0, 0);
+                    acc[1][n] = __builtin_amdgcn_mfma_f32_16x16x32_f16(w, fb[buf][k], acc[1][n], 0, 0, 0);
                 }
             }
         }
@@ -214,24 +214,26 @@ __device__ __forceinline__ void wave_product(floatx4 (&acc)[2][NT], const half8 
 #pragma unroll
             for (int n = 0; n < NT; ++n) {
                 const half8 w = wfrag_wave[(size_t(k) * NT + n) * kWave + lane];
-                acc[0][n] = __builtin_amdgcn_mfma_f32_16x16x32_f16(fa, w, acc[0][n], 0, 0, 0);
-                acc[1][n] = __builtin_amdgcn_mfma_f32_16x16x32_f16(fb, w, acc[1][n], 0, 0, 0);
+                acc[0][n] = __builtin_amdgcn_mfma_f32_16x16x32_f16(w, fa, acc[0][n], 0, 0, 0);
+                acc[1][n] = __builtin_amdgcn_mfma_f32_16x16x32_f16(w, fb, acc[1][n], 0, 0, 0);
             }
         }
     }
 }
 
+// The products are computed transposed (weights as the first MFMA operand), so a lane ends up with four
+// consecutive output columns of one batch row: tile (m, n) holds row m*16 + lane%16, columns
+// n*16 + 4*(lane/16) .. +3, and goes to LDS as one 16-byte store.  The 16 rows written together are
+// 4*pld banks apart; for the pitches in use that spreads them over all 64 banks.
 template <int NT>
 __device__ __forceinline__ void spill_partials(float* part, const floatx4 (&acc)[2][NT], int wave,
                                                int lane, int pld) {
-    float* base = part + size_t(wave) * kRows * pld;
+    float* base = part + size_t(wave) * kRows * pld + size_t(lane % 16) * pld + 4 * (lane / 16);
 #pragma unroll
     for (int m = 0; m < 2; ++m)
 #pragma unroll
         for (int n = 0; n < NT; ++n)
-#pragma unroll
-            for (int i = 0; i < 4; ++i)
-                base[(m * 16 + 4 * (lane / 16) + i) * pld + n * 16 + lane % 16] = acc[m][n][i];
+            *reinterpret_cast<floatx4*>(base + m * 16 * pld + n * 16) = acc[m][n];
 }
 
 __device__ __forceinline__ void unpack_h2(unsigned u, float& a, float& b) {
@@ -395,9 +397,6 @@ __global__ __launch_bounds__(kThreads) void rec_fwd_kernel(RecFwdArgs p, RecLayo
     const int pr = group_row(tid / 8);
     const int pj = (tid % 8) * UPT;
     const int j = hs * JB + pj;   // first hidden unit of the group
-    float bs[4][UPT];
-#pragma unroll
-    for (int gt = 0; gt < 4; ++gt) ld_f32(p.bias + size_t(hs) * NC + gt * JB + pj, bs[gt]);
     const int rb_count = (L.nrb - g + L.ng - 1) / L.ng;
     const bool c_in_regs = (rb_count == 1) && (t_end - t_begin > 1);
     float creg[UPT] = {};
@@ -443,7 +442,7 @@ __global__ __launch_bounds__(kThreads) void rec_fwd_kernel(RecFwdArgs p, RecLayo
             // its slot can be marked for reuse.  The mark is acknowledged long before the wait that
             // precedes the h_t store below, so whoever sees this step's h_t also sees the mark.
             const int b = row0 + pr;
-            const size_t xoff = xch_offset(b, j, nks_total);
+            const unsigned xoff = unsigned(xch_offset(b, j, nks_total));   // 32 bits: a slot is far below 4G halfs
             store_xch(xnext + xoff, pack_fill(kUnwritten, (PackT*)nullptr), device_scope);
             PackT act[4], hnew = pack_fill(0u, (PackT*)nullptr);   // batch rows past B travel as zeros
             const bool live = b < p.B;
@@ -454,7 +453,7 @@ __global__ __launch_bounds__(kThreads) void rec_fwd_kernel(RecFwdArgs p, RecLayo
                     float x[UPT];
                     unpack(xp[gt], x);
 #pragma unroll
-                    for (int u = 0; u < UPT; ++u) z[gt][u] = bs[gt][u] + x[u];
+                    for (int u = 0; u < UPT; ++u) z[gt][u] = x[u];
 #pragma unroll
                     for (int w = 0; w < 4; ++w) {
                         float v[UPT];

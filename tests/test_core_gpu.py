@@ -103,6 +103,22 @@ def test_persistent_and_stepwise_agree(shape):
         assert rell2(a[k], b[k]) < 1e-5, k
 
 
+def test_retry_limit_hit_is_repaired_by_stepwise_pass():
+    # Failure handling of the persistent kernels, forced from the host: with a retry limit of 1 a workgroup
+    # that finds an operand not yet written gives up at once, every kernel still exits normally, and the
+    # library repeats the pass one launch per step.  The results must be the same either way.
+    from flashlstm_poc_amd import LstmCore
+    p = make_problem(24, 40, 64, 256, seed=5)
+    ref, _ = oracle_reference(p)
+    core = LstmCore(40, 64, 256)
+    core.pack(*(p[k].cuda() for k in ("w_ih", "w_hh", "b_ih", "b_hh")))
+    core.set_option("spin_limit", 1)
+    for _ in range(2):
+        got, info = run_core(p, core=core)
+        check_against(ref, got, label=f"spin_limit=1 fallbacks={info['fallbacks']}")
+    core.close()
+
+
 def test_projection_chunk_size_does_not_change_results():
     p = make_problem(17, 6, 48, 40, seed=9)
     base, _ = run_core(p, proj_chunk=0)
