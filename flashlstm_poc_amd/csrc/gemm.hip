@@ -251,7 +251,6 @@ __global__ __launch_bounds__(kThreads) void gemm_nt_stream(GemmNT g, TileOrder o
     loader_advance();
 
     int slot = 0;            // LDS buffer of the slab consumed next
-    int stores_young = 0;    // 16 / 32: that many output stores of a full tile were issued after the copies in flight
     for (int n = 0; n < rounds; ++n) {
         int m0, n0, z, kb, nk;
         if (!decode(n, m0, n0, z, kb, nk)) continue;
@@ -264,14 +263,11 @@ __global__ __launch_bounds__(kThreads) void gemm_nt_stream(GemmNT g, TileOrder o
                 for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
 
         for (int ks = 0; ks < nk; ++ks) {
-            // Memory operations complete in issue order: a copier waits until nothing but the output stores
-            // issued after its copies (if any) is outstanding.
-            if (copied) {
-                if (stores_young == 32) wait_vm<32>();
-                else if (stores_young == 16) wait_vm<16>();
-                else wait_vm<0>();
-            }
-            stores_young = 0;
+            // Loads complete in issue order among themselves, but stores may be acknowledged out of order
+            // with them, so a count that discounts the output stores issued after the copies would not be
+            // safe: wait for everything.  (Store acknowledgements come from the L2 and take no longer than
+            // the copies that are in flight with them.)
+            if (copied) wait_vm<0>();
             // a bare barrier: every copier has waited for its own copies above, and a fence here would
             // make the compiler drain memory operations that are meant to stay in flight
             __builtin_amdgcn_s_barrier();   // slab complete in LDS; the other buffer is no longer read
@@ -317,10 +313,8 @@ __global__ __launch_bounds__(kThreads) void gemm_nt_stream(GemmNT g, TileOrder o
         const bool full = (m0 + BM <= g.M) && (n0 + BN <= g.N) && (g.ldc % 4 == 0);
         if (full && g.C16 && g.ldc % 8 == 0 && reinterpret_cast<uintptr_t>(g.C16) % 16 == 0) {
             store_tile_lines(g, acc, m0, n0, wm, wn, lane, lds + 2 * kSlabBytes + wave * kEpiBytesPerWave);
-            stores_young = 16;
         } else {
             store_tile(g, acc, m0, n0, wm, wn, lane, z);
-            stores_young = full ? 32 : -1;
         }
     }
     wait_vm<0>();   // no copy may still be heading for LDS when the workgroup retires

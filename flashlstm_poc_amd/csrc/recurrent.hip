@@ -126,41 +126,53 @@ __device__ __forceinline__ void wait_frags(half8 (&a)[4], half8 (&b)[4]) {
                  : "n"(N)
                  : "memory");
 }
+template <int N>
+__device__ __forceinline__ void wait_frags(half8 (&a)[2], half8 (&b)[2]) {
+    asm volatile("s_waitcnt vmcnt(%4)" : "+v"(a[0]), "+v"(a[1]), "+v"(b[0]), "+v"(b[1]) : "n"(N) : "memory");
+}
 
 // acc[mt][nt] += (A(32 rows x K) * Wslice)^T, this wave's interleaved k-steps only.
 // a0/a1: fragment (row tile, k-step 0) of the two 16-row tiles, already offset by lane*8 halfs.
 // The last KL of a wave's KS k-steps keep their weight fragments in LDS instead of registers (wlds:
 // this wave's [KL][NT][64 lanes] block); reading them back costs a few ds_read_b128 per step and frees
 // 4*KL*NT registers for fragments in flight.
-template <int NT, int KS, bool RESIDENT, int KL = 0>
+// `prefetch` issues exactly NPF vector loads (for every wave, whatever its lanes need) behind the last
+// fragment load.
+template <int NT, int KS, bool RESIDENT, int KL, int NPF, typename Prefetch>
 __device__ __forceinline__ void wave_product(floatx4 (&acc)[2][NT], const half8 (&wreg)[KS - KL][NT],
                                              const half8* wlds, const half8* wfrag_wave, const half_t* a0,
                                              const half_t* a1, int wave, int lane, int nks_total,
-                                             int ks_wave, const Poll& poll) {
+                                             int ks_wave, const Poll& poll, Prefetch&& prefetch) {
     if constexpr (RESIDENT && (KS % 8 == 0)) {
         // Loads and MFMAs are unconditional: k-steps beyond the real contraction length fetch a
-        // clamped (finite) address and meet all-zero weight fragments.  Chunks of 4 k-steps (8
+        // clamped (finite) address and meet all-zero weight fragments.  Chunks of CK k-steps (2*CK
         // fragments) alternate between two register sets: one is in flight while the other feeds the
-        // MFMAs.
-        constexpr int NCH = KS / 4;
-        half8 fa[2][4], fb[2][4];
+        // MFMAs.  (Short contractions take small chunks: their kernels have no registers to spare.)
+        constexpr int CK = (KS >= 16) ? 4 : 2;
+        constexpr int NCH = KS / CK;
+        half8 fa[2][CK], fb[2][CK];
         auto issue = [&](int c, int buf) {
 #pragma unroll
-            for (int k = 0; k < 4; ++k) {
-                const int kg = min((c * 4 + k) * 4 + wave, nks_total - 1);
+            for (int k = 0; k < CK; ++k) {
+                const int kg = min((c * CK + k) * 4 + wave, nks_total - 1);
                 ld_frag_async(fa[buf][k], a0 + size_t(kg) * 512);
                 ld_frag_async(fb[buf][k], a1 + size_t(kg) * 512);
             }
         };
         issue(0, 0);
+        if (NCH == 1) prefetch();
 #pragma unroll
         for (int c = 0; c < NCH; ++c) {
             const int buf = c & 1;
-            if (c + 1 < NCH) {
+            if (c + 2 < NCH) {
                 issue(c + 1, buf ^ 1);
-                wait_frags<8>(fa[buf], fb[buf]);
+                wait_frags<2 * CK>(fa[buf], fb[buf]);
+            } else if (c + 2 == NCH) {
+                issue(c + 1, buf ^ 1);
+                prefetch();
+                wait_frags<2 * CK + NPF>(fa[buf], fb[buf]);
             } else {
-                wait_frags<0>(fa[buf], fb[buf]);
+                wait_frags<NPF>(fa[buf], fb[buf]);
             }
             if (poll.on) {
                 // A pair of halfs that still holds the pattern has not been written yet by its producer:
@@ -170,7 +182,7 @@ __device__ __forceinline__ void wave_product(floatx4 (&acc)[2][NT], const half8 
                 for (;;) {
                     unsigned m = 0u;
 #pragma unroll
-                    for (int k = 0; k < 4; ++k) {
+                    for (int k = 0; k < CK; ++k) {
                         const uint4 ua = __builtin_bit_cast(uint4, fa[buf][k]);
                         const uint4 ub = __builtin_bit_cast(uint4, fb[buf][k]);
                         m = max(m, max(max(ua.x, ua.y), max(ua.z, ua.w)));
@@ -188,13 +200,13 @@ __device__ __forceinline__ void wave_product(floatx4 (&acc)[2][NT], const half8 
                         break;   // results are garbage from here on; the workgroup leaves at its next barrier
                     }
                     issue(c, buf);
-                    wait_frags<0>(fa[buf], fb[buf]);
+                    wait_frags<0>(fa[buf], fb[buf]);   // (also what was issued after this chunk the first time)
                 }
             }
 #pragma unroll
-            for (int k = 0; k < 4; ++k) {
+            for (int k = 0; k < CK; ++k) {
                 constexpr int KR = KS - KL;
-                const int ks = c * 4 + k;
+                const int ks = c * CK + k;
 #pragma unroll
                 for (int n = 0; n < NT; ++n) {
                     half8 w;
@@ -218,6 +230,7 @@ __device__ __forceinline__ void wave_product(floatx4 (&acc)[2][NT], const half8 
                 acc[1][n] = __builtin_amdgcn_mfma_f32_16x16x32_f16(w, fb, acc[1][n], 0, 0, 0);
             }
         }
+        prefetch();
     }
 }
 
@@ -257,12 +270,18 @@ __device__ __forceinline__ unsigned pack_h2(float a, float b) {
 // that to show.  Pack<N> is N halfs as raw bits.
 template <int N> struct Pack;
 template <> struct Pack<2> { unsigned v; };
-template <> struct Pack<4> { uint2 v; };
+typedef unsigned uintx2 __attribute__((ext_vector_type(2)));
+typedef float floatx2 __attribute__((ext_vector_type(2)));
+template <> struct Pack<4> { uintx2 v; };
+// N floats as one register tuple (destination of an asynchronous load)
+template <int N> struct F32;
+template <> struct F32<2> { floatx2 v; };
+template <> struct F32<4> { floatx4 v; };
 
 __device__ __forceinline__ Pack<2> ld_pack(const half_t* p, Pack<2>*) { return Pack<2>{*reinterpret_cast<const unsigned*>(p)}; }
-__device__ __forceinline__ Pack<4> ld_pack(const half_t* p, Pack<4>*) { return Pack<4>{*reinterpret_cast<const uint2*>(p)}; }
+__device__ __forceinline__ Pack<4> ld_pack(const half_t* p, Pack<4>*) { return Pack<4>{*reinterpret_cast<const uintx2*>(p)}; }
 __device__ __forceinline__ void st_pack(half_t* p, Pack<2> v) { *reinterpret_cast<unsigned*>(p) = v.v; }
-__device__ __forceinline__ void st_pack(half_t* p, Pack<4> v) { *reinterpret_cast<uint2*>(p) = v.v; }
+__device__ __forceinline__ void st_pack(half_t* p, Pack<4> v) { *reinterpret_cast<uintx2*>(p) = v.v; }
 __device__ __forceinline__ void unpack(Pack<2> v, float (&f)[2]) { unpack_h2(v.v, f[0], f[1]); }
 __device__ __forceinline__ void unpack(Pack<4> v, float (&f)[4]) {
     unpack_h2(v.v.x, f[0], f[1]);
@@ -270,10 +289,10 @@ __device__ __forceinline__ void unpack(Pack<4> v, float (&f)[4]) {
 }
 __device__ __forceinline__ Pack<2> pack(const float (&f)[2]) { return Pack<2>{pack_h2(f[0], f[1])}; }
 __device__ __forceinline__ Pack<4> pack(const float (&f)[4]) {
-    return Pack<4>{uint2{pack_h2(f[0], f[1]), pack_h2(f[2], f[3])}};
+    return Pack<4>{uintx2{pack_h2(f[0], f[1]), pack_h2(f[2], f[3])}};
 }
 __device__ __forceinline__ Pack<2> pack_fill(unsigned w, Pack<2>*) { return Pack<2>{w}; }
-__device__ __forceinline__ Pack<4> pack_fill(unsigned w, Pack<4>*) { return Pack<4>{uint2{w, w}}; }
+__device__ __forceinline__ Pack<4> pack_fill(unsigned w, Pack<4>*) { return Pack<4>{uintx2{w, w}}; }
 
 // One group into the exchange ring.  Consumers validate every 32-bit word on its own, so the two words
 // of an 8-byte group need not become visible together.
@@ -288,7 +307,7 @@ __device__ __forceinline__ void store_xch(half_t* dst, Pack<4> v, bool device_sc
         const u64 w = (u64(v.v.y) << 32) | v.v.x;
         __hip_atomic_store(reinterpret_cast<u64*>(dst), w, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     } else {
-        *reinterpret_cast<uint2*>(dst) = v.v;
+        *reinterpret_cast<uintx2*>(dst) = v.v;
     }
 }
 
@@ -322,6 +341,30 @@ __device__ __forceinline__ void ld_f32_coherent(const float* p, float (&f)[4]) {
 // order 0, 8, 1, 9, ...: the 16 lanes that the LDS serves together then read the partial sums of rows
 // r and r + 8, which are 32 banks apart for every row pitch in use (132, 68, 36, 20 floats).
 __device__ __forceinline__ int group_row(int idx) { return (idx % 2) * 8 + (idx / 2) % 8 + (idx / 16) * 16; }
+
+// Asynchronous loads of the per-step operands that come from HBM (x-projection, gate and cell caches, dY).
+// They are issued by hand, right after the LAST fragment load of a step's product: loads return in issue
+// order, so anything slow that sits in front of the fragment loads would hold them up, and a known number
+// of them behind lets the fragment waits discount them.  The values are used only after settle().
+__device__ __forceinline__ void ld_async(unsigned& d, const void* p) {
+    asm volatile("global_load_dword %0, %1, off" : "=v"(d) : "v"(p) : "memory");
+}
+__device__ __forceinline__ void ld_async(uintx2& d, const void* p) {
+    asm volatile("global_load_dwordx2 %0, %1, off" : "=v"(d) : "v"(p) : "memory");
+}
+__device__ __forceinline__ void ld_async(floatx2& d, const void* p) {
+    asm volatile("global_load_dwordx2 %0, %1, off" : "=v"(d) : "v"(p) : "memory");
+}
+__device__ __forceinline__ void ld_async(floatx4& d, const void* p) {
+    asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(d) : "v"(p) : "memory");
+}
+__device__ __forceinline__ void wait_all_vm() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
+template <typename T>
+__device__ __forceinline__ void settle(T& x) { asm volatile("" : "+v"(x)); }   // no use of x moves above this point
+__device__ __forceinline__ void to_floats(const F32<2>& r, float (&f)[2]) { f[0] = r.v.x; f[1] = r.v.y; }
+__device__ __forceinline__ void to_floats(const F32<4>& r, float (&f)[4]) {
+    f[0] = r.v.x; f[1] = r.v.y; f[2] = r.v.z; f[3] = r.v.w;
+}
 
 // Cycle counters of workgroup 0 per phase (only when the host passes a buffer): product (including the
 // wait for the operand), partial exchange, pointwise, cache stores + prefetch.  Thread 0 accumulates in
@@ -401,19 +444,16 @@ __global__ __launch_bounds__(kThreads) void rec_fwd_kernel(RecFwdArgs p, RecLayo
     const bool c_in_regs = (rb_count == 1) && (t_end - t_begin > 1);
     float creg[UPT] = {};
     PackT xp[4];
-    auto prefetch = [&](int t, int rb) {
-        const int b = rb * kRows + pr;
-        if (b < p.B) {
-            const half_t* src = p.G + (size_t(t) * p.B + b) * gld + size_t(hs) * NC + pj;
+    auto prefetch = [&](int t, int rb) {   // 4 loads per wave; rows past B fetch row B-1 and are not used
+        const int b = min(rb * kRows + pr, p.B - 1);
+        const half_t* src = p.G + (size_t(t) * p.B + b) * gld + size_t(hs) * NC + pj;
 #pragma unroll
-            for (int gt = 0; gt < 4; ++gt) xp[gt] = ld_pack(src + gt * JB, (PackT*)nullptr);
-        }
+        for (int gt = 0; gt < 4; ++gt) ld_async(xp[gt].v, src + gt * JB);
     };
     if (c_in_regs) {
         const int b = g * kRows + pr;
         if (b < p.B) ld_f32(p.C + (size_t(t_begin) * p.B + b) * p.Hp + j, creg);
     }
-    prefetch(t_begin, g);
     __syncthreads();
     clk.start();
 
@@ -431,7 +471,8 @@ __global__ __launch_bounds__(kThreads) void rec_fwd_kernel(RecFwdArgs p, RecLayo
             for (int m = 0; m < 2; ++m)
 #pragma unroll
                 for (int n = 0; n < NT; ++n) acc[m][n] = floatx4{0.f, 0.f, 0.f, 0.f};
-            wave_product<NT, KS, RESIDENT>(acc, wreg, nullptr, wfrag_wave, a0, a1, wave, lane, nks_total, ks_wave, poll);
+            wave_product<NT, KS, RESIDENT, 0, 4>(acc, wreg, nullptr, wfrag_wave, a0, a1, wave, lane, nks_total, ks_wave,
+                                                 poll, [&]() { prefetch(t, rb); });
             clk.lap(0);
             spill_partials<NT>(part, acc, wave, lane, PLD);
             __syncthreads();
@@ -441,6 +482,9 @@ __global__ __launch_bounds__(kThreads) void rec_fwd_kernel(RecFwdArgs p, RecLayo
             // Every peer of this group has delivered h_{t-1}, so all of them are done reading h_{t-2}:
             // its slot can be marked for reuse.  The mark is acknowledged long before the wait that
             // precedes the h_t store below, so whoever sees this step's h_t also sees the mark.
+            wait_all_vm();   // the x-projection of this step, issued during the product
+#pragma unroll
+            for (int gt = 0; gt < 4; ++gt) settle(xp[gt].v);
             const int b = row0 + pr;
             const unsigned xoff = unsigned(xch_offset(b, j, nks_total));   // 32 bits: a slot is far below 4G halfs
             store_xch(xnext + xoff, pack_fill(kUnwritten, (PackT*)nullptr), device_scope);
@@ -496,10 +540,6 @@ __global__ __launch_bounds__(kThreads) void rec_fwd_kernel(RecFwdArgs p, RecLayo
 #pragma unroll
                 for (int gt = 0; gt < 4; ++gt) st_pack(dst + gt * JB, act[gt]);
             }
-            // x-projection of the next work item
-            int nt_ = t, nrb_ = rb + L.ng;
-            if (nrb_ >= L.nrb) { nt_ = t + 1; nrb_ = g; }
-            if (nt_ < t_end) prefetch(nt_, nrb_);
             clk.lap(3);
         }
     }
@@ -568,19 +608,17 @@ __global__ __launch_bounds__(kThreads) void rec_bwd_kernel(RecBwdArgs p, RecLayo
     }
     // prefetched per work item: activated gates, c_{t-1}, c_t, dY_t
     PackT pg[4], pdy;
-    float pcp[UPT], pcc[UPT];
-    auto prefetch = [&](int t, int rb) {
-        const int b = rb * kRows + pr;
-        if (b < p.B) {
-            const half_t* gsrc = p.G + (size_t(t) * p.B + b) * gld + pq;
+    F32<UPT> pcp_r, pcc_r;
+    auto prefetch = [&](int t, int rb) {   // 7 loads per wave; rows past B fetch row B-1, the closing pass step 0
+        const int b = min(rb * kRows + pr, p.B - 1);
+        const int tt = max(t, 0);
+        const half_t* gsrc = p.G + (size_t(tt) * p.B + b) * gld + pq;
 #pragma unroll
-            for (int gt = 0; gt < 4; ++gt) pg[gt] = ld_pack(gsrc + gt * JF, (PackT*)nullptr);
-            ld_f32(p.C + (size_t(t) * p.B + b) * p.Hp + j, pcp);
-            ld_f32(p.C + (size_t(t + 1) * p.B + b) * p.Hp + j, pcc);
-            pdy = ld_pack(p.dY + (size_t(t) * p.B + b) * p.Hp + j, (PackT*)nullptr);
-        }
+        for (int gt = 0; gt < 4; ++gt) ld_async(pg[gt].v, gsrc + gt * JF);
+        ld_async(pcp_r.v, p.C + (size_t(tt) * p.B + b) * p.Hp + j);
+        ld_async(pcc_r.v, p.C + (size_t(tt + 1) * p.B + b) * p.Hp + j);
+        ld_async(pdy.v, p.dY + (size_t(tt) * p.B + b) * p.Hp + j);
     };
-    if (t_first >= 0) prefetch(t_first, g);
     __syncthreads();
     float dbacc[4][UPT] = {};
     clk.start();
@@ -601,13 +639,22 @@ __global__ __launch_bounds__(kThreads) void rec_bwd_kernel(RecBwdArgs p, RecLayo
                 for (int m = 0; m < 2; ++m)
 #pragma unroll
                     for (int n = 0; n < NT; ++n) acc[m][n] = floatx4{0.f, 0.f, 0.f, 0.f};
-                wave_product<NT, KS, RESIDENT, KL>(acc, wreg, wlds, wfrag_wave, a0, a1, wave, lane, nks_total, ks_wave, poll);
+                wave_product<NT, KS, RESIDENT, KL, 7>(acc, wreg, wlds, wfrag_wave, a0, a1, wave, lane, nks_total, ks_wave,
+                                                      poll, [&]() { prefetch(t, rb); });
                 clk.lap(0);
                 spill_partials<NT>(part, acc, wave, lane, PLD);
                 __syncthreads();
                 if (lds_abort != 0) return;
                 clk.lap(1);
+            } else {
+                prefetch(t, rb);
             }
+            wait_all_vm();   // gates, cell states and dY of this step, issued during the product
+#pragma unroll
+            for (int gt = 0; gt < 4; ++gt) settle(pg[gt].v);
+            settle(pdy.v);
+            settle(pcp_r.v);
+            settle(pcc_r.v);
             const int b = row0 + pr;
             const bool live = b < p.B;
             const size_t sidx = size_t(b) * p.Hp + j;
@@ -625,6 +672,9 @@ __global__ __launch_bounds__(kThreads) void rec_bwd_kernel(RecBwdArgs p, RecLayo
                 }
             }
             if (live) {
+                float pcp[UPT], pcc[UPT];
+                to_floats(pcp_r, pcp);
+                to_floats(pcc_r, pcc);
                 float dh[UPT];
                 if (from_product) {
 #pragma unroll
@@ -692,9 +742,6 @@ __global__ __launch_bounds__(kThreads) void rec_bwd_kernel(RecBwdArgs p, RecLayo
                 for (int gt = 0; gt < 4; ++gt) st_pack(gdst + gt * JF, dgnew[gt]);
                 if (!dc_in_regs) st_f32(p.dC + sidx, dcreg);
             }
-            int nt_ = t, nrb_ = rb + L.ng;
-            if (nrb_ >= L.nrb) { nt_ = t - 1; nrb_ = g; }
-            if (nt_ >= t_last && nt_ >= 0) prefetch(nt_, nrb_);
             clk.lap(3);
         }
     }
