@@ -150,9 +150,14 @@ def main():
     kflops = {"fwd_proj": 2.0 * T * B * 4 * H * I, "fwd_rec": 2.0 * T * B * 4 * H * H,
               "bwd_rec": 2.0 * T * B * 4 * H * H, "bwd_dx": 2.0 * T * B * 4 * H * I,
               "bwd_dw": 2.0 * T * B * 4 * H * (I + H)}
-    kname = {"fwd_proj": "gemm_nt_256x256 (X*W_ih^T)", "fwd_rec": "rec_fwd_kernel (persistent recurrence)",
-             "bwd_rec": "rec_bwd_kernel (persistent BPTT)", "bwd_dx": "gemm_nt_256x256 (dG*W_ih)",
-             "bwd_dw": "transpose_pad x3 + gemm_nt_256x256 split-K (dG^T*[X;H]) + reduce_dw"}
+    kname = {"fwd_proj": "gemm_nt_stream (X*W_ih^T + bias)", "fwd_rec": "rec_fwd_kernel (persistent recurrence)",
+             "bwd_rec": "rec_bwd_kernel (persistent BPTT)", "bwd_dx": "gemm_nt_stream (dG*W_ih)",
+             "bwd_dw": "gemm_tn_256x256 split-K x2 (dG^T*X, dG^T*H) + reduce_dw"}
+    # HBM-side traffic per launch at config3 from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (x2.0 / x1.0 after
+    # calibration against the fp16 output copy of the same run); see profiles/*_hbm_traffic.md
+    GiB = float(1 << 30)
+    traffic_config3 = {"fwd_proj": (3.01 + 1.25) * GiB, "bwd_dx": (3.01 + 1.25) * GiB, "fwd_rec": (2.07 + 3.50) * GiB,
+                       "bwd_rec": (3.57 + 2.75) * GiB, "bwd_dw": 2 * (3.04 + 0.25) * GiB}
     kernels = []
     for k in phases:
         tf = kflops[k] / (phase_ms[k] * 1e-3) / 1e12 if phase_ms[k] > 0 else 0.0
@@ -160,7 +165,9 @@ def main():
                         "frac_of_peak": round(tf / PEAK_FP16_TFLOPS, 4)})
     dom = max(kernels, key=lambda d: d["ms"])
     roofline = {"kernel": dom["kernel"], "bound": "mfma", "achieved": dom["tflops"], "peak": PEAK_FP16_TFLOPS,
-                "unit": "TFLOP/s", "frac": dom["frac_of_peak"], "traffic": None,
+                "unit": "TFLOP/s", "frac": dom["frac_of_peak"],
+                "traffic": traffic_config3[dom["phase"]] if args.workload == "config3" else None,
+                "traffic_unit": "bytes per launch (fetched + written beyond the L2)",
                 "launch_ms": dom["ms"], "flops_per_launch": kflops[dom["phase"]]}
     if dom["phase"] in ("fwd_rec", "bwd_rec"):
         roofline["us_per_timestep"] = round(dom["ms"] * 1e3 / T, 3)
