@@ -116,6 +116,14 @@ def main():
         print("bench.py: no GPU visible", file=sys.stderr)
         sys.exit(1)
     torch.cuda.set_device(0)
+    props = torch.cuda.get_device_properties(0)
+    clock_khz = getattr(props, "clock_rate", None)
+    device = {"name": props.name, "compute_units": props.multi_processor_count,
+              "max_engine_clock_mhz": (clock_khz / 1e3) if clock_khz else None,
+              # 4096 fp16 MFMA FLOP per clock and CU (CDNA4, dense)
+              "derived_fp16_peak_tflops": (round(props.multi_processor_count * 4096 * clock_khz * 1e3 / 1e12, 1)
+                                           if clock_khz else None),
+              "peak_used_tflops": PEAK_FP16_TFLOPS, "hbm_gib": round(props.total_memory / 2 ** 30, 1)}
     T, B, I, H, backward = WORKLOADS[args.workload]
     p = make_inputs(T, B, I, H)
     core = LstmCore(B, I, H)
@@ -187,7 +195,9 @@ def main():
         "persistent": {"fwd": core.info("persistent_fwd"), "bwd": core.info("persistent_bwd"),
                        "xcd_local_fwd": core.info("xcd_local_fwd"), "xcd_local_bwd": core.info("xcd_local_bwd"),
                        "fallbacks": core.info("fallbacks")},
-        "roofline": roofline, "kernels": kernels,
+        "roofline": roofline, "kernels": kernels, "device": device,
+        "us_per_timestep": {"fwd_rec": round(phase_ms["fwd_rec"] * 1e3 / T, 3),
+                            **({"bwd_rec": round(phase_ms["bwd_rec"] * 1e3 / T, 3)} if backward else {})},
     }
     core.close()
     if not args.no_parity:

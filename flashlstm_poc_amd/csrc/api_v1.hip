@@ -12,6 +12,7 @@
 
 #include "../../include/flashlstm/lstm_api.h"
 #include "../../include/flashlstm/lstm_core.h"
+#include "instrument.h"
 
 namespace {
 
@@ -108,6 +109,7 @@ extern "C" int lstm_forward(const float* x, const float* b_ih, const float* b_hh
                             const float* c0, float* output, float* hn, float* cn, size_t seq_len,
                             size_t batch, size_t input_size, size_t hidden_size, const lstm_buffers* buffers,
                             lstm_compute_precision_t precision) {
+    flstm_hip::RangeGuard range("FlashLSTM::lstm_forward");
     if (!buffers || !buffers->impl) return kInvalid;
     auto* impl = static_cast<V1Impl*>(buffers->impl);
     if (impl->precision != precision) return kInvalid;
@@ -130,6 +132,7 @@ extern "C" int lstm_forward(const float* x, const float* b_ih, const float* b_hh
                           (honor_immediate && impl->mode == LSTM_EXECUTION_MODE_IMMEDIATE) ? 1 : 0);
     int rc = flstm_core_pack_bias(impl->plan, b_ih, b_hh, impl->stream);
     if (rc) return rc;
+    flstm_hip::RangeGuard compute("FlashLSTM::lstm_forward::compute");
     return flstm_core_forward(impl->plan, seq_len, x, FLSTM_F32, h0, c0, FLSTM_F32, output, FLSTM_F32, hn, cn,
                               FLSTM_F32, 1, impl->stream);
 }
@@ -138,6 +141,7 @@ extern "C" int lstm_backward(const float* x, const float* d_output, const float*
                              float* dx, float* dW_ih, float* dW_hh, float* db, float* dh0, float* dc0,
                              size_t seq_len, size_t batch, size_t input_size, size_t hidden_size,
                              const lstm_buffers* buffers) {
+    flstm_hip::RangeGuard range("FlashLSTM::lstm_backward");
     if (!buffers || !buffers->impl) return kInvalid;
     auto* impl = static_cast<V1Impl*>(buffers->impl);
     if (impl->batch != batch || impl->input_size != input_size || impl->hidden_size != hidden_size) return kInvalid;

@@ -65,6 +65,10 @@ struct flstm_core_plan {
     DevBuf X16, G, Y, C, status, xch_f, xch_b;
     size_t T_cache = 0;
     bool have_cache = false;
+    // pass in progress (begin / steps / end)
+    struct { size_t T = 0; const void* x = nullptr; flstm_dtype x_dtype = FLSTM_F16; bool open = false; } fw;
+    struct { size_t T = 0; const half_t* dYk = nullptr; const void* dY = nullptr; flstm_dtype dy_dtype = FLSTM_F16;
+             float S = 1.f, dy_scale = 1.f; void* dx = nullptr; flstm_dtype dx_dtype = FLSTM_F16; bool open = false; } bw;
     // backward scratch
     DevBuf dYp, dG, dHn, dC, dH0, db_part, dw_part, prof;
     int opt_profile = 0, wall_khz = 100000;
@@ -215,23 +219,14 @@ extern "C" int flstm_core_pack_bias(flstm_core_plan* p, const float* b_ih, const
 
 namespace {
 
-int forward_once(flstm_core_plan* p, size_t T, const void* x, flstm_dtype x_dtype, const void* h0,
-                 const void* c0, flstm_dtype state_dtype, hipStream_t s) {
+// Forward pass in three parts so that a caller can feed it in ranges of steps: setup (state rows, exchange
+// ring), any number of step ranges in order (x rows -> projection -> recurrence), and the status check.
+int forward_setup(flstm_core_plan* p, size_t T, const void* x, flstm_dtype x_dtype, const void* h0,
+                  const void* c0, flstm_dtype state_dtype, hipStream_t s) {
     const Dims& d = p->d;
     const size_t TB = T * size_t(d.B);
-    // operand A of the projection
-    const half_t* A = nullptr;
-    size_t lda = 0;
-    if (x_dtype == FLSTM_F16 && d.I == d.Ip) {
-        A = static_cast<const half_t*>(x);
-        lda = size_t(d.I);
-    } else {
-        FL_TRY(p->X16.reserve(TB * d.Ip * sizeof(half_t)));
-        FL_TRY(convert_pad(x, x_dtype == FLSTM_F32, TB, d.I, size_t(d.I), 1.f, p->X16.as<half_t>(), TB,
-                           size_t(d.Ip), s));
-        A = p->X16.as<half_t>();
-        lda = size_t(d.Ip);
-    }
+    p->fw.T = T; p->fw.x = x; p->fw.x_dtype = x_dtype; p->fw.open = true;
+    if (!(x_dtype == FLSTM_F16 && d.I == d.Ip)) FL_TRY(p->X16.reserve(TB * d.Ip * sizeof(half_t)));
     FL_TRY(p->G.reserve(TB * 4 * d.Hp * sizeof(half_t)));
     FL_TRY(p->Y.reserve((TB + d.B) * d.Hp * sizeof(half_t)));
     FL_TRY(p->C.reserve((TB + d.B) * d.Hp * sizeof(float)));
@@ -246,37 +241,68 @@ int forward_once(flstm_core_plan* p, size_t T, const void* x, flstm_dtype x_dtyp
     FL_TRY(fill_zero(p->xch_f.p, xslot * sizeof(half_t), s));
     FL_TRY(fill_words(p->xch_f.as<half_t>() + xslot, 2 * xslot * sizeof(half_t), 0xFFFFFFFFu, s));
     FL_TRY(to_exchange_layout(p->Y.as<half_t>(), d.B, d.Hp, size_t(d.Hp), p->xch_f.as<half_t>(), s));
+    if (p->opt_profile) FL_TRY(fill_zero(p->prof.p, 8 * sizeof(long long), s));
+    return 0;
+}
 
-    FL_TRY(hipEventRecord(p->tm.ev[0], s));
+// x rows of steps [t0, t0+n) -> fp16 operand -> x-projection (+ bias) in G
+int forward_project(flstm_core_plan* p, size_t t0, size_t n, hipStream_t s) {
+    const Dims& d = p->d;
+    const half_t* A = nullptr;   // first row of step t0
+    size_t lda = 0;
+    if (p->fw.x_dtype == FLSTM_F16 && d.I == d.Ip) {
+        A = static_cast<const half_t*>(p->fw.x) + t0 * d.B * d.I;
+        lda = size_t(d.I);
+    } else {
+        const size_t esz = p->fw.x_dtype == FLSTM_F32 ? 4 : 2;
+        const char* src = static_cast<const char*>(p->fw.x) + t0 * d.B * d.I * esz;
+        half_t* dst = p->X16.as<half_t>() + t0 * d.B * d.Ip;
+        FL_TRY(convert_pad(src, p->fw.x_dtype == FLSTM_F32, n * d.B, d.I, size_t(d.I), 1.f, dst, n * d.B, size_t(d.Ip), s));
+        A = dst;
+        lda = size_t(d.Ip);
+    }
     // hoisted input projection, optionally in chunks of time steps
-    size_t chunk_steps = (p->opt_proj_chunk <= 0 || size_t(p->opt_proj_chunk) > T) ? T : size_t(p->opt_proj_chunk);
-    for (size_t t0 = 0; t0 < T; t0 += chunk_steps) {
-        const size_t steps = (t0 + chunk_steps <= T) ? chunk_steps : T - t0;
+    size_t chunk_steps = (p->opt_proj_chunk <= 0 || size_t(p->opt_proj_chunk) > n) ? n : size_t(p->opt_proj_chunk);
+    for (size_t c0 = 0; c0 < n; c0 += chunk_steps) {
+        const size_t steps = (c0 + chunk_steps <= n) ? chunk_steps : n - c0;
         GemmNT g{};
-        g.A = A + t0 * d.B * lda; g.lda = lda;
+        g.A = A + c0 * d.B * lda; g.lda = lda;
         g.B = p->wih_p.as<half_t>(); g.ldb = size_t(d.Ip);
         g.M = int(steps * d.B); g.N = 4 * d.Hp; g.K = d.Ip;
-        g.C16 = p->G.as<half_t>() + t0 * d.B * 4 * d.Hp; g.C32 = nullptr; g.ldc = size_t(4) * d.Hp;
+        g.C16 = p->G.as<half_t>() + (t0 + c0) * d.B * 4 * d.Hp; g.C32 = nullptr; g.ldc = size_t(4) * d.Hp;
         g.alpha = 1.f; g.splits = 1; g.split_stride = 0;
         g.bias = p->bias_p.as<float>();   // b_ih + b_hh, packed gate order: the recurrence reads x-projection + bias
         FL_TRY(launch_gemm_nt(g, s));
     }
-    FL_TRY(hipEventRecord(p->tm.ev[1], s));
+    return 0;
+}
+
+int forward_recur(flstm_core_plan* p, size_t t0, size_t n, hipStream_t s) {
+    const Dims& d = p->d;
     RecFwdArgs a{};
     a.wfrag = p->wfrag_f.as<half8>();
     a.Y = p->Y.as<half_t>(); a.G = p->G.as<half_t>(); a.C = p->C.as<float>();
-    a.X = p->xch_f.as<half_t>(); a.x_slot = xslot;
+    a.X = p->xch_f.as<half_t>(); a.x_slot = exchange_slot_halfs(d.B, d.Hp);
     a.status = p->status.as<int>();
     a.seats = p->status.as<unsigned>() + 8;
     FL_TRY(fill_zero(a.seats, 8 * sizeof(unsigned), s));
-    a.B = d.B; a.Hp = d.Hp; a.T = int(T);
+    a.B = d.B; a.Hp = d.Hp; a.T = int(p->fw.T); a.t0 = int(t0); a.t1 = int(t0 + n);
     a.spin_limit = p->opt_spin_limit;
-    a.prof = nullptr;
-    if (p->opt_profile) {
-        FL_TRY(fill_zero(p->prof.p, 16 * sizeof(long long), s));
-        a.prof = p->prof.as<long long>();
-    }
+    a.prof = p->opt_profile ? p->prof.as<long long>() : nullptr;
     FL_TRY(launch_rec_fwd(p->Lf, a, s));
+    return 0;
+}
+
+int forward_once(flstm_core_plan* p, size_t T, const void* x, flstm_dtype x_dtype, const void* h0,
+                 const void* c0, flstm_dtype state_dtype, hipStream_t s) {
+    int rc = forward_setup(p, T, x, x_dtype, h0, c0, state_dtype, s);
+    if (rc) return rc;
+    FL_TRY(hipEventRecord(p->tm.ev[0], s));
+    rc = forward_project(p, 0, T, s);
+    if (rc) return rc;
+    FL_TRY(hipEventRecord(p->tm.ev[1], s));
+    rc = forward_recur(p, 0, T, s);
+    if (rc) return rc;
     FL_TRY(hipEventRecord(p->tm.ev[2], s));
     return 0;
 }
@@ -324,26 +350,29 @@ extern "C" int flstm_core_forward(flstm_core_plan* p, size_t T, const void* x, f
     FL_TRY(unpad_from_float(p->C.as<float>() + TB * d.Hp, size_t(d.Hp), size_t(d.B), d.H, 1.f, cy,
                             out_state_dtype == FLSTM_F32, s));
     FL_TRY(hipStreamSynchronize(s));
+    p->fw.open = false;
     if (save_for_backward) { p->have_cache = true; p->T_cache = T; }
     return 0;
 }
 
 namespace {
 
-int backward_rec_once(flstm_core_plan* p, size_t T, const void* dY, flstm_dtype dy_dtype, const void* d_hn,
-                      const void* d_cn, flstm_dtype dstate_dtype, float S, hipStream_t s) {
+// Backward recurrence in parts, like the forward pass: setup, step ranges from the end of the sequence towards
+// its start (dY rows -> BPTT steps -> dX rows), and the weight-gradient GEMMs over the whole sequence.
+int backward_setup(flstm_core_plan* p, size_t T, const void* dY, flstm_dtype dy_dtype, const void* d_hn,
+                   const void* d_cn, flstm_dtype dstate_dtype, float S, void* dx, flstm_dtype dx_dtype,
+                   hipStream_t s) {
     const Dims& d = p->d;
     const size_t TB = T * size_t(d.B);
-    const half_t* dYk = nullptr;
-    float dy_scale = S;
+    p->bw.T = T; p->bw.dY = dY; p->bw.dy_dtype = dy_dtype; p->bw.S = S; p->bw.dx = dx; p->bw.dx_dtype = dx_dtype;
+    p->bw.open = true;
     if (dy_dtype == FLSTM_F16 && d.H == d.Hp) {
-        dYk = static_cast<const half_t*>(dY);
+        p->bw.dYk = static_cast<const half_t*>(dY);
+        p->bw.dy_scale = S;
     } else {
         FL_TRY(p->dYp.reserve(TB * d.Hp * sizeof(half_t)));
-        FL_TRY(convert_pad(dY, dy_dtype == FLSTM_F32, TB, d.H, size_t(d.H), S, p->dYp.as<half_t>(), TB,
-                           size_t(d.Hp), s));
-        dYk = p->dYp.as<half_t>();
-        dy_scale = 1.f;
+        p->bw.dYk = p->dYp.as<half_t>();
+        p->bw.dy_scale = 1.f;   // the scale is applied while the rows are converted
     }
     const size_t st_bytes = size_t(d.B) * d.Hp * sizeof(float);
     FL_TRY(p->dHn.reserve(st_bytes));
@@ -357,78 +386,75 @@ int backward_rec_once(flstm_core_plan* p, size_t T, const void* dY, flstm_dtype 
     FL_TRY(convert_pad_f32(d_hn, dstate_dtype == FLSTM_F32, size_t(d.B), d.H, S, p->dHn.as<float>(), size_t(d.Hp), s));
     FL_TRY(convert_pad_f32(d_cn, dstate_dtype == FLSTM_F32, size_t(d.B), d.H, S, p->dC.as<float>(), size_t(d.Hp), s));
     FL_TRY(fill_zero(p->db_part.p, size_t(p->Lb.ng) * 4 * d.Hp * sizeof(float), s));
+    if (p->opt_profile) FL_TRY(fill_zero(p->prof.as<long long>() + 8, 8 * sizeof(long long), s));
+    return 0;
+}
 
-    FL_TRY(hipEventRecord(p->tm.ev[3], s));
+// steps t_hi .. t_lo (t_lo = -1 includes the closing dh0 product); dY rows of these steps are converted first
+// when the caller's dY cannot be used in place
+int backward_recur(flstm_core_plan* p, long t_hi, long t_lo, hipStream_t s) {
+    const Dims& d = p->d;
+    const long lo = t_lo < 0 ? 0 : t_lo;
+    if (p->bw.dYk != p->bw.dY && t_hi >= lo) {
+        const size_t esz = p->bw.dy_dtype == FLSTM_F32 ? 4 : 2;
+        const size_t rows = size_t(t_hi - lo + 1) * d.B;
+        const char* src = static_cast<const char*>(p->bw.dY) + size_t(lo) * d.B * d.H * esz;
+        half_t* dst = p->dYp.as<half_t>() + size_t(lo) * d.B * d.Hp;
+        FL_TRY(convert_pad(src, p->bw.dy_dtype == FLSTM_F32, rows, d.H, size_t(d.H), p->bw.S, dst, rows, size_t(d.Hp), s));
+    }
     RecBwdArgs a{};
     a.wfrag = p->wfrag_b.as<half8>();
-    a.G = p->G.as<half_t>(); a.C = p->C.as<float>(); a.dY = dYk; a.dG = p->dG.as<half_t>();
+    a.G = p->G.as<half_t>(); a.C = p->C.as<float>(); a.dY = p->bw.dYk; a.dG = p->dG.as<half_t>();
     a.dHn = p->dHn.as<float>(); a.dC = p->dC.as<float>(); a.dH0 = p->dH0.as<float>();
-    a.X = p->xch_b.as<half_t>(); a.x_slot = xslot;
+    a.X = p->xch_b.as<half_t>(); a.x_slot = exchange_slot_halfs(d.B, 4 * d.Hp);
     a.db_part = p->db_part.as<float>();
     a.status = p->status.as<int>();
     a.seats = p->status.as<unsigned>() + 8;
     FL_TRY(fill_zero(a.seats, 8 * sizeof(unsigned), s));
-    a.B = d.B; a.Hp = d.Hp; a.T = int(T); a.jb_fwd = d.JF; a.dy_scale = dy_scale;
+    a.B = d.B; a.Hp = d.Hp; a.T = int(p->bw.T); a.jb_fwd = d.JF; a.dy_scale = p->bw.dy_scale;
+    a.t_hi = int(t_hi); a.t_lo = int(t_lo);
     a.spin_limit = p->opt_spin_limit;
-    a.prof = nullptr;
-    if (p->opt_profile) {
-        FL_TRY(fill_zero(p->prof.p, 16 * sizeof(long long), s));
-        a.prof = p->prof.as<long long>() + 8;
-    }
+    a.prof = p->opt_profile ? p->prof.as<long long>() + 8 : nullptr;
     FL_TRY(launch_rec_bwd(p->Lb, a, s));
+    return 0;
+}
+
+// dX rows of steps [t_lo, t_hi] = dG * W_ih  (contraction over the packed gate columns)
+int backward_dx(flstm_core_plan* p, long t_hi, long t_lo, hipStream_t s) {
+    const Dims& d = p->d;
+    if (!p->bw.dx || t_hi < t_lo) return 0;
+    const size_t row0 = size_t(t_lo) * d.B, rows = size_t(t_hi - t_lo + 1) * d.B;
+    GemmNT g{};
+    g.A = p->dG.as<half_t>() + row0 * 4 * d.Hp; g.lda = size_t(4) * d.Hp;
+    g.B = p->wih_t.as<half_t>(); g.ldb = size_t(4) * d.Hp;
+    g.M = int(rows); g.N = d.I; g.K = 4 * d.Hp;
+    if (p->bw.dx_dtype == FLSTM_F32) g.C32 = static_cast<float*>(p->bw.dx) + row0 * d.I;
+    else g.C16 = static_cast<half_t*>(p->bw.dx) + row0 * d.I;
+    g.ldc = size_t(d.I); g.alpha = 1.f / p->bw.S; g.splits = 1; g.split_stride = 0;
+    FL_TRY(launch_gemm_nt(g, s));
+    return 0;
+}
+
+int backward_rec_once(flstm_core_plan* p, size_t T, const void* dY, flstm_dtype dy_dtype, const void* d_hn,
+                      const void* d_cn, flstm_dtype dstate_dtype, float S, void* dx, flstm_dtype dx_dtype,
+                      hipStream_t s) {
+    int rc = backward_setup(p, T, dY, dy_dtype, d_hn, d_cn, dstate_dtype, S, dx, dx_dtype, s);
+    if (rc) return rc;
+    FL_TRY(hipEventRecord(p->tm.ev[3], s));
+    rc = backward_recur(p, long(T) - 1, -1, s);
+    if (rc) return rc;
     FL_TRY(hipEventRecord(p->tm.ev[4], s));
     return 0;
 }
 
-}  // namespace
-
-extern "C" int flstm_core_backward(flstm_core_plan* p, size_t T, const void* x, flstm_dtype x_dtype,
-                                   const void* dY, flstm_dtype dy_dtype, const void* d_hn, const void* d_cn,
-                                   flstm_dtype dstate_dtype, float grad_scale, void* dx, flstm_dtype dx_dtype,
-                                   float* dW_ih, float* dW_hh, float* db_ih, float* db_hh, float* dh0,
-                                   float* dc0, void* stream) {
-    if (!p) return FLSTM_E_INVALID;
-    if (T == 0) return 0;
-    if (!p->have_cache || p->T_cache != T) return FLSTM_E_NO_CACHE;
-    if (!dY) return FLSTM_E_INVALID;
-    if (dW_ih && !x) return FLSTM_E_INVALID;
-    hipStream_t s = static_cast<hipStream_t>(stream);
+// dW_ih = dG^T * X and dW_hh = dG^T * H_prev over the whole sequence, bias gradient and state gradients
+int backward_finish(flstm_core_plan* p, const void* x, flstm_dtype x_dtype, float* dW_ih, float* dW_hh,
+                    float* db_ih, float* db_hh, float* dh0, float* dc0, hipStream_t s) {
     const Dims& d = p->d;
-    const size_t TB = T * size_t(d.B);
-    const float S = grad_scale > 0.f ? grad_scale : 1.f;
-    const float invS = 1.f / S;
-
-    int rc = backward_rec_once(p, T, dY, dy_dtype, d_hn, d_cn, dstate_dtype, S, s);
-    if (rc) return rc;
-    int st = 0;
-    rc = read_status(p, s, &st);
-    if (rc) return rc;
-    if (st != 0) {
-        if (!p->Lb.persistent) return FLSTM_E_STALLED;
-        p->broken_bwd = true;
-        p->fallbacks++;
-        replan(p);
-        rc = backward_rec_once(p, T, dY, dy_dtype, d_hn, d_cn, dstate_dtype, S, s);
-        if (rc) return rc;
-        rc = read_status(p, s, &st);
-        if (rc) return rc;
-        if (st != 0) return FLSTM_E_STALLED;
-    }
-
-    // dX = dG * W_ih  (contraction over the packed gate columns)
-    if (dx) {
-        GemmNT g{};
-        g.A = p->dG.as<half_t>(); g.lda = size_t(4) * d.Hp;
-        g.B = p->wih_t.as<half_t>(); g.ldb = size_t(4) * d.Hp;
-        g.M = int(TB); g.N = d.I; g.K = 4 * d.Hp;
-        if (dx_dtype == FLSTM_F32) g.C32 = static_cast<float*>(dx); else g.C16 = static_cast<half_t*>(dx);
-        g.ldc = size_t(d.I); g.alpha = invS; g.splits = 1; g.split_stride = 0;
-        FL_TRY(launch_gemm_nt(g, s));
-    }
-    FL_TRY(hipEventRecord(p->tm.ev[5], s));
-
-    // dW_ih = dG^T * X and dW_hh = dG^T * H_prev: k-major operands exactly as the recurrence left them
-    // (H_prev of step t is row block t of the state array, row block 0 = h0), split over K, fp32 partials.
+    const size_t TB = p->bw.T * size_t(d.B);
+    const float invS = 1.f / p->bw.S;
+    // k-major operands exactly as the recurrence left them (H_prev of step t is row block t of the state array,
+    // row block 0 = h0), split over K, fp32 partials
     for (int which = 0; which < 2; ++which) {
         float* dst = which == 0 ? dW_ih : dW_hh;
         if (!dst) continue;
@@ -464,6 +490,46 @@ extern "C" int flstm_core_backward(flstm_core_plan* p, size_t T, const void* x, 
     FL_TRY(unpad_from_float(p->dC.as<float>(), size_t(d.Hp), size_t(d.B), d.H, invS, dc0, 1, s));
     FL_TRY(hipEventRecord(p->tm.ev[7], s));
     FL_TRY(hipStreamSynchronize(s));
+    p->bw.open = false;
+    return 0;
+}
+
+}  // namespace
+
+extern "C" int flstm_core_backward(flstm_core_plan* p, size_t T, const void* x, flstm_dtype x_dtype,
+                                   const void* dY, flstm_dtype dy_dtype, const void* d_hn, const void* d_cn,
+                                   flstm_dtype dstate_dtype, float grad_scale, void* dx, flstm_dtype dx_dtype,
+                                   float* dW_ih, float* dW_hh, float* db_ih, float* db_hh, float* dh0,
+                                   float* dc0, void* stream) {
+    if (!p) return FLSTM_E_INVALID;
+    if (T == 0) return 0;
+    if (!p->have_cache || p->T_cache != T) return FLSTM_E_NO_CACHE;
+    if (!dY) return FLSTM_E_INVALID;
+    if (dW_ih && !x) return FLSTM_E_INVALID;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const float S = grad_scale > 0.f ? grad_scale : 1.f;
+
+    int rc = backward_rec_once(p, T, dY, dy_dtype, d_hn, d_cn, dstate_dtype, S, dx, dx_dtype, s);
+    if (rc) return rc;
+    int st = 0;
+    rc = read_status(p, s, &st);
+    if (rc) return rc;
+    if (st != 0) {
+        if (!p->Lb.persistent) return FLSTM_E_STALLED;
+        p->broken_bwd = true;
+        p->fallbacks++;
+        replan(p);
+        rc = backward_rec_once(p, T, dY, dy_dtype, d_hn, d_cn, dstate_dtype, S, dx, dx_dtype, s);
+        if (rc) return rc;
+        rc = read_status(p, s, &st);
+        if (rc) return rc;
+        if (st != 0) return FLSTM_E_STALLED;
+    }
+    rc = backward_dx(p, long(T) - 1, 0, s);
+    if (rc) return rc;
+    FL_TRY(hipEventRecord(p->tm.ev[5], s));
+    rc = backward_finish(p, x, x_dtype, dW_ih, dW_hh, db_ih, db_hh, dh0, dc0, s);
+    if (rc) return rc;
     if (p->opt_profile)
         FL_TRY(hipMemcpy(p->prof_b, p->prof.as<long long>() + 8, sizeof(p->prof_b), hipMemcpyDeviceToHost));
     p->ms_bwd[0] = elapsed(p->tm.ev[3], p->tm.ev[4]);
@@ -473,8 +539,89 @@ extern "C" int flstm_core_backward(flstm_core_plan* p, size_t T, const void* x, 
     return 0;
 }
 
+// ---- the same passes fed in ranges of steps (for callers that stream the sequence through the device)
+
+extern "C" int flstm_core_forward_begin(flstm_core_plan* p, size_t T, const void* x, flstm_dtype x_dtype,
+                                        const void* h0, const void* c0, flstm_dtype state_dtype, void* stream) {
+    if (!p) return FLSTM_E_INVALID;
+    if (!p->weights_packed || !p->bias_packed) return FLSTM_E_NOT_PACKED;
+    if (T == 0 || !x || T > (size_t(1) << 24)) return FLSTM_E_INVALID;
+    p->have_cache = false;
+    for (float& m : p->ms_fwd) m = -1.f;
+    return forward_setup(p, T, x, x_dtype, h0, c0, state_dtype, static_cast<hipStream_t>(stream));
+}
+
+extern "C" int flstm_core_forward_steps(flstm_core_plan* p, size_t t0, size_t nsteps, void* stream) {
+    if (!p || !p->fw.open || t0 + nsteps > p->fw.T) return FLSTM_E_INVALID;
+    if (nsteps == 0) return 0;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    int rc = forward_project(p, t0, nsteps, s);
+    if (rc) return rc;
+    return forward_recur(p, t0, nsteps, s);
+}
+
+extern "C" int flstm_core_forward_end(flstm_core_plan* p, void* hy, void* cy, flstm_dtype out_state_dtype,
+                                      int save_for_backward, void* stream) {
+    if (!p || !p->fw.open) return FLSTM_E_INVALID;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const Dims& d = p->d;
+    const size_t TB = p->fw.T * size_t(d.B);
+    p->fw.open = false;
+    int st = 0;
+    int rc = read_status(p, s, &st);
+    if (rc) return rc;
+    if (st != 0) {   // a persistent launch gave up: the caller repeats the pass through flstm_core_forward
+        if (p->Lf.persistent) { p->broken_fwd = true; p->fallbacks++; replan(p); }
+        return FLSTM_E_STALLED;
+    }
+    FL_TRY(unpad_from_half(p->Y.as<half_t>() + TB * d.Hp, size_t(d.Hp), size_t(d.B), d.H, hy,
+                           out_state_dtype == FLSTM_F32, s));
+    FL_TRY(unpad_from_float(p->C.as<float>() + TB * d.Hp, size_t(d.Hp), size_t(d.B), d.H, 1.f, cy,
+                            out_state_dtype == FLSTM_F32, s));
+    FL_TRY(hipStreamSynchronize(s));
+    if (save_for_backward) { p->have_cache = true; p->T_cache = p->fw.T; }
+    return 0;
+}
+
+extern "C" int flstm_core_backward_begin(flstm_core_plan* p, size_t T, const void* dY, flstm_dtype dy_dtype,
+                                         const void* d_hn, const void* d_cn, flstm_dtype dstate_dtype,
+                                         float grad_scale, void* dx, flstm_dtype dx_dtype, void* stream) {
+    if (!p || !dY || T == 0) return FLSTM_E_INVALID;
+    if (!p->have_cache || p->T_cache != T) return FLSTM_E_NO_CACHE;
+    for (float& m : p->ms_bwd) m = -1.f;
+    const float S = grad_scale > 0.f ? grad_scale : 1.f;
+    return backward_setup(p, T, dY, dy_dtype, d_hn, d_cn, dstate_dtype, S, dx, dx_dtype, static_cast<hipStream_t>(stream));
+}
+
+extern "C" int flstm_core_backward_steps(flstm_core_plan* p, size_t t_hi, size_t nsteps, void* stream) {
+    if (!p || !p->bw.open || t_hi >= p->bw.T || nsteps == 0 || nsteps > t_hi + 1) return FLSTM_E_INVALID;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const long lo = long(t_hi) - long(nsteps) + 1;
+    // the range that reaches step 0 also runs the closing product for dh0
+    int rc = backward_recur(p, long(t_hi), lo == 0 ? -1 : lo, s);
+    if (rc) return rc;
+    return backward_dx(p, long(t_hi), lo, s);
+}
+
+extern "C" int flstm_core_backward_end(flstm_core_plan* p, const void* x, flstm_dtype x_dtype, float* dW_ih,
+                                       float* dW_hh, float* db_ih, float* db_hh, float* dh0, float* dc0,
+                                       void* stream) {
+    if (!p || !p->bw.open) return FLSTM_E_INVALID;
+    if (dW_ih && !x) return FLSTM_E_INVALID;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    int st = 0;
+    int rc = read_status(p, s, &st);
+    if (rc) return rc;
+    if (st != 0) {   // the caller repeats the pass through flstm_core_backward
+        p->bw.open = false;
+        if (p->Lb.persistent) { p->broken_bwd = true; p->fallbacks++; replan(p); }
+        return FLSTM_E_STALLED;
+    }
+    return backward_finish(p, x, x_dtype, dW_ih, dW_hh, db_ih, db_hh, dh0, dc0, s);
+}
+
 extern "C" int flstm_core_cache_ptr(const flstm_core_plan* p, int which, const void** ptr, size_t* ld) {
-    if (!p || !ptr || !ld || !p->have_cache) return FLSTM_E_INVALID;
+    if (!p || !ptr || !ld || !(p->have_cache || p->fw.open)) return FLSTM_E_INVALID;
     switch (which) {
         case 0: *ptr = p->Y.p; *ld = size_t(p->d.Hp); return 0;
         case 1: *ptr = p->C.p; *ld = size_t(p->d.Hp); return 0;

@@ -52,7 +52,16 @@ __device__ __forceinline__ bool work_item(const TileOrder& o, int lin, int& tm, 
 // Epilogue shared by both kernels.  With swapped MFMA operands register r of tile (i, j) holds row
 // (i*32 + lane%32) of the wave's 128 x 64 block and column j*32 + 8*(r/4) + 4*(lane/32) + r%4: four
 // consecutive columns per group of four registers, stored as one 8-byte (fp16) or 16-byte (fp32) access.
-// bias[col .. col+3] of a full tile (col % 4 == 0), zeros when the GEMM has no bias
+// bias[col .. col+3] of a full tile (col % 4 == 0), zeros when the GEMM has no bias.  Every epilogue forms
+// fma(alpha, acc, bias) explicitly in fp32 and only then rounds to fp16 (out16 keeps the compiler from
+// merging the two into one mixed-precision instruction with a single rounding), so an element gets the
+// same bits whichever path stores its tile.
+__device__ __forceinline__ half_t out16(float alpha, float acc, float bias) {
+    float v = __builtin_fmaf(alpha, acc, bias);
+    asm volatile("" : "+v"(v));
+    return (half_t)v;
+}
+
 __device__ __forceinline__ floatx4 bias4(const GemmNT& g, int col) {
     return g.bias ? *reinterpret_cast<const floatx4*>(g.bias + col) : floatx4{0.f, 0.f, 0.f, 0.f};
 }
@@ -75,13 +84,13 @@ __device__ __forceinline__ void store_tile(const GemmNT& g, floatx16 (&acc)[4][k
                     if (c32) {
                         floatx4 v;
 #pragma unroll
-                        for (int e = 0; e < 4; ++e) v[e] = g.alpha * acc[i][j][4 * q + e] + bias4(g, colb + j * 32 + 8 * q)[e];
+                        for (int e = 0; e < 4; ++e) v[e] = __builtin_fmaf(g.alpha, acc[i][j][4 * q + e], bias4(g, colb + j * 32 + 8 * q)[e]);
                         *reinterpret_cast<floatx4*>(c32 + off) = v;
                     } else {
                         half4 v;
 #pragma unroll
                         for (int e = 0; e < 4; ++e)
-                            v[e] = (half_t)(g.alpha * acc[i][j][4 * q + e] + bias4(g, colb + j * 32 + 8 * q)[e]);
+                            v[e] = out16(g.alpha, acc[i][j][4 * q + e], bias4(g, colb + j * 32 + 8 * q)[e]);
                         *reinterpret_cast<half4*>(g.C16 + off) = v;
                     }
                 }
@@ -100,9 +109,9 @@ __device__ __forceinline__ void store_tile(const GemmNT& g, floatx16 (&acc)[4][k
                     const int col = colb + j * 32 + 8 * (r / 4) + (r % 4);
                     if (col >= g.N) continue;
                     const size_t off = size_t(r_) * g.ldc + col;
-                    const float v = g.alpha * acc[i][j][r] + (g.bias ? g.bias[col] : 0.f);
-                    if (c32) c32[off] = v;
-                    else g.C16[off] = (half_t)v;
+                    const float bv = g.bias ? g.bias[col] : 0.f;
+                    if (c32) c32[off] = __builtin_fmaf(g.alpha, acc[i][j][r], bv);
+                    else g.C16[off] = out16(g.alpha, acc[i][j][r], bv);
                 }
                 __builtin_amdgcn_sched_barrier(0);
             }
@@ -166,7 +175,7 @@ __device__ __forceinline__ void store_tile_lines(const GemmNT& g, floatx16 (&acc
             for (int q = 0; q < 4; ++q) {
                 half4 v;
 #pragma unroll
-                for (int e = 0; e < 4; ++e) v[e] = (half_t)(g.alpha * acc[i][j][4 * q + e] + bv[j][q][e]);
+                for (int e = 0; e < 4; ++e) v[e] = out16(g.alpha, acc[i][j][4 * q + e], bv[j][q][e]);
                 const int chunk = 4 * j + q;
                 *reinterpret_cast<half4*>(stage + wr * 128 + ((chunk ^ wsw) * 16) + 8 * (lane / 32)) = v;
             }

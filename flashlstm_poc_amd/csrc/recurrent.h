@@ -31,6 +31,7 @@ struct RecFwdArgs {
     unsigned* seats;     // [8] zeroed before every launch: next free workgroup slot per XCD
     int* status;         // 0 ok, 1 spin limit hit, 2 workgroup not on the expected XCD
     int B, Hp, T;
+    int t0, t1;          // steps [t0, t1) of the sequence are run by this call (state and ring carry over)
     int spin_limit;      // reloads of a fragment chunk that still shows the 'unwritten' pattern before giving up
     long long* prof;     // optional [8] cycle counters of workgroup 0 per phase (null = off)
 };
@@ -53,6 +54,7 @@ struct RecBwdArgs {
     int B, Hp, T;
     int jb_fwd;          // hidden units per slice in the packed gate order of G / dG
     float dy_scale;      // factor applied to dY on load (the loss scale, or 1 when dY is pre-scaled)
+    int t_hi, t_lo;      // steps t_hi down to t_lo are run by this call; t_lo = -1 adds the closing dh0 product
     int spin_limit;
     long long* prof;     // optional [8] cycle counters of workgroup 0 per phase (null = off)
 };
@@ -70,9 +72,9 @@ hipError_t to_exchange_layout(const half_t* in, int rows, int cols, size_t ld, h
 int rec_fwd_ks(const RecLayout& L, int Hp);
 int rec_bwd_ks(const RecLayout& L, int Hp);
 
-// Runs steps [0, T). Persistent layouts use one launch; otherwise one launch per step.
+// Runs steps [t0, t1). Persistent layouts use one launch; otherwise one launch per step.
 hipError_t launch_rec_fwd(const RecLayout& L, const RecFwdArgs& a, hipStream_t stream);
-// Runs steps T-1 .. 0 and the final dh0 product.
+// Runs steps t_hi .. t_lo (the whole pass is T-1 .. -1: all steps and the final dh0 product).
 hipError_t launch_rec_bwd(const RecLayout& L, const RecBwdArgs& a, hipStream_t stream);
 
 }  // namespace flstm_hip

@@ -278,8 +278,6 @@ template <int N> struct F32;
 template <> struct F32<2> { floatx2 v; };
 template <> struct F32<4> { floatx4 v; };
 
-__device__ __forceinline__ Pack<2> ld_pack(const half_t* p, Pack<2>*) { return Pack<2>{*reinterpret_cast<const unsigned*>(p)}; }
-__device__ __forceinline__ Pack<4> ld_pack(const half_t* p, Pack<4>*) { return Pack<4>{*reinterpret_cast<const uintx2*>(p)}; }
 __device__ __forceinline__ void st_pack(half_t* p, Pack<2> v) { *reinterpret_cast<unsigned*>(p) = v.v; }
 __device__ __forceinline__ void st_pack(half_t* p, Pack<4> v) { *reinterpret_cast<uintx2*>(p) = v.v; }
 __device__ __forceinline__ void unpack(Pack<2> v, float (&f)[2]) { unpack_h2(v.v, f[0], f[1]); }
@@ -857,10 +855,10 @@ static hipError_t run_fwd(const RecLayout& L, const RecFwdArgs& a, hipStream_t s
     if (e != hipSuccess) return e;
     const int ks_wave = rec_fwd_ks(L, a.Hp);
     if (L.persistent) {
-        hipLaunchKernelGGL(kernel, dim3(L.grid), dim3(kThreads), lds, stream, a, L, 0, a.T, ks_wave);
+        hipLaunchKernelGGL(kernel, dim3(L.grid), dim3(kThreads), lds, stream, a, L, a.t0, a.t1, ks_wave);
         return hipGetLastError();
     }
-    for (int t = 0; t < a.T; ++t) {
+    for (int t = a.t0; t < a.t1; ++t) {
         hipLaunchKernelGGL(kernel, dim3(L.grid), dim3(kThreads), lds, stream, a, L, t, t + 1, ks_wave);
         e = hipGetLastError();
         if (e != hipSuccess) return e;
@@ -869,8 +867,8 @@ static hipError_t run_fwd(const RecLayout& L, const RecFwdArgs& a, hipStream_t s
 }
 
 hipError_t launch_rec_fwd(const RecLayout& L, const RecFwdArgs& a, hipStream_t stream) {
-    if (a.T <= 0 || a.B <= 0) return hipSuccess;
-    if (a.Hp % 32 != 0 || a.Hp % L.jb != 0) return hipErrorInvalidValue;
+    if (a.T <= 0 || a.B <= 0 || a.t1 <= a.t0) return hipSuccess;
+    if (a.Hp % 32 != 0 || a.Hp % L.jb != 0 || a.t0 < 0 || a.t1 > a.T) return hipErrorInvalidValue;
     if (!L.resident) return run_fwd<8, 1, false>(L, a, stream);
     if (L.nt == 8) return run_fwd<8, 8, true>(L, a, stream);
     if (L.nt == 4) return run_fwd<4, 16, true>(L, a, stream);
@@ -886,10 +884,10 @@ static hipError_t run_bwd(const RecLayout& L, const RecBwdArgs& a, hipStream_t s
     if (e != hipSuccess) return e;
     const int ks_wave = rec_bwd_ks(L, a.Hp);
     if (L.persistent) {
-        hipLaunchKernelGGL(kernel, dim3(L.grid), dim3(kThreads), lds, stream, a, L, a.T - 1, -1, ks_wave);
+        hipLaunchKernelGGL(kernel, dim3(L.grid), dim3(kThreads), lds, stream, a, L, a.t_hi, a.t_lo, ks_wave);
         return hipGetLastError();
     }
-    for (int t = a.T - 1; t >= -1; --t) {
+    for (int t = a.t_hi; t >= a.t_lo; --t) {
         hipLaunchKernelGGL(kernel, dim3(L.grid), dim3(kThreads), lds, stream, a, L, t, t, ks_wave);
         e = hipGetLastError();
         if (e != hipSuccess) return e;
@@ -898,8 +896,8 @@ static hipError_t run_bwd(const RecLayout& L, const RecBwdArgs& a, hipStream_t s
 }
 
 hipError_t launch_rec_bwd(const RecLayout& L, const RecBwdArgs& a, hipStream_t stream) {
-    if (a.T <= 0 || a.B <= 0) return hipSuccess;
-    if (a.Hp % 32 != 0 || a.Hp % L.jb != 0) return hipErrorInvalidValue;
+    if (a.T <= 0 || a.B <= 0 || a.t_hi < a.t_lo) return hipSuccess;
+    if (a.Hp % 32 != 0 || a.Hp % L.jb != 0 || a.t_lo < -1 || a.t_hi >= a.T) return hipErrorInvalidValue;
     if (!L.resident) return run_bwd<2, 1, false, 0>(L, a, stream);
     if (L.nt == 2) return run_bwd<2, 32, true, 8>(L, a, stream);
     if (L.nt == 1) return run_bwd<1, 64, true, 24>(L, a, stream);

@@ -76,6 +76,27 @@ int flstm_core_backward(flstm_core_plan* plan, size_t seq_len,
                         float* dW_ih, float* dW_hh, float* db_ih, float* db_hh,
                         float* dh0, float* dc0, void* stream);
 
+/* The same two passes fed in ranges of time steps, for callers that stream a sequence through the device
+ * while it is being processed.  (No counterpart in the reference, which walks 32-step chunks inside
+ * flashlstm_v2/src/lstm_forward.cu:646-940 and lstm_backward.cu:897-1213; this is the hook its replacement
+ * uses to overlap host transfers with compute.)  x / dY / dx name whole-sequence device buffers; only the
+ * rows of a range have to be valid (x, dY) or are written (h rows of the state cache, dx) when the range runs.
+ * _steps calls only enqueue work.  forward ranges go from step 0 upwards and must cover [0, T) in order;
+ * backward ranges go from step T-1 downwards.  _end waits, returns FLSTM_E_STALLED if a persistent launch
+ * gave up (repeat the pass with flstm_core_forward / flstm_core_backward, which fall back to step-wise
+ * launches), and otherwise finishes the pass (final states; weight and bias gradients). */
+int flstm_core_forward_begin(flstm_core_plan* plan, size_t seq_len, const void* x, flstm_dtype x_dtype,
+                             const void* h0, const void* c0, flstm_dtype state_dtype, void* stream);
+int flstm_core_forward_steps(flstm_core_plan* plan, size_t t0, size_t nsteps, void* stream);
+int flstm_core_forward_end(flstm_core_plan* plan, void* hy, void* cy, flstm_dtype out_state_dtype,
+                           int save_for_backward, void* stream);
+int flstm_core_backward_begin(flstm_core_plan* plan, size_t seq_len, const void* dY, flstm_dtype dy_dtype,
+                              const void* d_hn, const void* d_cn, flstm_dtype dstate_dtype, float grad_scale,
+                              void* dx, flstm_dtype dx_dtype, void* stream);
+int flstm_core_backward_steps(flstm_core_plan* plan, size_t t_hi, size_t nsteps, void* stream);
+int flstm_core_backward_end(flstm_core_plan* plan, const void* x, flstm_dtype x_dtype, float* dW_ih, float* dW_hh,
+                            float* db_ih, float* db_hh, float* dh0, float* dc0, void* stream);
+
 /* Read access to what forward cached (device pointers, valid until the next forward/destroy):
  *   which = 0: h states fp16 [(T+1)*B][Hp], row t*B+b = h before step t   (ld = *ld)
  *   which = 1: c states fp32 [(T+1)*B][Hp]

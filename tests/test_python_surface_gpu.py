@@ -98,3 +98,31 @@ def test_default_states_are_zero_and_argument_checks():
         streaming_lstm(x, None, None, torch.zeros(24, 5, device="cuda"), m.weight_hh, m.bias_ih, m.bias_hh)
     with pytest.raises(ValueError, match="float32"):
         streaming_lstm(x, None, None, m.weight_ih.half(), m.weight_hh, m.bias_ih, m.bias_hh)
+
+
+def test_mfu_report_is_printed_when_the_environment_asks_for_it():
+    # FLASHLSTM_PROFILE_MFU / FLASHLSTM_MFU_PEAK_TFLOPS as in flashlstm_v2/include/mfu_profiler.hpp:21-100:
+    # one line per streaming call, labelled "forward" / "backward"
+    import os
+    import re
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    code = (
+        "import sys, torch; sys.path.insert(0, %r)\n"
+        "import flashlstm_poc_amd; flashlstm_poc_amd.add_flashlstm_to_path()\n"
+        "from flashlstm import StreamingLSTM\n"
+        "m = StreamingLSTM(8, 16)\n"
+        "x = torch.empty(5, 2, 8, dtype=torch.float16, pin_memory=True).copy_(torch.randn(5, 2, 8).half())\n"
+        "y, cache, (hy, cy) = m(x)\n"
+        "y.float().sum().backward()\n"
+        "torch.cuda.synchronize()\n" % root)
+    env = dict(os.environ, FLASHLSTM_PROFILE_MFU="1", FLASHLSTM_MFU_PEAK_TFLOPS="2500")
+    out = subprocess.run([sys.executable, "-c", code], env=env, capture_output=True, text=True, timeout=300)
+    assert out.returncode == 0, out.stderr[-2000:]
+    pat = r"\[flashlstm\]\[%s\] MFU=[0-9.]+%% HFU=[0-9.]+%% \(useful=[0-9.]+ TFLOP/s, matmul=[0-9.]+ TFLOP/s, peak=2500\.000 TFLOP/s\)"
+    assert re.search(pat % "forward", out.stdout), out.stdout
+    assert re.search(pat % "backward", out.stdout), out.stdout
+    quiet = subprocess.run([sys.executable, "-c", code], env={k: v for k, v in os.environ.items() if not k.startswith("FLASHLSTM_")},
+                           capture_output=True, text=True, timeout=300)
+    assert quiet.returncode == 0 and "[flashlstm]" not in quiet.stdout

@@ -128,6 +128,24 @@ def test_backward_without_device_cache_recomputes_the_forward_pass():
         np.testing.assert_array_equal(a[k], b[k], err_msg=k)
 
 
+@pytest.mark.parametrize("shape", [(10, 3, 12, 20), (70, 5, 16, 24), (37, 40, 64, 256)])
+def test_chunked_streaming_gives_the_whole_sequence_results(shape, monkeypatch):
+    # FLASHLSTM_V2_CHUNK_STEPS cuts the sequence into chunks that are uploaded, processed and downloaded on the three
+    # streams (counterpart of the 32-step pipeline of lstm_forward.cu:646-940); the arithmetic must not depend on it
+    p = make_problem(*shape, seed=11)
+    f, g = reference(p)
+    monkeypatch.setenv("FLASHLSTM_V2_CHUNK_STEPS", "0")
+    whole = run_v2(p, R=4)
+    compare(whole, f, g, 4)
+    for chunk in ("1", "3", "64", "1000"):
+        monkeypatch.setenv("FLASHLSTM_V2_CHUNK_STEPS", chunk)
+        for fresh in (False, True):
+            out = run_v2(p, R=4, fresh_backward=fresh)
+            for k in ("y", "hn", "cn", "ck_h", "ck_c", "dx", "dh0", "dc0", "dw_ih", "dw_hh"):
+                np.testing.assert_array_equal(out[k], whole[k], err_msg=f"chunk {chunk} {k}")
+            assert rell2(out["db"], whole["db"]) < 1e-6   # summed per launch, then over launches
+
+
 def test_null_state_gradients_and_pageable_host_memory():
     p = make_problem(6, 4, 8, 16, seed=3)
     f, g = reference(p, state_grads=False)
