@@ -26,6 +26,8 @@ WORKLOADS = {
     "config3": (1024, 256, 1024, 1024, True),
     "config4": (2048, 16, 2048, 2048, True),
 }
+# 4-layer stack (no reference counterpart: the layer loop of flashlstm_poc_amd.LstmStack): T, B, I, H, layers
+STACKS = {"config5": (4096, 128, 512, 2048, 4)}
 
 
 def make_inputs(T, B, I, H, seed=0):
@@ -96,12 +98,65 @@ def cpu_baseline(B, I, H, backward, budget_s=20.0):
                       f"{reps} repeats after 1 warm-up, {dt * 1e3:.1f} ms each; os.cpu_count()={os.cpu_count()}"}
 
 
+def bench_stack(args, device):
+    """fwd+bwd of a stack of layers with MSE on the top layer's outputs (loss scale 2^12 on the gradients)."""
+    import torch
+    from flashlstm_poc_amd import LstmStack
+    T, B, I, H, L = STACKS[args.workload]
+    g = torch.Generator(device="cuda").manual_seed(0)
+    k = 1.0 / H ** 0.5
+    u = lambda *s: (torch.rand(*s, generator=g, device="cuda") * 2 - 1) * k
+    stack = LstmStack(B, I, H, L)
+    stack.pack([(u(4 * H, I if l == 0 else H), u(4 * H, H), u(4 * H), u(4 * H)) for l in range(L)])
+    x = torch.randn(T, B, I, generator=g, device="cuda").half()
+    target = torch.randn(T, B, H, generator=g, device="cuda").half()
+
+    def step():
+        y, _, _ = stack.forward(x)
+        dy = (y.float() - target.float()).mul_(2.0 / y.numel())
+        stack.backward(dy, loss_scale=2.0 ** 12, want_dx=False)
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(args.steps):
+        step()
+    e1.record()
+    torch.cuda.synchronize()
+    ms = e0.elapsed_time(e1) / args.steps
+    flops = sum(24.0 * T * B * H * ((I if l == 0 else H) + H) for l in range(L))
+    phases = {ph: sum(layer.last_ms(ph) for layer in stack.layers) for ph in ("fwd_proj", "fwd_rec", "bwd_rec", "bwd_dx", "bwd_dw")}
+    dom = max(phases, key=phases.get)
+    dom_flops = {"fwd_proj": sum(2.0 * T * B * 4 * H * (I if l == 0 else H) for l in range(L)),
+                 "fwd_rec": L * 2.0 * T * B * 4 * H * H, "bwd_rec": L * 2.0 * T * B * 4 * H * H,
+                 "bwd_dx": sum(2.0 * T * B * 4 * H * (I if l == 0 else H) for l in range(1, L)),
+                 "bwd_dw": sum(2.0 * T * B * 4 * H * ((I if l == 0 else H) + H) for l in range(L))}[dom]
+    tf = dom_flops / (phases[dom] * 1e-3) / 1e12
+    out = {"metric": "fwd+bwd batch*timesteps/sec", "value": round(B * T / (ms * 1e-3), 1), "unit": "batch*timesteps/s",
+           "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms, 3),
+           "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+           "dtype": "fp16 storage, fp32 accumulate, fp32 cell state", "data": "synthetic",
+           "config": {"workload": f"{args.workload}: {L}-layer LSTM stack fwd+bwd, MSE on the top outputs, I={I}, H={H}, "
+                                  f"B={B}, T={T}", "T": T, "B": B, "I": I, "H": H, "layers": L},
+           "mfu": round(flops / (ms * 1e-3) / (PEAK_FP16_TFLOPS * 1e12), 4), "tflops": round(flops / (ms * 1e-3) / 1e12, 1),
+           "flops_per_step": flops, "phase_ms_all_layers": {k_: round(v, 3) for k_, v in phases.items()},
+           "roofline": {"kernel": dom + " (summed over the layers)", "bound": "mfma", "achieved": round(tf, 1),
+                        "peak": PEAK_FP16_TFLOPS, "unit": "TFLOP/s", "frac": round(tf / PEAK_FP16_TFLOPS, 4), "traffic": None},
+           "us_per_timestep": {"fwd_rec": round(phases["fwd_rec"] * 1e3 / (T * L), 3),
+                               "bwd_rec": round(phases["bwd_rec"] * 1e3 / (T * L), 3)},
+           "device": device, "cpu_baseline": None}
+    stack.close()
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=10)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--workload", default="config3", choices=sorted(WORKLOADS))
+    ap.add_argument("--workload", default="config3", choices=sorted(WORKLOADS) + sorted(STACKS))
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-parity", action="store_true")
     args = ap.parse_args()
@@ -124,6 +179,9 @@ def main():
               "derived_fp16_peak_tflops": (round(props.multi_processor_count * 4096 * clock_khz * 1e3 / 1e12, 1)
                                            if clock_khz else None),
               "peak_used_tflops": PEAK_FP16_TFLOPS, "hbm_gib": round(props.total_memory / 2 ** 30, 1)}
+    if args.workload in STACKS:
+        print(json.dumps(bench_stack(args, device)))
+        return
     T, B, I, H, backward = WORKLOADS[args.workload]
     p = make_inputs(T, B, I, H)
     core = LstmCore(B, I, H)
