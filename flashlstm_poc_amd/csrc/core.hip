@@ -236,10 +236,10 @@ int forward_setup(flstm_core_plan* p, size_t T, const void* x, flstm_dtype x_dty
     else FL_TRY(fill_zero(p->Y.p, size_t(d.B) * d.Hp * sizeof(half_t), s));
     FL_TRY(convert_pad_f32(c0, state_dtype == FLSTM_F32, size_t(d.B), d.H, 1.f, p->C.as<float>(), size_t(d.Hp), s));
     const size_t xslot = exchange_slot_halfs(d.B, d.Hp);
-    // exchange ring: slot 0 = h0 (rows past B zero), slots 1 and 2 = the 'unwritten' pattern
-    FL_TRY(p->xch_f.reserve(3 * xslot * sizeof(half_t)));
+    // exchange ring: slot 0 = h0 (rows past B zero), slots 1 to 3 = the 'unwritten' pattern
+    FL_TRY(p->xch_f.reserve(4 * xslot * sizeof(half_t)));
     FL_TRY(fill_zero(p->xch_f.p, xslot * sizeof(half_t), s));
-    FL_TRY(fill_words(p->xch_f.as<half_t>() + xslot, 2 * xslot * sizeof(half_t), 0xFFFFFFFFu, s));
+    FL_TRY(fill_words(p->xch_f.as<half_t>() + xslot, 3 * xslot * sizeof(half_t), 0xFFFFFFFFu, s));
     FL_TRY(to_exchange_layout(p->Y.as<half_t>(), d.B, d.Hp, size_t(d.Hp), p->xch_f.as<half_t>(), s));
     if (p->opt_profile) FL_TRY(fill_zero(p->prof.p, 8 * sizeof(long long), s));
     return 0;
@@ -381,8 +381,8 @@ int backward_setup(flstm_core_plan* p, size_t T, const void* dY, flstm_dtype dy_
     FL_TRY(p->dG.reserve(TB * 4 * d.Hp * sizeof(half_t)));
     FL_TRY(p->db_part.reserve(size_t(p->Lb.ng) * 4 * d.Hp * sizeof(float)));
     const size_t xslot = exchange_slot_halfs(d.B, 4 * d.Hp);
-    FL_TRY(p->xch_b.reserve(3 * xslot * sizeof(half_t)));
-    FL_TRY(fill_words(p->xch_b.p, 3 * xslot * sizeof(half_t), 0xFFFFFFFFu, s));
+    FL_TRY(p->xch_b.reserve(4 * xslot * sizeof(half_t)));
+    FL_TRY(fill_words(p->xch_b.p, 4 * xslot * sizeof(half_t), 0xFFFFFFFFu, s));
     FL_TRY(convert_pad_f32(d_hn, dstate_dtype == FLSTM_F32, size_t(d.B), d.H, S, p->dHn.as<float>(), size_t(d.Hp), s));
     FL_TRY(convert_pad_f32(d_cn, dstate_dtype == FLSTM_F32, size_t(d.B), d.H, S, p->dC.as<float>(), size_t(d.Hp), s));
     FL_TRY(fill_zero(p->db_part.p, size_t(p->Lb.ng) * 4 * d.Hp * sizeof(float), s));

@@ -22,9 +22,9 @@ struct RecLayout {
 struct RecFwdArgs {
     const half8* wfrag;  // [nh][4 waves][ks][nt][64 lanes] MFMA B-fragments of W_hh (packed gate order)
     half_t* Y;           // [(T+1)*B][Hp]; rows [0,B) = h0, rows [(t+1)B, (t+2)B) = h_t (row-major, for later kernels)
-    half_t* X;           // exchange ring, 3 slots of x_slot halfs, fragment-major; step t reads slot t%3 (h_{t-1}),
-                         // writes slot (t+1)%3; before a launch slot 0 holds h0 (padding rows zero) and the
-                         // other two hold the 0xFFFF 'unwritten' pattern
+    half_t* X;           // exchange ring, 4 slots of x_slot halfs, fragment-major; step t reads slot t%4 (h_{t-1}),
+                         // writes slot (t+1)%4; before step 0 slot 0 holds h0 (padding rows zero) and the
+                         // other three hold the 0xFFFF 'unwritten' pattern
     size_t x_slot;
     half_t* G;           // [T*B][4Hp] packed gate order; in: x-projection + bias, out: activated i,f,g,o
     float* C;            // [(T+1)*B][Hp]; rows [0,B) = c0, rows [(t+1)B, ..) = c_t
@@ -42,8 +42,8 @@ struct RecBwdArgs {
     const float* C;      // cell states [(T+1)*B][Hp]
     const half_t* dY;    // [T*B][Hp] upstream gradient
     half_t* dG;          // [T*B][4Hp] pre-activation gradients (scaled), row-major, for the GEMMs
-    half_t* X;           // exchange ring, 3 slots of x_slot halfs, fragment-major; step t writes slot t%3 (dG_t);
-                         // before a launch all three hold the 0xFFFF 'unwritten' pattern
+    half_t* X;           // exchange ring, 4 slots of x_slot halfs, fragment-major; step t writes slot t%4 (dG_t);
+                         // before the first step all four hold the 0xFFFF 'unwritten' pattern
     size_t x_slot;
     float* dHn;          // [B][Hp] scaled gradient wrt final h (zeros when absent)
     float* dC;           // [B][Hp] running scaled dc; in: gradient wrt final c, out: dc0

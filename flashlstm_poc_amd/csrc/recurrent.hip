@@ -19,12 +19,15 @@
 //    served by that XCD's L2); no L2 write-back or invalidate is ever issued.  Groups that span XCDs
 //    store the exchanged values with device-scope atomic stores instead.
 //    There are no flags and no barrier between workgroups: the data validates itself.  The
-//    exchange ring has three slots; while a workgroup writes step t into one slot it refills its own
-//    region of the slot that step t+1 will use with a pattern no fp16 result can produce (0xFFFF pairs,
+//    exchange ring has four slots; while a workgroup writes step t into one slot it refills its own
+//    region of the slot that step t+2 will use with a pattern no fp16 result can produce (0xFFFF pairs,
 //    a NaN payload the arithmetic never generates).  A consumer simply loads its MFMA fragments and,
-//    as long as a fragment still shows the pattern, loads it again.  Compared with a flag per
-//    workgroup this takes two L2 round trips (store acknowledgement, flag poll) off the path between
-//    one step and the next.  Every retry loop is bounded and reports through `status`.
+//    as long as a fragment still shows the pattern, loads it again.  The refill of step t is
+//    acknowledged before the values of step t+1 are stored (every step drains its memory operations
+//    once, where it picks up its prefetched operands), so whoever has seen a producer's step t+1 sees,
+//    in the slot of step t+2, the pattern or the new values, never what the slot held four steps ago.
+//    No wait for a store acknowledgement and no flag poll sits on the path between one step and the next.
+//    Every retry loop is bounded and reports through `status`.
 //  * Fallback.  The same kernels launched once per step (no waits, kernel boundaries order
 //    memory) serve shapes whose weights do not fit on chip, and are the safe path after a failed
 //    persistent launch.
@@ -321,18 +324,29 @@ __device__ __forceinline__ void st_f32(float* p, const float (&f)[2]) { *reinter
 __device__ __forceinline__ void st_f32(float* p, const float (&f)[4]) {
     *reinterpret_cast<float4*>(p) = float4{f[0], f[1], f[2], f[3]};
 }
+// The same as one hand-issued load that has arrived when the call returns.  The compiler does not see
+// a pending load, so it puts no wait of its own where the value is used: such a wait would sit behind
+// the stores issued in between (the ring marks) and stall the step until they are acknowledged.
+__device__ __forceinline__ void ld_f32_now(const float* p, float (&f)[2]) {
+    floatx2 v;
+    asm volatile("global_load_dwordx2 %0, %1, off\n\ts_waitcnt vmcnt(0)" : "=&v"(v) : "v"(p) : "memory");
+    f[0] = v.x; f[1] = v.y;
+}
+__device__ __forceinline__ void ld_f32_now(const float* p, float (&f)[4]) {
+    floatx4 v;
+    asm volatile("global_load_dwordx4 %0, %1, off\n\ts_waitcnt vmcnt(0)" : "=&v"(v) : "v"(p) : "memory");
+    f[0] = v.x; f[1] = v.y; f[2] = v.z; f[3] = v.w;
+}
 // the same, past the L1 (the value was written by this thread through a plain store earlier on)
 __device__ __forceinline__ void ld_f32_coherent(const float* p, float (&f)[2]) {
-    union { u64 q; float v[2]; } u;
-    u.q = __hip_atomic_load(reinterpret_cast<const u64*>(p), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    f[0] = u.v[0]; f[1] = u.v[1];
+    floatx2 v;
+    asm volatile("global_load_dwordx2 %0, %1, off sc1\n\ts_waitcnt vmcnt(0)" : "=&v"(v) : "v"(p) : "memory");
+    f[0] = v.x; f[1] = v.y;
 }
 __device__ __forceinline__ void ld_f32_coherent(const float* p, float (&f)[4]) {
-    union { u64 q[2]; float v[4]; } u;
-    u.q[0] = __hip_atomic_load(reinterpret_cast<const u64*>(p), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    u.q[1] = __hip_atomic_load(reinterpret_cast<const u64*>(p) + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-#pragma unroll
-    for (int i = 0; i < 4; ++i) f[i] = u.v[i];
+    floatx4 v;
+    asm volatile("global_load_dwordx4 %0, %1, off sc1\n\ts_waitcnt vmcnt(0)" : "=&v"(v) : "v"(p) : "memory");
+    f[0] = v.x; f[1] = v.y; f[2] = v.z; f[3] = v.w;
 }
 
 // Thread -> (row, group): the 8 groups of a row go to consecutive lanes, and the rows are taken in the
@@ -365,18 +379,18 @@ __device__ __forceinline__ void to_floats(const F32<4>& r, float (&f)[4]) {
 }
 
 // Cycle counters of workgroup 0 per phase (only when the host passes a buffer): product (including the
-// wait for the operand), partial exchange, pointwise, cache stores + prefetch.  Thread 0 accumulates in
+// wait for the operand), partial exchange, pointwise, cache stores, wait for the prefetched operands.  Thread 0 accumulates in
 // LDS and writes the totals once at the end, so the measurement adds no memory round trips to a step.
 struct PhaseClock {
     long long* out;
     long long last;
     __device__ __forceinline__ long long* acc() {
-        __shared__ long long lds_acc[4];
+        __shared__ long long lds_acc[5];
         return lds_acc;
     }
     __device__ __forceinline__ void start() {
         if (out && threadIdx.x == 0) {
-            for (int i = 0; i < 4; ++i) acc()[i] = 0;
+            for (int i = 0; i < 5; ++i) acc()[i] = 0;
             last = wall_clock64();
         }
     }
@@ -389,7 +403,7 @@ struct PhaseClock {
     }
     __device__ __forceinline__ void flush() {
         if (out && threadIdx.x == 0)
-            for (int i = 0; i < 4; ++i) out[i] += acc()[i];
+            for (int i = 0; i < 5; ++i) out[i] += acc()[i];
     }
 };
 
@@ -450,7 +464,7 @@ __global__ __launch_bounds__(kThreads) void rec_fwd_kernel(RecFwdArgs p, RecLayo
     };
     if (c_in_regs) {
         const int b = g * kRows + pr;
-        if (b < p.B) ld_f32(p.C + (size_t(t_begin) * p.B + b) * p.Hp + j, creg);
+        if (b < p.B) ld_f32_now(p.C + (size_t(t_begin) * p.B + b) * p.Hp + j, creg);
     }
     __syncthreads();
     clk.start();
@@ -459,9 +473,9 @@ __global__ __launch_bounds__(kThreads) void rec_fwd_kernel(RecFwdArgs p, RecLayo
         for (int rb = g; rb < L.nrb; rb += L.ng, ++item) {
             const int row0 = rb * kRows;
             float* part = part_all + size_t(item & 1) * 4 * kRows * PLD;
-            const half_t* xin = p.X + size_t(t % 3) * p.x_slot;          // h_{t-1}, fragment-major
-            half_t* xout = p.X + size_t((t + 1) % 3) * p.x_slot;         // h_t
-            half_t* xnext = p.X + size_t((t + 2) % 3) * p.x_slot;        // will take h_{t+1}: marked unwritten
+            const half_t* xin = p.X + size_t(t & 3) * p.x_slot;          // h_{t-1}, fragment-major
+            half_t* xout = p.X + size_t((t + 1) & 3) * p.x_slot;         // h_t
+            half_t* xnext = p.X + size_t((t + 3) & 3) * p.x_slot;        // will take h_{t+2}: marked unwritten
             const half_t* a0 = xin + size_t(2 * rb) * nks_total * 512 + lane * 8;
             const half_t* a1 = a0 + size_t(nks_total) * 512;
             floatx4 acc[2][NT];
@@ -478,11 +492,12 @@ __global__ __launch_bounds__(kThreads) void rec_fwd_kernel(RecFwdArgs p, RecLayo
             clk.lap(1);
 
             // Every peer of this group has delivered h_{t-1}, so all of them are done reading h_{t-2}:
-            // its slot can be marked for reuse.  The mark is acknowledged long before the wait that
-            // precedes the h_t store below, so whoever sees this step's h_t also sees the mark.
+            // its slot can be marked for reuse (it takes h_{t+2}).  The wait below also drains the mark
+            // of the previous step, so that mark is in place before this step's h_t goes out.
             wait_all_vm();   // the x-projection of this step, issued during the product
 #pragma unroll
             for (int gt = 0; gt < 4; ++gt) settle(xp[gt].v);
+            clk.lap(4);
             const int b = row0 + pr;
             const unsigned xoff = unsigned(xch_offset(b, j, nks_total));   // 32 bits: a slot is far below 4G halfs
             store_xch(xnext + xoff, pack_fill(kUnwritten, (PackT*)nullptr), device_scope);
@@ -526,8 +541,7 @@ __global__ __launch_bounds__(kThreads) void rec_fwd_kernel(RecFwdArgs p, RecLayo
 #pragma unroll
                 for (int gt = 0; gt < 4; ++gt) act[gt] = pack(a4[gt]);
             }
-            // the exchanged value goes out first, after the mark above has been acknowledged
-            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+            // the exchanged value goes out first
             store_xch(xout + xoff, hnew, device_scope);
             clk.lap(2);
             // caches for the backward pass: off the critical path
@@ -602,7 +616,7 @@ __global__ __launch_bounds__(kThreads) void rec_bwd_kernel(RecBwdArgs p, RecLayo
     float dcreg[UPT] = {};
     if (dc_in_regs) {
         const int b = g * kRows + pr;
-        if (b < p.B) ld_f32(p.dC + size_t(b) * p.Hp + j, dcreg);
+        if (b < p.B) ld_f32_now(p.dC + size_t(b) * p.Hp + j, dcreg);
     }
     // prefetched per work item: activated gates, c_{t-1}, c_t, dY_t
     PackT pg[4], pdy;
@@ -626,10 +640,10 @@ __global__ __launch_bounds__(kThreads) void rec_bwd_kernel(RecBwdArgs p, RecLayo
         for (int rb = g; rb < L.nrb; rb += L.ng, ++item) {
             const int row0 = rb * kRows;
             float* part = part_all + size_t(item & 1) * 4 * kRows * PLD;
-            // ring slot of step u is (u + 3) % 3: this step reads dG_{t+1}, writes dG_t and marks the
-            // slot of dG_{t-1} unwritten
+            // ring slot of step u is (u + 8) & 3: this step reads dG_{t+1}, writes dG_t and marks the
+            // slot of dG_{t-2} unwritten
             if (from_product) {
-                const half_t* xin = p.X + size_t((t + 4) % 3) * p.x_slot;   // dG_{t+1}, fragment-major
+                const half_t* xin = p.X + size_t((t + 9) & 3) * p.x_slot;   // dG_{t+1}, fragment-major
                 const half_t* a0 = xin + size_t(2 * rb) * nks_total * 512 + lane * 8;
                 const half_t* a1 = a0 + size_t(nks_total) * 512;
                 floatx4 acc[2][NT];
@@ -653,15 +667,17 @@ __global__ __launch_bounds__(kThreads) void rec_bwd_kernel(RecBwdArgs p, RecLayo
             settle(pdy.v);
             settle(pcp_r.v);
             settle(pcc_r.v);
+            clk.lap(4);
             const int b = row0 + pr;
             const bool live = b < p.B;
             const size_t sidx = size_t(b) * p.Hp + j;
-            half_t* xout = p.X + size_t((t + 3) % 3) * p.x_slot;    // dG_t for the peers
-            half_t* xnext = p.X + size_t((t + 2) % 3) * p.x_slot;   // will take dG_{t-1}
+            half_t* xout = p.X + size_t((t + 8) & 3) * p.x_slot;    // dG_t for the peers
+            half_t* xnext = p.X + size_t((t + 6) & 3) * p.x_slot;   // will take dG_{t-2}
             unsigned xoff[4];   // 32 bits: a slot is far below 4G halfs
             PackT dgnew[4];
             if (t >= 0) {
                 // every peer has delivered dG_{t+1}, so all of them are done reading dG_{t+2}: mark its slot
+                // (the wait above has drained the marks of the previous step)
 #pragma unroll
                 for (int gt = 0; gt < 4; ++gt) {
                     xoff[gt] = unsigned(xch_offset(b, int(pq) + gt * JF, nks_total));
@@ -685,7 +701,7 @@ __global__ __launch_bounds__(kThreads) void rec_bwd_kernel(RecBwdArgs p, RecLayo
                         for (int u = 0; u < UPT; ++u) dh[u] += v[u];
                     }
                 } else {
-                    ld_f32(p.dHn + sidx, dh);
+                    ld_f32_now(p.dHn + sidx, dh);
                 }
                 if (t < 0) {  // closing pass: gradient wrt h0; dc0 is the running dc
                     st_f32(p.dH0 + sidx, dh);
@@ -728,8 +744,7 @@ __global__ __launch_bounds__(kThreads) void rec_bwd_kernel(RecBwdArgs p, RecLayo
                 }
             }
             if (t >= 0) {
-                // the exchanged values go out first, after the marks above have been acknowledged
-                asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+                // the exchanged values go out first
 #pragma unroll
                 for (int gt = 0; gt < 4; ++gt) store_xch(xout + xoff[gt], dgnew[gt], device_scope);
             }
