@@ -172,7 +172,9 @@ def main():
         sys.exit(1)
     torch.cuda.set_device(0)
     props = torch.cuda.get_device_properties(0)
-    clock_khz = getattr(props, "clock_rate", None)
+    probe = LstmCore(1, 8, 8)   # the library reads the engine clock from the HIP runtime
+    clock_khz = probe.info("clock_khz") or getattr(props, "clock_rate", None)
+    probe.close()
     device = {"name": props.name, "compute_units": props.multi_processor_count,
               "max_engine_clock_mhz": (clock_khz / 1e3) if clock_khz else None,
               # 4096 fp16 MFMA FLOP per clock and CU (CDNA4, dense)
@@ -222,8 +224,8 @@ def main():
     # HBM-side traffic per launch at config3 from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (x2.0 / x1.0 after
     # calibration against the fp16 output copy of the same run); see profiles/*_hbm_traffic.md
     GiB = float(1 << 30)
-    traffic_config3 = {"fwd_proj": (3.01 + 1.25) * GiB, "bwd_dx": (3.01 + 1.25) * GiB, "fwd_rec": (2.07 + 3.50) * GiB,
-                       "bwd_rec": (3.57 + 2.75) * GiB, "bwd_dw": 2 * (3.04 + 0.25) * GiB}
+    traffic_config3 = {"fwd_proj": (3.01 + 1.25) * GiB, "bwd_dx": (3.01 + 1.25) * GiB, "fwd_rec": (2.07 + 3.55) * GiB,
+                       "bwd_rec": (3.57 + 4.39) * GiB, "bwd_dw": 2 * (3.06 + 0.25) * GiB}
     kernels = []
     for k in phases:
         tf = kflops[k] / (phase_ms[k] * 1e-3) / 1e12 if phase_ms[k] > 0 else 0.0
@@ -257,6 +259,19 @@ def main():
         "us_per_timestep": {"fwd_rec": round(phase_ms["fwd_rec"] * 1e3 / T, 3),
                             **({"bwd_rec": round(phase_ms["bwd_rec"] * 1e3 / T, 3)} if backward else {})},
     }
+    # What the recurrence moves between workgroups each step: every workgroup (32 batch rows x one slice of hidden
+    # units) fetches the whole h_{t-1} (forward) or dG_{t+1} (backward) of its rows from the L2, and passes its
+    # fp32 partial sums (4 waves, written once and read once) through LDS.
+    Hp, rows = core.info("hidden_padded"), 32 * ((B + 31) // 32)
+    xch = {}
+    for d, k_cols, gate_cols in (("fwd", Hp, 4), ("bwd", 4 * Hp, 1)) if backward else (("fwd", Hp, 4),):
+        us = phase_ms[d + "_rec"] * 1e3 / T
+        slices = Hp // core.info("slice_" + d)
+        l2_bytes = rows * slices * k_cols * 2
+        lds_bytes = 2 * 4 * rows * slices * core.info("slice_" + d) * gate_cols * 4
+        xch[d] = {"l2_fetch_bytes_per_step": l2_bytes, "l2_fetch_gb_per_s": round(l2_bytes / us / 1e3, 1),
+                  "lds_bytes_per_step": lds_bytes, "lds_gb_per_s": round(lds_bytes / us / 1e3, 1)}
+    out["exchange_per_step"] = xch
     core.close()
     if not args.no_parity:
         out["parity"] = parity_check(B, I, H)

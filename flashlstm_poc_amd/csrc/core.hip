@@ -51,6 +51,7 @@ struct PhaseTimer {
 
 struct flstm_core_plan {
     int num_cus = 0;
+    int clock_khz = 0;   // maximum engine clock the runtime reports
     Dims d{};
     RecLayout Lf{}, Lb{};
     int ks_f = 0, ks_b = 0;
@@ -120,6 +121,8 @@ extern "C" int flstm_core_create(size_t batch, size_t input_size, size_t hidden_
     int dev = 0;
     hipError_t e = hipGetDevice(&dev);
     if (e == hipSuccess) e = hipDeviceGetAttribute(&p->num_cus, hipDeviceAttributeMultiprocessorCount, dev);
+    if (e == hipSuccess && hipDeviceGetAttribute(&p->clock_khz, hipDeviceAttributeClockRate, dev) != hipSuccess)
+        p->clock_khz = 0;
     if (e != hipSuccess) { delete p; return int(e); }
     p->d.B = int(batch);
     p->d.I = int(input_size);
@@ -175,10 +178,13 @@ extern "C" long flstm_core_get_info(const flstm_core_plan* p, const char* name) 
     if (!strcmp(name, "xcd_local_bwd")) return p->Lb.xcd_local;
     if (!strcmp(name, "resident_fwd")) return p->Lf.resident;
     if (!strcmp(name, "resident_bwd")) return p->Lb.resident;
+    if (!strcmp(name, "slice_fwd")) return p->Lf.jb;
+    if (!strcmp(name, "slice_bwd")) return p->Lb.jb;
     if (!strcmp(name, "groups_fwd")) return p->Lf.ng;
     if (!strcmp(name, "groups_bwd")) return p->Lb.ng;
     if (!strcmp(name, "fallbacks")) return p->fallbacks;
     if (!strcmp(name, "num_cus")) return p->num_cus;
+    if (!strcmp(name, "clock_khz")) return p->clock_khz;
     if (!strcmp(name, "hidden_padded")) return p->d.Hp;
     if (!strcmp(name, "input_padded")) return p->d.Ip;
     if (!strcmp(name, "gate_slice")) return p->d.JF;

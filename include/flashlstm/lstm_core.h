@@ -45,7 +45,9 @@ int flstm_core_destroy(flstm_core_plan* plan);
  * the weight-gradient GEMM, 0 = automatic). */
 int flstm_core_set_option(flstm_core_plan* plan, const char* name, long value);
 /* Reads back facts about the plan: "persistent_fwd", "persistent_bwd", "xcd_local_fwd",
- * "xcd_local_bwd", "fallbacks" (persistent launches that had to be redone step-wise). */
+ * "xcd_local_bwd", "fallbacks" (persistent launches that had to be redone step-wise), "slice_fwd",
+ * "slice_bwd" (hidden units per workgroup of the recurrence kernels), "hidden_padded", "num_cus" and
+ * "clock_khz" (compute units and maximum engine clock of the plan's device). */
 long flstm_core_get_info(const flstm_core_plan* plan, const char* name);
 
 /* fp32 PyTorch-layout weights -> fp16 MFMA operand layouts held by the plan. */
