@@ -161,8 +161,12 @@ class LstmCore:
         return y, hy, cy
 
     def backward(self, x, dy, d_hn=None, d_cn=None, *, grad_scale: float = 1.0, dx_dtype=None,
-                 want_dx: bool = True):
-        """Returns (dx, dW_ih, dW_hh, db, dh0, dc0); db is the gradient of both bias vectors."""
+                 want_dx: bool = True, accumulate_into=None):
+        """Returns (dx, dW_ih, dW_hh, db, dh0, dc0); db is the gradient of both bias vectors.
+
+        accumulate_into=(dW_ih, dW_hh, db): add this call's parameter gradients to these fp32 tensors (and return
+        them) instead of writing fresh ones -- a sequence run as consecutive segments, last segment first, with
+        each call's dh0 / dc0 passed to the next one as d_hn / d_cn."""
         import torch
         x = x.contiguous()
         dy = dy.contiguous()
@@ -179,11 +183,18 @@ class LstmCore:
             d_cn = d_cn.contiguous(); dst_code = _dtype_code(d_cn)
         dx_dtype = dx_dtype or x.dtype
         dx = torch.empty_like(x, dtype=dx_dtype) if want_dx else None
-        dW_ih = torch.empty((4 * self.H, self.I), device=dev, dtype=torch.float32)
-        dW_hh = torch.empty((4 * self.H, self.H), device=dev, dtype=torch.float32)
-        db = torch.empty((4 * self.H,), device=dev, dtype=torch.float32)
+        if accumulate_into is not None:
+            dW_ih, dW_hh, db = accumulate_into
+            for t, shape in ((dW_ih, (4 * self.H, self.I)), (dW_hh, (4 * self.H, self.H)), (db, (4 * self.H,))):
+                if t.dtype != torch.float32 or not t.is_cuda or not t.is_contiguous() or tuple(t.shape) != shape:
+                    raise ValueError(f"accumulate_into tensors must be contiguous CUDA float32 of shape {shape}")
+        else:
+            dW_ih = torch.empty((4 * self.H, self.I), device=dev, dtype=torch.float32)
+            dW_hh = torch.empty((4 * self.H, self.H), device=dev, dtype=torch.float32)
+            db = torch.empty((4 * self.H,), device=dev, dtype=torch.float32)
         dh0 = torch.empty((self.B, self.H), device=dev, dtype=torch.float32)
         dc0 = torch.empty_like(dh0)
+        self.set_option("accumulate_grads", 1 if accumulate_into is not None else 0)
         rc = self.lib.flstm_core_backward(self._h, T, x.data_ptr(), _dtype_code(x), dy.data_ptr(), _dtype_code(dy),
                                           _ptr(d_hn), _ptr(d_cn), dst_code, float(grad_scale), _ptr(dx),
                                           _dtype_code(dx) if dx is not None else F16, dW_ih.data_ptr(),

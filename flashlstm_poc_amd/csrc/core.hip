@@ -56,7 +56,7 @@ struct flstm_core_plan {
     RecLayout Lf{}, Lb{};
     int ks_f = 0, ks_b = 0;
     // options
-    int opt_stepwise = 0, opt_proj_chunk = 0, opt_spin_limit = 1 << 22, opt_dw_splits = 0;
+    int opt_stepwise = 0, opt_proj_chunk = 0, opt_spin_limit = 1 << 22, opt_dw_splits = 0, opt_accumulate = 0;
     bool broken_fwd = false, broken_bwd = false;  // persistent launch failed once: stay step-wise
     long fallbacks = 0;
     // weights
@@ -167,6 +167,7 @@ extern "C" int flstm_core_set_option(flstm_core_plan* p, const char* name, long 
         return 0;
     }
     if (!strcmp(name, "dw_splits")) { if (value < 0) return FLSTM_E_INVALID; p->opt_dw_splits = int(value); return 0; }
+    if (!strcmp(name, "accumulate_grads")) { p->opt_accumulate = value != 0; return 0; }
     return FLSTM_E_INVALID;
 }
 
@@ -488,10 +489,11 @@ int backward_finish(flstm_core_plan* p, const void* x, flstm_dtype x_dtype, floa
         g.C16 = nullptr; g.C32 = p->dw_part.as<float>(); g.ldc = size_t(ncols);
         g.alpha = 1.f; g.splits = splits; g.split_stride = per;
         FL_TRY(launch_gemm_tn(g, s));
-        FL_TRY(reduce_dw(d, p->dw_part.as<float>(), splits, ncols, out_cols, invS, dst, s));
+        FL_TRY(reduce_dw(d, p->dw_part.as<float>(), splits, ncols, out_cols, invS, p->opt_accumulate != 0, dst, s));
     }
     FL_TRY(hipEventRecord(p->tm.ev[6], s));
-    if (db_ih || db_hh) FL_TRY(reduce_db(d, p->db_part.as<float>(), p->Lb.ng, invS, db_ih, db_hh, s));
+    if (db_ih || db_hh)
+        FL_TRY(reduce_db(d, p->db_part.as<float>(), p->Lb.ng, invS, p->opt_accumulate != 0, db_ih, db_hh, s));
     FL_TRY(unpad_from_float(p->dH0.as<float>(), size_t(d.Hp), size_t(d.B), d.H, invS, dh0, 1, s));
     FL_TRY(unpad_from_float(p->dC.as<float>(), size_t(d.Hp), size_t(d.B), d.H, invS, dc0, 1, s));
     FL_TRY(hipEventRecord(p->tm.ev[7], s));

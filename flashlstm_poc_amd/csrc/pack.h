@@ -47,13 +47,13 @@ hipError_t transpose_pad(const void* in, int in_f32, size_t rows, int cols, size
                          int cols_out, size_t ld_out, hipStream_t s);
 
 // Sums split-K partials [splits][4Hp][ncols] (packed gate rows) into dst [4H][out_cols] (PyTorch row
-// order, the first out_cols columns), times `scale`.  Replaces the beta=1 accumulation of
-// flashlstm_v2/src/lstm_backward.cu:1112-1142.
+// order, the first out_cols columns), times `scale`; `accumulate` adds to dst instead of overwriting it (the
+// beta=1 accumulation over chunks of flashlstm_v2/src/lstm_backward.cu:1112-1142).
 hipError_t reduce_dw(const Dims& d, const float* partial, int splits, int ncols, int out_cols, float scale,
-                     float* dst, hipStream_t s);
+                     bool accumulate, float* dst, hipStream_t s);
 // db_part [ng][4Hp] packed -> db_ih == db_hh (4H), times scale (flashlstm_v2/src/lstm_backward.cu:1218-1231).
-hipError_t reduce_db(const Dims& d, const float* db_part, int ng, float scale, float* db_ih, float* db_hh,
-                     hipStream_t s);
+hipError_t reduce_db(const Dims& d, const float* db_part, int ng, float scale, bool accumulate, float* db_ih,
+                     float* db_hh, hipStream_t s);
 
 hipError_t fill_zero(void* p, size_t bytes, hipStream_t s);
 // Fills a buffer (multiple of 4 bytes) with one 32-bit pattern; a kernel, so it may be captured in a graph.

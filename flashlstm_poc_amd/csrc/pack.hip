@@ -145,7 +145,7 @@ __global__ void transpose_pad_kernel(const TIn* __restrict__ in, size_t rows, in
 
 // partial [splits][4Hp][ncols] with packed gate rows -> dst [4H][out_cols] in PyTorch row order
 __global__ void reduce_dw_kernel(Dims d, const float* __restrict__ partial, int splits, int ncols, int out_cols,
-                                 float scale, float* __restrict__ dst) {
+                                 float scale, int accumulate, float* __restrict__ dst) {
     const size_t idx = size_t(blockIdx.x) * kT + threadIdx.x;
     const size_t per = size_t(4) * d.Hp * ncols;
     if (idx >= per) return;
@@ -154,10 +154,11 @@ __global__ void reduce_dw_kernel(Dims d, const float* __restrict__ partial, int 
     if (row < 0 || n >= out_cols) return;
     float s = 0.f;
     for (int z = 0; z < splits; ++z) s += partial[size_t(z) * per + idx];
-    dst[size_t(row) * out_cols + n] = scale * s;
+    float* out = dst + size_t(row) * out_cols + n;
+    *out = accumulate ? *out + scale * s : scale * s;
 }
 
-__global__ void reduce_db_kernel(Dims d, const float* __restrict__ db_part, int ng, float scale,
+__global__ void reduce_db_kernel(Dims d, const float* __restrict__ db_part, int ng, float scale, int accumulate,
                                  float* __restrict__ db_ih, float* __restrict__ db_hh) {
     const int q = blockIdx.x * kT + threadIdx.x;
     if (q >= 4 * d.Hp) return;
@@ -166,8 +167,8 @@ __global__ void reduce_db_kernel(Dims d, const float* __restrict__ db_part, int 
     float s = 0.f;
     for (int g = 0; g < ng; ++g) s += db_part[size_t(g) * 4 * d.Hp + q];
     s *= scale;
-    if (db_ih) db_ih[row] = s;
-    if (db_hh) db_hh[row] = s;
+    if (db_ih) db_ih[row] = accumulate ? db_ih[row] + s : s;
+    if (db_hh && db_hh != db_ih) db_hh[row] = accumulate ? db_hh[row] + s : s;
 }
 
 // flat 16-byte copy (both ends 16-byte aligned, n16 chunks)
@@ -288,18 +289,18 @@ hipError_t transpose_pad(const void* in, int in_f32, size_t rows, int cols, size
 }
 
 hipError_t reduce_dw(const Dims& d, const float* partial, int splits, int ncols, int out_cols, float scale,
-                     float* dst, hipStream_t s) {
+                     bool accumulate, float* dst, hipStream_t s) {
     if (dst == nullptr) return hipSuccess;
     const size_t per = size_t(4) * d.Hp * ncols;
     hipLaunchKernelGGL(reduce_dw_kernel, dim3(grid_for(per)), dim3(kT), 0, s, d, partial, splits, ncols, out_cols,
-                       scale, dst);
+                       scale, int(accumulate), dst);
     return hipGetLastError();
 }
 
-hipError_t reduce_db(const Dims& d, const float* db_part, int ng, float scale, float* db_ih, float* db_hh,
-                     hipStream_t s) {
+hipError_t reduce_db(const Dims& d, const float* db_part, int ng, float scale, bool accumulate, float* db_ih,
+                     float* db_hh, hipStream_t s) {
     hipLaunchKernelGGL(reduce_db_kernel, dim3(grid_for(size_t(4) * d.Hp)), dim3(kT), 0, s, d, db_part, ng,
-                       scale, db_ih, db_hh);
+                       scale, int(accumulate), db_ih, db_hh);
     return hipGetLastError();
 }
 

@@ -42,7 +42,9 @@ int flstm_core_destroy(flstm_core_plan* plan);
 /* Options: "stepwise" (1 = one launch per time step instead of the persistent kernels),
  * "proj_chunk" (time steps per input-projection GEMM, <=0 = whole sequence; results do not depend
  * on it), "spin_limit" (polls before a waiting workgroup gives up), "dw_splits" (split-K slices of
- * the weight-gradient GEMM, 0 = automatic). */
+ * the weight-gradient GEMM, 0 = automatic), "accumulate_grads" (1 = the backward pass adds dW_ih, dW_hh, db_ih
+ * and db_hh to what the caller's buffers hold instead of overwriting them: a sequence processed as several
+ * consecutive segments, last segment first, each segment's dh0 / dc0 fed to the next call as d_hn / d_cn). */
 int flstm_core_set_option(flstm_core_plan* plan, const char* name, long value);
 /* Reads back facts about the plan: "persistent_fwd", "persistent_bwd", "xcd_local_fwd",
  * "xcd_local_bwd", "fallbacks" (persistent launches that had to be redone step-wise), "slice_fwd",

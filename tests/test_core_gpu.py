@@ -211,6 +211,47 @@ def test_gate_cache_and_state_arrays_hold_what_the_oracle_computes():
     core.close()
 
 
+@pytest.mark.parametrize("shape,cuts", [((23, 5, 12, 20), (7, 15)), ((96, 40, 64, 256), (32, 64)), ((40, 64, 128, 1024), (24,))])
+def test_sequence_in_segments_equals_the_whole_sequence(shape, cuts):
+    # A sequence run as consecutive segments: forward carries (h, c) from one segment to the next in fp32,
+    # backward runs the segments last to first, feeds each segment's dh0 / dc0 to the next call as d_hn / d_cn
+    # and adds the parameter gradients up ("accumulate_grads").  Every state and dx must come out bit-identical
+    # to the single pass; dW and db are sums in another order.
+    from flashlstm_poc_amd import LstmCore
+    p = make_problem(*shape, seed=21)
+    T, B, I, H = shape
+    whole, _ = run_core(p)
+    core = LstmCore(B, I, H)
+    core.pack(*(p[k].cuda() for k in ("w_ih", "w_hh", "b_ih", "b_hh")))
+    x, dy = p["x"].cuda().half(), p["dy"].cuda().half()
+    bounds = [0, *cuts, T]
+    segs = list(zip(bounds[:-1], bounds[1:]))
+    h, c = p["h0"].cuda().float(), p["c0"].cuda().float()
+    starts, ys = [], []
+    for a, b in segs:
+        starts.append((h, c))
+        y, hy, cy = core.forward(x[a:b], h, c, out_dtype=torch.float32)
+        ys.append(y)
+        h, c = hy, cy
+    np.testing.assert_array_equal(to_np(torch.cat(ys).half()), whole["y"])
+    np.testing.assert_array_equal(to_np(h.half()), whole["hn"])
+    assert relmax(to_np(c), whole["cn"]) < 1e-3   # the single pass returned c_T rounded to fp16
+    acc = (torch.zeros(4 * H, I, device="cuda"), torch.zeros(4 * H, H, device="cuda"), torch.zeros(4 * H, device="cuda"))
+    dh, dc = p["d_hn"].cuda().float(), p["d_cn"].cuda().float()
+    dxs = []
+    for (a, b), (h_in, c_in) in reversed(list(zip(segs, starts))):
+        core.forward(x[a:b], h_in, c_in, want_y=False)   # rebuild this segment's caches
+        dx, _, _, _, dh, dc = core.backward(x[a:b], dy[a:b], dh, dc, accumulate_into=acc)
+        dxs.insert(0, dx)
+    torch.cuda.synchronize()
+    np.testing.assert_array_equal(to_np(torch.cat(dxs)), whole["dx"])
+    np.testing.assert_array_equal(to_np(dh), whole["dh0"])
+    np.testing.assert_array_equal(to_np(dc), whole["dc0"])
+    for got, name in zip(acc, ("dw_ih", "dw_hh", "db")):
+        assert rell2(to_np(got), whole[name]) < 1e-5, name
+    core.close()
+
+
 def test_error_codes():
     from flashlstm_poc_amd import LstmCore
     core = LstmCore(2, 3, 5)

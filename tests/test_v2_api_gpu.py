@@ -146,6 +146,44 @@ def test_chunked_streaming_gives_the_whole_sequence_results(shape, monkeypatch):
             assert rell2(out["db"], whole["db"]) < 1e-6   # summed per launch, then over launches
 
 
+@pytest.mark.parametrize("shape,R,window", [((23, 3, 12, 20), 4, 5), ((23, 3, 12, 20), 7, 8), ((23, 3, 12, 20), 50, 6),
+                                            ((70, 40, 64, 256), 16, 32), ((33, 5, 16, 24), 1, 11)])
+def test_windows_smaller_than_the_sequence_give_the_whole_sequence_results(shape, R, window, monkeypatch):
+    # FLASHLSTM_V2_WINDOW_STEPS bounds what the device holds at once (the counterpart of the reference's bounded
+    # chunk buffers, lstm_forward.cu:646-940, and of its recomputation from the checkpoints,
+    # lstm_backward.cu:897-1056): forward carries the state from window to window, backward recomputes each
+    # window's gate cache from the state at its start -- kept on the device by the matching forward call, or
+    # rebuilt from the host checkpoints (fresh) -- and adds the weight gradients up.
+    p = make_problem(*shape, seed=13)
+    f, g = reference(p)
+    monkeypatch.setenv("FLASHLSTM_V2_CHUNK_STEPS", "4")
+    monkeypatch.delenv("FLASHLSTM_V2_WINDOW_STEPS", raising=False)
+    whole = run_v2(p, R=R)
+    compare(whole, f, g, R)
+    monkeypatch.setenv("FLASHLSTM_V2_WINDOW_STEPS", str(window))
+    for fresh in (False, True):
+        out = run_v2(p, R=R, fresh_backward=fresh)
+        compare(out, f, g, R)
+        # fp32 checkpoints describe the states exactly, so every window recomputes exactly the caches of the single pass
+        for k in ("y", "hn", "cn", "ck_h", "ck_c", "dx", "dh0", "dc0"):
+            np.testing.assert_array_equal(out[k], whole[k], err_msg=f"fresh={fresh} {k}")
+        for k in ("dw_ih", "dw_hh", "db"):
+            assert rell2(out[k], whole[k]) < 1e-5, k   # sums over windows instead of one sum
+    # fp16 checkpoints round the states a fresh backward call starts from
+    out = run_v2(p, R=R, h_dtype=torch.float16, c_dtype=torch.float16, fresh_backward=True)
+    compare(out, f, g, R)
+
+
+def test_device_budget_selects_the_window(monkeypatch):
+    p = make_problem(40, 8, 64, 128, seed=14)
+    f, g = reference(p)
+    monkeypatch.delenv("FLASHLSTM_V2_WINDOW_STEPS", raising=False)
+    monkeypatch.setenv("FLASHLSTM_V2_CHUNK_STEPS", "2")
+    monkeypatch.setenv("FLASHLSTM_V2_DEVICE_BUDGET_MB", "1")   # 29 KiB per step -> 36 steps, cut to whole chunks
+    out = run_v2(p, R=8, fresh_backward=True)
+    compare(out, f, g, 8)
+
+
 def test_null_state_gradients_and_pageable_host_memory():
     p = make_problem(6, 4, 8, 16, seed=3)
     f, g = reference(p, state_grads=False)
