@@ -62,6 +62,14 @@ __device__ __forceinline__ half_t out16(float alpha, float acc, float bias) {
     return (half_t)v;
 }
 
+// Vector stores of full tiles need rows of a multiple of 4 elements that start on 8 (fp16) / 16 (fp32) bytes;
+// any other output (odd row length, a sub-matrix that starts at an odd row) takes the element-wise path.
+__device__ __forceinline__ bool vector_output(const GemmNT& g) {
+    if (g.ldc % 4 != 0) return false;
+    if (g.C16) return reinterpret_cast<uintptr_t>(g.C16) % 8 == 0;
+    return reinterpret_cast<uintptr_t>(g.C32) % 16 == 0 && g.split_stride % 4 == 0;
+}
+
 __device__ __forceinline__ floatx4 bias4(const GemmNT& g, int col) {
     return g.bias ? *reinterpret_cast<const floatx4*>(g.bias + col) : floatx4{0.f, 0.f, 0.f, 0.f};
 }
@@ -71,7 +79,7 @@ __device__ __forceinline__ void store_tile(const GemmNT& g, floatx16 (&acc)[4][k
     const int row = m0 + wm * 128 + lane % 32;
     const int colb = n0 + wn * 32 * kTN + 4 * (lane / 32);
     float* c32 = g.C32 ? g.C32 + size_t(z) * g.split_stride : nullptr;
-    const bool full = (m0 + BM <= g.M) && (n0 + BN <= g.N) && (g.ldc % 4 == 0);
+    const bool full = (m0 + BM <= g.M) && (n0 + BN <= g.N) && vector_output(g);
     if (full) {
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
@@ -319,7 +327,7 @@ __global__ __launch_bounds__(kThreads) void gemm_nt_stream(GemmNT g, TileOrder o
             copied = ld_valid;
             loader_advance();
         }
-        const bool full = (m0 + BM <= g.M) && (n0 + BN <= g.N) && (g.ldc % 4 == 0);
+        const bool full = (m0 + BM <= g.M) && (n0 + BN <= g.N) && vector_output(g);
         if (full && g.C16 && g.ldc % 8 == 0 && reinterpret_cast<uintptr_t>(g.C16) % 16 == 0) {
             store_tile_lines(g, acc, m0, n0, wm, wn, lane, lds + 2 * kSlabBytes + wave * kEpiBytesPerWave);
         } else {
@@ -483,7 +491,7 @@ __global__ __launch_bounds__(kThreads) void gemm_tn_256x256(GemmNT g, TileOrder 
         if (more) stage(cur ^ 1);
         __syncthreads();
     }
-    const bool full = (m0 + BM <= g.M) && (n0 + BN <= g.N) && (g.ldc % 4 == 0);
+    const bool full = (m0 + BM <= g.M) && (n0 + BN <= g.N) && vector_output(g);
     if (full && g.C32) {
         // the slab buffers are free once every wave has left the main loop (the barrier that ends it)
         store_tile_lines_f32(g, acc, m0, n0, wm, wn, lane, z, reinterpret_cast<char*>(smem) + wave * 4096);
@@ -514,9 +522,6 @@ hipError_t launch_gemm_nt(const GemmNT& g, hipStream_t stream) {
     if (g.M <= 0 || g.N <= 0 || g.K <= 0) return hipSuccess;
     if (g.K % BK != 0 || g.lda % 8 != 0 || g.ldb % 8 != 0) return hipErrorInvalidValue;
     if ((g.C16 == nullptr) == (g.C32 == nullptr)) return hipErrorInvalidValue;
-    // the vector stores of full tiles need an aligned base (rows are covered by the ldc % 4 test in the kernel)
-    if (g.C32 && (reinterpret_cast<uintptr_t>(g.C32) % 16 != 0 || g.split_stride % 4 != 0)) return hipErrorInvalidValue;
-    if (g.C16 && (reinterpret_cast<uintptr_t>(g.C16) % 8 != 0)) return hipErrorInvalidValue;
     if (g.bias && (reinterpret_cast<uintptr_t>(g.bias) % 16 != 0 || g.splits > 1)) return hipErrorInvalidValue;
     int splits = g.splits < 1 ? 1 : g.splits;
     if (splits > 1 && g.C32 == nullptr) return hipErrorInvalidValue;
