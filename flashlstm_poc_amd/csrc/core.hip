@@ -179,6 +179,7 @@ extern "C" long flstm_core_get_info(const flstm_core_plan* p, const char* name) 
     if (!strcmp(name, "xcd_local_bwd")) return p->Lb.xcd_local;
     if (!strcmp(name, "resident_fwd")) return p->Lf.resident;
     if (!strcmp(name, "resident_bwd")) return p->Lb.resident;
+    if (!strcmp(name, "row_tiles")) return p->Lf.mt;
     if (!strcmp(name, "slice_fwd")) return p->Lf.jb;
     if (!strcmp(name, "slice_bwd")) return p->Lb.jb;
     if (!strcmp(name, "groups_fwd")) return p->Lf.ng;

@@ -11,6 +11,7 @@ struct RecLayout {
     int jb;          // hidden units per workgroup slice
     int nh;          // slices = Hp / jb  (workgroups per group)
     int nrb;         // 32-row batch blocks
+    int mt;          // 16-row tiles of a block that are fetched and multiplied: 2, or 1 when the batch has at most 16 rows
     int ng;          // concurrently running groups; group g owns row blocks g, g+ng, ...
     int gpx;         // XCD-local mode: groups per XCD
     int xcd_local;   // 1: every group lives inside one XCD (plain stores + L2-served loads)

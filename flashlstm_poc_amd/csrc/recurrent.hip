@@ -31,6 +31,8 @@
 //  * Fallback.  The same kernels launched once per step (no waits, kernel boundaries order
 //    memory) serve shapes whose weights do not fit on chip, and are the safe path after a failed
 //    persistent launch.
+#include <type_traits>
+
 #include "recurrent.h"
 
 namespace flstm_hip {
@@ -134,18 +136,27 @@ __device__ __forceinline__ void wait_frags(half8 (&a)[4], half8 (&b)[4]) {
                  : "memory");
 }
 template <int N>
+__device__ __forceinline__ void wait_frags(half8 (&a)[4]) {
+    asm volatile("s_waitcnt vmcnt(%4)" : "+v"(a[0]), "+v"(a[1]), "+v"(a[2]), "+v"(a[3]) : "n"(N) : "memory");
+}
+template <int N>
+__device__ __forceinline__ void wait_frags(half8 (&a)[2]) {
+    asm volatile("s_waitcnt vmcnt(%2)" : "+v"(a[0]), "+v"(a[1]) : "n"(N) : "memory");
+}
+template <int N>
 __device__ __forceinline__ void wait_frags(half8 (&a)[2], half8 (&b)[2]) {
     asm volatile("s_waitcnt vmcnt(%4)" : "+v"(a[0]), "+v"(a[1]), "+v"(b[0]), "+v"(b[1]) : "n"(N) : "memory");
 }
 
-// acc[mt][nt] += (A(32 rows x K) * Wslice)^T, this wave's interleaved k-steps only.
-// a0/a1: fragment (row tile, k-step 0) of the two 16-row tiles, already offset by lane*8 halfs.
+// acc[mt][nt] += (A(16*MT rows x K) * Wslice)^T, this wave's interleaved k-steps only.
+// a0/a1: fragment (row tile, k-step 0) of the two 16-row tiles, already offset by lane*8 halfs; with MT = 1
+// (batches of at most 16 rows) the second tile is neither fetched nor multiplied.
 // The last KL of a wave's KS k-steps keep their weight fragments in LDS instead of registers (wlds:
 // this wave's [KL][NT][64 lanes] block); reading them back costs a few ds_read_b128 per step and frees
 // 4*KL*NT registers for fragments in flight.
 // `prefetch` issues exactly NPF vector loads (for every wave, whatever its lanes need) behind the last
 // fragment load.
-template <int NT, int KS, bool RESIDENT, int KL, int NPF, typename Prefetch>
+template <int NT, int KS, bool RESIDENT, int KL, int NPF, int MT, typename Prefetch>
 __device__ __forceinline__ void wave_product(floatx4 (&acc)[2][NT], const half8 (&wreg)[KS - KL][NT],
                                              const half8* wlds, const half8* wfrag_wave, const half_t* a0,
                                              const half_t* a1, int wave, int lane, int nks_total,
@@ -163,8 +174,13 @@ __device__ __forceinline__ void wave_product(floatx4 (&acc)[2][NT], const half8 
             for (int k = 0; k < CK; ++k) {
                 const int kg = min((c * CK + k) * 4 + wave, nks_total - 1);
                 ld_frag_async(fa[buf][k], a0 + size_t(kg) * 512);
-                ld_frag_async(fb[buf][k], a1 + size_t(kg) * 512);
+                if constexpr (MT == 2) ld_frag_async(fb[buf][k], a1 + size_t(kg) * 512);
             }
+        };
+        auto wait = [&](auto younger, int buf) {   // until at most `younger` loads issued later are outstanding
+            constexpr int N = decltype(younger)::value;
+            if constexpr (MT == 2) wait_frags<N>(fa[buf], fb[buf]);
+            else wait_frags<N>(fa[buf]);
         };
         issue(0, 0);
         if (NCH == 1) prefetch();
@@ -173,13 +189,13 @@ __device__ __forceinline__ void wave_product(floatx4 (&acc)[2][NT], const half8 
             const int buf = c & 1;
             if (c + 2 < NCH) {
                 issue(c + 1, buf ^ 1);
-                wait_frags<2 * CK>(fa[buf], fb[buf]);
+                wait(std::integral_constant<int, MT * CK>{}, buf);
             } else if (c + 2 == NCH) {
                 issue(c + 1, buf ^ 1);
                 prefetch();
-                wait_frags<2 * CK + NPF>(fa[buf], fb[buf]);
+                wait(std::integral_constant<int, MT * CK + NPF>{}, buf);
             } else {
-                wait_frags<NPF>(fa[buf], fb[buf]);
+                wait(std::integral_constant<int, NPF>{}, buf);
             }
             if (poll.on) {
                 // A pair of halfs that still holds the pattern has not been written yet by its producer:
@@ -191,9 +207,11 @@ __device__ __forceinline__ void wave_product(floatx4 (&acc)[2][NT], const half8 
 #pragma unroll
                     for (int k = 0; k < CK; ++k) {
                         const uint4 ua = __builtin_bit_cast(uint4, fa[buf][k]);
-                        const uint4 ub = __builtin_bit_cast(uint4, fb[buf][k]);
                         m = max(m, max(max(ua.x, ua.y), max(ua.z, ua.w)));
-                        m = max(m, max(max(ub.x, ub.y), max(ub.z, ub.w)));
+                        if constexpr (MT == 2) {
+                            const uint4 ub = __builtin_bit_cast(uint4, fb[buf][k]);
+                            m = max(m, max(max(ub.x, ub.y), max(ub.z, ub.w)));
+                        }
                     }
                     if (!__any(m == kUnwritten)) break;
                     ++spins;
@@ -207,7 +225,7 @@ __device__ __forceinline__ void wave_product(floatx4 (&acc)[2][NT], const half8 
                         break;   // results are garbage from here on; the workgroup leaves at its next barrier
                     }
                     issue(c, buf);
-                    wait_frags<0>(fa[buf], fb[buf]);   // (also what was issued after this chunk the first time)
+                    wait(std::integral_constant<int, 0>{}, buf);   // (also what was issued after this chunk the first time)
                 }
             }
 #pragma unroll
@@ -220,7 +238,8 @@ __device__ __forceinline__ void wave_product(floatx4 (&acc)[2][NT], const half8 
                     if (ks < KR) w = wreg[ks < KR ? ks : 0][n];
                     else w = wlds[((ks - KR) * NT + n) * kWave + lane];
                     acc[0][n] = __builtin_amdgcn_mfma_f32_16x16x32_f16(w, fa[buf][k], acc[0][n], 0, 0, 0);
-                    acc[1][n] = __builtin_amdgcn_mfma_f32_16x16x32_f16(w, fb[buf][k], acc[1][n], 0, 0, 0);
+                    if constexpr (MT == 2)
+                        acc[1][n] = __builtin_amdgcn_mfma_f32_16x16x32_f16(w, fb[buf][k], acc[1][n], 0, 0, 0);
                 }
             }
         }
@@ -229,12 +248,13 @@ __device__ __forceinline__ void wave_product(floatx4 (&acc)[2][NT], const half8 
             const int kg = k * 4 + wave;
             if (kg >= nks_total) break;
             const half8 fa = ld_frag(a0 + size_t(kg) * 512);
-            const half8 fb = ld_frag(a1 + size_t(kg) * 512);
+            half8 fb{};
+            if constexpr (MT == 2) fb = ld_frag(a1 + size_t(kg) * 512);
 #pragma unroll
             for (int n = 0; n < NT; ++n) {
                 const half8 w = wfrag_wave[(size_t(k) * NT + n) * kWave + lane];
                 acc[0][n] = __builtin_amdgcn_mfma_f32_16x16x32_f16(w, fa, acc[0][n], 0, 0, 0);
-                acc[1][n] = __builtin_amdgcn_mfma_f32_16x16x32_f16(w, fb, acc[1][n], 0, 0, 0);
+                if constexpr (MT == 2) acc[1][n] = __builtin_amdgcn_mfma_f32_16x16x32_f16(w, fb, acc[1][n], 0, 0, 0);
             }
         }
         prefetch();
@@ -245,12 +265,12 @@ __device__ __forceinline__ void wave_product(floatx4 (&acc)[2][NT], const half8 
 // consecutive output columns of one batch row: tile (m, n) holds row m*16 + lane%16, columns
 // n*16 + 4*(lane/16) .. +3, and goes to LDS as one 16-byte store.  The 16 rows written together are
 // 4*pld banks apart; for the pitches in use that spreads them over all 64 banks.
-template <int NT>
+template <int NT, int MT>
 __device__ __forceinline__ void spill_partials(float* part, const floatx4 (&acc)[2][NT], int wave,
                                                int lane, int pld) {
     float* base = part + size_t(wave) * kRows * pld + size_t(lane % 16) * pld + 4 * (lane / 16);
 #pragma unroll
-    for (int m = 0; m < 2; ++m)
+    for (int m = 0; m < MT; ++m)
 #pragma unroll
         for (int n = 0; n < NT; ++n)
             *reinterpret_cast<floatx4*>(base + m * 16 * pld + n * 16) = acc[m][n];
@@ -417,7 +437,9 @@ struct PhaseClock {
 // activated gates -> prefetch the next step's x-projection.  Only the h_t store sits between this step
 // and the next one of the other workgroups; everything HBM-bound (x-projection fetch, cache stores) is
 // off that path.
-template <int NT, int KS, bool RESIDENT>
+// MT = 16-row tiles per row block: 2, or 1 for batches of at most 16 rows (the threads of rows 16..31 then only
+// keep the barriers company).
+template <int NT, int KS, bool RESIDENT, int MT>
 __global__ __launch_bounds__(kThreads) void rec_fwd_kernel(RecFwdArgs p, RecLayout L, int t_begin,
                                                            int t_end, int ks_wave) {
     constexpr int JB = 4 * NT;    // hidden units of this slice
@@ -487,10 +509,10 @@ __global__ __launch_bounds__(kThreads) void rec_fwd_kernel(RecFwdArgs p, RecLayo
             for (int m = 0; m < 2; ++m)
 #pragma unroll
                 for (int n = 0; n < NT; ++n) acc[m][n] = floatx4{0.f, 0.f, 0.f, 0.f};
-            wave_product<NT, KS, RESIDENT, 0, 4>(acc, wreg, nullptr, wfrag_wave, a0, a1, wave, lane, nks_total, ks_wave,
-                                                 poll, [&]() { prefetch(t, rb); });
+            wave_product<NT, KS, RESIDENT, 0, 4, MT>(acc, wreg, nullptr, wfrag_wave, a0, a1, wave, lane, nks_total,
+                                                     ks_wave, poll, [&]() { prefetch(t, rb); });
             clk.lap(0);
-            spill_partials<NT>(part, acc, wave, lane, PLD);
+            spill_partials<NT, MT>(part, acc, wave, lane, PLD);
             __syncthreads();
             if (lds_abort != 0) return;
             clk.lap(1);
@@ -504,7 +526,8 @@ __global__ __launch_bounds__(kThreads) void rec_fwd_kernel(RecFwdArgs p, RecLayo
             clk.lap(4);
             const int b = row0 + pr;
             const unsigned xoff = unsigned(xch_offset(b, j, nks_total));   // 32 bits: a slot is far below 4G halfs
-            store_xch(xnext + xoff, pack_fill(kUnwritten, (PackT*)nullptr), device_scope);
+            const bool row_used = (MT == 2) || pr < 16;   // rows nobody fetches are not exchanged
+            if (row_used) store_xch(xnext + xoff, pack_fill(kUnwritten, (PackT*)nullptr), device_scope);
             PackT act[4], hnew = pack_fill(0u, (PackT*)nullptr);   // batch rows past B travel as zeros
             const bool live = b < p.B;
             if (live) {
@@ -546,7 +569,7 @@ __global__ __launch_bounds__(kThreads) void rec_fwd_kernel(RecFwdArgs p, RecLayo
                 for (int gt = 0; gt < 4; ++gt) act[gt] = pack(a4[gt]);
             }
             // the exchanged value goes out first
-            store_xch(xout + xoff, hnew, device_scope);
+            if (row_used) store_xch(xout + xoff, hnew, device_scope);
             clk.lap(2);
             // caches for the backward pass: off the critical path
             if (live) {
@@ -565,7 +588,7 @@ __global__ __launch_bounds__(kThreads) void rec_fwd_kernel(RecFwdArgs p, RecLayo
 // ----------------------------------------------------------------------------------- backward
 // Gate order and the pointwise derivative follow flashlstm_v2/src/lstm_backward.cu:199-211, except
 // that c_{t-1}, c_t come from the cell-state cache instead of being rebuilt through atanh.
-template <int NT, int KS, bool RESIDENT, int KL>
+template <int NT, int KS, bool RESIDENT, int KL, int MT>
 __global__ __launch_bounds__(kThreads) void rec_bwd_kernel(RecBwdArgs p, RecLayout L, int t_first,
                                                            int t_last, int ks_wave) {
     constexpr int JB = 16 * NT;  // hidden units (= output columns of dG*W_hh) of this slice
@@ -655,10 +678,10 @@ __global__ __launch_bounds__(kThreads) void rec_bwd_kernel(RecBwdArgs p, RecLayo
                 for (int m = 0; m < 2; ++m)
 #pragma unroll
                     for (int n = 0; n < NT; ++n) acc[m][n] = floatx4{0.f, 0.f, 0.f, 0.f};
-                wave_product<NT, KS, RESIDENT, KL, 7>(acc, wreg, wlds, wfrag_wave, a0, a1, wave, lane, nks_total, ks_wave,
-                                                      poll, [&]() { prefetch(t, rb); });
+                wave_product<NT, KS, RESIDENT, KL, 7, MT>(acc, wreg, wlds, wfrag_wave, a0, a1, wave, lane, nks_total,
+                                                          ks_wave, poll, [&]() { prefetch(t, rb); });
                 clk.lap(0);
-                spill_partials<NT>(part, acc, wave, lane, PLD);
+                spill_partials<NT, MT>(part, acc, wave, lane, PLD);
                 __syncthreads();
                 if (lds_abort != 0) return;
                 clk.lap(1);
@@ -679,7 +702,8 @@ __global__ __launch_bounds__(kThreads) void rec_bwd_kernel(RecBwdArgs p, RecLayo
             half_t* xnext = p.X + size_t((t + 6) & 3) * p.x_slot;   // will take dG_{t-2}
             unsigned xoff[4];   // 32 bits: a slot is far below 4G halfs
             PackT dgnew[4];
-            if (t >= 0) {
+            const bool row_used = (MT == 2) || pr < 16;   // rows nobody fetches are not exchanged
+            if (t >= 0 && row_used) {
                 // every peer has delivered dG_{t+1}, so all of them are done reading dG_{t+2}: mark its slot
                 // (the wait above has drained the marks of the previous step)
 #pragma unroll
@@ -747,7 +771,7 @@ __global__ __launch_bounds__(kThreads) void rec_bwd_kernel(RecBwdArgs p, RecLayo
                     }
                 }
             }
-            if (t >= 0) {
+            if (t >= 0 && row_used) {
                 // the exchanged values go out first
 #pragma unroll
                 for (int gt = 0; gt < 4; ++gt) store_xch(xout + xoff[gt], dgnew[gt], device_scope);
@@ -823,6 +847,7 @@ static void finish_layout(RecLayout& L, int B, int Hp, int num_cus, bool force_s
     L.nh = Hp / L.jb;
     L.nrb = int(ceil_div(size_t(B), size_t(kRows)));
     L.resident = fits ? 1 : 0;
+    L.mt = (fits && B <= 16) ? 1 : 2;
     L.xcd_local = 0;
     L.gpx = 0;
     if (!fits || force_stepwise || L.nh > num_cus) {
@@ -866,9 +891,9 @@ RecLayout plan_rec_bwd(int B, int Hp, int num_cus, bool force_stepwise) {
     return L;
 }
 
-template <int NT, int KS, bool RES>
+template <int NT, int KS, bool RES, int MT>
 static hipError_t run_fwd(const RecLayout& L, const RecFwdArgs& a, hipStream_t stream) {
-    auto kernel = rec_fwd_kernel<NT, KS, RES>;
+    auto kernel = rec_fwd_kernel<NT, KS, RES, MT>;
     const size_t lds = size_t(2) * 4 * kRows * (16 * NT + kPartPad) * sizeof(float);
     hipError_t e = raise_lds(kernel, lds);
     if (e != hipSuccess) return e;
@@ -888,15 +913,16 @@ static hipError_t run_fwd(const RecLayout& L, const RecFwdArgs& a, hipStream_t s
 hipError_t launch_rec_fwd(const RecLayout& L, const RecFwdArgs& a, hipStream_t stream) {
     if (a.T <= 0 || a.B <= 0 || a.t1 <= a.t0) return hipSuccess;
     if (a.Hp % 32 != 0 || a.Hp % L.jb != 0 || a.t0 < 0 || a.t1 > a.T) return hipErrorInvalidValue;
-    if (!L.resident) return run_fwd<8, 1, false>(L, a, stream);
-    if (L.nt == 8) return run_fwd<8, 8, true>(L, a, stream);
-    if (L.nt == 4) return run_fwd<4, 16, true>(L, a, stream);
+    if (!L.resident) return run_fwd<8, 1, false, 2>(L, a, stream);
+    if (L.mt == 1 && a.B > 16) return hipErrorInvalidValue;
+    if (L.nt == 8) return L.mt == 1 ? run_fwd<8, 8, true, 1>(L, a, stream) : run_fwd<8, 8, true, 2>(L, a, stream);
+    if (L.nt == 4) return L.mt == 1 ? run_fwd<4, 16, true, 1>(L, a, stream) : run_fwd<4, 16, true, 2>(L, a, stream);
     return hipErrorInvalidValue;
 }
 
-template <int NT, int KS, bool RES, int KL>
+template <int NT, int KS, bool RES, int KL, int MT>
 static hipError_t run_bwd(const RecLayout& L, const RecBwdArgs& a, hipStream_t stream) {
-    auto kernel = rec_bwd_kernel<NT, KS, RES, KL>;
+    auto kernel = rec_bwd_kernel<NT, KS, RES, KL, MT>;
     static_assert(size_t(2) * 4 * kRows * (16 * NT + kPartPad) >= size_t(kThreads) * 8 * NT, "db reduction reuses the partial-sum area");
     const size_t lds = size_t(2) * 4 * kRows * (16 * NT + kPartPad) * sizeof(float) + size_t(4) * KL * NT * kWave * sizeof(half8);
     hipError_t e = raise_lds(kernel, lds);
@@ -917,9 +943,10 @@ static hipError_t run_bwd(const RecLayout& L, const RecBwdArgs& a, hipStream_t s
 hipError_t launch_rec_bwd(const RecLayout& L, const RecBwdArgs& a, hipStream_t stream) {
     if (a.T <= 0 || a.B <= 0 || a.t_hi < a.t_lo) return hipSuccess;
     if (a.Hp % 32 != 0 || a.Hp % L.jb != 0 || a.t_lo < -1 || a.t_hi >= a.T) return hipErrorInvalidValue;
-    if (!L.resident) return run_bwd<2, 1, false, 0>(L, a, stream);
-    if (L.nt == 2) return run_bwd<2, 32, true, 8>(L, a, stream);
-    if (L.nt == 1) return run_bwd<1, 64, true, 24>(L, a, stream);
+    if (!L.resident) return run_bwd<2, 1, false, 0, 2>(L, a, stream);
+    if (L.mt == 1 && a.B > 16) return hipErrorInvalidValue;
+    if (L.nt == 2) return L.mt == 1 ? run_bwd<2, 32, true, 8, 1>(L, a, stream) : run_bwd<2, 32, true, 8, 2>(L, a, stream);
+    if (L.nt == 1) return L.mt == 1 ? run_bwd<1, 64, true, 24, 1>(L, a, stream) : run_bwd<1, 64, true, 24, 2>(L, a, stream);
     return hipErrorInvalidValue;
 }
 
