@@ -46,11 +46,12 @@ int flstm_core_destroy(flstm_core_plan* plan);
  * and db_hh to what the caller's buffers hold instead of overwriting them: a sequence processed as several
  * consecutive segments, last segment first, each segment's dh0 / dc0 fed to the next call as d_hn / d_cn). */
 int flstm_core_set_option(flstm_core_plan* plan, const char* name, long value);
-/* Reads back facts about the plan: "persistent_fwd", "persistent_bwd", "xcd_local_fwd",
- * "xcd_local_bwd", "fallbacks" (persistent launches that had to be redone step-wise), "slice_fwd",
- * "slice_bwd" (hidden units per workgroup of the recurrence kernels), "row_tiles" (16-row tiles of a 32-row
- * batch block that the recurrence fetches and multiplies: 1 for batches of at most 16 rows, else 2), "hidden_padded", "num_cus" and
- * "clock_khz" (compute units and maximum engine clock of the plan's device). */
+/* Reads back facts about the plan: "persistent_fwd", "persistent_bwd", "xcd_local_fwd", "xcd_local_bwd",
+ * "fallbacks" (persistent launches that had to be redone step-wise), "slice_fwd", "slice_bwd" (hidden units
+ * per workgroup of the recurrence kernels), "row_tiles" (16-row tiles of a 32-row batch block that the
+ * recurrence fetches and multiplies: 1 for batches of at most 16 rows, else 2), "hidden_padded",
+ * "input_padded", "num_cus" and "clock_khz" (compute units and maximum engine clock of the plan's device).
+ * Unknown names give -1. */
 long flstm_core_get_info(const flstm_core_plan* plan, const char* name);
 
 /* fp32 PyTorch-layout weights -> fp16 MFMA operand layouts held by the plan. */
