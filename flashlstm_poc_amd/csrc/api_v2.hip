@@ -167,9 +167,11 @@ void sync_all(const Streams& st) {
 }
 
 // Steps per window: everything a pass keeps per time step on the device (staging + the core's caches),
-// against a budget of FLASHLSTM_V2_DEVICE_BUDGET_MB (default: 70 % of the device's memory).
-// FLASHLSTM_V2_WINDOW_STEPS forces a value.  Read per call: cheap, and tests switch them.
-size_t window_steps_for(size_t T, size_t B, size_t I, size_t H) {
+// against a budget of FLASHLSTM_V2_DEVICE_BUDGET_MB (default: 70 % of the device's memory, and no more than
+// 85 % of what is free now plus what this shape's buffers already hold).  FLASHLSTM_V2_WINDOW_STEPS forces a
+// value.  Read per call: cheap, and tests switch them.
+size_t window_steps_for(const Entry& e, size_t T) {
+    const size_t B = e.B, I = e.I, H = e.H;
     if (const char* v = getenv("FLASHLSTM_V2_WINDOW_STEPS")) {
         const long w = atol(v);
         if (w > 0) return size_t(w) < T ? size_t(w) : T;
@@ -181,7 +183,10 @@ size_t window_steps_for(size_t T, size_t B, size_t I, size_t H) {
     if (budget == 0) {
         size_t free_b = 0, total_b = 0;
         check(hipMemGetInfo(&free_b, &total_b), "hipMemGetInfo");
+        size_t held = size_t(flstm_core_get_info(e.plan, "device_bytes") > 0 ? flstm_core_get_info(e.plan, "device_bytes") : 0);
+        for (const Buf* b : {&e.x_dev, &e.y_dev, &e.dy_dev, &e.dx_dev}) held += b->bytes;
         budget = total_b / 10 * 7;
+        if (budget > (free_b + held) / 20 * 17) budget = (free_b + held) / 20 * 17;
     }
     size_t w = budget / per_step;
     if (w >= T) return T;
@@ -298,7 +303,7 @@ void run_forward(Entry& e, size_t T, size_t R, const __half* x_host, const __hal
     e.last.valid = false;
     check_core(flstm_core_pack_weights(e.plan, w_ih, w_hh, st.cs), "flstm_core_pack_weights");
     check_core(flstm_core_pack_bias(e.plan, b_ih, b_hh, st.cs), "flstm_core_pack_bias");
-    const size_t W = window_steps_for(T, B, I, H), nwin = (T + W - 1) / W;
+    const size_t W = window_steps_for(e, T), nwin = (T + W - 1) / W;
     e.start_known.assign(nwin, 0);
     if (nwin == 1) {
         const CachePtrs cp = forward_window(e, st, T, x_host, h0, c0, FLSTM_F16, y_host, hy, cy, FLSTM_F16);
@@ -471,7 +476,7 @@ void StreamingLstmBackward(size_t T, size_t B, size_t I, size_t H, size_t R, con
     Entry& e = entry_for(B, I, H);
     const Streams st{cs, h2d, d2h};
     const size_t x_bytes = T * B * I * sizeof(half_t), y_bytes = T * B * H * sizeof(half_t), BH = B * H;
-    const size_t W = window_steps_for(T, B, I, H), nwin = (T + W - 1) / W;
+    const size_t W = window_steps_for(e, T), nwin = (T + W - 1) / W;
     static const bool always_recompute = (getenv("FLASHLSTM_V2_RECOMPUTE") != nullptr);
     const ForwardKey& k = e.last;
     bool hit = !always_recompute && k.valid && k.x == x_host && k.y == y_host && k.ch == cache.h_ptr &&

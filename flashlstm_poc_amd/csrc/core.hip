@@ -180,6 +180,14 @@ extern "C" long flstm_core_get_info(const flstm_core_plan* p, const char* name) 
     if (!strcmp(name, "resident_fwd")) return p->Lf.resident;
     if (!strcmp(name, "resident_bwd")) return p->Lb.resident;
     if (!strcmp(name, "row_tiles")) return p->Lf.mt;
+    if (!strcmp(name, "device_bytes")) {
+        size_t sum = 0;
+        for (const DevBuf* b : {&p->wih_p, &p->wih_t, &p->wfrag_f, &p->wfrag_b, &p->bias_p, &p->X16, &p->G, &p->Y, &p->C,
+                                &p->status, &p->xch_f, &p->xch_b, &p->dYp, &p->dG, &p->dHn, &p->dC, &p->dH0, &p->db_part,
+                                &p->dw_part, &p->prof})
+            sum += b->bytes;
+        return long(sum);
+    }
     if (!strcmp(name, "slice_fwd")) return p->Lf.jb;
     if (!strcmp(name, "slice_bwd")) return p->Lb.jb;
     if (!strcmp(name, "groups_fwd")) return p->Lf.ng;

@@ -50,7 +50,8 @@ int flstm_core_set_option(flstm_core_plan* plan, const char* name, long value);
  * "fallbacks" (persistent launches that had to be redone step-wise), "slice_fwd", "slice_bwd" (hidden units
  * per workgroup of the recurrence kernels), "row_tiles" (16-row tiles of a 32-row batch block that the
  * recurrence fetches and multiplies: 1 for batches of at most 16 rows, else 2), "hidden_padded",
- * "input_padded", "num_cus" and "clock_khz" (compute units and maximum engine clock of the plan's device).
+ * "input_padded", "device_bytes" (device memory the plan holds), "num_cus" and "clock_khz" (compute units and
+ * maximum engine clock of the plan's device).
  * Unknown names give -1. */
 long flstm_core_get_info(const flstm_core_plan* plan, const char* name);
 
