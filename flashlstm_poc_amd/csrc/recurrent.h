@@ -10,8 +10,8 @@ struct RecLayout {
     int nt;          // forward: 16-wide gate-column tiles per workgroup (JB = 4*nt hidden units)
     int jb;          // hidden units per workgroup slice
     int nh;          // slices = Hp / jb  (workgroups per group)
-    int nrb;         // 32-row batch blocks
-    int mt;          // 16-row tiles of a block that are fetched and multiplied: 2, or 1 when the batch has at most 16 rows
+    int nrb;         // batch blocks of 16*mt rows
+    int mt;          // 16-row MFMA tiles per batch block: 1 when all 16-row blocks can run side by side, else 2
     int ng;          // concurrently running groups; group g owns row blocks g, g+ng, ...
     int gpx;         // XCD-local mode: groups per XCD
     int xcd_local;   // 1: every group lives inside one XCD (plain stores + L2-served loads)

@@ -39,7 +39,7 @@ namespace flstm_hip {
 namespace {
 
 constexpr int kThreads = 256;
-constexpr int kRows = 32;  // batch rows per row block
+constexpr int kRows = 32;  // batch rows per row block at most (two 16-row MFMA tiles; kernels with MT = 1 use one)
 // Floats added to a row of partial sums in LDS.  Any pad = 4 mod 8 keeps the 16-byte accesses free of bank
 // conflicts (measured: 4, 12 and 20 count the same; 8 triples the conflict cycles); what the counter still
 // shows is four cycles per 16-byte store, which run at half rate whatever the layout.
@@ -373,8 +373,8 @@ __device__ __forceinline__ void ld_f32_coherent(const float* p, float (&f)[4]) {
     f[0] = v.x; f[1] = v.y; f[2] = v.z; f[3] = v.w;
 }
 
-// Thread -> (row, group): the 8 groups of a row go to consecutive lanes, and the rows are taken in the
-// order 0, 8, 1, 9, ...: the 16 lanes that the LDS serves together then read the partial sums of rows
+// Thread -> (row, group): the 8 (or 16) groups of a row go to consecutive lanes, and the rows are taken in the
+// order 0, 8, 1, 9, ...: the lanes that the LDS serves together then read the partial sums of rows
 // r and r + 8, which are 32 banks apart for every row pitch in use (132, 68, 36, 20 floats).
 __device__ __forceinline__ int group_row(int idx) { return (idx % 2) * 8 + (idx / 2) % 8 + (idx / 16) * 16; }
 
@@ -445,8 +445,11 @@ __global__ __launch_bounds__(kThreads) void rec_fwd_kernel(RecFwdArgs p, RecLayo
     constexpr int JB = 4 * NT;    // hidden units of this slice
     constexpr int NC = 16 * NT;   // gate columns of this slice (i,f,g,o blocks of JB)
     constexpr int PLD = NC + kPartPad;
-    constexpr int UPT = JB / 8;               // hidden units per thread: 8 groups per batch row
-    static_assert(UPT == 2 || UPT == 4, "slices of 16 or 32 hidden units");
+    // cell updates per thread: the slice's units of one batch row are shared by GPR threads; 32 rows x 8 threads,
+    // or 16 rows x 16 threads when a block has one row tile and the slice is wide enough for 2 units each
+    constexpr int GPR = (MT == 1 && JB >= 32) ? 16 : 8;
+    constexpr int UPT = JB / GPR;
+    static_assert(UPT == 2 || UPT == 4, "2 or 4 hidden units per thread");
     typedef Pack<UPT> PackT;
     extern __shared__ __attribute__((aligned(16))) float part_all[];  // [2][4][32][PLD]
     __shared__ int lds_abort;
@@ -475,34 +478,36 @@ __global__ __launch_bounds__(kThreads) void rec_fwd_kernel(RecFwdArgs p, RecLayo
 
     const size_t gld = size_t(4) * p.Hp;
     // this thread's group: row pr of the row block, units pj .. pj+UPT-1 of the slice
-    const int pr = group_row(tid / 8);
-    const int pj = (tid % 8) * UPT;
+    constexpr int RB = 16 * MT;   // batch rows of a row block
+    const int pr = group_row(tid / GPR);
+    const bool row_used = pr < RB;   // with one row tile per block the threads of rows 16..31 only keep the barriers company
+    const int pj = (tid % GPR) * UPT;
     const int j = hs * JB + pj;   // first hidden unit of the group
     const int rb_count = (L.nrb - g + L.ng - 1) / L.ng;
     const bool c_in_regs = (rb_count == 1) && (t_end - t_begin > 1);
     float creg[UPT] = {};
     PackT xp[4];
     auto prefetch = [&](int t, int rb) {   // 4 loads per wave; rows past B fetch row B-1 and are not used
-        const int b = min(rb * kRows + pr, p.B - 1);
+        const int b = min(rb * RB + pr, p.B - 1);
         const half_t* src = p.G + (size_t(t) * p.B + b) * gld + size_t(hs) * NC + pj;
 #pragma unroll
         for (int gt = 0; gt < 4; ++gt) ld_async(xp[gt].v, src + gt * JB);
     };
     if (c_in_regs) {
-        const int b = g * kRows + pr;
-        if (b < p.B) ld_f32_now(p.C + (size_t(t_begin) * p.B + b) * p.Hp + j, creg);
+        const int b = g * RB + pr;
+        if (row_used && b < p.B) ld_f32_now(p.C + (size_t(t_begin) * p.B + b) * p.Hp + j, creg);
     }
     __syncthreads();
     clk.start();
 
     for (int t = t_begin; t < t_end; ++t) {
         for (int rb = g; rb < L.nrb; rb += L.ng, ++item) {
-            const int row0 = rb * kRows;
+            const int row0 = rb * RB;
             float* part = part_all + size_t(item & 1) * 4 * kRows * PLD;
             const half_t* xin = p.X + size_t(t & 3) * p.x_slot;          // h_{t-1}, fragment-major
             half_t* xout = p.X + size_t((t + 1) & 3) * p.x_slot;         // h_t
             half_t* xnext = p.X + size_t((t + 3) & 3) * p.x_slot;        // will take h_{t+2}: marked unwritten
-            const half_t* a0 = xin + size_t(2 * rb) * nks_total * 512 + lane * 8;
+            const half_t* a0 = xin + size_t(MT * rb) * nks_total * 512 + lane * 8;
             const half_t* a1 = a0 + size_t(nks_total) * 512;
             floatx4 acc[2][NT];
 #pragma unroll
@@ -526,10 +531,9 @@ __global__ __launch_bounds__(kThreads) void rec_fwd_kernel(RecFwdArgs p, RecLayo
             clk.lap(4);
             const int b = row0 + pr;
             const unsigned xoff = unsigned(xch_offset(b, j, nks_total));   // 32 bits: a slot is far below 4G halfs
-            const bool row_used = (MT == 2) || pr < 16;   // rows nobody fetches are not exchanged
             if (row_used) store_xch(xnext + xoff, pack_fill(kUnwritten, (PackT*)nullptr), device_scope);
             PackT act[4], hnew = pack_fill(0u, (PackT*)nullptr);   // batch rows past B travel as zeros
-            const bool live = b < p.B;
+            const bool live = row_used && b < p.B;
             if (live) {
                 float z[4][UPT];
 #pragma unroll
@@ -594,8 +598,9 @@ __global__ __launch_bounds__(kThreads) void rec_bwd_kernel(RecBwdArgs p, RecLayo
     constexpr int JB = 16 * NT;  // hidden units (= output columns of dG*W_hh) of this slice
     constexpr int PLD = JB + kPartPad;
     constexpr int KR = KS - KL;  // k-steps whose weight fragments stay in registers
-    constexpr int UPT = JB / 8;               // hidden units per thread: 8 groups per batch row
-    static_assert(UPT == 2 || UPT == 4, "slices of 16 or 32 hidden units");
+    constexpr int GPR = (MT == 1 && JB >= 32) ? 16 : 8;   // threads per batch row (as in the forward kernel)
+    constexpr int UPT = JB / GPR;
+    static_assert(UPT == 2 || UPT == 4, "2 or 4 hidden units per thread");
     typedef Pack<UPT> PackT;
     extern __shared__ __attribute__((aligned(16))) float part_all[];  // [2][4][32][PLD], reused for db
     __shared__ int lds_abort;
@@ -634,22 +639,24 @@ __global__ __launch_bounds__(kThreads) void rec_bwd_kernel(RecBwdArgs p, RecLayo
     const size_t gld = size_t(4) * p.Hp;
     const int JF = p.jb_fwd;   // a multiple of 4: a group never straddles two blocks of the packed gate order
     // this thread's group: row pr of the row block, units pj .. pj+UPT-1 of the slice
-    const int pr = group_row(tid / 8);
-    const int pj = (tid % 8) * UPT;
+    constexpr int RB = 16 * MT;   // batch rows of a row block
+    const int pr = group_row(tid / GPR);
+    const bool row_used = pr < RB;   // with one row tile per block the threads of rows 16..31 only keep the barriers company
+    const int pj = (tid % GPR) * UPT;
     const int j = hs * JB + pj;
     const size_t pq = size_t(j / JF) * 4 * JF + (j % JF);   // packed gate column of (unit j, gate 0)
     const int rb_count = (L.nrb - g + L.ng - 1) / L.ng;
     const bool dc_in_regs = (rb_count == 1) && (t_first - t_last > 0);
     float dcreg[UPT] = {};
     if (dc_in_regs) {
-        const int b = g * kRows + pr;
-        if (b < p.B) ld_f32_now(p.dC + size_t(b) * p.Hp + j, dcreg);
+        const int b = g * RB + pr;
+        if (row_used && b < p.B) ld_f32_now(p.dC + size_t(b) * p.Hp + j, dcreg);
     }
     // prefetched per work item: activated gates, c_{t-1}, c_t, dY_t
     PackT pg[4], pdy;
     F32<UPT> pcp_r, pcc_r;
     auto prefetch = [&](int t, int rb) {   // 7 loads per wave; rows past B fetch row B-1, the closing pass step 0
-        const int b = min(rb * kRows + pr, p.B - 1);
+        const int b = min(rb * RB + pr, p.B - 1);
         const int tt = max(t, 0);
         const half_t* gsrc = p.G + (size_t(tt) * p.B + b) * gld + pq;
 #pragma unroll
@@ -665,13 +672,13 @@ __global__ __launch_bounds__(kThreads) void rec_bwd_kernel(RecBwdArgs p, RecLayo
     for (int t = t_first; t >= t_last; --t) {
         const bool from_product = (t < p.T - 1);
         for (int rb = g; rb < L.nrb; rb += L.ng, ++item) {
-            const int row0 = rb * kRows;
+            const int row0 = rb * RB;
             float* part = part_all + size_t(item & 1) * 4 * kRows * PLD;
             // ring slot of step u is (u + 8) & 3: this step reads dG_{t+1}, writes dG_t and marks the
             // slot of dG_{t-2} unwritten
             if (from_product) {
                 const half_t* xin = p.X + size_t((t + 9) & 3) * p.x_slot;   // dG_{t+1}, fragment-major
-                const half_t* a0 = xin + size_t(2 * rb) * nks_total * 512 + lane * 8;
+                const half_t* a0 = xin + size_t(MT * rb) * nks_total * 512 + lane * 8;
                 const half_t* a1 = a0 + size_t(nks_total) * 512;
                 floatx4 acc[2][NT];
 #pragma unroll
@@ -696,13 +703,12 @@ __global__ __launch_bounds__(kThreads) void rec_bwd_kernel(RecBwdArgs p, RecLayo
             settle(pcc_r.v);
             clk.lap(4);
             const int b = row0 + pr;
-            const bool live = b < p.B;
+            const bool live = row_used && b < p.B;
             const size_t sidx = size_t(b) * p.Hp + j;
             half_t* xout = p.X + size_t((t + 8) & 3) * p.x_slot;    // dG_t for the peers
             half_t* xnext = p.X + size_t((t + 6) & 3) * p.x_slot;   // will take dG_{t-2}
             unsigned xoff[4];   // 32 bits: a slot is far below 4G halfs
             PackT dgnew[4];
-            const bool row_used = (MT == 2) || pr < 16;   // rows nobody fetches are not exchanged
             if (t >= 0 && row_used) {
                 // every peer has delivered dG_{t+1}, so all of them are done reading dG_{t+2}: mark its slot
                 // (the wait above has drained the marks of the previous step)
@@ -789,8 +795,8 @@ __global__ __launch_bounds__(kThreads) void rec_bwd_kernel(RecBwdArgs p, RecLayo
     clk.flush();
     // single-step launches leave dc in memory for the next launch
     if (dc_in_regs && t_last >= 0) {
-        const int b = g * kRows + pr;
-        if (b < p.B) st_f32(p.dC + size_t(b) * p.Hp + j, dcreg);
+        const int b = g * RB + pr;
+        if (row_used && b < p.B) st_f32(p.dC + size_t(b) * p.Hp + j, dcreg);
     }
 
     // Bias gradient: fold this launch's sums over the threads that share a group column (fixed order).
@@ -801,10 +807,10 @@ __global__ __launch_bounds__(kThreads) void rec_bwd_kernel(RecBwdArgs p, RecLayo
 #pragma unroll
         for (int u = 0; u < UPT; ++u) red[tid * (4 * UPT) + gt * UPT + u] = dbacc[gt][u];
     __syncthreads();
-    if (tid < 8 * 4 * UPT) {
+    if (tid < GPR * 4 * UPT) {
         const int gc = tid / (4 * UPT), e = tid % (4 * UPT);  // group column, (gate, unit)
         float sum = 0.f;
-        for (int k = gc; k < kThreads; k += 8) sum += red[k * (4 * UPT) + e];
+        for (int k = gc; k < kThreads; k += GPR) sum += red[k * (4 * UPT) + e];
         const int gt = e / UPT, u = e % UPT;
         const int ju = hs * JB + gc * UPT + u;
         const size_t q = size_t(ju / JF) * 4 * JF + size_t(gt) * JF + (ju % JF);
@@ -845,9 +851,13 @@ int rec_bwd_ks(const RecLayout&, int Hp) { return int(ceil_div(size_t(Hp) / 8, 4
 
 static void finish_layout(RecLayout& L, int B, int Hp, int num_cus, bool force_stepwise, bool fits) {
     L.nh = Hp / L.jb;
-    L.nrb = int(ceil_div(size_t(B), size_t(kRows)));
     L.resident = fits ? 1 : 0;
-    L.mt = (fits && B <= 16) ? 1 : 2;
+    // Row blocks of 16 rows (one MFMA row tile) when all of them can run side by side: twice the workgroups
+    // of 32-row blocks, each with half the product, fetch and cell-update work per step.
+    const bool xcd_mode = (num_cus == 256 && L.nh <= 32);
+    const int side_by_side = L.nh > num_cus ? 0 : (xcd_mode ? 8 * (32 / L.nh) : num_cus / L.nh);
+    L.mt = (fits && int(ceil_div(size_t(B), 16)) <= side_by_side) ? 1 : 2;
+    L.nrb = int(ceil_div(size_t(B), size_t(16 * L.mt)));
     L.xcd_local = 0;
     L.gpx = 0;
     if (!fits || force_stepwise || L.nh > num_cus) {
@@ -914,7 +924,6 @@ hipError_t launch_rec_fwd(const RecLayout& L, const RecFwdArgs& a, hipStream_t s
     if (a.T <= 0 || a.B <= 0 || a.t1 <= a.t0) return hipSuccess;
     if (a.Hp % 32 != 0 || a.Hp % L.jb != 0 || a.t0 < 0 || a.t1 > a.T) return hipErrorInvalidValue;
     if (!L.resident) return run_fwd<8, 1, false, 2>(L, a, stream);
-    if (L.mt == 1 && a.B > 16) return hipErrorInvalidValue;
     if (L.nt == 8) return L.mt == 1 ? run_fwd<8, 8, true, 1>(L, a, stream) : run_fwd<8, 8, true, 2>(L, a, stream);
     if (L.nt == 4) return L.mt == 1 ? run_fwd<4, 16, true, 1>(L, a, stream) : run_fwd<4, 16, true, 2>(L, a, stream);
     return hipErrorInvalidValue;
@@ -944,7 +953,6 @@ hipError_t launch_rec_bwd(const RecLayout& L, const RecBwdArgs& a, hipStream_t s
     if (a.T <= 0 || a.B <= 0 || a.t_hi < a.t_lo) return hipSuccess;
     if (a.Hp % 32 != 0 || a.Hp % L.jb != 0 || a.t_lo < -1 || a.t_hi >= a.T) return hipErrorInvalidValue;
     if (!L.resident) return run_bwd<2, 1, false, 0, 2>(L, a, stream);
-    if (L.mt == 1 && a.B > 16) return hipErrorInvalidValue;
     if (L.nt == 2) return L.mt == 1 ? run_bwd<2, 32, true, 8, 1>(L, a, stream) : run_bwd<2, 32, true, 8, 2>(L, a, stream);
     if (L.nt == 1) return L.mt == 1 ? run_bwd<1, 64, true, 24, 1>(L, a, stream) : run_bwd<1, 64, true, 24, 2>(L, a, stream);
     return hipErrorInvalidValue;
