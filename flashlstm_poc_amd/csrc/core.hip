@@ -130,7 +130,6 @@ extern "C" int flstm_core_create(size_t batch, size_t input_size, size_t hidden_
     p->d.Ip = int(round_up(input_size, 64));
     p->d.Hp = int(round_up(hidden_size, 32));
     replan(p);
-    p->d.JF = p->Lf.jb;
     e = p->status.reserve(64);
     if (e == hipSuccess) e = hipMemset(p->status.p, 0, 64);
     if (e == hipSuccess) e = p->tm.init();
@@ -197,7 +196,6 @@ extern "C" long flstm_core_get_info(const flstm_core_plan* p, const char* name) 
     if (!strcmp(name, "clock_khz")) return p->clock_khz;
     if (!strcmp(name, "hidden_padded")) return p->d.Hp;
     if (!strcmp(name, "input_padded")) return p->d.Ip;
-    if (!strcmp(name, "gate_slice")) return p->d.JF;
     return -1;
 }
 
@@ -427,7 +425,7 @@ int backward_recur(flstm_core_plan* p, long t_hi, long t_lo, hipStream_t s) {
     a.status = p->status.as<int>();
     a.seats = p->status.as<unsigned>() + 8;
     FL_TRY(fill_zero(a.seats, 8 * sizeof(unsigned), s));
-    a.B = d.B; a.Hp = d.Hp; a.T = int(p->bw.T); a.jb_fwd = d.JF; a.dy_scale = p->bw.dy_scale;
+    a.B = d.B; a.Hp = d.Hp; a.T = int(p->bw.T); a.dy_scale = p->bw.dy_scale;
     a.t_hi = int(t_hi); a.t_lo = int(t_lo);
     a.spin_limit = p->opt_spin_limit;
     a.prof = p->opt_profile ? p->prof.as<long long>() + 8 : nullptr;

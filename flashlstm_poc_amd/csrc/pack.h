@@ -5,12 +5,12 @@
 
 namespace flstm_hip {
 
-// Packed gate order: hidden units are cut into slices of JF; slice s holds its i,f,g,o rows next to
-// each other:  q = (j / JF) * 4JF + gate * JF + j % JF.   PyTorch row of (gate, j) is gate*H + j.
+// Packed gate order of the gate arrays (x-projection / gate cache, dG) and of everything indexed like them (rows
+// of the packed W_ih, bias, contraction index of the backward products): the four gates of a hidden unit are
+// neighbours, q = 4 * j + gate.   PyTorch row of (gate, j) is gate*H + j.
 struct Dims {
     int B, I, H;     // caller sizes
     int Ip, Hp;      // I rounded up to 64, H rounded up to 32
-    int JF;          // slice width of the packed gate order
 };
 
 // Replaces src/kernels.cu:57-84 (pack_weights_kernel) and :45-55 (combine_bias_kernel): fp32

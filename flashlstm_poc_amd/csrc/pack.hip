@@ -9,10 +9,12 @@ constexpr int kT = 256;
 
 __host__ __device__ inline int grid_for(size_t n) { return int((n + kT - 1) / kT); }
 
-// packed gate column -> PyTorch weight row, or -1 for a padding unit
-__device__ __forceinline__ int torch_row(int q, int JF, int H) {
-    const int blk = q / (4 * JF), rem = q % (4 * JF);
-    const int gate = rem / JF, j = blk * JF + rem % JF;
+// Column q of the gate arrays (x-projection / gate cache, dG, and with them the rows of the packed W_ih, the bias
+// and the contraction index of the backward products) -> PyTorch weight row, or -1 for a padding unit.  The four
+// gates of a hidden unit are neighbours, q = 4 * unit + gate, so a thread that owns a few consecutive units moves
+// all of their gate values with one 16-byte access.
+__device__ __forceinline__ int torch_row(int q, int H) {
+    const int j = q / 4, gate = q % 4;
     return j < H ? gate * H + j : -1;
 }
 
@@ -22,14 +24,16 @@ __global__ void pack_wih_kernel(Dims d, const float* __restrict__ w_ih, half_t* 
     const size_t total = size_t(4) * d.Hp * d.Ip;
     if (idx >= total) return;
     const int q = int(idx / d.Ip), i = int(idx % d.Ip);
-    const int row = torch_row(q, d.JF, d.H);
+    const int row = torch_row(q, d.H);
     const float v = (row >= 0 && i < d.I) ? w_ih[size_t(row) * d.I + i] : 0.f;
     wih_p[idx] = (half_t)v;
     wih_t[size_t(i) * 4 * d.Hp + q] = (half_t)v;
 }
 
-// Forward fragments: B operand of  gates[b][q] += h[b][k] * W_hh[row(q)][k].
-// fragment (hs, wave, ks, n): lane l holds column q = hs*16*NT + n*16 + l%16,
+// Forward fragments: B operand of  gates[b][c] += h[b][k] * W_hh[row(c)][k].  The product's columns are local to
+// a workgroup (they only meet the pointwise stage through LDS) and stay gate-major within the slice of JB = 4*NT
+// units: column c = gate * JB + unit.
+// fragment (hs, wave, ks, n): lane l holds column c = n*16 + l%16 of slice hs,
 // k = (ks*4 + wave)*32 + 8*(l/16) + e, e = 0..7.
 __global__ void pack_wfrag_fwd_kernel(Dims d, const float* __restrict__ w_hh, half_t* __restrict__ out,
                                       int ks_wave, int nt) {
@@ -44,10 +48,10 @@ __global__ void pack_wfrag_fwd_kernel(Dims d, const float* __restrict__ w_hh, ha
     const int ks = int(r % ks_wave); r /= ks_wave;
     const int wave = int(r % 4); r /= 4;
     const int hs = int(r);
-    const int q = hs * 16 * nt + n * 16 + lane % 16;
+    const int jb = 4 * nt, c = n * 16 + lane % 16;
+    const int gate = c / jb, unit = hs * jb + c % jb;
     const int k = (ks * 4 + wave) * 32 + 8 * (lane / 16) + e;
-    const int row = torch_row(q, d.JF, d.H);
-    out[idx] = (half_t)((row >= 0 && k < d.H) ? w_hh[size_t(row) * d.H + k] : 0.f);
+    out[idx] = (half_t)((unit < d.H && k < d.H) ? w_hh[size_t(gate * d.H + unit) * d.H + k] : 0.f);
 }
 
 // Backward fragments: B operand of  dh[b][k] += dG[b][q] * W_hh[row(q)][k].
@@ -70,7 +74,7 @@ __global__ void pack_wfrag_bwd_kernel(Dims d, const float* __restrict__ w_hh, ha
     const int q = (ks * 4 + wave) * 32 + 8 * (lane / 16) + e;
     float v = 0.f;
     if (q < 4 * d.Hp && k < d.H) {
-        const int row = torch_row(q, d.JF, d.H);
+        const int row = torch_row(q, d.H);
         if (row >= 0) v = w_hh[size_t(row) * d.H + k];
     }
     out[idx] = (half_t)v;
@@ -80,7 +84,7 @@ __global__ void pack_bias_kernel(Dims d, const float* __restrict__ b_ih, const f
                                  float* __restrict__ out) {
     const int q = blockIdx.x * kT + threadIdx.x;
     if (q >= 4 * d.Hp) return;
-    const int row = torch_row(q, d.JF, d.H);
+    const int row = torch_row(q, d.H);
     out[q] = row >= 0 ? b_ih[row] + b_hh[row] : 0.f;
 }
 
@@ -150,7 +154,7 @@ __global__ void reduce_dw_kernel(Dims d, const float* __restrict__ partial, int 
     const size_t per = size_t(4) * d.Hp * ncols;
     if (idx >= per) return;
     const int q = int(idx / ncols), n = int(idx % ncols);
-    const int row = torch_row(q, d.JF, d.H);
+    const int row = torch_row(q, d.H);
     if (row < 0 || n >= out_cols) return;
     float s = 0.f;
     for (int z = 0; z < splits; ++z) s += partial[size_t(z) * per + idx];
@@ -162,7 +166,7 @@ __global__ void reduce_db_kernel(Dims d, const float* __restrict__ db_part, int 
                                  float* __restrict__ db_ih, float* __restrict__ db_hh) {
     const int q = blockIdx.x * kT + threadIdx.x;
     if (q >= 4 * d.Hp) return;
-    const int row = torch_row(q, d.JF, d.H);
+    const int row = torch_row(q, d.H);
     if (row < 0) return;
     float s = 0.f;
     for (int g = 0; g < ng; ++g) s += db_part[size_t(g) * 4 * d.Hp + q];

@@ -53,7 +53,6 @@ struct RecBwdArgs {
     unsigned* seats;     // [8] zeroed before every launch
     int* status;
     int B, Hp, T;
-    int jb_fwd;          // hidden units per slice in the packed gate order of G / dG
     float dy_scale;      // factor applied to dY on load (the loss scale, or 1 when dY is pre-scaled)
     int t_hi, t_lo;      // steps t_hi down to t_lo are run by this call; t_lo = -1 adds the closing dh0 product
     int spin_limit;

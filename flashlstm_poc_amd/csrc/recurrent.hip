@@ -319,6 +319,52 @@ __device__ __forceinline__ Pack<4> pack(const float (&f)[4]) {
 __device__ __forceinline__ Pack<2> pack_fill(unsigned w, Pack<2>*) { return Pack<2>{w}; }
 __device__ __forceinline__ Pack<4> pack_fill(unsigned w, Pack<4>*) { return Pack<4>{uintx2{w, w}}; }
 
+// The gate values i, f, g, o of UPT consecutive hidden units as they lie in the gate arrays (x-projection / gate
+// cache, dG): unit-major, 8 bytes per unit, so UPT / 2 accesses of 16 bytes.
+typedef unsigned uintx4 __attribute__((ext_vector_type(4)));
+template <int UPT> struct GateRow { uintx4 v[UPT / 2]; };
+template <int UPT>
+__device__ __forceinline__ void unpack_gates(const GateRow<UPT>& g, float (&z)[4][UPT]) {
+#pragma unroll
+    for (int c = 0; c < UPT / 2; ++c) {
+        unpack_h2(g.v[c].x, z[0][2 * c], z[1][2 * c]);
+        unpack_h2(g.v[c].y, z[2][2 * c], z[3][2 * c]);
+        unpack_h2(g.v[c].z, z[0][2 * c + 1], z[1][2 * c + 1]);
+        unpack_h2(g.v[c].w, z[2][2 * c + 1], z[3][2 * c + 1]);
+    }
+}
+template <int UPT>
+__device__ __forceinline__ GateRow<UPT> pack_gates(const float (&a)[4][UPT]) {
+    GateRow<UPT> g;
+#pragma unroll
+    for (int c = 0; c < UPT / 2; ++c)
+        g.v[c] = uintx4{pack_h2(a[0][2 * c], a[1][2 * c]), pack_h2(a[2][2 * c], a[3][2 * c]),
+                        pack_h2(a[0][2 * c + 1], a[1][2 * c + 1]), pack_h2(a[2][2 * c + 1], a[3][2 * c + 1])};
+    return g;
+}
+template <int UPT>
+__device__ __forceinline__ GateRow<UPT> gates_fill(unsigned w) {
+    GateRow<UPT> g;
+#pragma unroll
+    for (int c = 0; c < UPT / 2; ++c) g.v[c] = uintx4{w, w, w, w};
+    return g;
+}
+template <int UPT>
+__device__ __forceinline__ void st_gates(half_t* p, const GateRow<UPT>& g) {
+#pragma unroll
+    for (int c = 0; c < UPT / 2; ++c) *reinterpret_cast<uintx4*>(p + 8 * c) = g.v[c];
+}
+// 16 bytes into the exchange ring (see below: every 32-bit word is validated on its own)
+__device__ __forceinline__ void store_xch16(half_t* dst, uintx4 v, bool device_scope) {
+    if (device_scope) {
+        // one write-through store (device scope); issued by hand: there is no 16-byte atomic store to ask the
+        // compiler for, and of two 8-byte ones it emitted the second without the scope bit
+        asm volatile("global_store_dwordx4 %0, %1, off sc1" ::"v"(dst), "v"(v) : "memory");
+    } else {
+        *reinterpret_cast<uintx4*>(dst) = v;
+    }
+}
+
 // One group into the exchange ring.  Consumers validate every 32-bit word on its own, so the two words
 // of an 8-byte group need not become visible together.
 __device__ __forceinline__ void store_xch(half_t* dst, Pack<2> v, bool device_scope) {
@@ -390,6 +436,9 @@ __device__ __forceinline__ void ld_async(uintx2& d, const void* p) {
 }
 __device__ __forceinline__ void ld_async(floatx2& d, const void* p) {
     asm volatile("global_load_dwordx2 %0, %1, off" : "=v"(d) : "v"(p) : "memory");
+}
+__device__ __forceinline__ void ld_async(uintx4& d, const void* p) {
+    asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(d) : "v"(p) : "memory");
 }
 __device__ __forceinline__ void ld_async(floatx4& d, const void* p) {
     asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(d) : "v"(p) : "memory");
@@ -486,12 +535,12 @@ __global__ __launch_bounds__(kThreads) void rec_fwd_kernel(RecFwdArgs p, RecLayo
     const int rb_count = (L.nrb - g + L.ng - 1) / L.ng;
     const bool c_in_regs = (rb_count == 1) && (t_end - t_begin > 1);
     float creg[UPT] = {};
-    PackT xp[4];
-    auto prefetch = [&](int t, int rb) {   // 4 loads per wave; rows past B fetch row B-1 and are not used
+    GateRow<UPT> xp;
+    auto prefetch = [&](int t, int rb) {   // UPT / 2 loads per wave; rows past B fetch row B-1 and are not used
         const int b = min(rb * RB + pr, p.B - 1);
-        const half_t* src = p.G + (size_t(t) * p.B + b) * gld + size_t(hs) * NC + pj;
+        const half_t* src = p.G + (size_t(t) * p.B + b) * gld + size_t(4) * j;
 #pragma unroll
-        for (int gt = 0; gt < 4; ++gt) ld_async(xp[gt].v, src + gt * JB);
+        for (int c = 0; c < UPT / 2; ++c) ld_async(xp.v[c], src + 8 * c);
     };
     if (c_in_regs) {
         const int b = g * RB + pr;
@@ -514,7 +563,7 @@ __global__ __launch_bounds__(kThreads) void rec_fwd_kernel(RecFwdArgs p, RecLayo
             for (int m = 0; m < 2; ++m)
 #pragma unroll
                 for (int n = 0; n < NT; ++n) acc[m][n] = floatx4{0.f, 0.f, 0.f, 0.f};
-            wave_product<NT, KS, RESIDENT, 0, 4, MT>(acc, wreg, nullptr, wfrag_wave, a0, a1, wave, lane, nks_total,
+            wave_product<NT, KS, RESIDENT, 0, UPT / 2, MT>(acc, wreg, nullptr, wfrag_wave, a0, a1, wave, lane, nks_total,
                                                      ks_wave, poll, [&]() { prefetch(t, rb); });
             clk.lap(0);
             spill_partials<NT, MT>(part, acc, wave, lane, PLD);
@@ -527,21 +576,19 @@ __global__ __launch_bounds__(kThreads) void rec_fwd_kernel(RecFwdArgs p, RecLayo
             // of the previous step, so that mark is in place before this step's h_t goes out.
             wait_all_vm();   // the x-projection of this step, issued during the product
 #pragma unroll
-            for (int gt = 0; gt < 4; ++gt) settle(xp[gt].v);
+            for (int c = 0; c < UPT / 2; ++c) settle(xp.v[c]);
             clk.lap(4);
             const int b = row0 + pr;
             const unsigned xoff = unsigned(xch_offset(b, j, nks_total));   // 32 bits: a slot is far below 4G halfs
             if (row_used) store_xch(xnext + xoff, pack_fill(kUnwritten, (PackT*)nullptr), device_scope);
-            PackT act[4], hnew = pack_fill(0u, (PackT*)nullptr);   // batch rows past B travel as zeros
+            GateRow<UPT> act;
+            PackT hnew = pack_fill(0u, (PackT*)nullptr);   // batch rows past B travel as zeros
             const bool live = row_used && b < p.B;
             if (live) {
                 float z[4][UPT];
+                unpack_gates(xp, z);
 #pragma unroll
                 for (int gt = 0; gt < 4; ++gt) {
-                    float x[UPT];
-                    unpack(xp[gt], x);
-#pragma unroll
-                    for (int u = 0; u < UPT; ++u) z[gt][u] = x[u];
 #pragma unroll
                     for (int w = 0; w < 4; ++w) {
                         float v[UPT];
@@ -569,8 +616,7 @@ __global__ __launch_bounds__(kThreads) void rec_fwd_kernel(RecFwdArgs p, RecLayo
                     a4[0][u] = ig; a4[1][u] = fg; a4[2][u] = gg; a4[3][u] = og;
                 }
                 hnew = pack(hn);
-#pragma unroll
-                for (int gt = 0; gt < 4; ++gt) act[gt] = pack(a4[gt]);
+                act = pack_gates(a4);
             }
             // the exchanged value goes out first
             if (row_used) store_xch(xout + xoff, hnew, device_scope);
@@ -579,9 +625,7 @@ __global__ __launch_bounds__(kThreads) void rec_fwd_kernel(RecFwdArgs p, RecLayo
             if (live) {
                 st_f32(p.C + (size_t(t + 1) * p.B + b) * p.Hp + j, creg);
                 st_pack(p.Y + (size_t(t + 1) * p.B + b) * p.Hp + j, hnew);
-                half_t* dst = p.G + (size_t(t) * p.B + b) * gld + size_t(hs) * NC + pj;
-#pragma unroll
-                for (int gt = 0; gt < 4; ++gt) st_pack(dst + gt * JB, act[gt]);
+                st_gates(p.G + (size_t(t) * p.B + b) * gld + size_t(4) * j, act);
             }
             clk.lap(3);
         }
@@ -637,14 +681,13 @@ __global__ __launch_bounds__(kThreads) void rec_bwd_kernel(RecBwdArgs p, RecLayo
     }
 
     const size_t gld = size_t(4) * p.Hp;
-    const int JF = p.jb_fwd;   // a multiple of 4: a group never straddles two blocks of the packed gate order
     // this thread's group: row pr of the row block, units pj .. pj+UPT-1 of the slice
     constexpr int RB = 16 * MT;   // batch rows of a row block
     const int pr = group_row(tid / GPR);
     const bool row_used = pr < RB;   // with one row tile per block the threads of rows 16..31 only keep the barriers company
     const int pj = (tid % GPR) * UPT;
     const int j = hs * JB + pj;
-    const size_t pq = size_t(j / JF) * 4 * JF + (j % JF);   // packed gate column of (unit j, gate 0)
+    const size_t pq = size_t(4) * j;   // column of (unit j, gate 0) in the gate arrays
     const int rb_count = (L.nrb - g + L.ng - 1) / L.ng;
     const bool dc_in_regs = (rb_count == 1) && (t_first - t_last > 0);
     float dcreg[UPT] = {};
@@ -653,14 +696,16 @@ __global__ __launch_bounds__(kThreads) void rec_bwd_kernel(RecBwdArgs p, RecLayo
         if (row_used && b < p.B) ld_f32_now(p.dC + size_t(b) * p.Hp + j, dcreg);
     }
     // prefetched per work item: activated gates, c_{t-1}, c_t, dY_t
-    PackT pg[4], pdy;
+    GateRow<UPT> pg;
+    PackT pdy;
     F32<UPT> pcp_r, pcc_r;
-    auto prefetch = [&](int t, int rb) {   // 7 loads per wave; rows past B fetch row B-1, the closing pass step 0
+    constexpr int NPF = UPT / 2 + 3;
+    auto prefetch = [&](int t, int rb) {   // NPF loads per wave; rows past B fetch row B-1, the closing pass step 0
         const int b = min(rb * RB + pr, p.B - 1);
         const int tt = max(t, 0);
         const half_t* gsrc = p.G + (size_t(tt) * p.B + b) * gld + pq;
 #pragma unroll
-        for (int gt = 0; gt < 4; ++gt) ld_async(pg[gt].v, gsrc + gt * JF);
+        for (int c = 0; c < UPT / 2; ++c) ld_async(pg.v[c], gsrc + 8 * c);
         ld_async(pcp_r.v, p.C + (size_t(tt) * p.B + b) * p.Hp + j);
         ld_async(pcc_r.v, p.C + (size_t(tt + 1) * p.B + b) * p.Hp + j);
         ld_async(pdy.v, p.dY + (size_t(tt) * p.B + b) * p.Hp + j);
@@ -685,7 +730,7 @@ __global__ __launch_bounds__(kThreads) void rec_bwd_kernel(RecBwdArgs p, RecLayo
                 for (int m = 0; m < 2; ++m)
 #pragma unroll
                     for (int n = 0; n < NT; ++n) acc[m][n] = floatx4{0.f, 0.f, 0.f, 0.f};
-                wave_product<NT, KS, RESIDENT, KL, 7, MT>(acc, wreg, wlds, wfrag_wave, a0, a1, wave, lane, nks_total,
+                wave_product<NT, KS, RESIDENT, KL, NPF, MT>(acc, wreg, wlds, wfrag_wave, a0, a1, wave, lane, nks_total,
                                                           ks_wave, poll, [&]() { prefetch(t, rb); });
                 clk.lap(0);
                 spill_partials<NT, MT>(part, acc, wave, lane, PLD);
@@ -697,7 +742,7 @@ __global__ __launch_bounds__(kThreads) void rec_bwd_kernel(RecBwdArgs p, RecLayo
             }
             wait_all_vm();   // gates, cell states and dY of this step, issued during the product
 #pragma unroll
-            for (int gt = 0; gt < 4; ++gt) settle(pg[gt].v);
+            for (int c = 0; c < UPT / 2; ++c) settle(pg.v[c]);
             settle(pdy.v);
             settle(pcp_r.v);
             settle(pcc_r.v);
@@ -707,16 +752,15 @@ __global__ __launch_bounds__(kThreads) void rec_bwd_kernel(RecBwdArgs p, RecLayo
             const size_t sidx = size_t(b) * p.Hp + j;
             half_t* xout = p.X + size_t((t + 8) & 3) * p.x_slot;    // dG_t for the peers
             half_t* xnext = p.X + size_t((t + 6) & 3) * p.x_slot;   // will take dG_{t-2}
-            unsigned xoff[4];   // 32 bits: a slot is far below 4G halfs
-            PackT dgnew[4];
+            unsigned xoff[UPT / 2];   // 32 bits: a slot is far below 4G halfs; 8 columns = 16 contiguous bytes
+            GateRow<UPT> dgnew = gates_fill<UPT>(0u);   // batch rows past B travel as zeros
             if (t >= 0 && row_used) {
                 // every peer has delivered dG_{t+1}, so all of them are done reading dG_{t+2}: mark its slot
                 // (the wait above has drained the marks of the previous step)
 #pragma unroll
-                for (int gt = 0; gt < 4; ++gt) {
-                    xoff[gt] = unsigned(xch_offset(b, int(pq) + gt * JF, nks_total));
-                    dgnew[gt] = pack_fill(0u, (PackT*)nullptr);   // batch rows past B travel as zeros
-                    store_xch(xnext + xoff[gt], pack_fill(kUnwritten, (PackT*)nullptr), device_scope);
+                for (int c = 0; c < UPT / 2; ++c) {
+                    xoff[c] = unsigned(xch_offset(b, int(pq) + 8 * c, nks_total));
+                    store_xch16(xnext + xoff[c], uintx4{kUnwritten, kUnwritten, kUnwritten, kUnwritten}, device_scope);
                 }
             }
             if (live) {
@@ -750,8 +794,7 @@ __global__ __launch_bounds__(kThreads) void rec_bwd_kernel(RecBwdArgs p, RecLayo
                         ld_f32_coherent(p.dC + sidx, dcin);
                     }
                     float gate[4][UPT];
-#pragma unroll
-                    for (int gt = 0; gt < 4; ++gt) unpack(pg[gt], gate[gt]);
+                    unpack_gates(pg, gate);
                     float da[4][UPT];
 #pragma unroll
                     for (int u = 0; u < UPT; ++u) {
@@ -766,27 +809,24 @@ __global__ __launch_bounds__(kThreads) void rec_bwd_kernel(RecBwdArgs p, RecLayo
                         da[3][u] = dov * og * (1.f - og);
                         dcreg[u] = dc * fg;
                     }
+                    // db sums the values the weight-gradient GEMMs will see (fp16-rounded)
+                    dgnew = pack_gates(da);
+                    float r[4][UPT];
+                    unpack_gates(dgnew, r);
 #pragma unroll
-                    for (int gt = 0; gt < 4; ++gt) {
-                        // db sums the values the weight-gradient GEMMs will see (fp16-rounded)
-                        dgnew[gt] = pack(da[gt]);
-                        float r[UPT];
-                        unpack(dgnew[gt], r);
+                    for (int gt = 0; gt < 4; ++gt)
 #pragma unroll
-                        for (int u = 0; u < UPT; ++u) dbacc[gt][u] += r[u];
-                    }
+                        for (int u = 0; u < UPT; ++u) dbacc[gt][u] += r[gt][u];
                 }
             }
             if (t >= 0 && row_used) {
                 // the exchanged values go out first
 #pragma unroll
-                for (int gt = 0; gt < 4; ++gt) store_xch(xout + xoff[gt], dgnew[gt], device_scope);
+                for (int c = 0; c < UPT / 2; ++c) store_xch16(xout + xoff[c], dgnew.v[c], device_scope);
             }
             clk.lap(2);
             if (t >= 0 && live) {   // row-major dG for the GEMMs that follow; running dc when it lives in memory
-                half_t* gdst = p.dG + (size_t(t) * p.B + b) * gld + pq;
-#pragma unroll
-                for (int gt = 0; gt < 4; ++gt) st_pack(gdst + gt * JF, dgnew[gt]);
+                st_gates(p.dG + (size_t(t) * p.B + b) * gld + pq, dgnew);
                 if (!dc_in_regs) st_f32(p.dC + sidx, dcreg);
             }
             clk.lap(3);
@@ -813,7 +853,7 @@ __global__ __launch_bounds__(kThreads) void rec_bwd_kernel(RecBwdArgs p, RecLayo
         for (int k = gc; k < kThreads; k += GPR) sum += red[k * (4 * UPT) + e];
         const int gt = e / UPT, u = e % UPT;
         const int ju = hs * JB + gc * UPT + u;
-        const size_t q = size_t(ju / JF) * 4 * JF + size_t(gt) * JF + (ju % JF);
+        const size_t q = size_t(4) * ju + gt;
         p.db_part[size_t(g) * gld + q] += sum;
     }
 }

@@ -107,7 +107,7 @@ int flstm_core_backward_end(flstm_core_plan* plan, const void* x, flstm_dtype x_
 /* Read access to what forward cached (device pointers, valid until the next forward/destroy):
  *   which = 0: h states fp16 [(T+1)*B][Hp], row t*B+b = h before step t   (ld = *ld)
  *   which = 1: c states fp32 [(T+1)*B][Hp]
- *   which = 2: activated gates fp16 [T*B][4Hp] in the plan's packed gate order */
+ *   which = 2: activated gates fp16 [T*B][4Hp], column 4 * unit + gate (gates i, f, g, o) */
 int flstm_core_cache_ptr(const flstm_core_plan* plan, int which, const void** ptr, size_t* ld);
 
 /* Average device time in milliseconds of the phases of the most recent forward / backward,

@@ -187,7 +187,7 @@ def test_gate_cache_and_state_arrays_hold_what_the_oracle_computes():
     core = LstmCore(B, I, H)
     core.pack(*(p[k].cuda() for k in ("w_ih", "w_hh", "b_ih", "b_hh")))
     core.forward(p["x"].cuda().half(), p["h0"].cuda().half(), p["c0"].cuda().half())
-    Hp, JF = core.info("hidden_padded"), core.info("gate_slice")
+    Hp = core.info("hidden_padded")
 
     def view(which, rows, cols, dtype):
         ptr, ld = ctypes.c_void_p(), ctypes.c_size_t()
@@ -202,10 +202,10 @@ def test_gate_cache_and_state_arrays_hold_what_the_oracle_computes():
     gates = view(2, T * B, 4 * Hp, torch.float16).reshape(T, B, 4 * Hp)
     assert relmax(h_all, f["h_all"]) <= 1e-2 and relmax(c_all, f["c_all"]) <= 1e-2
     np.testing.assert_array_equal(h_all[0], to_np(p["h0"]))          # entry 0 is the initial state
-    # packed gate order: unit j, gate g sits at (j // JF) * 4JF + g * JF + j % JF
+    # packed gate order: unit j, gate g sits at column 4 * j + g
     j = np.arange(H)
     for g in range(4):
-        cols = (j // JF) * 4 * JF + g * JF + j % JF
+        cols = 4 * j + g
         assert relmax(gates[..., cols], f["gates"][..., g * H:(g + 1) * H]) <= 1e-2
     assert gates.min() >= -1.0 and gates.max() <= 1.0
     core.close()
