@@ -225,7 +225,7 @@ def main():
     # calibration against the fp16 output copy of the same run); see profiles/*_hbm_traffic.md
     GiB = float(1 << 30)
     traffic_config3 = {"fwd_proj": (3.01 + 1.25) * GiB, "bwd_dx": (3.01 + 1.25) * GiB, "fwd_rec": (2.07 + 3.55) * GiB,
-                       "bwd_rec": (3.57 + 4.39) * GiB, "bwd_dw": 2 * (3.06 + 0.25) * GiB}
+                       "bwd_rec": (3.57 + 4.37) * GiB, "bwd_dw": 2 * (3.03 + 0.0625) * GiB}
     kernels = []
     for k in phases:
         tf = kflops[k] / (phase_ms[k] * 1e-3) / 1e12 if phase_ms[k] > 0 else 0.0
