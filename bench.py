@@ -262,7 +262,8 @@ def main():
     # What the recurrence moves between workgroups each step: every workgroup (16 or 32 batch rows x one slice of hidden
     # units) fetches the whole h_{t-1} (forward) or dG_{t+1} (backward) of its rows from the L2, and passes its
     # fp32 partial sums (4 waves, written once and read once) through LDS.
-    Hp, rows = core.info("hidden_padded"), 16 * core.info("row_tiles") * ((B + 31) // 32)
+    block = 16 * core.info("row_tiles")   # batch rows per workgroup
+    Hp, rows = core.info("hidden_padded"), block * ((B + block - 1) // block)
     xch = {}
     for d, k_cols, gate_cols in (("fwd", Hp, 4), ("bwd", 4 * Hp, 1)) if backward else (("fwd", Hp, 4),):
         us = phase_ms[d + "_rec"] * 1e3 / T
