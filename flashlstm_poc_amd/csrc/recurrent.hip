@@ -533,8 +533,9 @@ __global__ __launch_bounds__(kThreads) void rec_fwd_kernel(RecFwdArgs p, RecLayo
     const int pj = (tid % GPR) * UPT;
     const int j = hs * JB + pj;   // first hidden unit of the group
     const int rb_count = (L.nrb - g + L.ng - 1) / L.ng;
-    const bool c_in_regs = (rb_count == 1) && (t_end - t_begin > 1);
-    float creg[UPT] = {};
+    // the cell state of the workgroup's first and second row block stays in registers for the whole launch
+    const bool c_in_regs = (rb_count <= 2) && (t_end - t_begin > 1);
+    float creg[UPT] = {}, creg2[UPT] = {};
     GateRow<UPT> xp;
     auto prefetch = [&](int t, int rb) {   // UPT / 2 loads per wave; rows past B fetch row B-1 and are not used
         const int b = min(rb * RB + pr, p.B - 1);
@@ -543,8 +544,9 @@ __global__ __launch_bounds__(kThreads) void rec_fwd_kernel(RecFwdArgs p, RecLayo
         for (int c = 0; c < UPT / 2; ++c) ld_async(xp.v[c], src + 8 * c);
     };
     if (c_in_regs) {
-        const int b = g * RB + pr;
+        const int b = g * RB + pr, b2 = (g + L.ng) * RB + pr;
         if (row_used && b < p.B) ld_f32_now(p.C + (size_t(t_begin) * p.B + b) * p.Hp + j, creg);
+        if (rb_count == 2 && row_used && b2 < p.B) ld_f32_now(p.C + (size_t(t_begin) * p.B + b2) * p.Hp + j, creg2);
     }
     __syncthreads();
     clk.start();
@@ -582,6 +584,7 @@ __global__ __launch_bounds__(kThreads) void rec_fwd_kernel(RecFwdArgs p, RecLayo
             const unsigned xoff = unsigned(xch_offset(b, j, nks_total));   // 32 bits: a slot is far below 4G halfs
             if (row_used) store_xch(xnext + xoff, pack_fill(kUnwritten, (PackT*)nullptr), device_scope);
             GateRow<UPT> act;
+            float cnew[UPT] = {};
             PackT hnew = pack_fill(0u, (PackT*)nullptr);   // batch rows past B travel as zeros
             const bool live = row_used && b < p.B;
             if (live) {
@@ -597,10 +600,11 @@ __global__ __launch_bounds__(kThreads) void rec_fwd_kernel(RecFwdArgs p, RecLayo
                         for (int u = 0; u < UPT; ++u) z[gt][u] += v[u];
                     }
                 }
+                const bool second = (rb != g);
                 float cp[UPT];
                 if (c_in_regs) {
 #pragma unroll
-                    for (int u = 0; u < UPT; ++u) cp[u] = creg[u];
+                    for (int u = 0; u < UPT; ++u) cp[u] = second ? creg2[u] : creg[u];
                 } else {
                     ld_f32_coherent(p.C + (size_t(t) * p.B + b) * p.Hp + j, cp);
                 }
@@ -611,9 +615,11 @@ __global__ __launch_bounds__(kThreads) void rec_fwd_kernel(RecFwdArgs p, RecLayo
                     const float fg = sigmoidf_dev(z[1][u]);
                     const float gg = tanhf_dev(z[2][u]);
                     const float og = sigmoidf_dev(z[3][u]);
-                    creg[u] = fg * cp[u] + ig * gg;
-                    hn[u] = og * tanhf_dev(creg[u]);
+                    cnew[u] = fg * cp[u] + ig * gg;
+                    hn[u] = og * tanhf_dev(cnew[u]);
                     a4[0][u] = ig; a4[1][u] = fg; a4[2][u] = gg; a4[3][u] = og;
+                    if (second) creg2[u] = cnew[u];
+                    else creg[u] = cnew[u];
                 }
                 hnew = pack(hn);
                 act = pack_gates(a4);
@@ -623,7 +629,7 @@ __global__ __launch_bounds__(kThreads) void rec_fwd_kernel(RecFwdArgs p, RecLayo
             clk.lap(2);
             // caches for the backward pass: off the critical path
             if (live) {
-                st_f32(p.C + (size_t(t + 1) * p.B + b) * p.Hp + j, creg);
+                st_f32(p.C + (size_t(t + 1) * p.B + b) * p.Hp + j, cnew);
                 st_pack(p.Y + (size_t(t + 1) * p.B + b) * p.Hp + j, hnew);
                 st_gates(p.G + (size_t(t) * p.B + b) * gld + size_t(4) * j, act);
             }
@@ -689,11 +695,13 @@ __global__ __launch_bounds__(kThreads) void rec_bwd_kernel(RecBwdArgs p, RecLayo
     const int j = hs * JB + pj;
     const size_t pq = size_t(4) * j;   // column of (unit j, gate 0) in the gate arrays
     const int rb_count = (L.nrb - g + L.ng - 1) / L.ng;
-    const bool dc_in_regs = (rb_count == 1) && (t_first - t_last > 0);
-    float dcreg[UPT] = {};
+    // the running dc of the workgroup's first and second row block stays in registers for the whole launch
+    const bool dc_in_regs = (rb_count <= 2) && (t_first - t_last > 0);
+    float dcreg[UPT] = {}, dcreg2[UPT] = {};
     if (dc_in_regs) {
-        const int b = g * RB + pr;
+        const int b = g * RB + pr, b2 = (g + L.ng) * RB + pr;
         if (row_used && b < p.B) ld_f32_now(p.dC + size_t(b) * p.Hp + j, dcreg);
+        if (rb_count == 2 && row_used && b2 < p.B) ld_f32_now(p.dC + size_t(b2) * p.Hp + j, dcreg2);
     }
     // prefetched per work item: activated gates, c_{t-1}, c_t, dY_t
     GateRow<UPT> pg;
@@ -754,6 +762,7 @@ __global__ __launch_bounds__(kThreads) void rec_bwd_kernel(RecBwdArgs p, RecLayo
             half_t* xnext = p.X + size_t((t + 6) & 3) * p.x_slot;   // will take dG_{t-2}
             unsigned xoff[UPT / 2];   // 32 bits: a slot is far below 4G halfs; 8 columns = 16 contiguous bytes
             GateRow<UPT> dgnew = gates_fill<UPT>(0u);   // batch rows past B travel as zeros
+            float dcnew[UPT] = {};
             if (t >= 0 && row_used) {
                 // every peer has delivered dG_{t+1}, so all of them are done reading dG_{t+2}: mark its slot
                 // (the wait above has drained the marks of the previous step)
@@ -781,15 +790,19 @@ __global__ __launch_bounds__(kThreads) void rec_bwd_kernel(RecBwdArgs p, RecLayo
                 } else {
                     ld_f32_now(p.dHn + sidx, dh);
                 }
+                const bool second = (rb != g);
                 if (t < 0) {  // closing pass: gradient wrt h0; dc0 is the running dc
                     st_f32(p.dH0 + sidx, dh);
-                    if (dc_in_regs) st_f32(p.dC + sidx, dcreg);
+                    if (dc_in_regs) {
+                        if (second) st_f32(p.dC + sidx, dcreg2);
+                        else st_f32(p.dC + sidx, dcreg);
+                    }
                 } else {
                     float dy[UPT], dcin[UPT];
                     unpack(pdy, dy);
                     if (dc_in_regs) {
 #pragma unroll
-                        for (int u = 0; u < UPT; ++u) dcin[u] = dcreg[u];
+                        for (int u = 0; u < UPT; ++u) dcin[u] = second ? dcreg2[u] : dcreg[u];
                     } else {
                         ld_f32_coherent(p.dC + sidx, dcin);
                     }
@@ -807,7 +820,9 @@ __global__ __launch_bounds__(kThreads) void rec_bwd_kernel(RecBwdArgs p, RecLayo
                         da[1][u] = dc * pcp[u] * fg * (1.f - fg);
                         da[2][u] = dc * ig * (1.f - gg * gg);
                         da[3][u] = dov * og * (1.f - og);
-                        dcreg[u] = dc * fg;
+                        dcnew[u] = dc * fg;
+                        if (second) dcreg2[u] = dcnew[u];
+                        else dcreg[u] = dcnew[u];
                     }
                     // db sums the values the weight-gradient GEMMs will see (fp16-rounded)
                     dgnew = pack_gates(da);
@@ -827,7 +842,7 @@ __global__ __launch_bounds__(kThreads) void rec_bwd_kernel(RecBwdArgs p, RecLayo
             clk.lap(2);
             if (t >= 0 && live) {   // row-major dG for the GEMMs that follow; running dc when it lives in memory
                 st_gates(p.dG + (size_t(t) * p.B + b) * gld + pq, dgnew);
-                if (!dc_in_regs) st_f32(p.dC + sidx, dcreg);
+                if (!dc_in_regs) st_f32(p.dC + sidx, dcnew);
             }
             clk.lap(3);
         }
@@ -835,8 +850,9 @@ __global__ __launch_bounds__(kThreads) void rec_bwd_kernel(RecBwdArgs p, RecLayo
     clk.flush();
     // single-step launches leave dc in memory for the next launch
     if (dc_in_regs && t_last >= 0) {
-        const int b = g * RB + pr;
+        const int b = g * RB + pr, b2 = (g + L.ng) * RB + pr;
         if (row_used && b < p.B) st_f32(p.dC + size_t(b) * p.Hp + j, dcreg);
+        if (rb_count == 2 && row_used && b2 < p.B) st_f32(p.dC + size_t(b2) * p.Hp + j, dcreg2);
     }
 
     // Bias gradient: fold this launch's sums over the threads that share a group column (fixed order).

@@ -91,7 +91,18 @@ def test_config1_through_fp32_io():
     core.close()
 
 
-@pytest.mark.parametrize("shape", [(12, 40, 32, 64), (20, 16, 64, 1024)])
+@pytest.mark.parametrize("shape", [(6, 300, 32, 1024), (5, 128, 32, 2048), (4, 520, 32, 512)])
+def test_two_row_blocks_per_workgroup_match_torch_lstm(shape):
+    # more row blocks than groups that run side by side: a workgroup walks two (or more) blocks per step and keeps
+    # the cell state of the first two in registers
+    p = make_problem(*shape, seed=5)
+    ref = torch_reference(p, dtype=torch.float32, device="cuda")
+    got, info = run_core(p)
+    assert info["persistent_fwd"] == 1 and info["persistent_bwd"] == 1 and info["fallbacks"] == 0
+    check_against(ref, got, label=str(shape))
+
+
+@pytest.mark.parametrize("shape", [(12, 40, 32, 64), (20, 16, 64, 1024), (6, 300, 32, 1024), (5, 128, 32, 2048)])
 def test_persistent_and_stepwise_agree(shape):
     p = make_problem(*shape, seed=3)
     a, ia = run_core(p, stepwise=False)
