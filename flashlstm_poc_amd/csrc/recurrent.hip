@@ -5,11 +5,14 @@
 // flashlstm_v2/src/lstm_backward.cu:1057-1101 + :158-227) is done here by ONE kernel launch for
 // the whole sequence:
 //
-//  * Work split.  The batch is cut into blocks of 32 rows and the hidden dimension into slices of
-//    JB units.  A workgroup (4 wavefronts, one per SIMD, up to 512 registers each) owns one slice
-//    for all row blocks of its group, i.e. all four gates of its hidden units, so the cell update
-//    is local.  Its part of W_hh (forward: 4*JB gate rows x Hp; backward: 4Hp gate rows x JB
-//    columns) is loaded once into registers as ready-made MFMA B-fragments and stays there.
+//  * Work split.  The batch is cut into blocks of 32 rows (two 16-row MFMA tiles; blocks of 16 rows
+//    when all of those can run side by side, which halves every workgroup's work per step) and the
+//    hidden dimension into slices of JB units.  A workgroup (4 wavefronts, one per SIMD, up to 512
+//    registers each) owns one slice for all row blocks of its group, i.e. all four gates of its
+//    hidden units, so the cell update is local; the cell state of its first two row blocks never
+//    leaves registers.  Its part of W_hh (forward: 4*JB gate rows x Hp; backward: 4Hp gate rows x
+//    JB columns) is loaded once into registers (and, backward, partly LDS) as ready-made MFMA
+//    B-fragments and stays there.
 //  * K split.  The four wavefronts split the contraction dimension (interleaved 32-wide k-steps),
 //    so every element of h_{t-1} / dG_{t+1} is fetched exactly once per workgroup, straight from
 //    L2 into A-fragments; partial sums meet in LDS (fp32) and the pointwise stage reads them there.
