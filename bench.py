@@ -40,38 +40,115 @@ def make_inputs(T, B, I, H, seed=0):
                 h0=(n(B, H) * 0.1).half(), c0=(n(B, H) * 0.1).half(), dy=n(T, B, H).half())
 
 
-def parity_check(B, I, H, T=32):
-    """Same kernels at a short length against fp32 torch.nn.LSTM on the fp16-rounded operands."""
+def parity_check(p, outputs, grads):
+    """The tensors that were just timed (same x, h0, c0, dY, T) through fp32 torch.nn.LSTM on the GPU with the same
+    fp16-rounded weights; `outputs` / `grads` are what the last timed step produced.  Max relative error on y, h_T,
+    c_T, relative L2 on the gradients; the last time step's y is listed on its own (h is fed back through fp16)."""
     import torch
-    from flashlstm_poc_amd import LstmCore
-    p = make_inputs(T, B, I, H, seed=1)
-    core = LstmCore(B, I, H)
-    core.pack(p["w_ih"], p["w_hh"], p["b_ih"], p["b_hh"])
-    y, hy, cy = core.forward(p["x"], p["h0"], p["c0"])
-    dx, dW_ih, dW_hh, db, dh0, dc0 = core.backward(p["x"], p["dy"])
+    T, B, I = p["x"].shape
+    H = p["w_hh"].shape[1]
     m = torch.nn.LSTM(I, H, device="cuda")
     with torch.no_grad():
         m.weight_ih_l0.copy_(p["w_ih"].half().float()); m.weight_hh_l0.copy_(p["w_hh"].half().float())
         m.bias_ih_l0.copy_(p["b_ih"]); m.bias_hh_l0.copy_(p["b_hh"])
-    xr = p["x"].float().requires_grad_(True)
-    hr = p["h0"].float().requires_grad_(True); cr = p["c0"].float().requires_grad_(True)
+    want_grads = grads is not None
+    xr = p["x"].float().requires_grad_(want_grads)
+    hr = p["h0"].float().requires_grad_(want_grads); cr = p["c0"].float().requires_grad_(want_grads)
     yr, (hn, cn) = m(xr, (hr[None], cr[None]))
-    (yr * p["dy"].float()).sum().backward()
     relmax = lambda a, b: ((a.float() - b.float()).abs().max() / b.float().abs().max()).item()
-    rell2 = lambda a, b: ((a.float() - b.float()).norm() / b.float().norm()).item()
-    errs = {"y": relmax(y, yr), "h_T": relmax(hy, hn[0]), "c_T": relmax(cy, cn[0]), "dx": rell2(dx, xr.grad),
-            "dW_ih": rell2(dW_ih, m.weight_ih_l0.grad), "dW_hh": rell2(dW_hh, m.weight_hh_l0.grad),
-            "db": rell2(db, m.bias_ih_l0.grad), "dh0": rell2(dh0, hr.grad), "dc0": rell2(dc0, cr.grad)}
-    core.close()
+    rell2 = lambda a, b: ((a.double() - b.double()).norm() / b.double().norm()).item()
+    y, hy, cy = outputs
+    errs = {"y": relmax(y, yr), "y_last_step": relmax(y[-1], yr[-1]), "h_T": relmax(hy, hn[0]), "c_T": relmax(cy, cn[0])}
+    if want_grads:
+        (yr * p["dy"].float()).sum().backward()
+        dx, dW_ih, dW_hh, db, dh0, dc0 = grads
+        errs.update({"dx": rell2(dx, xr.grad), "dW_ih": rell2(dW_ih, m.weight_ih_l0.grad),
+                     "dW_hh": rell2(dW_hh, m.weight_hh_l0.grad), "db": rell2(db, m.bias_ih_l0.grad),
+                     "dh0": rell2(dh0, hr.grad), "dc0": rell2(dc0, cr.grad)})
     worst = max(errs.values())
-    return {"T": T, "max_err": round(worst, 6), "tolerance": 1e-2, "ok": bool(worst <= 1e-2)}
+    return {"on": "the timed tensors", "T": T, "reference": "torch.nn.LSTM fp32 on the GPU, fp16-rounded weights",
+            "errors": {k: float(f"{v:.3e}") for k, v in errs.items()}, "max_err": float(f"{worst:.3e}"),
+            "tolerance": 1e-2, "ok": bool(worst <= 1e-2)}
 
 
-def cpu_baseline(B, I, H, backward, budget_s=20.0):
-    """torch.nn.LSTM (fp32, CPU) on this host's cores, on a time-bounded sample of the same workload:
-    same B, I, H and seeded inputs, reduced T (LSTM cost is linear in T)."""
+def kernel_source_digest():
+    """First 16 hex digits of the SHA-256 over the kernel sources (csrc/*.hip, csrc/*.h, sorted by name): ties a
+    counter profile under profiles/ to the code it was taken from."""
+    import glob
+    import hashlib
+    h = hashlib.sha256()
+    d = os.path.join(ROOT, "flashlstm_poc_amd", "csrc")
+    for f in sorted(glob.glob(os.path.join(d, "*.hip")) + glob.glob(os.path.join(d, "*.h"))):
+        h.update(os.path.basename(f).encode())
+        h.update(open(f, "rb").read())
+    return h.hexdigest()[:16]
+
+
+def measured_traffic(workload, phase):
+    """HBM-side bytes per launch of a phase's kernels from the committed counter summary
+    profiles/hbm_traffic_per_kernel.md (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, calibrated against a copy kernel).
+    None unless that summary was taken from exactly the kernel sources that are running now."""
+    import re
+    path = os.path.join(ROOT, "profiles", "hbm_traffic_per_kernel.md")
+    try:
+        text = open(path).read()
+        block = re.search(r"```json traffic\n(.*?)```", text, flags=re.S)
+        data = json.loads(block.group(1))
+    except Exception:
+        return None, "no counter summary"
+    if data.get("kernel_source_digest") != kernel_source_digest():
+        return None, f"counter summary is from other kernel sources ({data.get('kernel_source_digest')})"
+    try:
+        return float(data["bytes_per_launch"][workload][phase]), data.get("taken", "")
+    except Exception:
+        return None, "phase not in the counter summary"
+
+
+def cpu_model():
+    try:
+        for line in open("/proc/cpuinfo"):
+            if line.startswith("model name"):
+                return line.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    return "unknown"
+
+
+def cpu_baseline(B, I, H, backward, budget_s=15.0):
+    """torch.nn.LSTM (fp32, CPU) on this host's cores.  Two figures: BASELINE config 1 exactly (I=128, H=256, B=8,
+    T=64, seed 0, h0=c0=0, loss = sum(y^2); 3 warm-ups, 20 repeats, forward and forward+backward), and a
+    time-bounded sample of the benchmarked workload: same B, I, H and seeded inputs at reduced T (LSTM cost is
+    linear in T).  `value` is the sample's rate, comparable with the GPU line."""
     import torch
     threads = torch.get_num_threads()
+
+    def timed(fn, warm, reps):
+        for _ in range(warm):
+            fn()
+        t0 = time.perf_counter()
+        for _ in range(reps):
+            fn()
+        return (time.perf_counter() - t0) / reps
+
+    # config 1
+    torch.manual_seed(0)
+    m1 = torch.nn.LSTM(128, 256)
+    x1 = torch.randn(64, 8, 128, requires_grad=True)
+
+    def c1_fwd():
+        with torch.no_grad():
+            m1(x1)
+
+    def c1_fwdbwd():
+        m1.zero_grad(set_to_none=True)
+        x1.grad = None
+        y, _ = m1(x1)
+        (y ** 2).sum().backward()
+
+    c1f = timed(c1_fwd, 3, 20)
+    c1fb = timed(c1_fwdbwd, 3, 20)
+
+    # sample of the benchmarked workload
     T = 8
     torch.manual_seed(0)
     m = torch.nn.LSTM(I, H)
@@ -87,15 +164,18 @@ def cpu_baseline(B, I, H, backward, budget_s=20.0):
 
     once()  # warm-up
     t0 = time.perf_counter(); once(); probe = time.perf_counter() - t0
-    reps = max(1, min(20, int(budget_s / max(probe, 1e-3))))
-    t0 = time.perf_counter()
-    for _ in range(reps):
-        once()
-    dt = (time.perf_counter() - t0) / reps
+    reps = max(3, min(20, int(budget_s / max(probe, 1e-3))))
+    dt = timed(once, 2, reps)
     return {"value": round(B * T / dt, 1), "unit": "batch*timesteps/s", "cores": threads, "kind": "port",
             "impl": "torch.nn.LSTM fp32 on CPU (the oracle named for this path)",
+            "cpu_model": cpu_model(), "os_cpu_count": os.cpu_count(), "torch_num_threads": threads,
+            "torch_version": torch.__version__,
             "sample": f"same B={B}, I={I}, H={H}, {'fwd+bwd' if backward else 'fwd'}, T reduced to {T}, "
-                      f"{reps} repeats after 1 warm-up, {dt * 1e3:.1f} ms each; os.cpu_count()={os.cpu_count()}"}
+                      f"{reps} repeats after 4 untimed runs, {dt * 1e3:.1f} ms each",
+            "config1": {"workload": "I=128, H=256, B=8, T=64, fp32, seed 0, loss=sum(y^2)", "warmups": 3, "repeats": 20,
+                        "fwd_ms": round(c1f * 1e3, 3), "fwd_bwd_ms": round(c1fb * 1e3, 3),
+                        "fwd_batch_timesteps_per_s": round(512 / c1f, 1),
+                        "fwd_bwd_batch_timesteps_per_s": round(512 / c1fb, 1)}}
 
 
 def bench_stack(args, device):
@@ -189,10 +269,12 @@ def main():
     core = LstmCore(B, I, H)
     core.pack(p["w_ih"], p["w_hh"], p["b_ih"], p["b_hh"])
 
+    last = {}
+
     def step():
-        core.forward(p["x"], p["h0"], p["c0"], save_for_backward=backward)
+        last["out"] = core.forward(p["x"], p["h0"], p["c0"], save_for_backward=backward)
         if backward:
-            core.backward(p["x"], p["dy"])
+            last["grads"] = core.backward(p["x"], p["dy"])
 
     for _ in range(args.warmup):
         step()
@@ -221,20 +303,16 @@ def main():
     kname = {"fwd_proj": "gemm_nt_stream (X*W_ih^T + bias)", "fwd_rec": "rec_fwd_kernel (persistent recurrence)",
              "bwd_rec": "rec_bwd_kernel (persistent BPTT)", "bwd_dx": "gemm_nt_stream (dG*W_ih)",
              "bwd_dw": "gemm_tn_256x256 split-K x2 (dG^T*X, dG^T*H) + reduce_dw"}
-    # HBM-side traffic per launch at config3 from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (x2.0 / x1.0 after
-    # calibration against the fp16 output copy of the same run); see profiles/*_hbm_traffic.md
-    GiB = float(1 << 30)
-    traffic_config3 = {"fwd_proj": (3.01 + 1.25) * GiB, "bwd_dx": (3.01 + 1.25) * GiB, "fwd_rec": (2.07 + 3.55) * GiB,
-                       "bwd_rec": (3.57 + 4.37) * GiB, "bwd_dw": 2 * (3.03 + 0.0625) * GiB}
     kernels = []
     for k in phases:
         tf = kflops[k] / (phase_ms[k] * 1e-3) / 1e12 if phase_ms[k] > 0 else 0.0
         kernels.append({"phase": k, "kernel": kname[k], "ms": round(phase_ms[k], 4), "tflops": round(tf, 1),
                         "frac_of_peak": round(tf / PEAK_FP16_TFLOPS, 4)})
     dom = max(kernels, key=lambda d: d["ms"])
+    traffic, traffic_note = measured_traffic(args.workload, dom["phase"])
     roofline = {"kernel": dom["kernel"], "bound": "mfma", "achieved": dom["tflops"], "peak": PEAK_FP16_TFLOPS,
                 "unit": "TFLOP/s", "frac": dom["frac_of_peak"],
-                "traffic": traffic_config3[dom["phase"]] if args.workload == "config3" else None,
+                "traffic": traffic, "traffic_source": traffic_note,
                 "traffic_unit": "bytes per launch (fetched + written beyond the L2)",
                 "launch_ms": dom["ms"], "flops_per_launch": kflops[dom["phase"]]}
     if dom["phase"] in ("fwd_rec", "bwd_rec"):
@@ -274,8 +352,10 @@ def main():
                   "lds_bytes_per_step": lds_bytes, "lds_gb_per_s": round(lds_bytes / us / 1e3, 1)}
     out["exchange_per_step"] = xch
     core.close()
+    out["kernel_source_digest"] = kernel_source_digest()
     if not args.no_parity:
-        out["parity"] = parity_check(B, I, H)
+        out["parity"] = parity_check(p, last["out"], last.get("grads"))
+    last.clear()
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(B, I, H, backward)
     print(json.dumps(out))

@@ -24,6 +24,7 @@ struct V1Impl {
     flstm_core_plan* plan;   // null when any dimension is zero
     hipStream_t stream;
     bool weights_packed;
+    size_t cached_T;         // sequence length of the forward pass whose caches the plan holds (0 = none)
 };
 
 constexpr int kInvalid = int(hipErrorInvalidValue);
@@ -55,6 +56,7 @@ extern "C" int lstm_create_buffers(lstm_compute_precision_t precision, size_t se
     impl->mode = LSTM_EXECUTION_MODE_IMMEDIATE;
     impl->plan = nullptr;
     impl->stream = nullptr;
+    impl->cached_T = 0;
     const bool empty = (batch == 0 || input_size == 0 || hidden_size == 0);
     impl->weights_packed = (hidden_size == 0 || input_size + hidden_size == 0);
     if (!empty) {
@@ -133,8 +135,19 @@ extern "C" int lstm_forward(const float* x, const float* b_ih, const float* b_hh
     int rc = flstm_core_pack_bias(impl->plan, b_ih, b_hh, impl->stream);
     if (rc) return rc;
     flstm_hip::RangeGuard compute("FlashLSTM::lstm_forward::compute");
-    return flstm_core_forward(impl->plan, seq_len, x, FLSTM_F32, h0, c0, FLSTM_F32, output, FLSTM_F32, hn, cn,
-                              FLSTM_F32, 1, impl->stream);
+    impl->cached_T = 0;
+    rc = flstm_core_forward(impl->plan, seq_len, x, FLSTM_F32, h0, c0, FLSTM_F32, output, FLSTM_F32, hn, cn,
+                            FLSTM_F32, 1, impl->stream);
+    if (rc == 0) impl->cached_T = seq_len;
+    return rc;
+}
+
+extern "C" int lstm_get_cache(const lstm_buffers* buffers, int which, const void** ptr, size_t* ld, size_t* seq_len) {
+    if (!buffers || !buffers->impl || !ptr || !ld) return kInvalid;
+    auto* impl = static_cast<V1Impl*>(buffers->impl);
+    if (!impl->plan || impl->cached_T == 0) return kInvalid;
+    if (seq_len) *seq_len = impl->cached_T;
+    return flstm_core_cache_ptr(impl->plan, which, ptr, ld);
 }
 
 extern "C" int lstm_backward(const float* x, const float* d_output, const float* d_hn, const float* d_cn,

@@ -13,8 +13,11 @@
 // 0 = whole window).
 //
 // Backward needs the gate cache of the steps it walks.  With one window, forward keeps it on the device in a
-// small registry and a backward call that names the same host buffers (and whose sampled contents still
-// match) reuses it; any other backward call first recomputes the forward pass from x, h0 and c0.  With several
+// small registry, and a backward call reuses it when it names the same buffers AND their contents are what
+// the forward pass saw: the device tensors (both weight matrices, both biases, h0, c0) are checksummed in full
+// on the device by either call, the host buffers x and y at 16 sampled places; any other backward call first
+// recomputes the forward pass from x, h0 and c0 (FLASHLSTM_V2_RECOMPUTE=1 forces that).  What the sampled
+// check cannot see is a rewrite of x or y between the two calls that misses all 16 samples.  With several
 // windows, backward takes them last to first and recomputes each window's forward pass from the state at the
 // window's start: the one the forward call left on the device when the registry matches, otherwise the host
 // checkpoint at or before it (flashlstm_v2/src/lstm_backward.cu:897-1056 recomputes from the checkpoints in
@@ -28,6 +31,7 @@
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
+#include <iterator>
 #include <list>
 #include <mutex>
 #include <stdexcept>
@@ -67,7 +71,7 @@ struct ForwardKey {
     const void *x = nullptr, *y = nullptr, *ch = nullptr, *cc = nullptr, *h0 = nullptr, *c0 = nullptr;
     const void *w_ih = nullptr, *w_hh = nullptr;
     size_t T = 0, R = 0, W = 0;
-    unsigned long long x_print = 0, y_print = 0;
+    unsigned long long x_print = 0, y_print = 0, dev_print = 0;
     bool valid = false;
 };
 
@@ -77,6 +81,7 @@ struct Entry {
     flstm_core_plan* plan = nullptr;
     Buf x_dev, y_dev, dy_dev, dx_dev, ck_h, ck_c;
     Buf carry_h, carry_c, carry_dh, carry_dc;   // fp32 (B, H): state / state gradient between windows
+    Buf sum_dev;                                // one 64-bit checksum accumulator
     Buf starts;                                 // fp32 [window][h, c][B * H]: state at the start of each window
     std::vector<char> start_known;              // which entries of `starts` hold the current sequence's states
     ForwardKey last;
@@ -91,9 +96,18 @@ struct Entry {
             chunk_out.push_back(b);
         }
     }
+    size_t device_bytes() const {
+        size_t sum = 0;
+        for (const Buf* b : {&x_dev, &y_dev, &dy_dev, &dx_dev, &ck_h, &ck_c, &carry_h, &carry_c, &carry_dh, &carry_dc,
+                             &starts, &sum_dev})
+            sum += b->bytes;
+        const long held = plan ? flstm_core_get_info(plan, "device_bytes") : 0;
+        return sum + size_t(held > 0 ? held : 0);
+    }
     ~Entry() {
         if (plan) flstm_core_destroy(plan);
-        for (Buf* b : {&x_dev, &y_dev, &dy_dev, &dx_dev, &ck_h, &ck_c, &carry_h, &carry_c, &carry_dh, &carry_dc, &starts})
+        for (Buf* b : {&x_dev, &y_dev, &dy_dev, &dx_dev, &ck_h, &ck_c, &carry_h, &carry_c, &carry_dh, &carry_dc, &starts,
+                       &sum_dev})
             b->release();
         if (ev_in) (void)hipEventDestroy(ev_in);
         if (ev_out) (void)hipEventDestroy(ev_out);
@@ -106,12 +120,32 @@ std::mutex g_mutex;
 std::list<Entry> g_entries;  // most recently used first
 constexpr size_t kMaxEntries = 4;
 
+// Every entry keeps whole-sequence caches alive (8 MiB per step at B = 256, H = 1024), so the registry is bounded
+// in bytes as well as in count: shapes other than the one in use are dropped, least recently used first, while
+// they hold more than FLASHLSTM_V2_REGISTRY_MB together (default: a quarter of the device's memory).
+void trim_registry() {
+    size_t cap = 0;
+    if (const char* v = getenv("FLASHLSTM_V2_REGISTRY_MB")) cap = size_t(atol(v) > 0 ? atol(v) : 0) << 20;
+    if (cap == 0) {
+        size_t free_b = 0, total_b = 0;
+        if (hipMemGetInfo(&free_b, &total_b) != hipSuccess) return;
+        cap = total_b / 4;
+    }
+    while (g_entries.size() > 1) {
+        size_t others = 0;
+        for (auto it = std::next(g_entries.begin()); it != g_entries.end(); ++it) others += it->device_bytes();
+        if (others <= cap) break;
+        g_entries.pop_back();
+    }
+}
+
 Entry& entry_for(size_t B, size_t I, size_t H) {
     int dev = 0;
     check(hipGetDevice(&dev), "hipGetDevice");
     for (auto it = g_entries.begin(); it != g_entries.end(); ++it) {
         if (it->B == B && it->I == I && it->H == H && it->device == dev) {
             g_entries.splice(g_entries.begin(), g_entries, it);
+            trim_registry();
             return g_entries.front();
         }
     }
@@ -122,19 +156,47 @@ Entry& entry_for(size_t B, size_t I, size_t H) {
     check_core(flstm_core_create(B, I, H, &e.plan), "flstm_core_create");
     check(hipEventCreateWithFlags(&e.ev_in, hipEventDisableTiming), "hipEventCreate");
     check(hipEventCreateWithFlags(&e.ev_out, hipEventDisableTiming), "hipEventCreate");
+    trim_registry();
     return e;
 }
 
-// FNV-1a over three 256-byte samples of a host buffer: cheap evidence that it still holds what the
-// cached forward pass saw.
+// FNV-1a over 16 evenly spread 256-byte samples of a host buffer (all of it when it is no longer than that):
+// cheap evidence that it still holds what the cached forward pass saw.
 unsigned long long fingerprint(const void* p, size_t bytes) {
     const unsigned char* b = static_cast<const unsigned char*>(p);
     unsigned long long h = 1469598103934665603ull;
-    const size_t win = bytes < 256 ? bytes : 256;
-    const size_t starts[3] = {0, bytes > win ? (bytes - win) / 2 : 0, bytes - win};
-    for (size_t s : starts)
-        for (size_t i = 0; i < win; ++i) { h ^= b[s + i]; h *= 1099511628211ull; }
+    constexpr size_t kSamples = 16, kWin = 256;
+    if (bytes <= kSamples * kWin) {
+        for (size_t i = 0; i < bytes; ++i) { h ^= b[i]; h *= 1099511628211ull; }
+        return h;
+    }
+    for (size_t k = 0; k < kSamples; ++k) {
+        const size_t s = (bytes - kWin) / (kSamples - 1) * k;
+        for (size_t i = 0; i < kWin; ++i) { h ^= b[s + i]; h *= 1099511628211ull; }
+    }
     return h;
+}
+
+// Checksum over the full contents of the device tensors a pass depends on (computed on the device, 8 bytes come
+// back): weights or initial states updated in place between forward and backward change it.
+unsigned long long device_print(Entry& e, hipStream_t s, const float* w_ih, const float* w_hh, const float* b_ih,
+                                const float* b_hh, const __half* h0, const __half* c0) {
+    using flstm_hip::checksum_add;
+    const size_t G = 4 * e.H;
+    e.sum_dev.reserve(sizeof(unsigned long long));
+    auto* acc = static_cast<flstm_hip::u64*>(e.sum_dev.p);
+    check(flstm_hip::fill_zero(acc, sizeof(unsigned long long), s), "checksum");
+    check(checksum_add(w_ih, G * e.I * sizeof(float), 0x1000000000ull, acc, s), "checksum");
+    check(checksum_add(w_hh, G * e.H * sizeof(float), 0x2000000000ull, acc, s), "checksum");
+    check(checksum_add(b_ih, G * sizeof(float), 0x3000000000ull, acc, s), "checksum");
+    check(checksum_add(b_hh, G * sizeof(float), 0x4000000000ull, acc, s), "checksum");
+    check(checksum_add(h0, e.B * e.H * sizeof(half_t), 0x5000000000ull, acc, s), "checksum");
+    check(checksum_add(c0, e.B * e.H * sizeof(half_t), 0x6000000000ull, acc, s), "checksum");
+    unsigned long long host = 0;
+    check(hipMemcpyAsync(&host, acc, sizeof(host), hipMemcpyDeviceToHost, s), "checksum");
+    check(hipStreamSynchronize(s), "checksum");
+    // which of the optional tensors are present is part of the identity
+    return host ^ (b_ih ? 1ull : 0) ^ (b_hh ? 2ull : 0) ^ (h0 ? 4ull : 0) ^ (c0 ? 8ull : 0);
 }
 
 void validate_common(size_t R, hipStream_t c, hipStream_t h2d, hipStream_t d2h) {
@@ -335,6 +397,7 @@ void run_forward(Entry& e, size_t T, size_t R, const __half* x_host, const __hal
     k.w_ih = w_ih; k.w_hh = w_hh; k.T = T; k.R = R; k.W = W;
     k.x_print = fingerprint(x_host, T * B * I * sizeof(half_t));
     k.y_print = y_host ? fingerprint(y_host, T * B * H * sizeof(half_t)) : 0;
+    k.dev_print = device_print(e, st.cs, w_ih, w_hh, b_ih, b_hh, h0, c0);
     k.valid = true;
     e.last = k;
 }
@@ -483,6 +546,7 @@ void StreamingLstmBackward(size_t T, size_t B, size_t I, size_t H, size_t R, con
                k.cc == cache.c_ptr && k.h0 == h0 && k.c0 == c0 && k.w_ih == w_ih && k.w_hh == w_hh && k.T == T &&
                k.W == W;
     if (hit) hit = (k.x_print == fingerprint(x_host, x_bytes)) && (!y_host || k.y_print == fingerprint(y_host, y_bytes));
+    if (hit) hit = (k.dev_print == device_print(e, cs, w_ih, w_hh, b_ih, b_hh, h0, c0));
     const double fwd_flops_per_step = flstm_hip::gemm_flops(4 * H, B, I + H);
     if (nwin == 1) {
         if (!hit) {

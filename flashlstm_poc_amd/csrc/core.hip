@@ -49,6 +49,8 @@ struct PhaseTimer {
 
 }  // namespace
 
+constexpr int kFirstHold = 8, kMaxHold = 1024;
+
 struct flstm_core_plan {
     int num_cus = 0;
     int clock_khz = 0;   // maximum engine clock the runtime reports
@@ -56,9 +58,14 @@ struct flstm_core_plan {
     RecLayout Lf{}, Lb{};
     int ks_f = 0, ks_b = 0;
     // options
-    int opt_stepwise = 0, opt_proj_chunk = 0, opt_spin_limit = 1 << 22, opt_dw_splits = 0, opt_accumulate = 0;
-    bool broken_fwd = false, broken_bwd = false;  // persistent launch failed once: stay step-wise
-    long fallbacks = 0;
+    int opt_stepwise = 0, opt_proj_chunk = 0, opt_spin_limit = 1 << 30, opt_spin_ms = 250, opt_dw_splits = 0, opt_accumulate = 0;
+    // A persistent launch that gave up (its workgroups were not all running at once, or not spread over the XCDs
+    // as expected) demotes that direction to step-wise launches for `hold` passes; then the persistent kernel is
+    // tried again.  Every further give-up doubles the hold (at most kMaxHold passes).
+    int hold_fwd = 0, hold_bwd = 0, backoff_fwd = kFirstHold, backoff_bwd = kFirstHold;
+    long fallbacks = 0, demotions_fwd = 0, demotions_bwd = 0;
+    int* status_host = nullptr;   // pinned: the device status word lands here with the end-of-pass copy
+    int inject_stall = 0;         // test hook: treat the next N persistent passes as if their launch had given up
     // weights
     DevBuf wih_p, wih_t, wfrag_f, wfrag_b, bias_p;
     bool weights_packed = false, bias_packed = false;
@@ -87,20 +94,49 @@ namespace {
     } while (0)
 
 void replan(flstm_core_plan* p) {
-    p->Lf = plan_rec_fwd(p->d.B, p->d.Hp, p->num_cus, p->opt_stepwise || p->broken_fwd);
-    p->Lb = plan_rec_bwd(p->d.B, p->d.Hp, p->num_cus, p->opt_stepwise || p->broken_bwd);
+    p->Lf = plan_rec_fwd(p->d.B, p->d.Hp, p->num_cus, p->opt_stepwise || p->hold_fwd > 0);
+    p->Lb = plan_rec_bwd(p->d.B, p->d.Hp, p->num_cus, p->opt_stepwise || p->hold_bwd > 0);
     p->ks_f = rec_fwd_ks(p->Lf, p->d.Hp);
     p->ks_b = rec_bwd_ks(p->Lb, p->d.Hp);
 }
 
-int read_status(flstm_core_plan* p, hipStream_t s, int* out) {
-    FL_TRY(hipStreamSynchronize(s));
-    FL_TRY(hipMemcpy(out, p->status.p, sizeof(int), hipMemcpyDeviceToHost));
-    if (*out != 0) {
-        int zero = 0;
-        FL_TRY(hipMemcpy(p->status.p, &zero, sizeof(int), hipMemcpyHostToDevice));
+// The status word of the recurrence kernels travels to pinned host memory behind the pass's last kernel, so the
+// wait that ends the pass anyway is also the one that makes it readable: no second round trip to the device.
+int enqueue_status_copy(flstm_core_plan* p, hipStream_t s) {
+    FL_TRY(hipMemcpyAsync(p->status_host, p->status.p, sizeof(int), hipMemcpyDeviceToHost, s));
+    return 0;
+}
+// after the stream has been waited for: the status of the pass; a non-zero one is cleared on the device
+int take_status(flstm_core_plan* p, bool fwd, hipStream_t s, int* out) {
+    *out = *static_cast<volatile int*>(p->status_host);
+    if (*out != 0) FL_TRY(fill_zero(p->status.p, sizeof(int), s));
+    if (*out == 0 && p->inject_stall > 0 && (fwd ? p->Lf.persistent : p->Lb.persistent)) {
+        p->inject_stall--;
+        *out = 1;
     }
     return 0;
+}
+int wait_status(flstm_core_plan* p, bool fwd, hipStream_t s, int* out) {
+    int rc = enqueue_status_copy(p, s);
+    if (rc) return rc;
+    FL_TRY(hipStreamSynchronize(s));
+    return take_status(p, fwd, s, out);
+}
+
+// A persistent launch gave up: step-wise launches for the next `hold` passes of that direction.
+void demote(flstm_core_plan* p, bool fwd) {
+    int& hold = fwd ? p->hold_fwd : p->hold_bwd;
+    int& backoff = fwd ? p->backoff_fwd : p->backoff_bwd;
+    hold = backoff;
+    backoff = backoff * 2 > kMaxHold ? kMaxHold : backoff * 2;
+    (fwd ? p->demotions_fwd : p->demotions_bwd)++;
+    p->fallbacks++;
+    replan(p);
+}
+// A pass of a demoted direction went through: one pass less to hold; at zero the persistent kernel is back.
+void pass_done(flstm_core_plan* p, bool fwd) {
+    int& hold = fwd ? p->hold_fwd : p->hold_bwd;
+    if (hold > 0 && --hold == 0) replan(p);
 }
 
 float elapsed(hipEvent_t a, hipEvent_t b) {
@@ -123,6 +159,9 @@ extern "C" int flstm_core_create(size_t batch, size_t input_size, size_t hidden_
     if (e == hipSuccess) e = hipDeviceGetAttribute(&p->num_cus, hipDeviceAttributeMultiprocessorCount, dev);
     if (e == hipSuccess && hipDeviceGetAttribute(&p->clock_khz, hipDeviceAttributeClockRate, dev) != hipSuccess)
         p->clock_khz = 0;
+    if (e == hipSuccess && (hipDeviceGetAttribute(&p->wall_khz, hipDeviceAttributeWallClockRate, dev) != hipSuccess ||
+                            p->wall_khz <= 0))
+        p->wall_khz = 100000;
     if (e != hipSuccess) { delete p; return int(e); }
     p->d.B = int(batch);
     p->d.I = int(input_size);
@@ -132,6 +171,8 @@ extern "C" int flstm_core_create(size_t batch, size_t input_size, size_t hidden_
     replan(p);
     e = p->status.reserve(64);
     if (e == hipSuccess) e = hipMemset(p->status.p, 0, 64);
+    if (e == hipSuccess) e = hipHostMalloc(reinterpret_cast<void**>(&p->status_host), 64, hipHostMallocDefault);
+    if (e == hipSuccess) p->status_host[0] = 0;
     if (e == hipSuccess) e = p->tm.init();
     if (e != hipSuccess) { flstm_core_destroy(p); return int(e); }
     *out = p;
@@ -145,6 +186,7 @@ extern "C" int flstm_core_destroy(flstm_core_plan* p) {
                       &p->dH0, &p->db_part, &p->dw_part, &p->prof})
         b->release();
     p->tm.destroy();
+    if (p->status_host) (void)hipHostFree(p->status_host);
     delete p;
     return 0;
 }
@@ -154,17 +196,15 @@ extern "C" int flstm_core_set_option(flstm_core_plan* p, const char* name, long 
     if (!strcmp(name, "stepwise")) { p->opt_stepwise = value != 0; replan(p); return 0; }
     if (!strcmp(name, "proj_chunk")) { p->opt_proj_chunk = int(value); return 0; }
     if (!strcmp(name, "spin_limit")) { if (value < 1) return FLSTM_E_INVALID; p->opt_spin_limit = int(value); return 0; }
+    if (!strcmp(name, "spin_ms")) { if (value < 1 || value > 60000) return FLSTM_E_INVALID; p->opt_spin_ms = int(value); return 0; }
     if (!strcmp(name, "profile")) {
         p->opt_profile = value != 0;
         if (p->opt_profile) {
             FL_TRY(p->prof.reserve(16 * sizeof(long long)));
-            int dev = 0;
-            FL_TRY(hipGetDevice(&dev));
-            (void)hipDeviceGetAttribute(&p->wall_khz, hipDeviceAttributeWallClockRate, dev);
-            if (p->wall_khz <= 0) p->wall_khz = 100000;
         }
         return 0;
     }
+    if (!strcmp(name, "inject_stall")) { if (value < 0) return FLSTM_E_INVALID; p->inject_stall = int(value); return 0; }
     if (!strcmp(name, "dw_splits")) { if (value < 0) return FLSTM_E_INVALID; p->opt_dw_splits = int(value); return 0; }
     if (!strcmp(name, "accumulate_grads")) { p->opt_accumulate = value != 0; return 0; }
     return FLSTM_E_INVALID;
@@ -192,6 +232,10 @@ extern "C" long flstm_core_get_info(const flstm_core_plan* p, const char* name) 
     if (!strcmp(name, "groups_fwd")) return p->Lf.ng;
     if (!strcmp(name, "groups_bwd")) return p->Lb.ng;
     if (!strcmp(name, "fallbacks")) return p->fallbacks;
+    if (!strcmp(name, "demotions_fwd")) return p->demotions_fwd;
+    if (!strcmp(name, "demotions_bwd")) return p->demotions_bwd;
+    if (!strcmp(name, "hold_fwd")) return p->hold_fwd;
+    if (!strcmp(name, "hold_bwd")) return p->hold_bwd;
     if (!strcmp(name, "num_cus")) return p->num_cus;
     if (!strcmp(name, "clock_khz")) return p->clock_khz;
     if (!strcmp(name, "hidden_padded")) return p->d.Hp;
@@ -302,6 +346,7 @@ int forward_recur(flstm_core_plan* p, size_t t0, size_t n, hipStream_t s) {
     FL_TRY(fill_zero(a.seats, 8 * sizeof(unsigned), s));
     a.B = d.B; a.Hp = d.Hp; a.T = int(p->fw.T); a.t0 = int(t0); a.t1 = int(t0 + n);
     a.spin_limit = p->opt_spin_limit;
+    a.spin_ticks = (long long)p->opt_spin_ms * p->wall_khz;
     a.prof = p->opt_profile ? p->prof.as<long long>() : nullptr;
     FL_TRY(launch_rec_fwd(p->Lf, a, s));
     return 0;
@@ -336,34 +381,28 @@ extern "C" int flstm_core_forward(flstm_core_plan* p, size_t T, const void* x, f
     const size_t TB = T * size_t(d.B);
     p->have_cache = false;
 
-    int rc = forward_once(p, T, x, x_dtype, h0, c0, state_dtype, s);
-    if (rc) return rc;
-    int st = 0;
-    rc = read_status(p, s, &st);
-    if (rc) return rc;
-    if (st != 0) {
-        if (!p->Lf.persistent) return FLSTM_E_STALLED;
-        // persistent launch gave up (workgroups not co-resident or not where expected): redo step-wise
-        p->broken_fwd = true;
-        p->fallbacks++;
-        replan(p);
-        rc = forward_once(p, T, x, x_dtype, h0, c0, state_dtype, s);
+    // The outputs are written behind the recurrence without waiting for its status: if the persistent launch gave
+    // up, the whole pass is repeated step-wise and overwrites them.
+    for (int attempt = 0;; ++attempt) {
+        int rc = forward_once(p, T, x, x_dtype, h0, c0, state_dtype, s);
         if (rc) return rc;
-        rc = read_status(p, s, &st);
+        FL_TRY(unpad_from_half(p->Y.as<half_t>() + size_t(d.B) * d.Hp, size_t(d.Hp), TB, d.H, y, y_dtype == FLSTM_F32, s));
+        FL_TRY(unpad_from_half(p->Y.as<half_t>() + TB * d.Hp, size_t(d.Hp), size_t(d.B), d.H, hy,
+                               out_state_dtype == FLSTM_F32, s));
+        FL_TRY(unpad_from_float(p->C.as<float>() + TB * d.Hp, size_t(d.Hp), size_t(d.B), d.H, 1.f, cy,
+                                out_state_dtype == FLSTM_F32, s));
+        int st = 0;
+        rc = wait_status(p, true, s, &st);
         if (rc) return rc;
-        if (st != 0) return FLSTM_E_STALLED;
+        if (st == 0) break;
+        if (!p->Lf.persistent || attempt > 0) return FLSTM_E_STALLED;
+        demote(p, true);   // workgroups not co-resident or not where expected: redo with one launch per step
     }
+    pass_done(p, true);
     if (p->opt_profile) FL_TRY(hipMemcpy(p->prof_f, p->prof.p, sizeof(p->prof_f), hipMemcpyDeviceToHost));
     p->ms_fwd[0] = elapsed(p->tm.ev[0], p->tm.ev[1]);
     p->ms_fwd[1] = elapsed(p->tm.ev[1], p->tm.ev[2]);
     p->ms_fwd[2] = elapsed(p->tm.ev[0], p->tm.ev[2]);
-
-    FL_TRY(unpad_from_half(p->Y.as<half_t>() + size_t(d.B) * d.Hp, size_t(d.Hp), TB, d.H, y, y_dtype == FLSTM_F32, s));
-    FL_TRY(unpad_from_half(p->Y.as<half_t>() + TB * d.Hp, size_t(d.Hp), size_t(d.B), d.H, hy,
-                           out_state_dtype == FLSTM_F32, s));
-    FL_TRY(unpad_from_float(p->C.as<float>() + TB * d.Hp, size_t(d.Hp), size_t(d.B), d.H, 1.f, cy,
-                            out_state_dtype == FLSTM_F32, s));
-    FL_TRY(hipStreamSynchronize(s));
     p->fw.open = false;
     if (save_for_backward) { p->have_cache = true; p->T_cache = T; }
     return 0;
@@ -428,6 +467,7 @@ int backward_recur(flstm_core_plan* p, long t_hi, long t_lo, hipStream_t s) {
     a.B = d.B; a.Hp = d.Hp; a.T = int(p->bw.T); a.dy_scale = p->bw.dy_scale;
     a.t_hi = int(t_hi); a.t_lo = int(t_lo);
     a.spin_limit = p->opt_spin_limit;
+    a.spin_ticks = (long long)p->opt_spin_ms * p->wall_khz;
     a.prof = p->opt_profile ? p->prof.as<long long>() + 8 : nullptr;
     FL_TRY(launch_rec_bwd(p->Lb, a, s));
     return 0;
@@ -511,6 +551,8 @@ int backward_finish(flstm_core_plan* p, const void* x, flstm_dtype x_dtype, floa
     FL_TRY(unpad_from_float(p->dH0.as<float>(), size_t(d.Hp), size_t(d.B), d.H, invS, dh0, 1, s));
     FL_TRY(unpad_from_float(p->dC.as<float>(), size_t(d.Hp), size_t(d.B), d.H, invS, dc0, 1, s));
     FL_TRY(hipEventRecord(p->tm.ev[7], s));
+    int rc = enqueue_status_copy(p, s);
+    if (rc) return rc;
     FL_TRY(hipStreamSynchronize(s));
     p->bw.open = false;
     return 0;
@@ -531,27 +573,31 @@ extern "C" int flstm_core_backward(flstm_core_plan* p, size_t T, const void* x, 
     hipStream_t s = static_cast<hipStream_t>(stream);
     const float S = grad_scale > 0.f ? grad_scale : 1.f;
 
-    int rc = backward_rec_once(p, T, dY, dy_dtype, d_hn, d_cn, dstate_dtype, S, dx, dx_dtype, s);
-    if (rc) return rc;
-    int st = 0;
-    rc = read_status(p, s, &st);
-    if (rc) return rc;
-    if (st != 0) {
-        if (!p->Lb.persistent) return FLSTM_E_STALLED;
-        p->broken_bwd = true;
-        p->fallbacks++;
-        replan(p);
-        rc = backward_rec_once(p, T, dY, dy_dtype, d_hn, d_cn, dstate_dtype, S, dx, dx_dtype, s);
+    // dX and the weight gradients follow the recurrence without waiting for its status (one wait per pass); a
+    // persistent launch that gave up is found at the end and the pass repeated step-wise over the same outputs.
+    // Only when the caller's gradients are added to (accumulate_grads) the status is checked first.
+    for (int attempt = 0;; ++attempt) {
+        int rc = backward_rec_once(p, T, dY, dy_dtype, d_hn, d_cn, dstate_dtype, S, dx, dx_dtype, s);
         if (rc) return rc;
-        rc = read_status(p, s, &st);
-        if (rc) return rc;
-        if (st != 0) return FLSTM_E_STALLED;
+        int st = 0;
+        if (p->opt_accumulate) {
+            rc = wait_status(p, false, s, &st);
+            if (rc) return rc;
+        }
+        if (st == 0) {
+            rc = backward_dx(p, long(T) - 1, 0, s);
+            if (rc) return rc;
+            FL_TRY(hipEventRecord(p->tm.ev[5], s));
+            rc = backward_finish(p, x, x_dtype, dW_ih, dW_hh, db_ih, db_hh, dh0, dc0, s);
+            if (rc) return rc;
+            rc = take_status(p, false, s, &st);
+            if (rc) return rc;
+            if (st == 0) break;
+        }
+        if (!p->Lb.persistent || attempt > 0) return FLSTM_E_STALLED;
+        demote(p, false);
     }
-    rc = backward_dx(p, long(T) - 1, 0, s);
-    if (rc) return rc;
-    FL_TRY(hipEventRecord(p->tm.ev[5], s));
-    rc = backward_finish(p, x, x_dtype, dW_ih, dW_hh, db_ih, db_hh, dh0, dc0, s);
-    if (rc) return rc;
+    pass_done(p, false);
     if (p->opt_profile)
         FL_TRY(hipMemcpy(p->prof_b, p->prof.as<long long>() + 8, sizeof(p->prof_b), hipMemcpyDeviceToHost));
     p->ms_bwd[0] = elapsed(p->tm.ev[3], p->tm.ev[4]);
@@ -589,18 +635,18 @@ extern "C" int flstm_core_forward_end(flstm_core_plan* p, void* hy, void* cy, fl
     const Dims& d = p->d;
     const size_t TB = p->fw.T * size_t(d.B);
     p->fw.open = false;
-    int st = 0;
-    int rc = read_status(p, s, &st);
-    if (rc) return rc;
-    if (st != 0) {   // a persistent launch gave up: the caller repeats the pass through flstm_core_forward
-        if (p->Lf.persistent) { p->broken_fwd = true; p->fallbacks++; replan(p); }
-        return FLSTM_E_STALLED;
-    }
     FL_TRY(unpad_from_half(p->Y.as<half_t>() + TB * d.Hp, size_t(d.Hp), size_t(d.B), d.H, hy,
                            out_state_dtype == FLSTM_F32, s));
     FL_TRY(unpad_from_float(p->C.as<float>() + TB * d.Hp, size_t(d.Hp), size_t(d.B), d.H, 1.f, cy,
                             out_state_dtype == FLSTM_F32, s));
-    FL_TRY(hipStreamSynchronize(s));
+    int st = 0;
+    int rc = wait_status(p, true, s, &st);
+    if (rc) return rc;
+    if (st != 0) {   // a persistent launch gave up: the caller repeats the pass through flstm_core_forward
+        if (p->Lf.persistent) demote(p, true);
+        return FLSTM_E_STALLED;
+    }
+    pass_done(p, true);
     if (save_for_backward) { p->have_cache = true; p->T_cache = p->fw.T; }
     return 0;
 }
@@ -631,15 +677,19 @@ extern "C" int flstm_core_backward_end(flstm_core_plan* p, const void* x, flstm_
     if (!p || !p->bw.open) return FLSTM_E_INVALID;
     if (dW_ih && !x) return FLSTM_E_INVALID;
     hipStream_t s = static_cast<hipStream_t>(stream);
+    // the caller's gradients may be accumulated into: the status of the recurrence is checked before they are touched
     int st = 0;
-    int rc = read_status(p, s, &st);
+    int rc = wait_status(p, false, s, &st);
     if (rc) return rc;
     if (st != 0) {   // the caller repeats the pass through flstm_core_backward
         p->bw.open = false;
-        if (p->Lb.persistent) { p->broken_bwd = true; p->fallbacks++; replan(p); }
+        if (p->Lb.persistent) demote(p, false);
         return FLSTM_E_STALLED;
     }
-    return backward_finish(p, x, x_dtype, dW_ih, dW_hh, db_ih, db_hh, dh0, dc0, s);
+    rc = backward_finish(p, x, x_dtype, dW_ih, dW_hh, db_ih, db_hh, dh0, dc0, s);
+    if (rc) return rc;
+    pass_done(p, false);
+    return 0;
 }
 
 extern "C" int flstm_core_cache_ptr(const flstm_core_plan* p, int which, const void** ptr, size_t* ld) {
@@ -667,4 +717,51 @@ extern "C" double flstm_core_last_ms(const flstm_core_plan* p, const char* phase
     if (!strncmp(phase, "bwd_clk", 7) && phase[7] >= '0' && phase[7] <= '7')
         return double(p->prof_b[phase[7] - '0']) / p->wall_khz;
     return -1.0;
+}
+
+// ---- the GEMMs the passes are built from, callable on their own
+
+extern "C" int flstm_gemm_nt(const void* A, size_t lda, const void* B, size_t ldb, size_t M, size_t N, size_t K,
+                             void* C, flstm_dtype c_dtype, size_t ldc, float alpha, const float* bias, void* stream) {
+    if (!A || !B || !C || M > (1u << 30) || N > (1u << 30) || K > (1u << 30)) return FLSTM_E_INVALID;
+    GemmNT g{};
+    g.A = static_cast<const half_t*>(A); g.lda = lda;
+    g.B = static_cast<const half_t*>(B); g.ldb = ldb;
+    g.M = int(M); g.N = int(N); g.K = int(K);
+    if (c_dtype == FLSTM_F32) g.C32 = static_cast<float*>(C);
+    else g.C16 = static_cast<half_t*>(C);
+    g.ldc = ldc; g.alpha = alpha; g.splits = 1; g.split_stride = 0; g.bias = bias;
+    if (lda < K || ldb < K || ldc < N) return FLSTM_E_INVALID;
+    FL_TRY(launch_gemm_nt(g, static_cast<hipStream_t>(stream)));
+    return 0;
+}
+
+extern "C" size_t flstm_gemm_tn_workspace_bytes(size_t M, size_t N, size_t K, int splits) {
+    if (splits <= 1 || K == 0 || K > (1u << 30)) return 0;
+    const int eff = gemm_effective_splits(int(K), splits);
+    return eff <= 1 ? 0 : size_t(eff) * M * N * sizeof(float);
+}
+
+extern "C" int flstm_gemm_tn(const void* A, size_t lda, const void* B, size_t ldb, size_t M, size_t N, size_t K,
+                             float* C, size_t ldc, float alpha, int splits, void* workspace, void* stream) {
+    if (!A || !B || !C || M > (1u << 30) || N > (1u << 30) || K > (1u << 30)) return FLSTM_E_INVALID;
+    if (lda < M || ldb < N || ldc < N) return FLSTM_E_INVALID;
+    if (M == 0 || N == 0 || K == 0) return 0;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const int eff = gemm_effective_splits(int(K), splits < 1 ? 1 : splits);
+    GemmNT g{};
+    g.A = static_cast<const half_t*>(A); g.lda = lda;
+    g.B = static_cast<const half_t*>(B); g.ldb = ldb;
+    g.M = int(M); g.N = int(N); g.K = int(K);
+    g.alpha = alpha; g.bias = nullptr;
+    if (eff <= 1) {
+        g.C32 = C; g.ldc = ldc; g.splits = 1; g.split_stride = 0;
+        FL_TRY(launch_gemm_tn(g, s));
+        return 0;
+    }
+    if (!workspace) return FLSTM_E_INVALID;
+    g.C32 = static_cast<float*>(workspace); g.ldc = N; g.splits = eff; g.split_stride = M * N;
+    FL_TRY(launch_gemm_tn(g, s));
+    FL_TRY(reduce_partials(static_cast<const float*>(workspace), eff, M * N, int(M), int(N), ldc, C, s));
+    return 0;
 }

@@ -536,13 +536,10 @@ hipError_t launch_gemm_nt(const GemmNT& g, hipStream_t stream) {
     }
     const int tiles_m = (g.M + BM - 1) / BM, tiles_n = (g.N + BN - 1) / BN;
     const TileOrder order = make_order(tiles_m, tiles_n, splits);
-    static bool attr_set = false;
-    if (!attr_set) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_nt_stream),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, int(kLdsBytesStream));
-        if (e != hipSuccess) return e;
-        attr_set = true;
-    }
+    // (set before every launch: the call is cheap, needs no process-wide flag and holds for whichever device is current)
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_nt_stream),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, int(kLdsBytesStream));
+    if (e != hipSuccess) return e;
     hipLaunchKernelGGL(gemm_nt_stream, dim3(256), dim3(kThreads), kLdsBytesStream, stream, g, order,
                        slabs_per_split * BK);
     return hipGetLastError();
@@ -557,13 +554,9 @@ hipError_t launch_gemm_tn(const GemmNT& g, hipStream_t stream) {
     const int splits = g.splits < 1 ? 1 : g.splits;
     if (splits > 1 && g.C32 == nullptr) return hipErrorInvalidValue;
     if (gemm_effective_splits(g.K, splits) != splits) return hipErrorInvalidValue;
-    static bool attr_set = false;
-    if (!attr_set) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_tn_256x256),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, int(kLdsBytesTN));
-        if (e != hipSuccess) return e;
-        attr_set = true;
-    }
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_tn_256x256),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, int(kLdsBytesTN));
+    if (e != hipSuccess) return e;
     const int nslab = (g.K + BK - 1) / BK;
     const int slabs_per_split = (nslab + splits - 1) / splits;
     const int tiles_m = (g.M + BM - 1) / BM, tiles_n = (g.N + BN - 1) / BN;

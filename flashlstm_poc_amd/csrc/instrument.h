@@ -74,14 +74,15 @@ private:
     using Clock = std::chrono::steady_clock;
     // FLASHLSTM_MFU_PEAK_TFLOPS, or clock x CUs x 4096 FLOP/clk/CU (dense fp16 MFMA rate of a CDNA4 CU)
     static double peak_flops() {
-        static double cached = -1.0;
-        if (cached >= 0.0) return cached;
-        const char* ov = std::getenv("FLASHLSTM_MFU_PEAK_TFLOPS");
-        if (ov && ov[0]) return cached = std::strtod(ov, nullptr) * 1e12;
-        int dev = 0;
-        hipDeviceProp_t prop{};
-        if (hipGetDevice(&dev) != hipSuccess || hipGetDeviceProperties(&prop, dev) != hipSuccess) return cached = 0.0;
-        return cached = double(prop.clockRate) * 1000.0 * double(prop.multiProcessorCount) * 4096.0;
+        static const double cached = [] {   // initialised once, also when several threads arrive together
+            const char* ov = std::getenv("FLASHLSTM_MFU_PEAK_TFLOPS");
+            if (ov && ov[0]) return std::strtod(ov, nullptr) * 1e12;
+            int dev = 0;
+            hipDeviceProp_t prop{};
+            if (hipGetDevice(&dev) != hipSuccess || hipGetDeviceProperties(&prop, dev) != hipSuccess) return 0.0;
+            return double(prop.clockRate) * 1000.0 * double(prop.multiProcessorCount) * 4096.0;
+        }();
+        return cached;
     }
     bool enabled_ = false, finished_ = false;
     std::string label_;

@@ -55,6 +55,15 @@ hipError_t reduce_dw(const Dims& d, const float* partial, int splits, int ncols,
 hipError_t reduce_db(const Dims& d, const float* db_part, int ng, float scale, bool accumulate, float* db_ih,
                      float* db_hh, hipStream_t s);
 
+// dst[r][c] (pitch ldc) = sum over z < splits of partial[z * per + r * cols + c]: split-K partials of a plain GEMM.
+hipError_t reduce_partials(const float* partial, int splits, size_t per, int rows, int cols, size_t ldc, float* dst,
+                           hipStream_t s);
+
+// *out += a position-weighted 64-bit sum over the 16-bit units of a device buffer (`salt` tells buffers apart when
+// several are folded into one sum); null or empty buffers add nothing.  Evidence that device tensors still hold what
+// an earlier call saw.
+hipError_t checksum_add(const void* p, size_t bytes, u64 salt, u64* out, hipStream_t s);
+
 hipError_t fill_zero(void* p, size_t bytes, hipStream_t s);
 // Fills a buffer (multiple of 4 bytes) with one 32-bit pattern; a kernel, so it may be captured in a graph.
 hipError_t fill_words(void* p, size_t bytes, unsigned value, hipStream_t s);

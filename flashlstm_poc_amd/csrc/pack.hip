@@ -308,6 +308,46 @@ hipError_t reduce_db(const Dims& d, const float* db_part, int ng, float scale, b
     return hipGetLastError();
 }
 
+__global__ void reduce_partials_kernel(const float* __restrict__ partial, int splits, size_t per, int rows, int cols,
+                                       size_t ldc, float* __restrict__ dst) {
+    const size_t idx = size_t(blockIdx.x) * kT + threadIdx.x;
+    if (idx >= size_t(rows) * cols) return;
+    float s = 0.f;
+    for (int z = 0; z < splits; ++z) s += partial[size_t(z) * per + idx];
+    dst[(idx / cols) * ldc + idx % cols] = s;
+}
+
+hipError_t reduce_partials(const float* partial, int splits, size_t per, int rows, int cols, size_t ldc, float* dst,
+                           hipStream_t s) {
+    if (rows <= 0 || cols <= 0) return hipSuccess;
+    hipLaunchKernelGGL(reduce_partials_kernel, dim3(grid_for(size_t(rows) * cols)), dim3(kT), 0, s, partial, splits, per,
+                       rows, cols, ldc, dst);
+    return hipGetLastError();
+}
+
+// Position-weighted sum of the 16-bit units of a buffer, added to *out: any changed, moved or swapped element
+// changes the sum (up to a 2^-64 accident); the order of the additions does not matter, so atomics may be used.
+__global__ void checksum_kernel(const unsigned short* __restrict__ p, size_t n, u64 salt, u64* out) {
+    u64 acc = 0;
+    const size_t stride = size_t(gridDim.x) * blockDim.x;
+    for (size_t i = size_t(blockIdx.x) * blockDim.x + threadIdx.x; i < n; i += stride) {
+        u64 v = (u64(p[i]) + 1u) * (2 * (i + salt) + 1) * 0x9E3779B97F4A7C15ull;
+        v ^= v >> 29;
+        acc += v * 0xBF58476D1CE4E5B9ull;
+    }
+    for (int off = 32; off > 0; off >>= 1) acc += __shfl_down(acc, off, 64);
+    if (threadIdx.x % 64 == 0 && acc != 0) atomicAdd(reinterpret_cast<unsigned long long*>(out), acc);
+}
+
+hipError_t checksum_add(const void* p, size_t bytes, u64 salt, u64* out, hipStream_t s) {
+    if (p == nullptr || bytes < 2) return hipSuccess;
+    const size_t n = bytes / 2;   // every tensor of this library is made of 2- or 4-byte elements
+    int blocks = grid_for(n);
+    if (blocks > 2048) blocks = 2048;
+    hipLaunchKernelGGL(checksum_kernel, dim3(blocks), dim3(kT), 0, s, static_cast<const unsigned short*>(p), n, salt, out);
+    return hipGetLastError();
+}
+
 hipError_t fill_words(void* p, size_t bytes, unsigned value, hipStream_t s) {
     if (bytes == 0) return hipSuccess;
     const size_t words = bytes / 4;  // all buffers of this library are multiples of 4 bytes

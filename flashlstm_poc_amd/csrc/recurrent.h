@@ -34,6 +34,7 @@ struct RecFwdArgs {
     int B, Hp, T;
     int t0, t1;          // steps [t0, t1) of the sequence are run by this call (state and ring carry over)
     int spin_limit;      // reloads of a fragment chunk that still shows the 'unwritten' pattern before giving up
+    long long spin_ticks;   // the same bound as time: ticks of the device's constant-rate wall clock
     long long* prof;     // optional [8] cycle counters of workgroup 0 per phase (null = off)
 };
 
@@ -56,6 +57,7 @@ struct RecBwdArgs {
     float dy_scale;      // factor applied to dY on load (the loss scale, or 1 when dY is pre-scaled)
     int t_hi, t_lo;      // steps t_hi down to t_lo are run by this call; t_lo = -1 adds the closing dh0 product
     int spin_limit;
+    long long spin_ticks;
     long long* prof;     // optional [8] cycle counters of workgroup 0 per phase (null = off)
 };
 

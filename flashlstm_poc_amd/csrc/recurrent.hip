@@ -96,7 +96,8 @@ constexpr unsigned kUnwritten = 0xFFFFFFFFu;
 // boundary orders memory).
 struct Poll {
     bool on;
-    int limit;        // reloads of one fragment chunk before the launch gives up
+    int limit;        // reloads of one fragment chunk before the launch gives up ...
+    long long ticks;  // ... or this many ticks of the constant-rate wall clock spent reloading it, whichever comes first
     int* status;      // global: 1 = gave up
     int* lds_abort;   // workgroup: some wave gave up
 };
@@ -205,6 +206,7 @@ __device__ __forceinline__ void wave_product(floatx4 (&acc)[2][NT], const half8 
                 // fetch the chunk again (the chunk in flight behind it has to land first, loads return
                 // in order).  The decision is wave-uniform.
                 int spins = 0;
+                long long spin_start = 0;
                 for (;;) {
                     unsigned m = 0u;
 #pragma unroll
@@ -218,9 +220,12 @@ __device__ __forceinline__ void wave_product(floatx4 (&acc)[2][NT], const half8 
                     }
                     if (!__any(m == kUnwritten)) break;
                     ++spins;
+                    if (spins == 1) spin_start = wall_clock64();
+                    // (the clock and the global status word are looked at every 256th reload only)
                     if (spins > poll.limit || *reinterpret_cast<volatile int*>(poll.lds_abort) != 0 ||
                         ((spins & 255) == 0 &&
-                         __hip_atomic_load(poll.status, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0)) {
+                         (wall_clock64() - spin_start > poll.ticks ||
+                          __hip_atomic_load(poll.status, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0))) {
                         if (lane == 0) {
                             __hip_atomic_store(poll.status, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                             *reinterpret_cast<volatile int*>(poll.lds_abort) = 1;
@@ -514,7 +519,7 @@ __global__ __launch_bounds__(kThreads) void rec_fwd_kernel(RecFwdArgs p, RecLayo
     const int hs = role.hs, g = role.g;
     const int nks_total = p.Hp / 32;
     const bool device_scope = (L.persistent != 0) && (L.xcd_local == 0);
-    const Poll poll{L.persistent != 0, p.spin_limit, p.status, &lds_abort};
+    const Poll poll{L.persistent != 0, p.spin_limit, p.spin_ticks, p.status, &lds_abort};
     PhaseClock clk{(blockIdx.x == 0) ? p.prof : nullptr, 0};
     int item = 0;   // work items done: selects the partial-sum buffer
 
@@ -666,7 +671,7 @@ __global__ __launch_bounds__(kThreads) void rec_bwd_kernel(RecBwdArgs p, RecLayo
     const int hs = role.hs, g = role.g;
     const int nks_total = p.Hp / 8;  // contraction over 4Hp packed gate columns
     const bool device_scope = (L.persistent != 0) && (L.xcd_local == 0);
-    const Poll poll{L.persistent != 0, p.spin_limit, p.status, &lds_abort};
+    const Poll poll{L.persistent != 0, p.spin_limit, p.spin_ticks, p.status, &lds_abort};
     const float S = p.dy_scale;
     PhaseClock clk{(blockIdx.x == 0) ? p.prof : nullptr, 0};
     int item = 0;   // work items done: selects the partial-sum buffer
@@ -887,9 +892,26 @@ __global__ void to_exchange_layout_kernel(const half_t* __restrict__ in, int row
     *reinterpret_cast<unsigned*>(out + xch_offset(r, k, nks)) = *reinterpret_cast<const unsigned*>(in + size_t(r) * ld + k);
 }
 
+// (set before every launch: the call is cheap, needs no process-wide flag and holds for whichever device is current)
 template <typename K>
 hipError_t raise_lds(K kernel, size_t bytes) {
     return hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, int(bytes));
+}
+
+// A persistent launch needs all its workgroups running at once: they wait for each other's data.  The cooperative
+// launch makes that a condition of the launch (the runtime refuses a grid that cannot be co-resident and does not
+// run it beside another kernel); where the runtime has no cooperative launch the ordinary one is used, and the
+// bounded waits inside the kernel cover the case that some workgroup is late.
+template <typename K, typename A>
+hipError_t launch_persistent(K kernel, int grid, size_t lds, hipStream_t stream, A a, RecLayout L, int t_a, int t_b,
+                             int ks_wave) {
+    void* params[] = {&a, &L, &t_a, &t_b, &ks_wave};
+    hipError_t e = hipLaunchCooperativeKernel(reinterpret_cast<const void*>(kernel), dim3(grid), dim3(kThreads), params,
+                                              unsigned(lds), stream);
+    if (e == hipSuccess) return hipSuccess;
+    (void)hipGetLastError();
+    hipLaunchKernelGGL(kernel, dim3(grid), dim3(kThreads), lds, stream, a, L, t_a, t_b, ks_wave);
+    return hipGetLastError();
 }
 
 }  // namespace
@@ -967,10 +989,7 @@ static hipError_t run_fwd(const RecLayout& L, const RecFwdArgs& a, hipStream_t s
     hipError_t e = raise_lds(kernel, lds);
     if (e != hipSuccess) return e;
     const int ks_wave = rec_fwd_ks(L, a.Hp);
-    if (L.persistent) {
-        hipLaunchKernelGGL(kernel, dim3(L.grid), dim3(kThreads), lds, stream, a, L, a.t0, a.t1, ks_wave);
-        return hipGetLastError();
-    }
+    if (L.persistent) return launch_persistent(kernel, L.grid, lds, stream, a, L, a.t0, a.t1, ks_wave);
     for (int t = a.t0; t < a.t1; ++t) {
         hipLaunchKernelGGL(kernel, dim3(L.grid), dim3(kThreads), lds, stream, a, L, t, t + 1, ks_wave);
         e = hipGetLastError();
@@ -996,10 +1015,7 @@ static hipError_t run_bwd(const RecLayout& L, const RecBwdArgs& a, hipStream_t s
     hipError_t e = raise_lds(kernel, lds);
     if (e != hipSuccess) return e;
     const int ks_wave = rec_bwd_ks(L, a.Hp);
-    if (L.persistent) {
-        hipLaunchKernelGGL(kernel, dim3(L.grid), dim3(kThreads), lds, stream, a, L, a.t_hi, a.t_lo, ks_wave);
-        return hipGetLastError();
-    }
+    if (L.persistent) return launch_persistent(kernel, L.grid, lds, stream, a, L, a.t_hi, a.t_lo, ks_wave);
     for (int t = a.t_hi; t >= a.t_lo; --t) {
         hipLaunchKernelGGL(kernel, dim3(L.grid), dim3(kThreads), lds, stream, a, L, t, t, ks_wave);
         e = hipGetLastError();

@@ -99,6 +99,17 @@ int lstm_backward(const float* x,
                   size_t hidden_size,
                   const lstm_buffers* buffers);
 
+/* Read access to what the most recent lstm_forward on this handle cached for lstm_backward (device pointers,
+ * valid until the next lstm_forward or lstm_destroy_buffers on the handle; the reference keeps no such cache:
+ * its pointwise kernel overwrites the pre-activations every step, src/lstm.cu:1330).  `which`:
+ *   LSTM_CACHE_HIDDEN (0): h states, fp16 [(T+1)*B][ld], row t*B+b = h before step t (row block 0 = h0)
+ *   LSTM_CACHE_CELL   (1): c states, fp32 [(T+1)*B][ld], row block t = c before step t
+ *   LSTM_CACHE_GATES  (2): activated gates, fp16 [T*B][ld], column 4*unit + gate with gates i, f, g, o
+ * *ld receives the row pitch in elements (hidden size rounded up to a multiple of 32, times 4 for the gates),
+ * *seq_len the length of the cached sequence.  Returns 1 when nothing is cached. */
+enum { LSTM_CACHE_HIDDEN = 0, LSTM_CACHE_CELL = 1, LSTM_CACHE_GATES = 2 };
+int lstm_get_cache(const lstm_buffers* buffers, int which, const void** ptr, size_t* ld, size_t* seq_len);
+
 #ifdef __cplusplus
 }  /* extern "C" */
 #endif

@@ -41,13 +41,18 @@ int flstm_core_destroy(flstm_core_plan* plan);
 
 /* Options: "stepwise" (1 = one launch per time step instead of the persistent kernels),
  * "proj_chunk" (time steps per input-projection GEMM, <=0 = whole sequence; results do not depend
- * on it), "spin_limit" (polls before a waiting workgroup gives up), "dw_splits" (split-K slices of
+ * on it), "spin_limit" / "spin_ms" (reloads of a not-yet-written operand, and milliseconds spent on them, before a
+ * waiting workgroup of a persistent launch gives up; default 2^30 reloads / 250 ms), "dw_splits" (split-K slices of
  * the weight-gradient GEMM, 0 = automatic), "accumulate_grads" (1 = the backward pass adds dW_ih, dW_hh, db_ih
  * and db_hh to what the caller's buffers hold instead of overwriting them: a sequence processed as several
- * consecutive segments, last segment first, each segment's dh0 / dc0 fed to the next call as d_hn / d_cn). */
+ * consecutive segments, last segment first, each segment's dh0 / dc0 fed to the next call as d_hn / d_cn),
+ * "inject_stall" (test hook: the next N passes that use a persistent kernel are treated as if that launch had
+ * given up, which exercises the step-wise repeat and the demotion rule without making any kernel wait). */
 int flstm_core_set_option(flstm_core_plan* plan, const char* name, long value);
 /* Reads back facts about the plan: "persistent_fwd", "persistent_bwd", "xcd_local_fwd", "xcd_local_bwd",
- * "fallbacks" (persistent launches that had to be redone step-wise), "slice_fwd", "slice_bwd" (hidden units
+ * "fallbacks" (persistent launches that had to be redone step-wise), "demotions_fwd", "demotions_bwd" (how often a
+ * direction was demoted to step-wise launches after such a give-up), "hold_fwd", "hold_bwd" (passes a demoted
+ * direction still runs step-wise before the persistent kernel is tried again; 0 = not demoted), "slice_fwd", "slice_bwd" (hidden units
  * per workgroup of the recurrence kernels), "row_tiles" (16-row tiles of a 32-row batch block that the
  * recurrence fetches and multiplies: 1 for batches of at most 16 rows, else 2), "hidden_padded",
  * "input_padded", "device_bytes" (device memory the plan holds), "num_cus" and "clock_khz" (compute units and
@@ -114,6 +119,23 @@ int flstm_core_cache_ptr(const flstm_core_plan* plan, int which, const void** pt
  * measured with events on the call's stream: names "fwd_proj", "fwd_rec", "fwd_total",
  * "bwd_rec", "bwd_dx", "bwd_dw", "bwd_total".  Negative when not available. */
 double flstm_core_last_ms(const flstm_core_plan* plan, const char* phase);
+
+/* The fp16 x fp16 -> fp32-accumulate MFMA GEMMs the passes are built from, callable on their own (the counterpart
+ * of flstm::GemmTN / GemmNN / GemmNT, reference flashlstm_v2/src/gemm.h:8-51; device pointers, work is enqueued on
+ * `stream` and not waited for).
+ *
+ * flstm_gemm_nt:  C[M][N] = alpha * A[M][K] * B[N][K]^T (+ bias[n]); A, B fp16 row-major with K contiguous (this
+ *   is the input projection X * W_ih^T and, with the transposed weights, dX = dG * W_ih).  K must be a multiple
+ *   of 64, lda and ldb multiples of 8; C is fp16 or fp32 with any ldc >= N; bias (fp32, 16-byte aligned) may be null.
+ * flstm_gemm_tn:  C[M][N] = alpha * sum_k A[k][m] * B[k][n]; A is [K][lda], B is [K][ldb] fp16 (the weight gradients
+ *   dG^T * X).  M and N must be multiples of 8, K is arbitrary; C is fp32, 16-byte aligned.  splits > 1 cuts K
+ *   into that many slices (at most: every slice gets whole 64-row slabs) whose partial products go to `workspace`
+ *   (flstm_gemm_tn_workspace_bytes() bytes of device memory, 16-byte aligned) and are then summed into C. */
+int flstm_gemm_nt(const void* A, size_t lda, const void* B, size_t ldb, size_t M, size_t N, size_t K,
+                  void* C, flstm_dtype c_dtype, size_t ldc, float alpha, const float* bias, void* stream);
+size_t flstm_gemm_tn_workspace_bytes(size_t M, size_t N, size_t K, int splits);
+int flstm_gemm_tn(const void* A, size_t lda, const void* B, size_t ldb, size_t M, size_t N, size_t K,
+                  float* C, size_t ldc, float alpha, int splits, void* workspace, void* stream);
 
 #ifdef __cplusplus
 }

@@ -5,4 +5,4 @@ through ctypes and exposes numpy-in / numpy-out helpers.  Allowed importers: tes
 __graft_entry__.smoke() and the cpu_baseline leg of bench.py.
 """
 from .lstm_oracle import (build, forward, backward, pack_weights_v1, checkpoints, chunk_steps, round_fp16,
-                          FLAG_FP16_OPERANDS, FLAG_FP16_FEEDBACK, FLAG_FP16_OUTPUT)
+                          FLAG_FP16_OPERANDS, FLAG_FP16_FEEDBACK, FLAG_FP16_OUTPUT, FLAG_FP16_DG)

@@ -12,7 +12,9 @@
  *   oracle_lstm_backward  closed-form BPTT of flashlstm_v2/src/lstm_backward.cu:199-211 (pointwise),
  *                         :1083-1097 (dh = dG W_hh), :1112-1172 (dW_ih, dW_hh, db, dX), :1218-1246
  *                         (db_ih == db_hh, dh0/dc0) -- with c taken from the forward pass instead of
- *                         the atanh reconstruction of :188-197
+ *                         the atanh reconstruction of :188-197; flag bit3 rounds the pre-activation
+ *                         gradients dG to fp16 before the products that consume them, as the fp16 copy
+ *                         written at :213-222 for the half-operand GEMMs does
  *   oracle_pack_weights_v1 layout of src/kernels.cu:57-84 with stride = align_up(I+H, 8)
  *                         (src/lstm.cu:698-699)
  *   oracle_checkpoints    "entry k = state before step k*R" of flashlstm_v2/src/lstm_forward.cu:370-375,
@@ -161,6 +163,12 @@ int oracle_lstm_backward(size_t T, size_t B, size_t I, size_t H, const double* x
                 d[2 * H + j] = dcv * ig * (1.0 - gg * gg);
                 d[3 * H + j] = dov * og * (1.0 - og);
                 dc[b * H + j] = dcv * fg;
+                if (flags & 8) {   /* the GEMMs that consume dG take fp16 operands */
+                    d[j] = round_fp16(d[j]);
+                    d[H + j] = round_fp16(d[H + j]);
+                    d[2 * H + j] = round_fp16(d[2 * H + j]);
+                    d[3 * H + j] = round_fp16(d[3 * H + j]);
+                }
             }
         }
         memset(dhp, 0, sizeof(double) * B * H);

@@ -14,6 +14,7 @@ _lib = None
 FLAG_FP16_OPERANDS = 1   # round x, W_ih, W_hh to fp16 before use
 FLAG_FP16_FEEDBACK = 2   # h is fed back through an fp16 cast (reference src/kernels.cu:150-155)
 FLAG_FP16_OUTPUT = 4     # y holds fp16-rounded values
+FLAG_FP16_DG = 8         # backward: pre-activation gradients are rounded to fp16 before the GEMMs that consume them
 
 
 def build(force: bool = False) -> str:

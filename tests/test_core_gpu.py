@@ -130,6 +130,45 @@ def test_retry_limit_hit_is_repaired_by_stepwise_pass():
     core.close()
 
 
+def test_give_up_demotes_for_a_few_passes_and_then_the_persistent_kernel_returns():
+    # The give-up of a persistent launch is injected from the host (no kernel waits for anything): the pass is
+    # repeated step-wise with the same results, that direction stays step-wise for 8 passes, then the persistent
+    # kernel is back; a second give-up holds it for 16.  The other direction is not touched.
+    from flashlstm_poc_amd import LstmCore
+    p = make_problem(10, 40, 64, 256, seed=6)
+    ref, _ = oracle_reference(p)
+    core = LstmCore(40, 64, 256)
+    core.pack(*(p[k].cuda() for k in ("w_ih", "w_hh", "b_ih", "b_hh")))
+    x = p["x"].cuda().half(); h0 = p["h0"].cuda().half(); c0 = p["c0"].cuda().half()
+    assert core.info("persistent_fwd") == 1 and core.info("hold_fwd") == 0
+    y0, _, _ = core.forward(x, h0, c0)
+    core.set_option("inject_stall", 1)
+    y1, _, _ = core.forward(x, h0, c0)
+    assert torch.equal(y0, y1)                        # step-wise repeat: bit-identical forward results
+    assert core.info("demotions_fwd") == 1 and core.info("fallbacks") == 1
+    assert core.info("persistent_fwd") == 0 and core.info("hold_fwd") == 7 and core.info("persistent_bwd") == 1
+    for left in range(6, -1, -1):
+        y2, _, _ = core.forward(x, h0, c0)
+        assert torch.equal(y0, y2) and core.info("hold_fwd") == left
+    assert core.info("persistent_fwd") == 1           # back on the persistent kernel
+    core.set_option("inject_stall", 1)
+    core.forward(x, h0, c0)
+    assert core.info("demotions_fwd") == 2 and core.info("hold_fwd") == 15
+    # the same for the backward direction, checked against the oracle
+    core.set_option("inject_stall", 0)
+    got, _ = run_core(p, core=core)
+    check_against(ref, got, label="before the injected backward give-up")
+    core.forward(x, h0, c0)
+    core.set_option("inject_stall", 1)                # forward is step-wise now, so the backward pass takes it
+    assert core.info("persistent_fwd") == 0 and core.info("persistent_bwd") == 1
+    dy = p["dy"].cuda().half()
+    grads = core.backward(x, dy, p["d_hn"].cuda().half(), p["d_cn"].cuda().half())
+    assert core.info("demotions_bwd") == 1 and core.info("persistent_bwd") == 0 and core.info("hold_bwd") == 7
+    for k, t in zip(("dx", "dw_ih", "dw_hh", "db", "dh0", "dc0"), grads):
+        assert rell2(to_np(t), ref[k]) <= 1e-2, k
+    core.close()
+
+
 def test_projection_chunk_size_does_not_change_results():
     p = make_problem(17, 6, 48, 40, seed=9)
     base, _ = run_core(p, proj_chunk=0)

@@ -89,3 +89,56 @@ def test_headline_shapes_against_torch_lstm_on_gpu(shape):
                            (db, m.bias_ih_l0.grad, "db"), (dh0, hr.grad, "dh0"), (dc0, cr.grad, "dc0")):
         assert rell2(to_np(got), to_np(ref)) <= 1e-2, name
     core.close()
+
+
+def _torch_lstm_reference(p, with_grads=True):
+    T, B, I = p["x"].shape
+    H = p["w_hh"].shape[1]
+    m = torch.nn.LSTM(I, H, device="cuda")
+    with torch.no_grad():
+        m.weight_ih_l0.copy_(p["w_ih"].half().float()); m.weight_hh_l0.copy_(p["w_hh"].half().float())
+        m.bias_ih_l0.copy_(p["b_ih"]); m.bias_hh_l0.copy_(p["b_hh"])
+    xr = p["x"].float().requires_grad_(with_grads)
+    hr = p["h0"].float().requires_grad_(with_grads); cr = p["c0"].float().requires_grad_(with_grads)
+    yr, (hn, cn) = m(xr, (hr[None], cr[None]))
+    grads = None
+    if with_grads:
+        (yr * p["dy"].float()).sum().backward()
+        grads = dict(dx=xr.grad, dW_ih=m.weight_ih_l0.grad, dW_hh=m.weight_hh_l0.grad, db=m.bias_ih_l0.grad,
+                     dh0=hr.grad, dc0=cr.grad)
+    return yr.detach(), hn[0].detach(), cn[0].detach(), grads
+
+
+def _gpu_relmax(a, b):
+    return ((a.float() - b.float()).abs().max() / b.float().abs().max()).item()
+
+
+def _gpu_rell2(a, b):
+    return ((a.double() - b.double()).norm() / b.double().norm()).item()
+
+
+@pytest.mark.parametrize("name,shape,backward", [("config2", (512, 64, 1024, 1024), False),
+                                                 ("config3", (1024, 256, 1024, 1024), True),
+                                                 ("config4", (2048, 16, 2048, 2048), True)])
+def test_full_length_configs_against_fp32_torch_lstm(name, shape, backward):
+    # The BASELINE configurations at their FULL sequence length against fp32 nn.LSTM on the GPU, same fp16-rounded
+    # operands: max relative error <= 1e-2 on y / h_T / c_T, relative L2 <= 1e-2 on every gradient.  The error of
+    # the LAST step is reported beside the maximum: h is fed back through fp16 at every step, and this is where a
+    # growth of that error over 1024 / 2048 steps would show.
+    T, B, I, H = shape
+    p = problem(T, B, I, H, seed=11)
+    core = make_core(p)
+    y, hy, cy = core.forward(p["x"], p["h0"], p["c0"], save_for_backward=backward)
+    got = core.backward(p["x"], p["dy"]) if backward else None
+    assert core.info("persistent_fwd") == 1 and core.info("fallbacks") == 0
+    yr, hn, cn, gr = _torch_lstm_reference(p, with_grads=backward)
+    errs = {"y_max": _gpu_relmax(y, yr), "y_last_step": _gpu_relmax(y[-1], yr[-1]), "y_first_step": _gpu_relmax(y[0], yr[0]),
+            "h_T": _gpu_relmax(hy, hn), "c_T": _gpu_relmax(cy, cn)}
+    if backward:
+        for k, t in zip(("dx", "dW_ih", "dW_hh", "db", "dh0", "dc0"), got):
+            errs[k] = _gpu_rell2(t, gr[k])
+        # gradient of the FIRST time step's input: the end of the backward chain
+        errs["dx_first_step"] = _gpu_rell2(got[0][0], gr["dx"][0])
+    print(f"\n{name} T={T} B={B} I={I} H={H}: " + ", ".join(f"{k}={v:.2e}" for k, v in errs.items()))
+    assert max(errs.values()) <= 1e-2, errs
+    core.close()

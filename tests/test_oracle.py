@@ -185,3 +185,52 @@ def test_projection_chunk_semantics():
     assert oracle.chunk_steps(17, 17) == 17
     assert oracle.chunk_steps(4, 17) == 4
     assert oracle.chunk_steps(1, 17) == 1
+
+
+def _fp16_path_oracle(n, gates16=True):
+    """The oracle run the way the fp16 path stores things: fp16 operands, h fed back through fp16, the activated
+    gates kept as fp16 (the gate cache), dG rounded to fp16 for the products that consume it."""
+    f = dict(oracle.forward(n["x"], n["w_ih"], n["w_hh"], n["b_ih"], n["b_hh"], n["h0"], n["c0"],
+                            flags=oracle.FLAG_FP16_OPERANDS | oracle.FLAG_FP16_FEEDBACK))
+    if gates16:
+        f["gates"] = f["gates"].astype(np.float16).astype(np.float64)
+    g = oracle.backward(n["x"], n["w_ih"], n["w_hh"], f, n["dy"], n["d_hn"], n["d_cn"],
+                        flags=oracle.FLAG_FP16_OPERANDS | oracle.FLAG_FP16_DG)
+    return f, g
+
+
+def test_fp16_dg_flag_only_rounds_the_preactivation_gradients():
+    # pins flag bit 3: the flagged run differs from the plain one by no more than fp16 rounding of dG can explain
+    # (relative 2^-11 per element), and db -- a plain sum of dG -- is a sum of fp16-representable values
+    p = make_problem(6, 3, 5, 4, seed=77)
+    n = {k: to_np(v) for k, v in p.items()}
+    f = oracle.forward(n["x"], n["w_ih"], n["w_hh"], n["b_ih"], n["b_hh"], n["h0"], n["c0"])
+    g0 = oracle.backward(n["x"], n["w_ih"], n["w_hh"], f, n["dy"], n["d_hn"], n["d_cn"])
+    g1 = oracle.backward(n["x"], n["w_ih"], n["w_hh"], f, n["dy"], n["d_hn"], n["d_cn"], flags=oracle.FLAG_FP16_DG)
+    for k in ("dx", "dw_ih", "dw_hh", "db", "dh0", "dc0"):
+        err = np.linalg.norm(g1[k] - g0[k]) / np.linalg.norm(g0[k])
+        assert 0 < err < 2e-3, (k, err)
+    # one step, one row: db IS dG, so every entry must be exactly representable in fp16
+    q = make_problem(1, 1, 3, 4, seed=78)
+    m = {k: to_np(v) for k, v in q.items()}
+    f = oracle.forward(m["x"], m["w_ih"], m["w_hh"], m["b_ih"], m["b_hh"], m["h0"], m["c0"])
+    g = oracle.backward(m["x"], m["w_ih"], m["w_hh"], f, m["dy"], m["d_hn"], m["d_cn"], flags=oracle.FLAG_FP16_DG)
+    np.testing.assert_array_equal(g["db"], g["db"].astype(np.float16).astype(np.float64))
+    g_plain = oracle.backward(m["x"], m["w_ih"], m["w_hh"], f, m["dy"], m["d_hn"], m["d_cn"])
+    np.testing.assert_array_equal(g["db"], g_plain["db"].astype(np.float16).astype(np.float64))
+
+
+def test_single_unit_dh0_is_ill_conditioned_under_an_fp16_gate_cache():
+    # T=40, B=1, I=65, H=1 (seed 550): dh0 is ONE number, the sum of four products dG_0[gate] * w_hh[gate] that
+    # nearly cancel.  Storing the activated gates in fp16 (the gate cache) moves it by ~10 % while every other
+    # gradient stays within 1e-3: a property of the conditioning of this element, not of any code path.
+    p = make_problem(40, 1, 65, 1, seed=550)
+    n = {k: to_np(v) for k, v in p.items()}
+    ref = torch_reference(p)
+    _, g_cache = _fp16_path_oracle(n, gates16=True)
+    _, g_nocache = _fp16_path_oracle(n, gates16=False)
+    rel = lambda a, b: float(np.abs(a - b).max() / np.abs(b).max())
+    assert 5e-2 < rel(g_cache["dh0"], ref["dh0"]) < 2e-1          # the gate cache alone explains the deviation
+    assert rel(g_nocache["dh0"], ref["dh0"]) < 2e-3               # without it the element is fine
+    for k in ("dx", "dw_ih", "dw_hh", "db", "dc0"):                 # and nothing else is affected
+        assert np.linalg.norm(g_cache[k] - ref[k]) / np.linalg.norm(ref[k]) < 2e-3, k

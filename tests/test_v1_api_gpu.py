@@ -105,6 +105,47 @@ def test_backward_addition_matches_oracle():
     lib.lstm_destroy_buffers(ctypes.byref(buf))
 
 
+def test_cache_accessor_on_the_v1_handle():
+    # lstm_get_cache: what the last lstm_forward on the handle kept for lstm_backward, read through the handle
+    lib = bind()
+    lib.lstm_get_cache.argtypes = [ctypes.POINTER(Buffers), ctypes.c_int, ctypes.POINTER(ctypes.c_void_p),
+                                   ctypes.POINTER(ctypes.c_size_t), ctypes.POINTER(ctypes.c_size_t)]
+    T, B, I, H = 6, 3, 10, 20
+    p = make_problem(T, B, I, H, seed=31, fp16_values=False)
+    buf = Buffers()
+    assert lib.lstm_create_buffers(ACC32, T, B, I, H, 0, ctypes.byref(buf)) == 0
+    ptr, ld, seq = ctypes.c_void_p(), ctypes.c_size_t(), ctypes.c_size_t()
+    assert lib.lstm_get_cache(ctypes.byref(buf), 2, ctypes.byref(ptr), ctypes.byref(ld), ctypes.byref(seq)) == 1   # nothing cached
+    w_ih, w_hh = p["w_ih"].cuda().contiguous(), p["w_hh"].cuda().contiguous()
+    assert lib.lstm_pack_weights(ACC32, w_ih.data_ptr(), w_hh.data_ptr(), I, H, ctypes.byref(buf)) == 0
+    rc, out, hn, cn = forward(lib, buf, p, T, ACC32)
+    assert rc == 0
+    f = oracle_fwd(p, T)
+
+    def read(which, rows, dtype):
+        assert lib.lstm_get_cache(ctypes.byref(buf), which, ctypes.byref(ptr), ctypes.byref(ld), ctypes.byref(seq)) == 0
+        assert seq.value == T
+        esz = 2 if dtype == torch.float16 else 4
+        host = torch.empty(rows, ld.value, dtype=dtype)
+        # plain device-to-host copy of the cached rows (the pointer belongs to the library)
+        from torch.cuda import cudart
+        assert int(cudart().cudaMemcpy(host.data_ptr(), ptr.value, rows * ld.value * esz, 2)) == 0
+        return host.double().numpy(), ld.value
+
+    Hp = (H + 31) // 32 * 32
+    h_all, ldh = read(0, (T + 1) * B, torch.float16)
+    c_all, ldc = read(1, (T + 1) * B, torch.float32)
+    gates, ldg = read(2, T * B, torch.float16)
+    assert (ldh, ldc, ldg) == (Hp, Hp, 4 * Hp)
+    assert relmax(h_all[:, :H].reshape(T + 1, B, H)[:T], f["h_all"][:T]) <= 1e-2
+    assert relmax(c_all[:, :H].reshape(T + 1, B, H)[:T], f["c_all"][:T]) <= 1e-2
+    # column 4 * unit + gate  <->  PyTorch order gate * H + unit
+    packed = gates.reshape(T, B, Hp, 4)[:, :, :H, :]
+    assert relmax(np.moveaxis(packed, 3, 2).reshape(T, B, 4 * H), f["gates"]) <= 1e-2
+    assert lib.lstm_get_cache(ctypes.byref(buf), 9, ctypes.byref(ptr), ctypes.byref(ld), None) == 1
+    lib.lstm_destroy_buffers(ctypes.byref(buf))
+
+
 def test_error_codes_follow_the_reference():
     # reference src/lstm.cu:861-904,1912-1920: everything invalid returns 1
     lib = bind()
