@@ -16,6 +16,7 @@ class LstmStack:
         self.B, self.I, self.H, self.L = int(batch), int(input_size), int(hidden_size), int(num_layers)
         self.layers: List[LstmCore] = [LstmCore(self.B, self.I if l == 0 else self.H, self.H) for l in range(self.L)]
         self._inputs: List = []
+        self.last_loss_scale = 1.0
 
     def close(self) -> None:
         for layer in self.layers:
@@ -44,16 +45,29 @@ class LstmStack:
             cys.append(cy)
         return cur, hys, cys
 
-    def backward(self, dy_top, *, loss_scale: float = 1.0, d_hn: Optional[Sequence] = None,
+    def backward(self, dy_top, *, loss_scale="auto", d_hn: Optional[Sequence] = None,
                  d_cn: Optional[Sequence] = None, want_dx: bool = True):
         """dy_top (T,B,H): gradient wrt the top layer's outputs.  loss_scale (a power of two) multiplies it before
         it is rounded to fp16 and stays on every inter-layer gradient, so that small gradients survive the fp16
-        hand-over between layers; it is divided out of everything returned.
+        hand-over between layers; it is divided out of everything returned.  "auto" (the default) picks the power
+        of two that brings the largest |dy_top| to about 64: far enough from the fp16 maximum (65504) for the
+        gradients to grow a thousandfold on the way down, and far enough from the smallest normal fp16 number
+        (6e-5) for them to shrink a few hundredfold per layer (the mean-squared-error gradient of a 4096 x 128 x
+        2048 output is ~2e-9 per element: with a scale of 2^12 the bottom layer of a 4-layer stack loses all of
+        its gradient).  The scale used is kept in self.last_loss_scale.
         Returns (dx of layer 0 (fp32 when a loss scale is in use) or None, [(dW_ih, dW_hh, db) per layer], [dh0 per layer], [dc0 per layer])."""
+        import math
         import torch
         if not self._inputs:
             raise RuntimeError("backward needs a forward pass first")
-        S = float(loss_scale) if loss_scale and loss_scale > 0 else 1.0
+        if isinstance(loss_scale, str):
+            if loss_scale != "auto":
+                raise ValueError("loss_scale must be a positive number or 'auto'")
+            amax = float(dy_top.abs().max())
+            S = 2.0 ** min(60, max(-14, math.floor(math.log2(64.0 / amax)))) if 0.0 < amax < float("inf") else 1.0
+        else:
+            S = float(loss_scale) if loss_scale and loss_scale > 0 else 1.0
+        self.last_loss_scale = S
         cur = (dy_top.float() * S).half() if S != 1.0 else dy_top.half()
         grads: List = [None] * self.L
         dh0s: List = [None] * self.L

@@ -73,3 +73,53 @@ def check_against(ref, got, label=""):
             errs[k] = rell2(got[k], ref[k])
             assert errs[k] <= TOL_GRAD, f"{label} {k}: rel L2 err {errs[k]:.3e} > {TOL_GRAD}"
     return errs
+
+
+class SafeTorchLstm(torch.nn.Module):
+    """fp32 reference LSTM stack on the GPU for FULL-SIZE problems, built from torch.nn.LSTM calls that stay inside
+    the range where PyTorch-ROCm's nn.LSTM is itself right.  Two things were found to go wrong in that library at
+    the BASELINE sizes (this library's results were confirmed independently both times, by forming the same sums
+    with its weight-gradient GEMM and by running the sequence in segments):
+      * the bias gradient is 2.6 times too large in norm at T*B = 262144 rows (fine at 131072);
+      * at T*B = 524288 rows with H = 2048 (one call) its outputs are right for the first 1024 steps and wrong by
+        O(1) after them, while the same module called on 131072 rows at a time agrees with this library to 5e-4.
+    So: every call sees at most `max_rows` rows (the sequence is walked in segments, (h, c) carried from one to the
+    next with the autograd graph intact), and the bias enters as the weight of an extra all-ones input column
+    (bias=False), which makes its gradient a column of the weight gradient.  On small problems this equals
+    nn.LSTM(num_layers=L) exactly (tests/test_stack_gpu.py checks that)."""
+
+    def __init__(self, params, max_rows=131072):
+        # params[l] = (w_ih, w_hh, b_ih, b_hh) fp32 CUDA tensors; weights are rounded to fp16 values as the kernels see them
+        super().__init__()
+        self.max_rows = max_rows
+        self.layers = torch.nn.ModuleList()
+        for w_ih, w_hh, b_ih, b_hh in params:
+            m = torch.nn.LSTM(w_ih.shape[1] + 1, w_hh.shape[1], bias=False, device=w_ih.device)
+            with torch.no_grad():
+                m.weight_ih_l0[:, :-1].copy_(w_ih.half().float())
+                m.weight_ih_l0[:, -1].copy_(b_ih + b_hh)
+                m.weight_hh_l0.copy_(w_hh.half().float())
+            self.layers.append(m)
+
+    def forward(self, x, h0=None, c0=None):
+        """x (T,B,I) fp32; h0/c0: lists per layer of (B,H) or None.  Returns y_top, [h_T per layer], [c_T per layer]."""
+        T, B, _ = x.shape
+        seg = max(1, self.max_rows // B)
+        hs, cs = [], []
+        for l, m in enumerate(self.layers):
+            H = m.hidden_size
+            h = (h0[l] if h0 is not None and h0[l] is not None else x.new_zeros(B, H))[None]
+            c = (c0[l] if c0 is not None and c0[l] is not None else x.new_zeros(B, H))[None]
+            outs = []
+            for t0 in range(0, T, seg):
+                xs = x[t0:t0 + seg]
+                ys, (h, c) = m(torch.cat([xs, torch.ones_like(xs[:, :, :1])], dim=2), (h, c))
+                outs.append(ys)
+            x = outs[0] if len(outs) == 1 else torch.cat(outs, dim=0)
+            hs.append(h[0]); cs.append(c[0])
+        return x, hs, cs
+
+    def grads(self, l):
+        """(dW_ih, dW_hh, db) of layer l after backward()."""
+        g = self.layers[l].weight_ih_l0.grad
+        return g[:, :-1], self.layers[l].weight_hh_l0.grad, g[:, -1]

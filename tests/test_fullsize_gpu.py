@@ -92,20 +92,17 @@ def test_headline_shapes_against_torch_lstm_on_gpu(shape):
 
 
 def _torch_lstm_reference(p, with_grads=True):
-    T, B, I = p["x"].shape
-    H = p["w_hh"].shape[1]
-    m = torch.nn.LSTM(I, H, device="cuda")
-    with torch.no_grad():
-        m.weight_ih_l0.copy_(p["w_ih"].half().float()); m.weight_hh_l0.copy_(p["w_hh"].half().float())
-        m.bias_ih_l0.copy_(p["b_ih"]); m.bias_hh_l0.copy_(p["b_hh"])
+    """fp32 nn.LSTM on the GPU with the fp16-rounded weights, called the safe way (helpers.SafeTorchLstm)."""
+    from helpers import SafeTorchLstm
+    m = SafeTorchLstm([(p["w_ih"], p["w_hh"], p["b_ih"], p["b_hh"])])
     xr = p["x"].float().requires_grad_(with_grads)
     hr = p["h0"].float().requires_grad_(with_grads); cr = p["c0"].float().requires_grad_(with_grads)
-    yr, (hn, cn) = m(xr, (hr[None], cr[None]))
+    yr, hn, cn = m(xr, [hr], [cr])
     grads = None
     if with_grads:
         (yr * p["dy"].float()).sum().backward()
-        grads = dict(dx=xr.grad, dW_ih=m.weight_ih_l0.grad, dW_hh=m.weight_hh_l0.grad, db=m.bias_ih_l0.grad,
-                     dh0=hr.grad, dc0=cr.grad)
+        dW_ih, dW_hh, db = m.grads(0)
+        grads = dict(dx=xr.grad, dW_ih=dW_ih, dW_hh=dW_hh, db=db, dh0=hr.grad, dc0=cr.grad)
     return yr.detach(), hn[0].detach(), cn[0].detach(), grads
 
 

@@ -5,14 +5,15 @@ relative error <= 1e-2 on outputs, relative L2 <= 1e-2 on every gradient."""
 import pytest
 import torch
 
-from helpers import rell2, relmax, to_np
+from helpers import SafeTorchLstm, rell2, relmax, to_np
 
 pytestmark = pytest.mark.gpu
 
 
-def _run(T, B, I, H, L, loss_scale, seed=5):
+def _run(T, B, I, H, L, loss_scale, seed=5, safe_reference=False, max_rows=131072):
     """Our stack first (forward, MSE gradient, backward), then -- after its device memory has been given back -- the
-    fp32 nn.LSTM(num_layers=L) reference on the same inputs; returns the error of every output and gradient."""
+    fp32 reference on the same inputs: nn.LSTM(num_layers=L) itself, or (safe_reference) the same function built
+    from nn.LSTM calls of bounded size, helpers.SafeTorchLstm.  Returns the error of every output and gradient."""
     from flashlstm_poc_amd import LstmStack
     torch.manual_seed(seed)
     ref = torch.nn.LSTM(I, H, num_layers=L, device="cuda")
@@ -34,7 +35,14 @@ def _run(T, B, I, H, L, loss_scale, seed=5):
     torch.cuda.empty_cache()
 
     xr = x.float().requires_grad_(True)
-    yr, (hn, cn) = ref(xr)
+    if safe_reference:
+        safe = SafeTorchLstm([tuple(getattr(ref, f"{n}_l{l}").detach() for n in ("weight_ih", "weight_hh", "bias_ih", "bias_hh"))
+                              for l in range(L)], max_rows=max_rows)
+        grad_of = lambda name, l: safe.grads(l)[("weight_ih", "weight_hh", "bias_ih").index(name)]
+        yr, hn, cn = safe(xr)
+    else:
+        grad_of = lambda name, l: getattr(ref, f"{name}_l{l}").grad
+        yr, (hn, cn) = ref(xr)
     errs = {"y": relmax_t(y, yr), "y_last_step": relmax_t(y[-1], yr[-1])}
     for l in range(L):
         errs[f"h_T{l}"] = relmax_t(hys[l], hn[l])
@@ -44,9 +52,9 @@ def _run(T, B, I, H, L, loss_scale, seed=5):
     errs["dx"] = rell2_t(dx, xr.grad)
     for l in range(L):
         dW_ih, dW_hh, db = grads[l]
-        errs[f"dW_ih{l}"] = rell2_t(dW_ih, getattr(ref, f"weight_ih_l{l}").grad)
-        errs[f"dW_hh{l}"] = rell2_t(dW_hh, getattr(ref, f"weight_hh_l{l}").grad)
-        errs[f"db{l}"] = rell2_t(db, getattr(ref, f"bias_ih_l{l}").grad)
+        errs[f"dW_ih{l}"] = rell2_t(dW_ih, grad_of("weight_ih", l))
+        errs[f"dW_hh{l}"] = rell2_t(dW_hh, grad_of("weight_hh", l))
+        errs[f"db{l}"] = rell2_t(db, grad_of("bias_ih", l))
     return errs
 
 
@@ -56,6 +64,15 @@ def relmax_t(a, b):   # on the GPU: the full-size tensors are too large to move 
 
 def rell2_t(a, b):
     return ((a.double() - b.double()).norm() / b.double().norm()).item()
+
+
+def test_safe_reference_is_the_multilayer_lstm():
+    # the reference used at full size equals nn.LSTM(num_layers=L), outputs and gradients, where both are sound;
+    # max_rows=20 forces three time segments per layer on this 12-step problem
+    a = _run(12, 5, 16, 24, 3, loss_scale=2.0 ** 12)
+    b = _run(12, 5, 16, 24, 3, loss_scale=2.0 ** 12, safe_reference=True, max_rows=20)
+    for k in a:
+        assert abs(a[k] - b[k]) <= 2e-4, (k, a[k], b[k])
 
 
 @pytest.mark.parametrize("shape", [(12, 5, 16, 24, 3), (20, 33, 48, 64, 4)])
@@ -68,15 +85,17 @@ def test_stack_matches_multilayer_torch_lstm_with_loss_scale(shape):
 def test_loss_scale_is_what_keeps_small_gradients():
     errs = _run(12, 5, 16, 24, 3, loss_scale=1.0)
     scaled = _run(12, 5, 16, 24, 3, loss_scale=2.0 ** 12)
-    assert max(scaled.values()) <= 1e-2
+    auto = _run(12, 5, 16, 24, 3, loss_scale="auto")
+    assert max(scaled.values()) <= 1e-2 and max(auto.values()) <= 1e-2
     assert max(errs.values()) > max(scaled.values())   # unscaled: fp16 underflow costs accuracy
 
 
 def test_config5_stack_full_size_against_fp32_torch_lstm():
     # BASELINE config 5 as written: 4 layers, I = 512, H = 2048, B = 128, T = 4096, MSE on the top layer's outputs
     # against seeded N(0,1) targets; the reference for every output and all 13 gradients is fp32
-    # nn.LSTM(num_layers=4) on the same GPU with the same fp16-rounded weights.  (About 50 GB of device memory for
-    # the reference's autograd state and about 70 GB for the four layers' caches.)
-    errs = _run(4096, 128, 512, 2048, 4, loss_scale=2.0 ** 12, seed=7)
+    # nn.LSTM on the same GPU with the same fp16-rounded weights, called in pieces of at most 131072 rows
+    # (helpers.SafeTorchLstm says why).
+    # The automatic loss scale is part of what is tested: d MSE / d y is ~2e-9 per element here.
+    errs = _run(4096, 128, 512, 2048, 4, loss_scale="auto", seed=7, safe_reference=True)
     print("\nconfig5 stack: " + ", ".join(f"{k}={v:.2e}" for k, v in errs.items()))
     assert max(errs.values()) <= 1e-2, errs
