@@ -128,8 +128,8 @@ def test_cache_accessor_on_the_v1_handle():
         esz = 2 if dtype == torch.float16 else 4
         host = torch.empty(rows, ld.value, dtype=dtype)
         # plain device-to-host copy of the cached rows (the pointer belongs to the library)
-        from torch.cuda import cudart
-        assert int(cudart().cudaMemcpy(host.data_ptr(), ptr.value, rows * ld.value * esz, 2)) == 0
+        assert ctypes.CDLL("libamdhip64.so").hipMemcpy(ctypes.c_void_p(host.data_ptr()), ptr,
+                                                       ctypes.c_size_t(rows * ld.value * esz), 2) == 0
         return host.double().numpy(), ld.value
 
     Hp = (H + 31) // 32 * 32
