@@ -52,6 +52,8 @@ def load_library() -> ctypes.CDLL:
     lib.flstm_core_pack_weights.argtypes = [vp, vp, vp, vp]
     lib.flstm_core_pack_bias.argtypes = [vp, vp, vp, vp]
     lib.flstm_core_forward.argtypes = [vp, sz, vp, i32, vp, vp, i32, vp, i32, vp, vp, i32, i32, vp]
+    lib.flstm_core_forward_static.argtypes = [vp, sz, vp, i32, vp, vp, i32, vp, i32, vp, vp, i32, vp]
+    lib.flstm_core_forward_static.restype = i32
     lib.flstm_core_backward.argtypes = [vp, sz, vp, i32, vp, i32, vp, vp, i32, c.c_float, vp, i32,
                                         vp, vp, vp, vp, vp, vp, vp]
     lib.flstm_core_cache_ptr.argtypes = [vp, i32, c.POINTER(vp), c.POINTER(sz)]
@@ -159,6 +161,27 @@ class LstmCore:
         if rc != 0:
             raise RuntimeError(f"flstm_core_forward failed with status {rc}")
         return y, hy, cy
+
+    def forward_static(self, x, h0, c0, y, hy, cy) -> None:
+        """flstm_core_forward_static: the forward pass into caller-provided outputs (y (T,B,H), hy, cy (B,H), all
+        of one dtype), with the library's fixed scratch array instead of plan-owned buffers -- the call allocates
+        nothing.  h0 / c0 may be None (zeros).  Raises MemoryError when the pass does not fit the array."""
+        T = x.shape[0]
+        if not x.is_cuda or not x.is_contiguous() or tuple(x.shape[1:]) != (self.B, self.I):
+            raise ValueError(f"x must be a contiguous CUDA tensor of shape (T, {self.B}, {self.I})")
+        if tuple(y.shape) != (T, self.B, self.H) or tuple(hy.shape) != (self.B, self.H) or tuple(cy.shape) != (self.B, self.H):
+            raise ValueError("outputs must have shapes (T,B,H), (B,H), (B,H)")
+        if hy.dtype != cy.dtype or not (y.is_contiguous() and hy.is_contiguous() and cy.is_contiguous()):
+            raise ValueError("hy and cy must share a dtype; outputs must be contiguous")
+        st = h0 if h0 is not None else c0
+        rc = self.lib.flstm_core_forward_static(self._h, T, x.data_ptr(), _dtype_code(x), _ptr(h0), _ptr(c0),
+                                                _dtype_code(st) if st is not None else F16, y.data_ptr(),
+                                                _dtype_code(y), hy.data_ptr(), cy.data_ptr(), _dtype_code(hy),
+                                                self._stream())
+        if rc == 2004:
+            raise MemoryError("the pass needs more scratch memory than flstm_core_forward_static's fixed array holds")
+        if rc != 0:
+            raise RuntimeError(f"flstm_core_forward_static failed with status {rc}")
 
     def backward(self, x, dy, d_hn=None, d_cn=None, *, grad_scale: float = 1.0, dx_dtype=None,
                  want_dx: bool = True, accumulate_into=None):

@@ -10,6 +10,7 @@
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
+#include <mutex>
 #include <new>
 
 #include "../../include/flashlstm/lstm_core.h"
@@ -19,21 +20,49 @@
 
 using namespace flstm_hip;
 
+// Scratch memory of flstm_core_forward_static: everything that entry point's kernels need beyond the caller's
+// tensors and the plan's packed weights (status word and seat counters, converted x rows, x-projection / gate rows,
+// state rows, exchange ring).  One array per device, owned by the code object; host code reaches it only through
+// the address hipGetSymbolAddress returns for the device that is current (static_scratch()).
+static constexpr size_t kStaticScratchBytes = size_t(64) << 20;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+static constexpr int kMaxDevices = 64;
+static std::mutex g_scratch_mutex;
+static void* g_scratch_ptr[kMaxDevices] = {};
+
+// address of `scratch` on the current device (looked up once per device)
+static int static_scratch(int dev, void** out) {
+    if (dev < 0 || dev >= kMaxDevices) return FLSTM_E_INVALID;
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (!g_scratch_ptr[dev]) {
+        void* ptr = nullptr;
+        hipError_t e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+        if (e != hipSuccess) return int(e);
+        if (!ptr) return int(hipErrorInvalidSymbol);
+        g_scratch_ptr[dev] = ptr;
+    }
+    *out = g_scratch_ptr[dev];
+    return 0;
+}
+
 namespace {
 
 struct DevBuf {
     void* p = nullptr;
     size_t bytes = 0;
+    bool borrowed = false;   // a view of memory owned elsewhere: never grown, never freed
     // grows (never shrinks); contents are lost on growth
     hipError_t reserve(size_t need) {
         if (need <= bytes) return hipSuccess;
+        if (borrowed) return hipErrorOutOfMemory;
         if (p) { hipError_t e = hipFree(p); p = nullptr; bytes = 0; if (e != hipSuccess) return e; }
         hipError_t e = hipMalloc(&p, need);
         if (e == hipSuccess) bytes = need;
         return e;
     }
-    void release() { if (p) (void)hipFree(p); p = nullptr; bytes = 0; }
+    void release() { if (p && !borrowed) (void)hipFree(p); p = nullptr; bytes = 0; borrowed = false; }
     template <typename T> T* as() const { return static_cast<T*>(p); }
+    static DevBuf view(void* ptr, size_t n) { DevBuf b; b.p = ptr; b.bytes = n; b.borrowed = true; return b; }
 };
 
 struct PhaseTimer {
@@ -52,6 +81,7 @@ struct PhaseTimer {
 constexpr int kFirstHold = 8, kMaxHold = 1024;
 
 struct flstm_core_plan {
+    int device = 0;
     int num_cus = 0;
     int clock_khz = 0;   // maximum engine clock the runtime reports
     Dims d{};
@@ -163,6 +193,12 @@ extern "C" int flstm_core_create(size_t batch, size_t input_size, size_t hidden_
                             p->wall_khz <= 0))
         p->wall_khz = 100000;
     if (e != hipSuccess) { delete p; return int(e); }
+    p->device = dev;
+    {   // this device's copy of the static scratch array: looked up now, while its device is current
+        void* sp = nullptr;
+        const int rc = static_scratch(dev, &sp);
+        if (rc) { delete p; return rc; }
+    }
     p->d.B = int(batch);
     p->d.I = int(input_size);
     p->d.H = int(hidden_size);
@@ -236,6 +272,7 @@ extern "C" long flstm_core_get_info(const flstm_core_plan* p, const char* name) 
     if (!strcmp(name, "demotions_bwd")) return p->demotions_bwd;
     if (!strcmp(name, "hold_fwd")) return p->hold_fwd;
     if (!strcmp(name, "hold_bwd")) return p->hold_bwd;
+    if (!strcmp(name, "static_scratch_bytes")) return long(kStaticScratchBytes);
     if (!strcmp(name, "num_cus")) return p->num_cus;
     if (!strcmp(name, "clock_khz")) return p->clock_khz;
     if (!strcmp(name, "hidden_padded")) return p->d.Hp;
@@ -366,23 +403,14 @@ int forward_once(flstm_core_plan* p, size_t T, const void* x, flstm_dtype x_dtyp
     return 0;
 }
 
-}  // namespace
-
-extern "C" int flstm_core_forward(flstm_core_plan* p, size_t T, const void* x, flstm_dtype x_dtype,
-                                  const void* h0, const void* c0, flstm_dtype state_dtype, void* y,
-                                  flstm_dtype y_dtype, void* hy, void* cy, flstm_dtype out_state_dtype,
-                                  int save_for_backward, void* stream) {
-    if (!p) return FLSTM_E_INVALID;
-    if (!p->weights_packed || !p->bias_packed) return FLSTM_E_NOT_PACKED;
-    if (T == 0) return 0;
-    if (!x || T > (size_t(1) << 24)) return FLSTM_E_INVALID;
-    hipStream_t s = static_cast<hipStream_t>(stream);
+// One whole forward pass: projection, recurrence, outputs, one wait, status.  The outputs are written behind the
+// recurrence without waiting for its status: if the persistent launch gave up, the whole pass is repeated
+// step-wise and overwrites them.
+int forward_pass(flstm_core_plan* p, size_t T, const void* x, flstm_dtype x_dtype, const void* h0, const void* c0,
+                 flstm_dtype state_dtype, void* y, flstm_dtype y_dtype, void* hy, void* cy,
+                 flstm_dtype out_state_dtype, hipStream_t s) {
     const Dims& d = p->d;
     const size_t TB = T * size_t(d.B);
-    p->have_cache = false;
-
-    // The outputs are written behind the recurrence without waiting for its status: if the persistent launch gave
-    // up, the whole pass is repeated step-wise and overwrites them.
     for (int attempt = 0;; ++attempt) {
         int rc = forward_once(p, T, x, x_dtype, h0, c0, state_dtype, s);
         if (rc) return rc;
@@ -404,8 +432,74 @@ extern "C" int flstm_core_forward(flstm_core_plan* p, size_t T, const void* x, f
     p->ms_fwd[1] = elapsed(p->tm.ev[1], p->tm.ev[2]);
     p->ms_fwd[2] = elapsed(p->tm.ev[0], p->tm.ev[2]);
     p->fw.open = false;
+    return 0;
+}
+
+}  // namespace
+
+extern "C" int flstm_core_forward(flstm_core_plan* p, size_t T, const void* x, flstm_dtype x_dtype,
+                                  const void* h0, const void* c0, flstm_dtype state_dtype, void* y,
+                                  flstm_dtype y_dtype, void* hy, void* cy, flstm_dtype out_state_dtype,
+                                  int save_for_backward, void* stream) {
+    if (!p) return FLSTM_E_INVALID;
+    if (!p->weights_packed || !p->bias_packed) return FLSTM_E_NOT_PACKED;
+    if (T == 0) return 0;
+    if (!x || T > (size_t(1) << 24)) return FLSTM_E_INVALID;
+    p->have_cache = false;
+    int rc = forward_pass(p, T, x, x_dtype, h0, c0, state_dtype, y, y_dtype, hy, cy, out_state_dtype,
+                          static_cast<hipStream_t>(stream));
+    if (rc) return rc;
     if (save_for_backward) { p->have_cache = true; p->T_cache = T; }
     return 0;
+}
+
+namespace {
+
+size_t align256(size_t v) { return (v + 255) / 256 * 256; }
+
+}  // namespace
+
+extern "C" int flstm_core_forward_static(flstm_core_plan* p, size_t T, const void* x, flstm_dtype x_dtype,
+                                         const void* h0, const void* c0, flstm_dtype state_dtype, void* y,
+                                         flstm_dtype y_dtype, void* hy, void* cy, flstm_dtype out_state_dtype,
+                                         void* stream) {
+    if (!p) return FLSTM_E_INVALID;
+    if (!p->weights_packed || !p->bias_packed) return FLSTM_E_NOT_PACKED;
+    if (T == 0) return 0;
+    if (!x || T > (size_t(1) << 24) || p->fw.open || p->bw.open) return FLSTM_E_INVALID;
+    int dev = -1;
+    FL_TRY(hipGetDevice(&dev));
+    if (dev != p->device) return FLSTM_E_INVALID;
+    void* base = nullptr;
+    int rc = static_scratch(dev, &base);
+    if (rc) return rc;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const Dims& d = p->d;
+    const size_t TB = T * size_t(d.B);
+    // the same buffers forward_setup() sizes, carved out of the static array instead of allocated
+    const bool x_in_place = (x_dtype == FLSTM_F16 && d.I == d.Ip);
+    const size_t need[6] = {256,
+                            x_in_place ? 0 : TB * d.Ip * sizeof(half_t),
+                            TB * 4 * d.Hp * sizeof(half_t),
+                            (TB + d.B) * d.Hp * sizeof(half_t),
+                            (TB + d.B) * d.Hp * sizeof(float),
+                            4 * exchange_slot_halfs(d.B, d.Hp) * sizeof(half_t)};
+    size_t off[6], total = 0;
+    for (int i = 0; i < 6; ++i) { off[i] = total; total += align256(need[i]); }
+    if (total > kStaticScratchBytes) return FLSTM_E_TOO_LARGE;
+    char* b = static_cast<char*>(base);
+    DevBuf* slot[6] = {&p->status, &p->X16, &p->G, &p->Y, &p->C, &p->xch_f};
+    DevBuf saved[6];
+    for (int i = 0; i < 6; ++i) { saved[i] = *slot[i]; *slot[i] = DevBuf::view(b + off[i], need[i]); }
+    const bool had_cache = p->have_cache;
+    p->have_cache = false;   // (the plan's own caches are untouched, but no pass may use the borrowed ones later)
+    // status word and seat counters start at zero; the array keeps whatever the last call left
+    rc = int(fill_zero(p->status.p, 64, s));
+    if (rc == 0)
+        rc = forward_pass(p, T, x, x_dtype, h0, c0, state_dtype, y, y_dtype, hy, cy, out_state_dtype, s);
+    for (int i = 0; i < 6; ++i) *slot[i] = saved[i];
+    p->have_cache = had_cache;
+    return rc;
 }
 
 namespace {

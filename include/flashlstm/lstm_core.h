@@ -32,7 +32,8 @@ enum {
     FLSTM_E_INVALID = 1,        /* same value as hipErrorInvalidValue */
     FLSTM_E_NOT_PACKED = 2001,  /* forward before weights were packed */
     FLSTM_E_NO_CACHE = 2002,    /* backward without a matching forward(save_for_backward=1) */
-    FLSTM_E_STALLED = 2003      /* recurrence kernels gave up waiting even in step-wise mode */
+    FLSTM_E_STALLED = 2003,     /* recurrence kernels gave up waiting even in step-wise mode */
+    FLSTM_E_TOO_LARGE = 2004    /* flstm_core_forward_static: the pass needs more scratch memory than the fixed array holds */
 };
 
 /* Creates a plan for fixed (batch, input, hidden); sequence length may vary per call. */
@@ -55,7 +56,8 @@ int flstm_core_set_option(flstm_core_plan* plan, const char* name, long value);
  * direction still runs step-wise before the persistent kernel is tried again; 0 = not demoted), "slice_fwd", "slice_bwd" (hidden units
  * per workgroup of the recurrence kernels), "row_tiles" (16-row tiles of a 32-row batch block that the
  * recurrence fetches and multiplies: 1 for batches of at most 16 rows, else 2), "hidden_padded",
- * "input_padded", "device_bytes" (device memory the plan holds), "num_cus" and "clock_khz" (compute units and
+ * "input_padded", "device_bytes" (device memory the plan holds), "static_scratch_bytes" (size of the fixed scratch
+ * array of flstm_core_forward_static), "num_cus" and "clock_khz" (compute units and
  * maximum engine clock of the plan's device).
  * Unknown names give -1. */
 long flstm_core_get_info(const flstm_core_plan* plan, const char* name);
@@ -74,6 +76,22 @@ int flstm_core_forward(flstm_core_plan* plan, size_t seq_len,
                        void* y, flstm_dtype y_dtype,
                        void* hy, void* cy, flstm_dtype out_state_dtype,
                        int save_for_backward, void* stream);
+
+/* flstm_core_forward for callers that cannot allocate device memory (code under HIP graph capture, tight serving
+ * loops, harnesses that forbid hipMalloc).  It has no counterpart in the reference.  Same arguments, results and
+ * kernels as flstm_core_forward with save_for_backward = 0, but everything the kernels need beyond the caller's
+ * tensors and the plan's packed weights -- status word, converted x rows, x-projection / gate rows, state rows,
+ * exchange ring -- lives in one fixed 64 MiB array in the library's device image instead of buffers grown by the
+ * plan: the call allocates and frees nothing.  A pass that needs more (about T*B*(14*Hp + 2*Ip) bytes; the limit
+ * is flstm_core_get_info(plan, "static_scratch_bytes")) is rejected with FLSTM_E_TOO_LARGE before any work is
+ * enqueued.  Nothing is kept for a backward pass, and a cache that an earlier flstm_core_forward left in the plan
+ * stays valid.  Every call on a GPU uses that GPU's one array, whichever plan it comes from: calls that overlap
+ * on one GPU (two threads, two streams) race; calls on different GPUs do not.  The plan's device must be current. */
+int flstm_core_forward_static(flstm_core_plan* plan, size_t seq_len,
+                              const void* x, flstm_dtype x_dtype,
+                              const void* h0, const void* c0, flstm_dtype state_dtype,
+                              void* y, flstm_dtype y_dtype,
+                              void* hy, void* cy, flstm_dtype out_state_dtype, void* stream);
 
 /* BPTT for the last forward of this plan.  d_hn/d_cn may be null (zeros).  Any output may be null.
  * grad_scale (a power of two, 1 if <= 0) multiplies dY on load and is divided out of every
