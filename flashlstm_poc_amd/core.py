@@ -54,6 +54,10 @@ def load_library() -> ctypes.CDLL:
     lib.flstm_core_forward.argtypes = [vp, sz, vp, i32, vp, vp, i32, vp, i32, vp, vp, i32, i32, vp]
     lib.flstm_core_forward_static.argtypes = [vp, sz, vp, i32, vp, vp, i32, vp, i32, vp, vp, i32, vp]
     lib.flstm_core_forward_static.restype = i32
+    lib.flstm_core_tune.argtypes = [vp, sz, i32, i32, vp]
+    lib.flstm_core_tune.restype = i32
+    lib.flstm_core_tuned_ms.argtypes = [vp, sz, c.c_char_p]
+    lib.flstm_core_tuned_ms.restype = c.c_double
     lib.flstm_core_backward.argtypes = [vp, sz, vp, i32, vp, i32, vp, vp, i32, c.c_float, vp, i32,
                                         vp, vp, vp, vp, vp, vp, vp]
     lib.flstm_core_cache_ptr.argtypes = [vp, i32, c.POINTER(vp), c.POINTER(sz)]
@@ -117,6 +121,18 @@ class LstmCore:
 
     def last_ms(self, phase: str) -> float:
         return float(self.lib.flstm_core_last_ms(self._h, phase.encode()))
+
+    def tune(self, seq_len: int, repeats: int = 3, try_stepwise: bool = False) -> dict:
+        """flstm_core_tune: times the launch choices for this sequence length on synthetic data, caches the best in
+        the plan (later passes of similar length use them) and returns them with the best time found per phase."""
+        rc = self.lib.flstm_core_tune(self._h, int(seq_len), int(repeats), 1 if try_stepwise else 0, self._stream())
+        if rc != 0:
+            raise RuntimeError(f"flstm_core_tune failed with status {rc}")
+        out = {k: self.info("tuned_" + k) for k in ("T", "row_tiles_fwd", "row_tiles_bwd", "stepwise_fwd", "stepwise_bwd",
+                                                    "dw_splits")}
+        for ph in ("fwd_rec", "bwd_rec", "bwd_dw"):
+            out[ph + "_ms"] = float(self.lib.flstm_core_tuned_ms(self._h, int(seq_len), ph.encode()))
+        return out
 
     def pack(self, w_ih, w_hh, b_ih=None, b_hh=None) -> None:
         import torch

@@ -10,8 +10,10 @@
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
+#include <cmath>
 #include <mutex>
 #include <new>
+#include <vector>
 
 #include "../../include/flashlstm/lstm_core.h"
 #include "gemm.h"
@@ -94,6 +96,14 @@ struct flstm_core_plan {
     // tried again.  Every further give-up doubles the hold (at most kMaxHold passes).
     int hold_fwd = 0, hold_bwd = 0, backoff_fwd = kFirstHold, backoff_bwd = kFirstHold;
     long fallbacks = 0, demotions_fwd = 0, demotions_bwd = 0;
+    // Tuned launch choices per sequence length (flstm_core_tune): 16- or 32-row blocks and persistent or step-wise
+    // launches per direction, split-K count of the weight-gradient GEMM.  eff_* hold the entry in force for the
+    // sequence length of the current pass (0 = no tuned value: the rules of thumb decide); explicit options win.
+    struct Tuned { size_t T; int mt_f, mt_b, step_f, step_b, dw_splits; float ms_f, ms_b, ms_dw; };
+    std::vector<Tuned> tuned;
+    int opt_mt_f = 0, opt_mt_b = 0;
+    int eff_mt_f = 0, eff_mt_b = 0, eff_step_f = 0, eff_step_b = 0, eff_dw = 0;
+    size_t eff_T = 0;
     int* status_host = nullptr;   // pinned: the device status word lands here with the end-of-pass copy
     int inject_stall = 0;         // test hook: treat the next N persistent passes as if their launch had given up
     // weights
@@ -124,10 +134,31 @@ namespace {
     } while (0)
 
 void replan(flstm_core_plan* p) {
-    p->Lf = plan_rec_fwd(p->d.B, p->d.Hp, p->num_cus, p->opt_stepwise || p->hold_fwd > 0);
-    p->Lb = plan_rec_bwd(p->d.B, p->d.Hp, p->num_cus, p->opt_stepwise || p->hold_bwd > 0);
+    p->Lf = plan_rec_fwd(p->d.B, p->d.Hp, p->num_cus, p->opt_stepwise || p->hold_fwd > 0 || p->eff_step_f,
+                         p->opt_mt_f ? p->opt_mt_f : p->eff_mt_f);
+    p->Lb = plan_rec_bwd(p->d.B, p->d.Hp, p->num_cus, p->opt_stepwise || p->hold_bwd > 0 || p->eff_step_b,
+                         p->opt_mt_b ? p->opt_mt_b : p->eff_mt_b);
     p->ks_f = rec_fwd_ks(p->Lf, p->d.Hp);
     p->ks_b = rec_bwd_ks(p->Lb, p->d.Hp);
+}
+
+// Puts the tuned entry for sequence length T in force: the entry tuned at exactly T, else the nearest one within a
+// factor of two, else none.
+void use_tuned(flstm_core_plan* p, size_t T) {
+    const flstm_core_plan::Tuned* best = nullptr;
+    double best_d = 1.0;   // |log2(T / T')| <= 1
+    for (const auto& t : p->tuned) {
+        const double dist = std::fabs(std::log2(double(T) / double(t.T)));
+        if (dist <= best_d && (!best || dist < best_d)) { best = &t; best_d = dist; }
+    }
+    const int mt_f = best ? best->mt_f : 0, mt_b = best ? best->mt_b : 0, sf = best ? best->step_f : 0,
+              sb = best ? best->step_b : 0;
+    p->eff_dw = best ? best->dw_splits : 0;
+    p->eff_T = best ? best->T : 0;
+    if (mt_f != p->eff_mt_f || mt_b != p->eff_mt_b || sf != p->eff_step_f || sb != p->eff_step_b) {
+        p->eff_mt_f = mt_f; p->eff_mt_b = mt_b; p->eff_step_f = sf; p->eff_step_b = sb;
+        replan(p);
+    }
 }
 
 // The status word of the recurrence kernels travels to pinned host memory behind the pass's last kernel, so the
@@ -240,6 +271,13 @@ extern "C" int flstm_core_set_option(flstm_core_plan* p, const char* name, long 
         }
         return 0;
     }
+    if (!strcmp(name, "row_tiles_fwd") || !strcmp(name, "row_tiles_bwd")) {
+        if (value < 0 || value > 2) return FLSTM_E_INVALID;
+        (name[10] == 'f' ? p->opt_mt_f : p->opt_mt_b) = int(value);
+        replan(p);
+        return 0;
+    }
+    if (!strcmp(name, "clear_tuned")) { p->tuned.clear(); use_tuned(p, 1); return 0; }
     if (!strcmp(name, "inject_stall")) { if (value < 0) return FLSTM_E_INVALID; p->inject_stall = int(value); return 0; }
     if (!strcmp(name, "dw_splits")) { if (value < 0) return FLSTM_E_INVALID; p->opt_dw_splits = int(value); return 0; }
     if (!strcmp(name, "accumulate_grads")) { p->opt_accumulate = value != 0; return 0; }
@@ -255,6 +293,15 @@ extern "C" long flstm_core_get_info(const flstm_core_plan* p, const char* name) 
     if (!strcmp(name, "resident_fwd")) return p->Lf.resident;
     if (!strcmp(name, "resident_bwd")) return p->Lb.resident;
     if (!strcmp(name, "row_tiles")) return p->Lf.mt;
+    if (!strcmp(name, "row_tiles_fwd")) return p->Lf.mt;
+    if (!strcmp(name, "row_tiles_bwd")) return p->Lb.mt;
+    if (!strcmp(name, "tuned_entries")) return long(p->tuned.size());
+    if (!strcmp(name, "tuned_T")) return long(p->eff_T);
+    if (!strcmp(name, "tuned_row_tiles_fwd")) return p->eff_mt_f;
+    if (!strcmp(name, "tuned_row_tiles_bwd")) return p->eff_mt_b;
+    if (!strcmp(name, "tuned_stepwise_fwd")) return p->eff_step_f;
+    if (!strcmp(name, "tuned_stepwise_bwd")) return p->eff_step_b;
+    if (!strcmp(name, "tuned_dw_splits")) return p->eff_dw;
     if (!strcmp(name, "device_bytes")) {
         size_t sum = 0;
         for (const DevBuf* b : {&p->wih_p, &p->wih_t, &p->wfrag_f, &p->wfrag_b, &p->bias_p, &p->X16, &p->G, &p->Y, &p->C,
@@ -411,6 +458,7 @@ int forward_pass(flstm_core_plan* p, size_t T, const void* x, flstm_dtype x_dtyp
                  flstm_dtype out_state_dtype, hipStream_t s) {
     const Dims& d = p->d;
     const size_t TB = T * size_t(d.B);
+    use_tuned(p, T);
     for (int attempt = 0;; ++attempt) {
         int rc = forward_once(p, T, x, x_dtype, h0, c0, state_dtype, s);
         if (rc) return rc;
@@ -602,25 +650,17 @@ int backward_finish(flstm_core_plan* p, const void* x, flstm_dtype x_dtype, floa
     const size_t TB = p->bw.T * size_t(d.B);
     const float invS = 1.f / p->bw.S;
     // k-major operands exactly as the recurrence left them (H_prev of step t is row block t of the state array,
-    // row block 0 = h0), split over K, fp32 partials
-    for (int which = 0; which < 2; ++which) {
-        float* dst = which == 0 ? dW_ih : dW_hh;
-        if (!dst) continue;
-        const half_t* Bop;
-        int ncols, out_cols;
-        size_t ldb;
-        if (which == 0) {
-            const bool direct = (x_dtype == FLSTM_F16 && d.I == d.Ip);
-            Bop = direct ? static_cast<const half_t*>(x) : p->X16.as<half_t>();
-            ncols = d.Ip; ldb = size_t(d.Ip); out_cols = d.I;
-        } else {
-            Bop = p->Y.as<half_t>();
-            ncols = d.Hp; ldb = size_t(d.Hp); out_cols = d.H;
-        }
-        const int tiles = int(ceil_div(size_t(4) * d.Hp, 256) * ceil_div(size_t(ncols), 256));
+    // row block 0 = h0), split over K, fp32 partials.  Both gradients come out of ONE launch, dG^T * [X | H_prev]:
+    // dG (the large operand) is read once, and the tiles of both products fill the machine together.
+    const bool direct = (x_dtype == FLSTM_F16 && d.I == d.Ip);
+    const half_t* Xop = direct ? static_cast<const half_t*>(x) : p->X16.as<half_t>();
+    const half_t* Hop = p->Y.as<half_t>();
+    const int n_ih = dW_ih ? d.Ip : 0, n_hh = dW_hh ? d.Hp : 0, ncols = n_ih + n_hh;
+    if (ncols > 0) {
+        const int tiles = int(ceil_div(size_t(4) * d.Hp, 256) * (ceil_div(size_t(n_ih), 256) + ceil_div(size_t(n_hh), 256)));
         // automatic: one work item (tile x split) per compute unit, at least four 64-row slabs per split
         // (measured best or within a few percent of it from 4 to 256 tiles)
-        int want = p->opt_dw_splits;
+        int want = p->opt_dw_splits > 0 ? p->opt_dw_splits : p->eff_dw;
         if (want <= 0) {
             want = int(ceil_div(size_t(p->num_cus > 0 ? p->num_cus : 256), size_t(tiles)));
             const int cap = int(TB / 256);
@@ -632,12 +672,18 @@ int backward_finish(flstm_core_plan* p, const void* x, flstm_dtype x_dtype, floa
         FL_TRY(p->dw_part.reserve(per * splits * sizeof(float)));
         GemmNT g{};
         g.A = p->dG.as<half_t>(); g.lda = size_t(4) * d.Hp;
-        g.B = Bop; g.ldb = ldb;
         g.M = 4 * d.Hp; g.N = ncols; g.K = int(TB);
+        if (n_ih && n_hh) {
+            g.B = Xop; g.ldb = size_t(d.Ip); g.N1 = n_ih;
+            g.B2 = Hop; g.ldb2 = size_t(d.Hp);
+        } else {
+            g.B = n_ih ? Xop : Hop; g.ldb = size_t(n_ih ? d.Ip : d.Hp);
+        }
         g.C16 = nullptr; g.C32 = p->dw_part.as<float>(); g.ldc = size_t(ncols);
         g.alpha = 1.f; g.splits = splits; g.split_stride = per;
         FL_TRY(launch_gemm_tn(g, s));
-        FL_TRY(reduce_dw(d, p->dw_part.as<float>(), splits, ncols, out_cols, invS, p->opt_accumulate != 0, dst, s));
+        FL_TRY(reduce_dw(d, p->dw_part.as<float>(), splits, size_t(ncols), 0, n_ih, d.I, invS, p->opt_accumulate != 0, dW_ih, s));
+        FL_TRY(reduce_dw(d, p->dw_part.as<float>(), splits, size_t(ncols), n_ih, n_hh, d.H, invS, p->opt_accumulate != 0, dW_hh, s));
     }
     FL_TRY(hipEventRecord(p->tm.ev[6], s));
     if (db_ih || db_hh)
@@ -666,6 +712,7 @@ extern "C" int flstm_core_backward(flstm_core_plan* p, size_t T, const void* x, 
     if (dW_ih && !x) return FLSTM_E_INVALID;
     hipStream_t s = static_cast<hipStream_t>(stream);
     const float S = grad_scale > 0.f ? grad_scale : 1.f;
+    use_tuned(p, T);
 
     // dX and the weight gradients follow the recurrence without waiting for its status (one wait per pass); a
     // persistent launch that gave up is found at the end and the pass repeated step-wise over the same outputs.
@@ -710,6 +757,7 @@ extern "C" int flstm_core_forward_begin(flstm_core_plan* p, size_t T, const void
     if (T == 0 || !x || T > (size_t(1) << 24)) return FLSTM_E_INVALID;
     p->have_cache = false;
     for (float& m : p->ms_fwd) m = -1.f;
+    use_tuned(p, T);
     return forward_setup(p, T, x, x_dtype, h0, c0, state_dtype, static_cast<hipStream_t>(stream));
 }
 
@@ -752,6 +800,7 @@ extern "C" int flstm_core_backward_begin(flstm_core_plan* p, size_t T, const voi
     if (!p->have_cache || p->T_cache != T) return FLSTM_E_NO_CACHE;
     for (float& m : p->ms_bwd) m = -1.f;
     const float S = grad_scale > 0.f ? grad_scale : 1.f;
+    use_tuned(p, T);
     return backward_setup(p, T, dY, dy_dtype, d_hn, d_cn, dstate_dtype, S, dx, dx_dtype, static_cast<hipStream_t>(stream));
 }
 
@@ -858,4 +907,109 @@ extern "C" int flstm_gemm_tn(const void* A, size_t lda, const void* B, size_t ld
     FL_TRY(launch_gemm_tn(g, s));
     FL_TRY(reduce_partials(static_cast<const float*>(workspace), eff, M * N, int(M), int(N), ldc, C, s));
     return 0;
+}
+
+// ---- tuner
+
+extern "C" int flstm_core_tune(flstm_core_plan* p, size_t T, int repeats, int try_stepwise, void* stream) {
+    if (!p || T == 0 || T > (size_t(1) << 24) || p->fw.open || p->bw.open) return FLSTM_E_INVALID;
+    if (!p->weights_packed || !p->bias_packed) return FLSTM_E_NOT_PACKED;
+    if (repeats < 1) repeats = 1;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const Dims& d = p->d;
+    const size_t TB = T * size_t(d.B);
+    // synthetic inputs: zeros (the kernels' time does not depend on the values)
+    DevBuf x, dy, dwi, dwh;
+    int rc = 0;
+    auto fail = [&](int code) { x.release(); dy.release(); dwi.release(); dwh.release(); return code; };
+    if (x.reserve(TB * d.I * sizeof(half_t)) != hipSuccess || dy.reserve(TB * d.H * sizeof(half_t)) != hipSuccess ||
+        dwi.reserve(size_t(4) * d.H * d.I * sizeof(float)) != hipSuccess ||
+        dwh.reserve(size_t(4) * d.H * d.H * sizeof(float)) != hipSuccess)
+        return fail(int(hipErrorOutOfMemory));
+    if (fill_zero(x.p, TB * d.I * sizeof(half_t), s) != hipSuccess || fill_zero(dy.p, TB * d.H * sizeof(half_t), s) != hipSuccess)
+        return fail(int(hipErrorUnknown));
+    // the plan's explicit options and tuned state are set aside while candidates run
+    const int keep_step = p->opt_stepwise, keep_mtf = p->opt_mt_f, keep_mtb = p->opt_mt_b, keep_dw = p->opt_dw_splits,
+              keep_acc = p->opt_accumulate;
+    const bool keep_cache = p->have_cache;
+    const std::vector<flstm_core_plan::Tuned> keep_tuned = p->tuned;
+    p->tuned.clear();
+    p->opt_accumulate = 0;
+    auto restore = [&]() {
+        p->opt_stepwise = keep_step; p->opt_mt_f = keep_mtf; p->opt_mt_b = keep_mtb; p->opt_dw_splits = keep_dw;
+        p->opt_accumulate = keep_acc;
+        p->tuned = keep_tuned;
+        p->have_cache = false;   // the caches now hold the synthetic sequence
+        (void)keep_cache;
+        use_tuned(p, T);
+        replan(p);
+    };
+    flstm_core_plan::Tuned best{};
+    best.T = T; best.ms_f = best.ms_b = best.ms_dw = -1.f;
+    auto run = [&](float& f_ms, float& b_ms, float& dw_ms) -> int {
+        f_ms = b_ms = dw_ms = 1e30f;
+        for (int r = 0; r <= repeats; ++r) {   // first pass is a warm-up
+            int e = flstm_core_forward(p, T, x.p, FLSTM_F16, nullptr, nullptr, FLSTM_F16, nullptr, FLSTM_F16, nullptr, nullptr,
+                                       FLSTM_F16, 1, s);
+            if (e) return e;
+            e = flstm_core_backward(p, T, x.p, FLSTM_F16, dy.p, FLSTM_F16, nullptr, nullptr, FLSTM_F16, 1.f, nullptr, FLSTM_F16,
+                                    dwi.as<float>(), dwh.as<float>(), nullptr, nullptr, nullptr, nullptr, s);
+            if (e) return e;
+            if (r == 0) continue;
+            if (p->ms_fwd[1] > 0 && p->ms_fwd[1] < f_ms) f_ms = p->ms_fwd[1];
+            if (p->ms_bwd[0] > 0 && p->ms_bwd[0] < b_ms) b_ms = p->ms_bwd[0];
+            if (p->ms_bwd[2] > 0 && p->ms_bwd[2] < dw_ms) dw_ms = p->ms_bwd[2];
+        }
+        return 0;
+    };
+    // 1) row-block height and launch mode of the two recurrences (independent of each other and of the GEMMs)
+    p->opt_dw_splits = 0;
+    for (int step = 0; step <= (try_stepwise ? 1 : 0); ++step) {
+        for (int mt = 1; mt <= 2; ++mt) {
+            p->opt_stepwise = step; p->opt_mt_f = mt; p->opt_mt_b = mt;
+            replan(p);
+            const bool f_is = (p->Lf.mt == mt), b_is = (p->Lb.mt == mt);   // 16-row blocks may not fit
+            if (!f_is && !b_is) continue;
+            float f_ms, b_ms, dw_ms;
+            rc = run(f_ms, b_ms, dw_ms);
+            if (rc) { restore(); return fail(rc); }
+            if (f_is && (best.ms_f < 0 || f_ms < best.ms_f)) { best.ms_f = f_ms; best.mt_f = mt; best.step_f = step; }
+            if (b_is && (best.ms_b < 0 || b_ms < best.ms_b)) { best.ms_b = b_ms; best.mt_b = mt; best.step_b = step; }
+        }
+    }
+    // 2) split-K count of the weight-gradient GEMM around the rule of thumb (one work item per compute unit)
+    p->opt_stepwise = best.step_f && best.step_b; p->opt_mt_f = best.mt_f; p->opt_mt_b = best.mt_b;
+    replan(p);
+    const int tiles = int(ceil_div(size_t(4) * d.Hp, 256) * (ceil_div(size_t(d.Ip), 256) + ceil_div(size_t(d.Hp), 256)));
+    int rule = int(ceil_div(size_t(p->num_cus > 0 ? p->num_cus : 256), size_t(tiles)));
+    if (rule < 1) rule = 1;
+    int last_eff = -1;
+    for (int cand : {rule / 2, rule, rule * 2, rule * 4}) {
+        if (cand < 1 || cand > 64) continue;
+        const int eff = gemm_effective_splits(int(TB), cand);
+        if (eff == last_eff) continue;
+        last_eff = eff;
+        p->opt_dw_splits = cand;
+        float f_ms, b_ms, dw_ms;
+        rc = run(f_ms, b_ms, dw_ms);
+        if (rc) { restore(); return fail(rc); }
+        if (best.ms_dw < 0 || dw_ms < best.ms_dw) { best.ms_dw = dw_ms; best.dw_splits = cand; }
+    }
+    restore();
+    for (auto it = p->tuned.begin(); it != p->tuned.end();)
+        it = (it->T == T) ? p->tuned.erase(it) : it + 1;
+    p->tuned.push_back(best);
+    use_tuned(p, T);
+    return fail(0);
+}
+
+extern "C" double flstm_core_tuned_ms(const flstm_core_plan* p, size_t T, const char* phase) {
+    if (!p || !phase) return -1.0;
+    for (const auto& t : p->tuned)
+        if (t.T == T) {
+            if (!strcmp(phase, "fwd_rec")) return t.ms_f;
+            if (!strcmp(phase, "bwd_rec")) return t.ms_b;
+            if (!strcmp(phase, "bwd_dw")) return t.ms_dw;
+        }
+    return -1.0;
 }

@@ -16,6 +16,10 @@ struct GemmNT {
     int splits; size_t split_stride;
     // optional per-column term: C = alpha * (A * B^T) + bias[n]  (NT form only)
     const float* bias;
+    // TN form only: a second B operand.  With B2 set, columns [0, N1) of C come from B (N1 columns) and columns
+    // [N1, N) from B2 (N - N1 columns, row pitch ldb2): one launch forms A^T * [B | B2] and reads A once.  N1 must
+    // be a multiple of 8; output tiles never straddle the seam (each side is tiled on its own).
+    const half_t* B2; size_t ldb2; int N1;
 };
 
 // Enqueue on `stream`. Returns hipSuccess or the launch error.

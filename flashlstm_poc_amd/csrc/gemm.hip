@@ -397,6 +397,18 @@ __global__ __launch_bounds__(kThreads) void gemm_tn_256x256(GemmNT g, TileOrder 
 
     int tm, tn, z;
     if (!work_item(order, blockIdx.x, tm, tn, z)) return;
+    // two B operands side by side: each side has its own tiles, so a tile reads one operand only
+    if (g.B2) {
+        const int tiles_n1 = (g.N1 + BN - 1) / BN;
+        if (tn >= tiles_n1) {
+            tn -= tiles_n1;
+            g.B = g.B2; g.ldb = g.ldb2;
+            g.C32 += g.N1;
+            g.N -= g.N1;
+        } else {
+            g.N = g.N1;
+        }
+    }
     const int m0 = tm * BM, n0 = tn * BN;
     const int nslab_total = (g.K + BK - 1) / BK;
     const int slab_begin = z * slabs_per_split;
@@ -559,7 +571,9 @@ hipError_t launch_gemm_tn(const GemmNT& g, hipStream_t stream) {
     if (e != hipSuccess) return e;
     const int nslab = (g.K + BK - 1) / BK;
     const int slabs_per_split = (nslab + splits - 1) / splits;
-    const int tiles_m = (g.M + BM - 1) / BM, tiles_n = (g.N + BN - 1) / BN;
+    if (g.B2 && (g.C32 == nullptr || g.N1 <= 0 || g.N1 >= g.N || g.N1 % 8 != 0 || g.ldb2 % 8 != 0)) return hipErrorInvalidValue;
+    const int tiles_m = (g.M + BM - 1) / BM;
+    const int tiles_n = g.B2 ? (g.N1 + BN - 1) / BN + (g.N - g.N1 + BN - 1) / BN : (g.N + BN - 1) / BN;
     const TileOrder order = make_order(tiles_m, tiles_n, splits);
     hipLaunchKernelGGL(gemm_tn_256x256, dim3(order.per_xcd * 256), dim3(kThreads), kLdsBytesTN, stream, g, order,
                        slabs_per_split);

@@ -46,11 +46,11 @@ hipError_t gather_from_float(const float* in, size_t ld_in, size_t rows, int col
 hipError_t transpose_pad(const void* in, int in_f32, size_t rows, int cols, size_t ld_in, half_t* out,
                          int cols_out, size_t ld_out, hipStream_t s);
 
-// Sums split-K partials [splits][4Hp][ncols] (packed gate rows) into dst [4H][out_cols] (PyTorch row
-// order, the first out_cols columns), times `scale`; `accumulate` adds to dst instead of overwriting it (the
-// beta=1 accumulation over chunks of flashlstm_v2/src/lstm_backward.cu:1112-1142).
-hipError_t reduce_dw(const Dims& d, const float* partial, int splits, int ncols, int out_cols, float scale,
-                     bool accumulate, float* dst, hipStream_t s);
+// Sums columns [col0, col0 + ncols) of the split-K partials [splits][4Hp][ld] (packed gate rows) into dst
+// [4H][out_cols] (PyTorch row order, the first out_cols of those columns), times `scale`; `accumulate` adds to dst
+// instead of overwriting it (the beta=1 accumulation over chunks of flashlstm_v2/src/lstm_backward.cu:1112-1142).
+hipError_t reduce_dw(const Dims& d, const float* partial, int splits, size_t ld, int col0, int ncols, int out_cols,
+                     float scale, bool accumulate, float* dst, hipStream_t s);
 // db_part [ng][4Hp] packed -> db_ih == db_hh (4H), times scale (flashlstm_v2/src/lstm_backward.cu:1218-1231).
 hipError_t reduce_db(const Dims& d, const float* db_part, int ng, float scale, bool accumulate, float* db_ih,
                      float* db_hh, hipStream_t s);

@@ -147,17 +147,18 @@ __global__ void transpose_pad_kernel(const TIn* __restrict__ in, size_t rows, in
     }
 }
 
-// partial [splits][4Hp][ncols] with packed gate rows -> dst [4H][out_cols] in PyTorch row order
-__global__ void reduce_dw_kernel(Dims d, const float* __restrict__ partial, int splits, int ncols, int out_cols,
-                                 float scale, int accumulate, float* __restrict__ dst) {
+// columns [col0, col0 + ncols) of partial [splits][4Hp][ld] with packed gate rows -> dst [4H][out_cols] in PyTorch
+// row order
+__global__ void reduce_dw_kernel(Dims d, const float* __restrict__ partial, int splits, size_t ld, int col0, int ncols,
+                                 int out_cols, float scale, int accumulate, float* __restrict__ dst) {
     const size_t idx = size_t(blockIdx.x) * kT + threadIdx.x;
-    const size_t per = size_t(4) * d.Hp * ncols;
-    if (idx >= per) return;
+    if (idx >= size_t(4) * d.Hp * ncols) return;
     const int q = int(idx / ncols), n = int(idx % ncols);
     const int row = torch_row(q, d.H);
     if (row < 0 || n >= out_cols) return;
+    const size_t per = size_t(4) * d.Hp * ld, src = size_t(q) * ld + col0 + n;
     float s = 0.f;
-    for (int z = 0; z < splits; ++z) s += partial[size_t(z) * per + idx];
+    for (int z = 0; z < splits; ++z) s += partial[size_t(z) * per + src];
     float* out = dst + size_t(row) * out_cols + n;
     *out = accumulate ? *out + scale * s : scale * s;
 }
@@ -292,12 +293,12 @@ hipError_t transpose_pad(const void* in, int in_f32, size_t rows, int cols, size
     return hipGetLastError();
 }
 
-hipError_t reduce_dw(const Dims& d, const float* partial, int splits, int ncols, int out_cols, float scale,
-                     bool accumulate, float* dst, hipStream_t s) {
+hipError_t reduce_dw(const Dims& d, const float* partial, int splits, size_t ld, int col0, int ncols, int out_cols,
+                     float scale, bool accumulate, float* dst, hipStream_t s) {
     if (dst == nullptr) return hipSuccess;
-    const size_t per = size_t(4) * d.Hp * ncols;
-    hipLaunchKernelGGL(reduce_dw_kernel, dim3(grid_for(per)), dim3(kT), 0, s, d, partial, splits, ncols, out_cols,
-                       scale, int(accumulate), dst);
+    const size_t n = size_t(4) * d.Hp * ncols;
+    hipLaunchKernelGGL(reduce_dw_kernel, dim3(grid_for(n)), dim3(kT), 0, s, d, partial, splits, ld, col0, ncols,
+                       out_cols, scale, int(accumulate), dst);
     return hipGetLastError();
 }
 

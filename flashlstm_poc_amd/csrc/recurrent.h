@@ -61,9 +61,11 @@ struct RecBwdArgs {
     long long* prof;     // optional [8] cycle counters of workgroup 0 per phase (null = off)
 };
 
-// Picks tile shapes and the group structure for a problem size on the current device.
-RecLayout plan_rec_fwd(int B, int Hp, int num_cus, bool force_stepwise);
-RecLayout plan_rec_bwd(int B, int Hp, int num_cus, bool force_stepwise);
+// Picks tile shapes and the group structure for a problem size on the current device.  force_mt: 0 = the rule of
+// thumb (16-row blocks whenever all of them can run side by side), 1 / 2 = that many 16-row tiles per row block
+// (1 only where it fits).  The choice does not change the weight-fragment layout.
+RecLayout plan_rec_fwd(int B, int Hp, int num_cus, bool force_stepwise, int force_mt = 0);
+RecLayout plan_rec_bwd(int B, int Hp, int num_cus, bool force_stepwise, int force_mt = 0);
 
 // Halfs in one slot of an exchange ring for a [rows][cols] operand (rows padded to 32).
 size_t exchange_slot_halfs(int rows, int cols);

@@ -313,8 +313,9 @@ template <int N> struct F32;
 template <> struct F32<2> { floatx2 v; };
 template <> struct F32<4> { floatx4 v; };
 
-__device__ __forceinline__ void st_pack(half_t* p, Pack<2> v) { *reinterpret_cast<unsigned*>(p) = v.v; }
-__device__ __forceinline__ void st_pack(half_t* p, Pack<4> v) { *reinterpret_cast<uintx2*>(p) = v.v; }
+// (non-temporal: the state and gate arrays are written once per pass and read by later kernels)
+__device__ __forceinline__ void st_pack(half_t* p, Pack<2> v) { __builtin_nontemporal_store(v.v, reinterpret_cast<unsigned*>(p)); }
+__device__ __forceinline__ void st_pack(half_t* p, Pack<4> v) { __builtin_nontemporal_store(v.v, reinterpret_cast<uintx2*>(p)); }
 __device__ __forceinline__ void unpack(Pack<2> v, float (&f)[2]) { unpack_h2(v.v, f[0], f[1]); }
 __device__ __forceinline__ void unpack(Pack<4> v, float (&f)[4]) {
     unpack_h2(v.v.x, f[0], f[1]);
@@ -360,7 +361,7 @@ __device__ __forceinline__ GateRow<UPT> gates_fill(unsigned w) {
 template <int UPT>
 __device__ __forceinline__ void st_gates(half_t* p, const GateRow<UPT>& g) {
 #pragma unroll
-    for (int c = 0; c < UPT / 2; ++c) *reinterpret_cast<uintx4*>(p + 8 * c) = g.v[c];
+    for (int c = 0; c < UPT / 2; ++c) __builtin_nontemporal_store(g.v[c], reinterpret_cast<uintx4*>(p + 8 * c));
 }
 // 16 bytes into the exchange ring (see below: every 32-bit word is validated on its own)
 __device__ __forceinline__ void store_xch16(half_t* dst, uintx4 v, bool device_scope) {
@@ -436,20 +437,22 @@ __device__ __forceinline__ int group_row(int idx) { return (idx % 2) * 8 + (idx 
 // They are issued by hand, right after the LAST fragment load of a step's product: loads return in issue
 // order, so anything slow that sits in front of the fragment loads would hold them up, and a known number
 // of them behind lets the fragment waits discount them.  The values are used only after settle().
-__device__ __forceinline__ void ld_async(unsigned& d, const void* p) {
-    asm volatile("global_load_dword %0, %1, off" : "=v"(d) : "v"(p) : "memory");
+// They carry the non-temporal hint: these arrays stream through once per pass, and their lines should not push the
+// exchange ring, which is re-read every step, out of the L2.
+__device__ __forceinline__ void ld_stream(uintx2& d, const void* p) {
+    asm volatile("global_load_dwordx2 %0, %1, off nt" : "=v"(d) : "v"(p) : "memory");
 }
-__device__ __forceinline__ void ld_async(uintx2& d, const void* p) {
-    asm volatile("global_load_dwordx2 %0, %1, off" : "=v"(d) : "v"(p) : "memory");
+__device__ __forceinline__ void ld_stream(floatx2& d, const void* p) {
+    asm volatile("global_load_dwordx2 %0, %1, off nt" : "=v"(d) : "v"(p) : "memory");
 }
-__device__ __forceinline__ void ld_async(floatx2& d, const void* p) {
-    asm volatile("global_load_dwordx2 %0, %1, off" : "=v"(d) : "v"(p) : "memory");
+__device__ __forceinline__ void ld_stream(unsigned& d, const void* p) {
+    asm volatile("global_load_dword %0, %1, off nt" : "=v"(d) : "v"(p) : "memory");
 }
-__device__ __forceinline__ void ld_async(uintx4& d, const void* p) {
-    asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(d) : "v"(p) : "memory");
+__device__ __forceinline__ void ld_stream(uintx4& d, const void* p) {
+    asm volatile("global_load_dwordx4 %0, %1, off nt" : "=v"(d) : "v"(p) : "memory");
 }
-__device__ __forceinline__ void ld_async(floatx4& d, const void* p) {
-    asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(d) : "v"(p) : "memory");
+__device__ __forceinline__ void ld_stream(floatx4& d, const void* p) {
+    asm volatile("global_load_dwordx4 %0, %1, off nt" : "=v"(d) : "v"(p) : "memory");
 }
 __device__ __forceinline__ void wait_all_vm() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
 template <typename T>
@@ -549,7 +552,7 @@ __global__ __launch_bounds__(kThreads) void rec_fwd_kernel(RecFwdArgs p, RecLayo
         const int b = min(rb * RB + pr, p.B - 1);
         const half_t* src = p.G + (size_t(t) * p.B + b) * gld + size_t(4) * j;
 #pragma unroll
-        for (int c = 0; c < UPT / 2; ++c) ld_async(xp.v[c], src + 8 * c);
+        for (int c = 0; c < UPT / 2; ++c) ld_stream(xp.v[c], src + 8 * c);
     };
     if (c_in_regs) {
         const int b = g * RB + pr, b2 = (g + L.ng) * RB + pr;
@@ -721,10 +724,10 @@ __global__ __launch_bounds__(kThreads) void rec_bwd_kernel(RecBwdArgs p, RecLayo
         const int tt = max(t, 0);
         const half_t* gsrc = p.G + (size_t(tt) * p.B + b) * gld + pq;
 #pragma unroll
-        for (int c = 0; c < UPT / 2; ++c) ld_async(pg.v[c], gsrc + 8 * c);
-        ld_async(pcp_r.v, p.C + (size_t(tt) * p.B + b) * p.Hp + j);
-        ld_async(pcc_r.v, p.C + (size_t(tt + 1) * p.B + b) * p.Hp + j);
-        ld_async(pdy.v, p.dY + (size_t(tt) * p.B + b) * p.Hp + j);
+        for (int c = 0; c < UPT / 2; ++c) ld_stream(pg.v[c], gsrc + 8 * c);
+        ld_stream(pcp_r.v, p.C + (size_t(tt) * p.B + b) * p.Hp + j);
+        ld_stream(pcc_r.v, p.C + (size_t(tt + 1) * p.B + b) * p.Hp + j);
+        ld_stream(pdy.v, p.dY + (size_t(tt) * p.B + b) * p.Hp + j);
     };
     __syncthreads();
     float dbacc[4][UPT] = {};
@@ -930,14 +933,16 @@ size_t exchange_slot_halfs(int rows, int cols) { return round_up(size_t(rows), 3
 int rec_fwd_ks(const RecLayout&, int Hp) { return int(ceil_div(size_t(Hp) / 32, 4)); }
 int rec_bwd_ks(const RecLayout&, int Hp) { return int(ceil_div(size_t(Hp) / 8, 4)); }
 
-static void finish_layout(RecLayout& L, int B, int Hp, int num_cus, bool force_stepwise, bool fits) {
+static void finish_layout(RecLayout& L, int B, int Hp, int num_cus, bool force_stepwise, bool fits, int force_mt) {
     L.nh = Hp / L.jb;
     L.resident = fits ? 1 : 0;
     // Row blocks of 16 rows (one MFMA row tile) when all of them can run side by side: twice the workgroups
     // of 32-row blocks, each with half the product, fetch and cell-update work per step.
     const bool xcd_mode = (num_cus == 256 && L.nh <= 32);
     const int side_by_side = L.nh > num_cus ? 0 : (xcd_mode ? 8 * (32 / L.nh) : num_cus / L.nh);
-    L.mt = (fits && int(ceil_div(size_t(B), 16)) <= side_by_side) ? 1 : 2;
+    const bool can_16 = fits && int(ceil_div(size_t(B), 16)) <= side_by_side;
+    L.mt = can_16 ? 1 : 2;
+    if (force_mt == 2 || (force_mt == 1 && can_16)) L.mt = force_mt;   // a tuned choice; 16-row blocks only where they fit
     L.nrb = int(ceil_div(size_t(B), size_t(16 * L.mt)));
     L.xcd_local = 0;
     L.gpx = 0;
@@ -960,25 +965,25 @@ static void finish_layout(RecLayout& L, int B, int Hp, int num_cus, bool force_s
     }
 }
 
-RecLayout plan_rec_fwd(int B, int Hp, int num_cus, bool force_stepwise) {
+RecLayout plan_rec_fwd(int B, int Hp, int num_cus, bool force_stepwise, int force_mt) {
     RecLayout L{};
     bool fits = true;
     if (Hp <= 1024) L.nt = 8;
     else if (Hp <= 2048) L.nt = 4;
     else { L.nt = 8; fits = false; }
     L.jb = 4 * L.nt;
-    finish_layout(L, B, Hp, num_cus, force_stepwise, fits);
+    finish_layout(L, B, Hp, num_cus, force_stepwise, fits, force_mt);
     return L;
 }
 
-RecLayout plan_rec_bwd(int B, int Hp, int num_cus, bool force_stepwise) {
+RecLayout plan_rec_bwd(int B, int Hp, int num_cus, bool force_stepwise, int force_mt) {
     RecLayout L{};
     bool fits = true;
     if (Hp <= 1024) L.nt = 2;
     else if (Hp <= 2048) L.nt = 1;
     else { L.nt = 2; fits = false; }
     L.jb = 16 * L.nt;
-    finish_layout(L, B, Hp, num_cus, force_stepwise, fits);
+    finish_layout(L, B, Hp, num_cus, force_stepwise, fits, force_mt);
     return L;
 }
 

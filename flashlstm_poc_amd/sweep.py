@@ -1,12 +1,14 @@
 """Sequence-length sweep and tuner for the device-resident LSTM core.
 
     python -m flashlstm_poc_amd.sweep --batch 64 --input-size 1024 --hidden-size 1024 --seq-lens 128 512 2048
-    python -m flashlstm_poc_amd.sweep --tune --seq-lens 1024          # split-K sweep of the weight-gradient GEMMs
+    python -m flashlstm_poc_amd.sweep --tune --seq-lens 256 1024      # tune a plan per length, then sweep with it
 
 Counterpart of the reference's python/benchmark_lstm.py:455-620 (sequence-length sweep against torch.nn.LSTM,
-here the MIOpen-backed one of PyTorch-ROCm on the same GPU) and of src/tune_projchunksz.cu:56-226 (sweep of the
-one launch parameter worth tuning; in this library that is the split-K count of the dW GEMMs, not the
-projection chunk).  Inputs are synthetic (seeded); every tensor is resident on the GPU before timing starts.
+here the MIOpen-backed one of PyTorch-ROCm on the same GPU) and of its tuners (src/tune_projchunksz.cu:56-226,
+python/benchmark_lstm.py:203-301): --tune runs the library's own tuner (LstmCore.tune -> flstm_core_tune: 16- or
+32-row blocks per recurrence, persistent or step-wise launches, split-K count of the weight-gradient GEMM) for
+every length before timing it, prints what it chose, and the sweep then runs with those choices cached in the
+plan.  Inputs are synthetic (seeded); every tensor is resident on the GPU before timing starts.
 """
 import argparse
 import csv
@@ -76,7 +78,7 @@ def check_parity(core, p, I: int, H: int) -> Dict[str, float]:
 
 
 def sweep(B: int, I: int, H: int, seq_lens: Sequence[int], *, warmup: int = 3, repeats: int = 10, seed: int = 2025,
-          baseline: bool = True, check: bool = False) -> List[Dict]:
+          baseline: bool = True, check: bool = False, tune: bool = False, try_stepwise: bool = False) -> List[Dict]:
     import torch
     from . import LstmCore
     rows = []
@@ -85,6 +87,9 @@ def sweep(B: int, I: int, H: int, seq_lens: Sequence[int], *, warmup: int = 3, r
         core = LstmCore(B, I, H)
         core.pack(p["w_ih"], p["w_hh"], p["b_ih"], p["b_hh"])
         row: Dict = {"T": T, "B": B, "I": I, "H": H}
+        if tune:
+            row["untuned"] = {"row_tiles_fwd": core.info("row_tiles_fwd"), "row_tiles_bwd": core.info("row_tiles_bwd")}
+            row["tuned"] = core.tune(T, repeats=3, try_stepwise=try_stepwise)
         if check:
             row["parity"] = check_parity(core, p, I, H)
             row["parity_ok"] = all(v <= 1e-2 for v in row["parity"].values())
@@ -135,6 +140,11 @@ def format_row(r: Dict) -> str:
     if "torch_fwd_ms" in r:
         s += (f"  | nn.LSTM fwd {r['torch_fwd_ms']:9.3f} ms (x{r['speedup_fwd']:.2f})  "
               f"fwd+bwd {r['torch_fwd_bwd_ms']:9.3f} ms (x{r['speedup_fwd_bwd']:.2f})")
+    if "tuned" in r:
+        t = r["tuned"]
+        s += (f"  | tuned: rows/block fwd {16 * t['row_tiles_fwd']} bwd {16 * t['row_tiles_bwd']}, "
+              f"{'step-wise' if t['stepwise_fwd'] else 'persistent'}/{'step-wise' if t['stepwise_bwd'] else 'persistent'}, "
+              f"dW split-K {t['dw_splits']}")
     if "parity_ok" in r:
         s += "  parity " + ("ok" if r["parity_ok"] else "FAILED " + json.dumps(r["parity"]))
     return s
@@ -177,7 +187,11 @@ def main(argv: Optional[Sequence[str]] = None) -> int:
     ap.add_argument("--seed", type=int, default=2025)
     ap.add_argument("--no-baseline", action="store_true", help="skip torch.nn.LSTM on the GPU")
     ap.add_argument("--check", action="store_true", help="parity against torch.nn.LSTM (fp32) at every length")
-    ap.add_argument("--tune", action="store_true", help="sweep the split-K count of the weight-gradient GEMMs instead")
+    ap.add_argument("--tune", action="store_true", help="run the library's tuner for every length first (choices are "
+                    "cached in the plan and printed)")
+    ap.add_argument("--tune-stepwise", action="store_true", help="with --tune: also time one launch per step")
+    ap.add_argument("--dw-splits-table", action="store_true", help="print the weight-gradient time for every "
+                    "split-K count instead of sweeping")
     ap.add_argument("--csv", type=str, default=None)
     ap.add_argument("--json", type=str, default=None)
     args = ap.parse_args(argv)
@@ -191,16 +205,17 @@ def main(argv: Optional[Sequence[str]] = None) -> int:
         while t <= args.seq_len_max:
             lens.append(t)
             t *= 2
-    if args.tune:
+    if args.dw_splits_table:
         results = [tune_dw_splits(args.batch, args.input_size, args.hidden_size, T, seed=args.seed) for T in lens]
         for r in results:
             print(f"T={r['T']}: " + "  ".join(f"{k}:{v:.3f}ms" for k, v in r["dw_ms_by_splits"].items()) +
                   f"  best={r['best']}  automatic/best={r['automatic_over_best']:.3f}")
     else:
         results = sweep(args.batch, args.input_size, args.hidden_size, lens, warmup=args.warmup, repeats=args.repeats,
-                        seed=args.seed, baseline=not args.no_baseline, check=args.check)
+                        seed=args.seed, baseline=not args.no_baseline, check=args.check, tune=args.tune,
+                        try_stepwise=args.tune_stepwise)
         if args.csv:
-            keys = [k for k in results[0] if k != "parity"]
+            keys = [k for k in results[0] if k not in ("parity", "tuned", "untuned")]
             with open(args.csv, "w", newline="") as f:
                 w = csv.DictWriter(f, fieldnames=keys, extrasaction="ignore")
                 w.writeheader()

@@ -47,6 +47,7 @@ int flstm_core_destroy(flstm_core_plan* plan);
  * the weight-gradient GEMM, 0 = automatic), "accumulate_grads" (1 = the backward pass adds dW_ih, dW_hh, db_ih
  * and db_hh to what the caller's buffers hold instead of overwriting them: a sequence processed as several
  * consecutive segments, last segment first, each segment's dh0 / dc0 fed to the next call as d_hn / d_cn),
+ * "row_tiles_fwd" / "row_tiles_bwd" (16-row tiles per row block of that recurrence: 1, 2, or 0 = automatic),
  * "inject_stall" (test hook: the next N passes that use a persistent kernel are treated as if that launch had
  * given up, which exercises the step-wise repeat and the demotion rule without making any kernel wait). */
 int flstm_core_set_option(flstm_core_plan* plan, const char* name, long value);
@@ -137,6 +138,20 @@ int flstm_core_cache_ptr(const flstm_core_plan* plan, int which, const void** pt
  * measured with events on the call's stream: names "fwd_proj", "fwd_rec", "fwd_total",
  * "bwd_rec", "bwd_dx", "bwd_dw", "bwd_total".  Negative when not available. */
 double flstm_core_last_ms(const flstm_core_plan* plan, const char* phase);
+
+/* Tuner (the counterpart of the reference's projection-chunk tuner, src/tune_projchunksz.cu:56-226, and of the
+ * autotune loop of python/benchmark_lstm.py:203-301, for the launch choices that matter in this library).  For
+ * sequence length seq_len it times, on synthetic data in the plan's own buffers, `repeats` passes of every
+ * candidate: 16- or 32-row blocks for each recurrence (where both fit), persistent or -- with try_stepwise -- one
+ * launch per step, and the split-K count of the weight-gradient GEMM around the rule of thumb; the fastest choice
+ * per phase is cached in the plan and used by every later pass whose length is within a factor of two of a tuned
+ * one (explicit options "stepwise", "row_tiles_fwd", "row_tiles_bwd", "dw_splits" still win; option "clear_tuned"
+ * forgets everything).  Read back with flstm_core_get_info: "tuned_entries", and for the entry in force for the
+ * last pass "tuned_T", "tuned_row_tiles_fwd", "tuned_row_tiles_bwd", "tuned_stepwise_fwd", "tuned_stepwise_bwd",
+ * "tuned_dw_splits" (0 = rule of thumb); flstm_core_tuned_ms gives the best time found per phase ("fwd_rec",
+ * "bwd_rec", "bwd_dw").  The plan's forward cache is invalidated.  Allocates temporary device buffers. */
+int flstm_core_tune(flstm_core_plan* plan, size_t seq_len, int repeats, int try_stepwise, void* stream);
+double flstm_core_tuned_ms(const flstm_core_plan* plan, size_t seq_len, const char* phase);
 
 /* The fp16 x fp16 -> fp32-accumulate MFMA GEMMs the passes are built from, callable on their own (the counterpart
  * of flstm::GemmTN / GemmNN / GemmNT, reference flashlstm_v2/src/gemm.h:8-51; device pointers, work is enqueued on

@@ -25,3 +25,49 @@ def test_tuner_returns_a_table_and_the_automatic_choice_is_close_to_the_best():
     r = sweep.tune_dw_splits(32, 256, 256, 64, candidates=(0, 1, 2, 4, 8, 16), warmup=1, repeats=3)
     assert set(r["dw_ms_by_splits"]) == {0, 1, 2, 4, 8, 16} and r["best"] in (1, 2, 4, 8, 16)
     assert r["automatic_over_best"] < 4.0   # launches of ~50 us: only a grossly wrong automatic choice fails this
+
+
+def test_plan_caches_the_tuned_choice_per_sequence_length():
+    # flstm_core_tune: the choice lands in the plan, is read back through get_info, applies to passes of similar
+    # length only, loses against explicit options, and never changes results beyond summation order.
+    import torch
+    from flashlstm_poc_amd import LstmCore, sweep
+    B, I, H, T = 16, 128, 256, 48          # 16 rows: both 16- and 32-row blocks are possible
+    p = sweep.make_problem(T, B, I, H, seed=3)
+    core = LstmCore(B, I, H)
+    core.pack(p["w_ih"], p["w_hh"], p["b_ih"], p["b_hh"])
+    y0, hy0, cy0 = core.forward(p["x"], p["h0"], p["c0"])
+    g0 = core.backward(p["x"], p["dy"])
+    assert core.info("tuned_entries") == 0 and core.info("tuned_T") == 0
+    t = core.tune(T, repeats=2, try_stepwise=True)
+    assert core.info("tuned_entries") == 1 and t["T"] == T
+    assert t["row_tiles_fwd"] in (1, 2) and t["row_tiles_bwd"] in (1, 2) and t["dw_splits"] >= 1
+    assert t["stepwise_fwd"] in (0, 1) and t["fwd_rec_ms"] > 0 and t["bwd_rec_ms"] > 0 and t["bwd_dw_ms"] > 0
+    y1, hy1, cy1 = core.forward(p["x"], p["h0"], p["c0"])
+    g1 = core.backward(p["x"], p["dy"])
+    assert core.info("tuned_T") == T
+    assert core.info("row_tiles_fwd") == t["row_tiles_fwd"] and core.info("row_tiles_bwd") == t["row_tiles_bwd"]
+    assert core.info("persistent_fwd") == 1 - t["stepwise_fwd"]
+    assert torch.equal(y0, y1) and torch.equal(cy0, cy1)          # the forward pass does not depend on the choice
+    for a, b in zip(g0, g1):
+        assert ((a.float() - b.float()).norm() / b.float().norm()).item() <= 1e-5
+    # a sequence eight times longer is outside the tuned entry's range: rules of thumb again
+    long = sweep.make_problem(8 * T, B, I, H, seed=4)
+    core.forward(long["x"], long["h0"], long["c0"])
+    assert core.info("tuned_T") == 0 and core.info("tuned_dw_splits") == 0
+    # explicit options win over the tuned entry
+    core.set_option("row_tiles_fwd", 3 - t["row_tiles_fwd"])
+    core.forward(p["x"], p["h0"], p["c0"])
+    assert core.info("row_tiles_fwd") == 3 - t["row_tiles_fwd"] and core.info("tuned_row_tiles_fwd") == t["row_tiles_fwd"]
+    core.set_option("row_tiles_fwd", 0)
+    core.set_option("clear_tuned", 1)
+    assert core.info("tuned_entries") == 0
+    core.close()
+
+
+def test_sweep_with_tuning_prints_the_choices(capsys):
+    from flashlstm_poc_amd import sweep
+    rc = sweep.main(["--batch", "16", "--input-size", "64", "--hidden-size", "128", "--seq-lens", "32", "--warmup", "1",
+                     "--repeats", "2", "--tune", "--no-baseline"])
+    assert rc == 0
+    assert "tuned: rows/block" in capsys.readouterr().out
