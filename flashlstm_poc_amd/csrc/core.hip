@@ -114,7 +114,8 @@ struct flstm_core_plan {
     size_t T_cache = 0;
     bool have_cache = false;
     // pass in progress (begin / steps / end)
-    struct { size_t T = 0; const void* x = nullptr; flstm_dtype x_dtype = FLSTM_F16; bool open = false; } fw;
+    struct { size_t T = 0; const void* x = nullptr; flstm_dtype x_dtype = FLSTM_F16; bool open = false;
+             half_t* y_direct = nullptr; } fw;   // y_direct: the recurrence writes the caller's y itself
     struct { size_t T = 0; const half_t* dYk = nullptr; const void* dY = nullptr; flstm_dtype dy_dtype = FLSTM_F16;
              float S = 1.f, dy_scale = 1.f; void* dx = nullptr; flstm_dtype dx_dtype = FLSTM_F16; bool open = false; } bw;
     // backward scratch
@@ -424,6 +425,7 @@ int forward_recur(flstm_core_plan* p, size_t t0, size_t n, hipStream_t s) {
     RecFwdArgs a{};
     a.wfrag = p->wfrag_f.as<half8>();
     a.Y = p->Y.as<half_t>(); a.G = p->G.as<half_t>(); a.C = p->C.as<float>();
+    a.y_out = p->fw.y_direct;
     a.X = p->xch_f.as<half_t>(); a.x_slot = exchange_slot_halfs(d.B, d.Hp);
     a.status = p->status.as<int>();
     a.seats = p->status.as<unsigned>() + 8;
@@ -459,10 +461,15 @@ int forward_pass(flstm_core_plan* p, size_t T, const void* x, flstm_dtype x_dtyp
     const Dims& d = p->d;
     const size_t TB = T * size_t(d.B);
     use_tuned(p, T);
+    // an fp16 output whose rows are the state rows is written by the recurrence itself (no copy afterwards)
+    half_t* const y_direct = (y && y_dtype == FLSTM_F16 && d.H == d.Hp) ? static_cast<half_t*>(y) : nullptr;
     for (int attempt = 0;; ++attempt) {
+        p->fw.y_direct = y_direct;
         int rc = forward_once(p, T, x, x_dtype, h0, c0, state_dtype, s);
+        p->fw.y_direct = nullptr;
         if (rc) return rc;
-        FL_TRY(unpad_from_half(p->Y.as<half_t>() + size_t(d.B) * d.Hp, size_t(d.Hp), TB, d.H, y, y_dtype == FLSTM_F32, s));
+        if (!y_direct)
+            FL_TRY(unpad_from_half(p->Y.as<half_t>() + size_t(d.B) * d.Hp, size_t(d.Hp), TB, d.H, y, y_dtype == FLSTM_F32, s));
         FL_TRY(unpad_from_half(p->Y.as<half_t>() + TB * d.Hp, size_t(d.Hp), size_t(d.B), d.H, hy,
                                out_state_dtype == FLSTM_F32, s));
         FL_TRY(unpad_from_float(p->C.as<float>() + TB * d.Hp, size_t(d.Hp), size_t(d.B), d.H, 1.f, cy,

@@ -27,6 +27,8 @@ struct RecFwdArgs {
                          // writes slot (t+1)%4; before step 0 slot 0 holds h0 (padding rows zero) and the
                          // other three hold the 0xFFFF 'unwritten' pattern
     size_t x_slot;
+    half_t* y_out;       // optional: the caller's output tensor [T*B][Hp] fp16 (only when its rows equal the state
+                         // rows: fp16, hidden size = Hp); h_t is then stored there as well, which saves the copy
     half_t* G;           // [T*B][4Hp] packed gate order; in: x-projection + bias, out: activated i,f,g,o
     float* C;            // [(T+1)*B][Hp]; rows [0,B) = c0, rows [(t+1)B, ..) = c_t
     unsigned* seats;     // [8] zeroed before every launch: next free workgroup slot per XCD

@@ -642,6 +642,7 @@ __global__ __launch_bounds__(kThreads) void rec_fwd_kernel(RecFwdArgs p, RecLayo
             if (live) {
                 st_f32(p.C + (size_t(t + 1) * p.B + b) * p.Hp + j, cnew);
                 st_pack(p.Y + (size_t(t + 1) * p.B + b) * p.Hp + j, hnew);
+                if (p.y_out) st_pack(p.y_out + (size_t(t) * p.B + b) * p.Hp + j, hnew);
                 st_gates(p.G + (size_t(t) * p.B + b) * gld + size_t(4) * j, act);
             }
             clk.lap(3);

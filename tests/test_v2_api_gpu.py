@@ -278,6 +278,107 @@ def test_weights_changed_in_place_between_forward_and_backward_are_noticed():
         assert rell2(got[k], g[k]) <= 1e-2, ("h0 changed in place", k, rell2(got[k], g[k]))
 
 
+def test_reference_validator_long_shape_against_torch_lstm_on_gpu():
+    # (T, B, I, H) = (2048, 32, 1024, 1024): the largest shape of the reference's forward validator
+    # (flashlstm_v2/scripts/validate_lstm_fwd.py:243-250), with its R = 4 and mixed checkpoint dtypes (h fp16,
+    # c fp32), forward AND backward, against fp32 nn.LSTM on the GPU with the same fp16-rounded operands.
+    from helpers import SafeTorchLstm
+    T, B, I, H, R = 2048, 32, 1024, 1024, 4
+    p = make_problem(T, B, I, H, seed=0)
+    out = run_v2(p, R=R, h_dtype=torch.float16, c_dtype=torch.float32)
+    m = SafeTorchLstm([tuple(p[k].cuda() for k in ("w_ih", "w_hh", "b_ih", "b_hh"))])
+    xr = p["x"].cuda().requires_grad_(True)
+    hr = p["h0"].cuda().requires_grad_(True); cr = p["c0"].cuda().requires_grad_(True)
+    yr, hn, cn = m(xr, [hr], [cr])
+    ((yr * p["dy"].cuda()).sum() + (hn[0] * p["d_hn"].cuda()).sum() + (cn[0] * p["d_cn"].cuda()).sum()).backward()
+    dW_ih, dW_hh, db = m.grads(0)
+    ref = dict(y=yr, hn=hn[0], cn=cn[0], dx=xr.grad, dw_ih=dW_ih, dw_hh=dW_hh, db=db, dh0=hr.grad, dc0=cr.grad)
+    errs = {k: relmax(out[k], to_np(ref[k])) for k in ("y", "hn", "cn")}
+    errs.update({k: rell2(out[k], to_np(ref[k])) for k in ("dx", "dw_ih", "dw_hh", "db", "dh0", "dc0")})
+    errs["y_last_step"] = relmax(out["y"][-1], to_np(yr[-1]))
+    print("\nvalidator shape (2048, 32, 1024, 1024): " + ", ".join(f"{k}={v:.2e}" for k, v in errs.items()))
+    assert max(errs.values()) <= 1e-2, errs
+    # checkpoint k = state before step k * R: entry 1 is (h, c) after R steps
+    yk = to_np(yr[R - 1])
+    assert relmax(out["ck_h"][1], yk) <= 1e-2
+    np.testing.assert_array_equal(out["db"], out["db_hh"])
+
+
+def test_reference_smoke_shape_with_budget_driven_windows():
+    # The reference's smoke executable (flashlstm_v2/src/main.cu:279-283,296,317,433,663-685): T = 8192, B = 1024,
+    # I = H = 1024, R = 8, x ~ N(0, 0.01), W ~ U(+-1/sqrt(H)), b = 0, dY ~ N(0, 0.005); it counts NaN / Inf in dx.
+    # Here the sequence needs 32 MiB of device memory per step, 256 GiB in all: more than the default budget (70 %
+    # of the device), so the library itself cuts it into windows -- no environment variable forces that.  Checked:
+    # nothing non-finite in y, dx and the weight gradients, and the first 64 steps of y against nn.LSTM.
+    import os
+    for k in ("FLASHLSTM_V2_WINDOW_STEPS", "FLASHLSTM_V2_DEVICE_BUDGET_MB", "FLASHLSTM_V2_CHUNK_STEPS"):
+        assert k not in os.environ
+    lib = bind()
+    T, B, I, H, R = 8192, 1024, 1024, 1024, 8
+    free, total = torch.cuda.mem_get_info()
+    per_step = B * (4 * I + 2 * I + 24 * H + 2 * H)
+    assert T * per_step > total * 7 // 10, "the whole sequence would fit the budget: windows would not engage"
+    g = torch.Generator(device="cuda").manual_seed(1337)
+    k = 1.0 / H ** 0.5
+    w_ih = (torch.rand(4 * H, I, generator=g, device="cuda") * 2 - 1) * k
+    w_hh = (torch.rand(4 * H, H, generator=g, device="cuda") * 2 - 1) * k
+    b = torch.zeros(4 * H, device="cuda")
+    # 4 x 16 GiB of host sequences: the inputs pinned when the machine lets that much be pinned, the outputs in
+    # ordinary pageable memory (the entry points take either)
+    def host(shape, pin):
+        if pin:
+            try:
+                return torch.empty(shape, dtype=torch.float16, pin_memory=True)
+            except RuntimeError:
+                pass
+        return torch.empty(shape, dtype=torch.float16)
+    x_host = host((T, B, I), True)
+    dy_host = host((T, B, H), True)
+    y_host = host((T, B, H), False)
+    dx_host = host((T, B, I), False)
+    step = 256
+    for t0 in range(0, T, step):
+        x_host[t0:t0 + step].copy_((torch.randn(step, B, I, generator=g, device="cuda") * 0.01).half())
+        dy_host[t0:t0 + step].copy_((torch.randn(step, B, H, generator=g, device="cuda") * 0.005).half())
+    n_ck = T // R
+    ck_h = torch.empty(n_ck, B, H, dtype=torch.float16, pin_memory=True); ck_c = torch.empty(n_ck, B, H, dtype=torch.float16, pin_memory=True)
+    h0 = torch.zeros(B, H, device="cuda", dtype=torch.float16); c0 = torch.zeros_like(h0)
+    hy = torch.empty_like(h0); cy = torch.empty_like(h0)
+    dW_ih = torch.empty_like(w_ih); dW_hh = torch.empty_like(w_hh); db_ih = torch.empty_like(b); db_hh = torch.empty_like(b)
+    dh0 = torch.empty(B, H, device="cuda"); dc0 = torch.empty(B, H, device="cuda")
+    streams = [torch.cuda.Stream() for _ in range(3)]
+    s = [st.cuda_stream for st in streams]
+    cache = GateCacheHost(ck_h.data_ptr(), ck_c.data_ptr())
+    opt = Options(1, 1)
+    torch.cuda.synchronize()
+    lib.flstm_StreamingLstmForward(T, B, I, H, R, x_host.data_ptr(), h0.data_ptr(), c0.data_ptr(), w_ih.data_ptr(),
+                                   w_hh.data_ptr(), b.data_ptr(), b.data_ptr(), y_host.data_ptr(), cache, ctypes.byref(opt),
+                                   hy.data_ptr(), cy.data_ptr(), s[0], s[1], s[2])
+    lib.flstm_StreamingLstmBackward(T, B, I, H, R, x_host.data_ptr(), y_host.data_ptr(), cache, dy_host.data_ptr(), None, None,
+                                    h0.data_ptr(), c0.data_ptr(), w_ih.data_ptr(), w_hh.data_ptr(), b.data_ptr(), b.data_ptr(),
+                                    dx_host.data_ptr(), dW_ih.data_ptr(), dW_hh.data_ptr(), db_ih.data_ptr(), db_hh.data_ptr(),
+                                    dh0.data_ptr(), dc0.data_ptr(), s[0], s[1], s[2], ctypes.byref(opt))
+    torch.cuda.synchronize()
+    bad = 0
+    for t0 in range(0, T, step):
+        bad += int((~torch.isfinite(dx_host[t0:t0 + step].cuda())).sum()) + int((~torch.isfinite(y_host[t0:t0 + step].cuda())).sum())
+    assert bad == 0, f"{bad} non-finite values in y / dx"
+    for t in (dW_ih, dW_hh, db_ih, dh0, dc0, hy, cy):
+        assert torch.isfinite(t.float()).all() and t.float().abs().max() > 0
+    assert dx_host[0].float().abs().max() > 0 and dx_host[-1].float().abs().max() > 0
+    # the last window's end state equals the last output row; the first 64 steps against nn.LSTM
+    assert torch.equal(hy.cpu(), y_host[-1])
+    m = torch.nn.LSTM(I, H, device="cuda")
+    with torch.no_grad():
+        m.weight_ih_l0.copy_(w_ih.half().float()); m.weight_hh_l0.copy_(w_hh.half().float())
+        m.bias_ih_l0.zero_(); m.bias_hh_l0.zero_()
+        yr, _ = m(x_host[:64].cuda().float())
+    assert relmax(to_np(y_host[:64]), to_np(yr)) <= 1e-2
+    # checkpoint 1 = h before step R = output of step R - 1
+    assert torch.equal(ck_h[1], y_host[R - 1])
+    lib.flstm_ReleaseStreamingCaches()
+
+
 def test_null_state_gradients_and_pageable_host_memory():
     p = make_problem(6, 4, 8, 16, seed=3)
     f, g = reference(p, state_grads=False)
