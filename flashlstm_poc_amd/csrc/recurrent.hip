@@ -47,6 +47,9 @@ constexpr int kRows = 32;  // batch rows per row block at most (two 16-row MFMA 
 // conflicts (measured: 4, 12 and 20 count the same; 8 triples the conflict cycles); what the counter still
 // shows is four cycles per 16-byte store, which run at half rate whatever the layout.
 constexpr int kPartPad = 4;
+// Register sets of fragments in the forward kernel's tile-by-tile product: one feeds the MFMAs, the others are in
+// flight.  (Three sets measured the same as two at I = H = 1024, B = 256: 3.93 against 3.86 us per step.)
+constexpr int kFwdBufs = 2;
 
 __device__ __forceinline__ unsigned xcc_id() {
     unsigned v;
@@ -150,6 +153,99 @@ __device__ __forceinline__ void wait_frags(half8 (&a)[2]) {
 template <int N>
 __device__ __forceinline__ void wait_frags(half8 (&a)[2], half8 (&b)[2]) {
     asm volatile("s_waitcnt vmcnt(%4)" : "+v"(a[0]), "+v"(a[1]), "+v"(b[0]), "+v"(b[1]) : "n"(N) : "memory");
+}
+
+template <int N>
+__device__ __forceinline__ void wait_frags(half8 (&a)[8]) {
+    asm volatile("s_waitcnt vmcnt(%8)"
+                 : "+v"(a[0]), "+v"(a[1]), "+v"(a[2]), "+v"(a[3]), "+v"(a[4]), "+v"(a[5]), "+v"(a[6]), "+v"(a[7])
+                 : "n"(N)
+                 : "memory");
+}
+
+// The same product for row blocks of two 16-row tiles whose producers publish the tiles one after the other (the
+// pointwise stage of a step handles rows 0..15 first, stores them, then rows 16..31): all k-steps of tile 0 are
+// fetched and multiplied before tile 1 is touched, so the first half of a step's product runs while the peers are
+// still busy with the second half of their cell updates.  Chunks of CKT k-steps of ONE tile alternate between two
+// register sets (as many registers as the two-tile chunks of wave_product).  Resident weights only.
+template <int NT, int KS, int KL, int NPF, int NBUF, typename Prefetch>
+__device__ __forceinline__ void wave_product_tiles(floatx4 (&acc)[2][NT], const half8 (&wreg)[KS - KL][NT],
+                                                   const half8* wlds, const half_t* a0, const half_t* a1, int wave,
+                                                   int lane, int nks_total, const Poll& poll, Prefetch&& prefetch) {
+    static_assert(KS % 8 == 0, "whole chunks");
+    constexpr int CKT = (KS >= 16) ? 8 : 4;
+    constexpr int NCHK = KS / CKT;      // chunks per tile
+    constexpr int NCH = 2 * NCHK;
+    static_assert(NBUF >= 2 && NBUF <= NCH, "register sets: one feeds the MFMAs, the others are in flight");
+    half8 f[NBUF][CKT];
+    auto issue = [&](int c) {
+        const half_t* base = (c / NCHK) ? a1 : a0;
+#pragma unroll
+        for (int k = 0; k < CKT; ++k) {
+            const int kg = min(((c % NCHK) * CKT + k) * 4 + wave, nks_total - 1);
+            ld_frag_async(f[c % NBUF][k], base + size_t(kg) * 512);
+        }
+    };
+#pragma unroll
+    for (int c = 0; c < NBUF - 1; ++c) issue(c);
+#pragma unroll
+    for (int c = 0; c < NCH; ++c) {
+        const int buf = c % NBUF;
+        const int last_issued = (c + NBUF - 1 < NCH) ? c + NBUF - 1 : NCH - 1;   // after this iteration's issue
+        if (c + NBUF - 1 < NCH) {
+            issue(c + NBUF - 1);
+            if (c + NBUF - 1 == NCH - 1) prefetch();
+        }
+        // loads return in issue order: chunk c has landed once at most the loads issued after it are outstanding
+        const int younger = (last_issued - c) * CKT + ((last_issued == NCH - 1) ? NPF : 0);
+        switch (younger) {   // (a compile-time constant in every unrolled iteration)
+            case NPF: wait_frags<NPF>(f[buf]); break;
+            case CKT + NPF: wait_frags<CKT + NPF>(f[buf]); break;
+            case 2 * CKT + NPF: wait_frags<2 * CKT + NPF>(f[buf]); break;
+            case CKT: wait_frags<CKT>(f[buf]); break;
+            case 2 * CKT: wait_frags<2 * CKT>(f[buf]); break;
+            default: wait_frags<0>(f[buf]); break;
+        }
+        if (poll.on) {
+            int spins = 0;
+            long long spin_start = 0;
+            for (;;) {
+                unsigned m = 0u;
+#pragma unroll
+                for (int k = 0; k < CKT; ++k) {
+                    const uint4 ua = __builtin_bit_cast(uint4, f[buf][k]);
+                    m = max(m, max(max(ua.x, ua.y), max(ua.z, ua.w)));
+                }
+                if (!__any(m == kUnwritten)) break;
+                ++spins;
+                if (spins == 1) spin_start = wall_clock64();
+                if (spins > poll.limit || *reinterpret_cast<volatile int*>(poll.lds_abort) != 0 ||
+                    ((spins & 255) == 0 &&
+                     (wall_clock64() - spin_start > poll.ticks ||
+                      __hip_atomic_load(poll.status, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0))) {
+                    if (lane == 0) {
+                        __hip_atomic_store(poll.status, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                        *reinterpret_cast<volatile int*>(poll.lds_abort) = 1;
+                    }
+                    break;   // results are garbage from here on; the workgroup leaves at its next barrier
+                }
+                issue(c);
+                wait_frags<0>(f[buf]);   // (whatever was in flight behind this chunk has landed as well)
+            }
+        }
+#pragma unroll
+        for (int k = 0; k < CKT; ++k) {
+            constexpr int KR = KS - KL;
+            const int ks = (c % NCHK) * CKT + k;
+#pragma unroll
+            for (int n = 0; n < NT; ++n) {
+                half8 w;
+                if (ks < KR) w = wreg[ks < KR ? ks : 0][n];
+                else w = wlds[((ks - KR) * NT + n) * kWave + lane];
+                acc[c / NCHK][n] = __builtin_amdgcn_mfma_f32_16x16x32_f16(w, f[buf][k], acc[c / NCHK][n], 0, 0, 0);
+            }
+        }
+    }
 }
 
 // acc[mt][nt] += (A(16*MT rows x K) * Wslice)^T, this wave's interleaved k-steps only.
@@ -499,16 +595,22 @@ struct PhaseClock {
 // off that path.
 // MT = 16-row tiles per row block: 2, or 1 for batches of at most 16 rows (the threads of rows 16..31 then only
 // keep the barriers company).
+// Slices of 32 units with two row tiles run the pointwise stage in two PHASES: all 256 threads update rows 0..15
+// of the block (two units each) and store that half of h_t, then rows 16..31.  The consumers fetch and multiply
+// tile by tile (wave_product_tiles), so the second phase of a step overlaps the first half of the peers' next
+// product instead of sitting on the path from one step to the next.
 template <int NT, int KS, bool RESIDENT, int MT>
 __global__ __launch_bounds__(kThreads) void rec_fwd_kernel(RecFwdArgs p, RecLayout L, int t_begin,
                                                            int t_end, int ks_wave) {
     constexpr int JB = 4 * NT;    // hidden units of this slice
     constexpr int NC = 16 * NT;   // gate columns of this slice (i,f,g,o blocks of JB)
     constexpr int PLD = NC + kPartPad;
+    constexpr bool SPLIT = RESIDENT && MT == 2 && JB >= 32 && (KS % 8 == 0);
     // cell updates per thread: the slice's units of one batch row are shared by GPR threads; 32 rows x 8 threads,
-    // or 16 rows x 16 threads when a block has one row tile and the slice is wide enough for 2 units each
-    constexpr int GPR = (MT == 1 && JB >= 32) ? 16 : 8;
+    // or 16 rows x 16 threads (per phase, or when a block has one row tile) where the slice is wide enough for 2 units each
+    constexpr int GPR = (SPLIT || (MT == 1 && JB >= 32)) ? 16 : 8;
     constexpr int UPT = JB / GPR;
+    constexpr int NPH = SPLIT ? 2 : 1;   // pointwise phases per step
     static_assert(UPT == 2 || UPT == 4, "2 or 4 hidden units per thread");
     typedef Pack<UPT> PackT;
     extern __shared__ __attribute__((aligned(16))) float part_all[];  // [2][4][32][PLD]
@@ -537,27 +639,33 @@ __global__ __launch_bounds__(kThreads) void rec_fwd_kernel(RecFwdArgs p, RecLayo
     }
 
     const size_t gld = size_t(4) * p.Hp;
-    // this thread's group: row pr of the row block, units pj .. pj+UPT-1 of the slice
+    // this thread's groups: row pr (+ 16 in the second phase) of the row block, units pj .. pj+UPT-1 of the slice
     constexpr int RB = 16 * MT;   // batch rows of a row block
     const int pr = group_row(tid / GPR);
-    const bool row_used = pr < RB;   // with one row tile per block the threads of rows 16..31 only keep the barriers company
+    const bool row_used = pr + 16 * (NPH - 1) < RB;   // with one row tile per block the threads of rows 16..31 only keep the barriers company
     const int pj = (tid % GPR) * UPT;
     const int j = hs * JB + pj;   // first hidden unit of the group
     const int rb_count = (L.nrb - g + L.ng - 1) / L.ng;
     // the cell state of the workgroup's first and second row block stays in registers for the whole launch
     const bool c_in_regs = (rb_count <= 2) && (t_end - t_begin > 1);
-    float creg[UPT] = {}, creg2[UPT] = {};
-    GateRow<UPT> xp;
-    auto prefetch = [&](int t, int rb) {   // UPT / 2 loads per wave; rows past B fetch row B-1 and are not used
-        const int b = min(rb * RB + pr, p.B - 1);
-        const half_t* src = p.G + (size_t(t) * p.B + b) * gld + size_t(4) * j;
+    float creg[NPH][UPT] = {}, creg2[NPH][UPT] = {};
+    GateRow<UPT> xp[NPH];
+    auto prefetch = [&](int t, int rb) {   // NPH * UPT / 2 loads per wave; rows past B fetch row B-1 and are not used
 #pragma unroll
-        for (int c = 0; c < UPT / 2; ++c) ld_stream(xp.v[c], src + 8 * c);
+        for (int ph = 0; ph < NPH; ++ph) {
+            const int b = min(rb * RB + pr + 16 * ph, p.B - 1);
+            const half_t* src = p.G + (size_t(t) * p.B + b) * gld + size_t(4) * j;
+#pragma unroll
+            for (int c = 0; c < UPT / 2; ++c) ld_stream(xp[ph].v[c], src + 8 * c);
+        }
     };
     if (c_in_regs) {
-        const int b = g * RB + pr, b2 = (g + L.ng) * RB + pr;
-        if (row_used && b < p.B) ld_f32_now(p.C + (size_t(t_begin) * p.B + b) * p.Hp + j, creg);
-        if (rb_count == 2 && row_used && b2 < p.B) ld_f32_now(p.C + (size_t(t_begin) * p.B + b2) * p.Hp + j, creg2);
+#pragma unroll
+        for (int ph = 0; ph < NPH; ++ph) {
+            const int b = g * RB + pr + 16 * ph, b2 = (g + L.ng) * RB + pr + 16 * ph;
+            if (row_used && b < p.B) ld_f32_now(p.C + (size_t(t_begin) * p.B + b) * p.Hp + j, creg[ph]);
+            if (rb_count == 2 && row_used && b2 < p.B) ld_f32_now(p.C + (size_t(t_begin) * p.B + b2) * p.Hp + j, creg2[ph]);
+        }
     }
     __syncthreads();
     clk.start();
@@ -576,8 +684,12 @@ __global__ __launch_bounds__(kThreads) void rec_fwd_kernel(RecFwdArgs p, RecLayo
             for (int m = 0; m < 2; ++m)
 #pragma unroll
                 for (int n = 0; n < NT; ++n) acc[m][n] = floatx4{0.f, 0.f, 0.f, 0.f};
-            wave_product<NT, KS, RESIDENT, 0, UPT / 2, MT>(acc, wreg, nullptr, wfrag_wave, a0, a1, wave, lane, nks_total,
-                                                     ks_wave, poll, [&]() { prefetch(t, rb); });
+            if constexpr (SPLIT)
+                wave_product_tiles<NT, KS, 0, NPH * UPT / 2, kFwdBufs>(acc, wreg, nullptr, a0, a1, wave, lane, nks_total, poll,
+                                                             [&]() { prefetch(t, rb); });
+            else
+                wave_product<NT, KS, RESIDENT, 0, UPT / 2, MT>(acc, wreg, nullptr, wfrag_wave, a0, a1, wave, lane, nks_total,
+                                                               ks_wave, poll, [&]() { prefetch(t, rb); });
             clk.lap(0);
             spill_partials<NT, MT>(part, acc, wave, lane, PLD);
             __syncthreads();
@@ -589,61 +701,76 @@ __global__ __launch_bounds__(kThreads) void rec_fwd_kernel(RecFwdArgs p, RecLayo
             // of the previous step, so that mark is in place before this step's h_t goes out.
             wait_all_vm();   // the x-projection of this step, issued during the product
 #pragma unroll
-            for (int c = 0; c < UPT / 2; ++c) settle(xp.v[c]);
+            for (int ph = 0; ph < NPH; ++ph)
+#pragma unroll
+                for (int c = 0; c < UPT / 2; ++c) settle(xp[ph].v[c]);
             clk.lap(4);
-            const int b = row0 + pr;
-            const unsigned xoff = unsigned(xch_offset(b, j, nks_total));   // 32 bits: a slot is far below 4G halfs
-            if (row_used) store_xch(xnext + xoff, pack_fill(kUnwritten, (PackT*)nullptr), device_scope);
-            GateRow<UPT> act;
-            float cnew[UPT] = {};
-            PackT hnew = pack_fill(0u, (PackT*)nullptr);   // batch rows past B travel as zeros
-            const bool live = row_used && b < p.B;
-            if (live) {
-                float z[4][UPT];
-                unpack_gates(xp, z);
+            unsigned xoff[NPH];   // 32 bits: a slot is far below 4G halfs
 #pragma unroll
-                for (int gt = 0; gt < 4; ++gt) {
-#pragma unroll
-                    for (int w = 0; w < 4; ++w) {
-                        float v[UPT];
-                        ld_f32(part + (size_t(w) * kRows + pr) * PLD + gt * JB + pj, v);
-#pragma unroll
-                        for (int u = 0; u < UPT; ++u) z[gt][u] += v[u];
-                    }
-                }
-                const bool second = (rb != g);
-                float cp[UPT];
-                if (c_in_regs) {
-#pragma unroll
-                    for (int u = 0; u < UPT; ++u) cp[u] = second ? creg2[u] : creg[u];
-                } else {
-                    ld_f32_coherent(p.C + (size_t(t) * p.B + b) * p.Hp + j, cp);
-                }
-                float hn[UPT], a4[4][UPT];
-#pragma unroll
-                for (int u = 0; u < UPT; ++u) {
-                    const float ig = sigmoidf_dev(z[0][u]);
-                    const float fg = sigmoidf_dev(z[1][u]);
-                    const float gg = tanhf_dev(z[2][u]);
-                    const float og = sigmoidf_dev(z[3][u]);
-                    cnew[u] = fg * cp[u] + ig * gg;
-                    hn[u] = og * tanhf_dev(cnew[u]);
-                    a4[0][u] = ig; a4[1][u] = fg; a4[2][u] = gg; a4[3][u] = og;
-                    if (second) creg2[u] = cnew[u];
-                    else creg[u] = cnew[u];
-                }
-                hnew = pack(hn);
-                act = pack_gates(a4);
+            for (int ph = 0; ph < NPH; ++ph) {
+                xoff[ph] = unsigned(xch_offset(row0 + pr + 16 * ph, j, nks_total));
+                if (row_used) store_xch(xnext + xoff[ph], pack_fill(kUnwritten, (PackT*)nullptr), device_scope);
             }
-            // the exchanged value goes out first
-            if (row_used) store_xch(xout + xoff, hnew, device_scope);
+            GateRow<UPT> act[NPH];
+            float cnew[NPH][UPT] = {};
+            PackT hnew[NPH];
+            bool live[NPH];
+            const bool second = (rb != g);
+#pragma unroll
+            for (int ph = 0; ph < NPH; ++ph) {
+                const int prow = pr + 16 * ph, b = row0 + prow;
+                hnew[ph] = pack_fill(0u, (PackT*)nullptr);   // batch rows past B travel as zeros
+                live[ph] = row_used && b < p.B;
+                if (live[ph]) {
+                    float z[4][UPT];
+                    unpack_gates(xp[ph], z);
+#pragma unroll
+                    for (int gt = 0; gt < 4; ++gt) {
+#pragma unroll
+                        for (int w = 0; w < 4; ++w) {
+                            float v[UPT];
+                            ld_f32(part + (size_t(w) * kRows + prow) * PLD + gt * JB + pj, v);
+#pragma unroll
+                            for (int u = 0; u < UPT; ++u) z[gt][u] += v[u];
+                        }
+                    }
+                    float cp[UPT];
+                    if (c_in_regs) {
+#pragma unroll
+                        for (int u = 0; u < UPT; ++u) cp[u] = second ? creg2[ph][u] : creg[ph][u];
+                    } else {
+                        ld_f32_coherent(p.C + (size_t(t) * p.B + b) * p.Hp + j, cp);
+                    }
+                    float hn[UPT], a4[4][UPT];
+#pragma unroll
+                    for (int u = 0; u < UPT; ++u) {
+                        const float ig = sigmoidf_dev(z[0][u]);
+                        const float fg = sigmoidf_dev(z[1][u]);
+                        const float gg = tanhf_dev(z[2][u]);
+                        const float og = sigmoidf_dev(z[3][u]);
+                        cnew[ph][u] = fg * cp[u] + ig * gg;
+                        hn[u] = og * tanhf_dev(cnew[ph][u]);
+                        a4[0][u] = ig; a4[1][u] = fg; a4[2][u] = gg; a4[3][u] = og;
+                        if (second) creg2[ph][u] = cnew[ph][u];
+                        else creg[ph][u] = cnew[ph][u];
+                    }
+                    hnew[ph] = pack(hn);
+                    act[ph] = pack_gates(a4);
+                }
+                // the exchanged value goes out first (one row tile after the other)
+                if (row_used) store_xch(xout + xoff[ph], hnew[ph], device_scope);
+            }
             clk.lap(2);
             // caches for the backward pass: off the critical path
-            if (live) {
-                st_f32(p.C + (size_t(t + 1) * p.B + b) * p.Hp + j, cnew);
-                st_pack(p.Y + (size_t(t + 1) * p.B + b) * p.Hp + j, hnew);
-                if (p.y_out) st_pack(p.y_out + (size_t(t) * p.B + b) * p.Hp + j, hnew);
-                st_gates(p.G + (size_t(t) * p.B + b) * gld + size_t(4) * j, act);
+#pragma unroll
+            for (int ph = 0; ph < NPH; ++ph) {
+                if (live[ph]) {
+                    const int b = row0 + pr + 16 * ph;
+                    st_f32(p.C + (size_t(t + 1) * p.B + b) * p.Hp + j, cnew[ph]);
+                    st_pack(p.Y + (size_t(t + 1) * p.B + b) * p.Hp + j, hnew[ph]);
+                    if (p.y_out) st_pack(p.y_out + (size_t(t) * p.B + b) * p.Hp + j, hnew[ph]);
+                    st_gates(p.G + (size_t(t) * p.B + b) * gld + size_t(4) * j, act[ph]);
+                }
             }
             clk.lap(3);
         }
