@@ -104,6 +104,8 @@ struct flstm_core_plan {
     int opt_mt_f = 0, opt_mt_b = 0;
     int eff_mt_f = 0, eff_mt_b = 0, eff_step_f = 0, eff_step_b = 0, eff_dw = 0;
     size_t eff_T = 0;
+    StepGraphCache graphs_f, graphs_b;   // captured step-wise launches (only used where the persistent kernels are not)
+    int opt_graphs = 1;
     int* status_host = nullptr;   // pinned: the device status word lands here with the end-of-pass copy
     int inject_stall = 0;         // test hook: treat the next N persistent passes as if their launch had given up
     // weights
@@ -279,6 +281,7 @@ extern "C" int flstm_core_set_option(flstm_core_plan* p, const char* name, long 
         return 0;
     }
     if (!strcmp(name, "clear_tuned")) { p->tuned.clear(); use_tuned(p, 1); return 0; }
+    if (!strcmp(name, "step_graphs")) { p->opt_graphs = value != 0; return 0; }
     if (!strcmp(name, "inject_stall")) { if (value < 0) return FLSTM_E_INVALID; p->inject_stall = int(value); return 0; }
     if (!strcmp(name, "dw_splits")) { if (value < 0) return FLSTM_E_INVALID; p->opt_dw_splits = int(value); return 0; }
     if (!strcmp(name, "accumulate_grads")) { p->opt_accumulate = value != 0; return 0; }
@@ -296,6 +299,9 @@ extern "C" long flstm_core_get_info(const flstm_core_plan* p, const char* name) 
     if (!strcmp(name, "row_tiles")) return p->Lf.mt;
     if (!strcmp(name, "row_tiles_fwd")) return p->Lf.mt;
     if (!strcmp(name, "row_tiles_bwd")) return p->Lb.mt;
+    if (!strcmp(name, "graph_captures")) return p->graphs_f.captures + p->graphs_b.captures;
+    if (!strcmp(name, "graph_replays")) return p->graphs_f.replays + p->graphs_b.replays;
+    if (!strcmp(name, "graphs_disabled")) return (p->graphs_f.disabled ? 1 : 0) + (p->graphs_b.disabled ? 2 : 0);
     if (!strcmp(name, "tuned_entries")) return long(p->tuned.size());
     if (!strcmp(name, "tuned_T")) return long(p->eff_T);
     if (!strcmp(name, "tuned_row_tiles_fwd")) return p->eff_mt_f;
@@ -434,7 +440,7 @@ int forward_recur(flstm_core_plan* p, size_t t0, size_t n, hipStream_t s) {
     a.spin_limit = p->opt_spin_limit;
     a.spin_ticks = (long long)p->opt_spin_ms * p->wall_khz;
     a.prof = p->opt_profile ? p->prof.as<long long>() : nullptr;
-    FL_TRY(launch_rec_fwd(p->Lf, a, s));
+    FL_TRY(launch_rec_fwd(p->Lf, a, s, p->opt_graphs ? &p->graphs_f : nullptr));
     return 0;
 }
 
@@ -461,9 +467,12 @@ int forward_pass(flstm_core_plan* p, size_t T, const void* x, flstm_dtype x_dtyp
     const Dims& d = p->d;
     const size_t TB = T * size_t(d.B);
     use_tuned(p, T);
-    // an fp16 output whose rows are the state rows is written by the recurrence itself (no copy afterwards)
-    half_t* const y_direct = (y && y_dtype == FLSTM_F16 && d.H == d.Hp) ? static_cast<half_t*>(y) : nullptr;
     for (int attempt = 0;; ++attempt) {
+        // An fp16 output whose rows are the state rows is written by the persistent recurrence itself (no copy
+        // afterwards).  Step-wise launches leave it to the copy: every argument of theirs is then plan-owned, and
+        // the graph they were captured into can be replayed on the next pass.
+        half_t* const y_direct =
+            (y && y_dtype == FLSTM_F16 && d.H == d.Hp && p->Lf.persistent) ? static_cast<half_t*>(y) : nullptr;
         p->fw.y_direct = y_direct;
         int rc = forward_once(p, T, x, x_dtype, h0, c0, state_dtype, s);
         p->fw.y_direct = nullptr;
@@ -568,7 +577,8 @@ int backward_setup(flstm_core_plan* p, size_t T, const void* dY, flstm_dtype dy_
     const size_t TB = T * size_t(d.B);
     p->bw.T = T; p->bw.dY = dY; p->bw.dy_dtype = dy_dtype; p->bw.S = S; p->bw.dx = dx; p->bw.dx_dtype = dx_dtype;
     p->bw.open = true;
-    if (dy_dtype == FLSTM_F16 && d.H == d.Hp) {
+    // (step-wise launches always read a plan-owned copy, so that their captured graph can be replayed)
+    if (dy_dtype == FLSTM_F16 && d.H == d.Hp && p->Lb.persistent) {
         p->bw.dYk = static_cast<const half_t*>(dY);
         p->bw.dy_scale = S;
     } else {
@@ -618,7 +628,7 @@ int backward_recur(flstm_core_plan* p, long t_hi, long t_lo, hipStream_t s) {
     a.spin_limit = p->opt_spin_limit;
     a.spin_ticks = (long long)p->opt_spin_ms * p->wall_khz;
     a.prof = p->opt_profile ? p->prof.as<long long>() + 8 : nullptr;
-    FL_TRY(launch_rec_bwd(p->Lb, a, s));
+    FL_TRY(launch_rec_bwd(p->Lb, a, s, p->opt_graphs ? &p->graphs_b : nullptr));
     return 0;
 }
 

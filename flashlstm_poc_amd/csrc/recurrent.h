@@ -1,5 +1,7 @@
 // Persistent, W_hh-resident recurrence kernels (forward and BPTT) for gfx950.
 #pragma once
+#include <vector>
+
 #include "common.h"
 
 namespace flstm_hip {
@@ -63,6 +65,30 @@ struct RecBwdArgs {
     long long* prof;     // optional [8] cycle counters of workgroup 0 per phase (null = off)
 };
 
+// Step-wise launches as hipGraphs.  Where the persistent kernels cannot be used (weights that do not fit on chip,
+// a plan demoted after a give-up, "stepwise" forced) a pass is one launch per time step; the launches of a range of
+// steps are captured once into a graph and replayed on later passes with the same arguments (what the reference
+// does with its CUDA graph, src/lstm.cu:1373-1895).  A cache belongs to one plan and holds a few instantiated
+// graphs keyed by the complete kernel arguments; streams that cannot be captured (the legacy default stream) and
+// ranges shorter than kGraphMinSteps take plain launches.
+struct StepGraphCache {
+    struct Entry {
+        std::vector<unsigned char> key;
+        hipGraph_t graph = nullptr;
+        hipGraphExec_t exec = nullptr;
+        unsigned long stamp = 0;
+    };
+    std::vector<Entry> entries;
+    unsigned long clock = 0;
+    long captures = 0, replays = 0;   // graphs built / graph launches (for tests and tuning)
+    bool disabled = false;            // capture failed once on this plan's stream: plain launches from then on
+    ~StepGraphCache() { clear(); }
+    void clear();
+};
+constexpr int kGraphMinSteps = 8;
+constexpr int kGraphMaxSteps = 1 << 16;
+constexpr size_t kGraphCacheEntries = 4;
+
 // Picks tile shapes and the group structure for a problem size on the current device.  force_mt: 0 = the rule of
 // thumb (16-row blocks whenever all of them can run side by side), 1 / 2 = that many 16-row tiles per row block
 // (1 only where it fits).  The choice does not change the weight-fragment layout.
@@ -79,8 +105,8 @@ int rec_fwd_ks(const RecLayout& L, int Hp);
 int rec_bwd_ks(const RecLayout& L, int Hp);
 
 // Runs steps [t0, t1). Persistent layouts use one launch; otherwise one launch per step.
-hipError_t launch_rec_fwd(const RecLayout& L, const RecFwdArgs& a, hipStream_t stream);
+hipError_t launch_rec_fwd(const RecLayout& L, const RecFwdArgs& a, hipStream_t stream, StepGraphCache* graphs = nullptr);
 // Runs steps t_hi .. t_lo (the whole pass is T-1 .. -1: all steps and the final dh0 product).
-hipError_t launch_rec_bwd(const RecLayout& L, const RecBwdArgs& a, hipStream_t stream);
+hipError_t launch_rec_bwd(const RecLayout& L, const RecBwdArgs& a, hipStream_t stream, StepGraphCache* graphs = nullptr);
 
 }  // namespace flstm_hip

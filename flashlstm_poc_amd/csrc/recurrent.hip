@@ -34,6 +34,7 @@
 //  * Fallback.  The same kernels launched once per step (no waits, kernel boundaries order
 //    memory) serve shapes whose weights do not fit on chip, and are the safe path after a failed
 //    persistent launch.
+#include <cstring>
 #include <type_traits>
 
 #include "recurrent.h"
@@ -1115,33 +1116,102 @@ RecLayout plan_rec_bwd(int B, int Hp, int num_cus, bool force_stepwise, int forc
     return L;
 }
 
+void StepGraphCache::clear() {
+    for (auto& e : entries) {
+        if (e.exec) (void)hipGraphExecDestroy(e.exec);
+        if (e.graph) (void)hipGraphDestroy(e.graph);
+    }
+    entries.clear();
+}
+
+// Runs `launch_all` (plain launches of a range of steps on `stream`) either directly or, when a cache is given and
+// the stream can be captured, as a graph: built on first use for this key, replayed afterwards.
+template <typename LaunchAll>
+static hipError_t launch_steps(StepGraphCache* graphs, const void* kernel, const void* args, size_t args_bytes,
+                               const RecLayout& L, int t_a, int t_b, int nsteps, hipStream_t stream,
+                               LaunchAll&& launch_all) {
+    if (!graphs || graphs->disabled || stream == nullptr || nsteps < kGraphMinSteps || nsteps > kGraphMaxSteps)
+        return launch_all();
+    std::vector<unsigned char> key(sizeof(kernel) + args_bytes + sizeof(RecLayout) + 2 * sizeof(int));
+    unsigned char* k = key.data();
+    memcpy(k, &kernel, sizeof(kernel)); k += sizeof(kernel);
+    memcpy(k, args, args_bytes); k += args_bytes;
+    memcpy(k, &L, sizeof(RecLayout)); k += sizeof(RecLayout);
+    memcpy(k, &t_a, sizeof(int)); k += sizeof(int);
+    memcpy(k, &t_b, sizeof(int));
+    for (auto& e : graphs->entries)
+        if (e.key == key) {
+            e.stamp = ++graphs->clock;
+            graphs->replays++;
+            return hipGraphLaunch(e.exec, stream);
+        }
+    // not seen before: capture the launches (nothing runs yet), instantiate, launch
+    if (hipStreamBeginCapture(stream, hipStreamCaptureModeThreadLocal) != hipSuccess) {
+        (void)hipGetLastError();
+        graphs->disabled = true;
+        return launch_all();
+    }
+    hipError_t le = launch_all();
+    hipGraph_t graph = nullptr;
+    hipError_t ce = hipStreamEndCapture(stream, &graph);
+    if (le != hipSuccess || ce != hipSuccess || !graph) {
+        if (graph) (void)hipGraphDestroy(graph);
+        (void)hipGetLastError();
+        graphs->disabled = true;
+        return le != hipSuccess ? le : launch_all();
+    }
+    hipGraphExec_t exec = nullptr;
+    if (hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0) != hipSuccess || !exec) {
+        (void)hipGraphDestroy(graph);
+        (void)hipGetLastError();
+        graphs->disabled = true;
+        return launch_all();
+    }
+    if (graphs->entries.size() >= kGraphCacheEntries) {   // drop the least recently used graph
+        size_t victim = 0;
+        for (size_t i = 1; i < graphs->entries.size(); ++i)
+            if (graphs->entries[i].stamp < graphs->entries[victim].stamp) victim = i;
+        (void)hipGraphExecDestroy(graphs->entries[victim].exec);
+        (void)hipGraphDestroy(graphs->entries[victim].graph);
+        graphs->entries.erase(graphs->entries.begin() + victim);
+    }
+    StepGraphCache::Entry e;
+    e.key = std::move(key); e.graph = graph; e.exec = exec; e.stamp = ++graphs->clock;
+    graphs->entries.push_back(std::move(e));
+    graphs->captures++;
+    return hipGraphLaunch(exec, stream);
+}
+
 template <int NT, int KS, bool RES, int MT>
-static hipError_t run_fwd(const RecLayout& L, const RecFwdArgs& a, hipStream_t stream) {
+static hipError_t run_fwd(const RecLayout& L, const RecFwdArgs& a, hipStream_t stream, StepGraphCache* graphs) {
     auto kernel = rec_fwd_kernel<NT, KS, RES, MT>;
     const size_t lds = size_t(2) * 4 * kRows * (16 * NT + kPartPad) * sizeof(float);
     hipError_t e = raise_lds(kernel, lds);
     if (e != hipSuccess) return e;
     const int ks_wave = rec_fwd_ks(L, a.Hp);
     if (L.persistent) return launch_persistent(kernel, L.grid, lds, stream, a, L, a.t0, a.t1, ks_wave);
-    for (int t = a.t0; t < a.t1; ++t) {
-        hipLaunchKernelGGL(kernel, dim3(L.grid), dim3(kThreads), lds, stream, a, L, t, t + 1, ks_wave);
-        e = hipGetLastError();
-        if (e != hipSuccess) return e;
-    }
-    return hipSuccess;
+    return launch_steps(graphs, reinterpret_cast<const void*>(kernel), &a, sizeof(a), L, a.t0, a.t1, a.t1 - a.t0, stream,
+                        [&]() -> hipError_t {
+                            for (int t = a.t0; t < a.t1; ++t) {
+                                hipLaunchKernelGGL(kernel, dim3(L.grid), dim3(kThreads), lds, stream, a, L, t, t + 1, ks_wave);
+                                hipError_t le = hipGetLastError();
+                                if (le != hipSuccess) return le;
+                            }
+                            return hipSuccess;
+                        });
 }
 
-hipError_t launch_rec_fwd(const RecLayout& L, const RecFwdArgs& a, hipStream_t stream) {
+hipError_t launch_rec_fwd(const RecLayout& L, const RecFwdArgs& a, hipStream_t stream, StepGraphCache* graphs) {
     if (a.T <= 0 || a.B <= 0 || a.t1 <= a.t0) return hipSuccess;
     if (a.Hp % 32 != 0 || a.Hp % L.jb != 0 || a.t0 < 0 || a.t1 > a.T) return hipErrorInvalidValue;
-    if (!L.resident) return run_fwd<8, 1, false, 2>(L, a, stream);
-    if (L.nt == 8) return L.mt == 1 ? run_fwd<8, 8, true, 1>(L, a, stream) : run_fwd<8, 8, true, 2>(L, a, stream);
-    if (L.nt == 4) return L.mt == 1 ? run_fwd<4, 16, true, 1>(L, a, stream) : run_fwd<4, 16, true, 2>(L, a, stream);
+    if (!L.resident) return run_fwd<8, 1, false, 2>(L, a, stream, graphs);
+    if (L.nt == 8) return L.mt == 1 ? run_fwd<8, 8, true, 1>(L, a, stream, graphs) : run_fwd<8, 8, true, 2>(L, a, stream, graphs);
+    if (L.nt == 4) return L.mt == 1 ? run_fwd<4, 16, true, 1>(L, a, stream, graphs) : run_fwd<4, 16, true, 2>(L, a, stream, graphs);
     return hipErrorInvalidValue;
 }
 
 template <int NT, int KS, bool RES, int KL, int MT>
-static hipError_t run_bwd(const RecLayout& L, const RecBwdArgs& a, hipStream_t stream) {
+static hipError_t run_bwd(const RecLayout& L, const RecBwdArgs& a, hipStream_t stream, StepGraphCache* graphs) {
     auto kernel = rec_bwd_kernel<NT, KS, RES, KL, MT>;
     static_assert(size_t(2) * 4 * kRows * (16 * NT + kPartPad) >= size_t(kThreads) * 8 * NT, "db reduction reuses the partial-sum area");
     const size_t lds = size_t(2) * 4 * kRows * (16 * NT + kPartPad) * sizeof(float) + size_t(4) * KL * NT * kWave * sizeof(half8);
@@ -1149,20 +1219,23 @@ static hipError_t run_bwd(const RecLayout& L, const RecBwdArgs& a, hipStream_t s
     if (e != hipSuccess) return e;
     const int ks_wave = rec_bwd_ks(L, a.Hp);
     if (L.persistent) return launch_persistent(kernel, L.grid, lds, stream, a, L, a.t_hi, a.t_lo, ks_wave);
-    for (int t = a.t_hi; t >= a.t_lo; --t) {
-        hipLaunchKernelGGL(kernel, dim3(L.grid), dim3(kThreads), lds, stream, a, L, t, t, ks_wave);
-        e = hipGetLastError();
-        if (e != hipSuccess) return e;
-    }
-    return hipSuccess;
+    return launch_steps(graphs, reinterpret_cast<const void*>(kernel), &a, sizeof(a), L, a.t_hi, a.t_lo, a.t_hi - a.t_lo + 1,
+                        stream, [&]() -> hipError_t {
+                            for (int t = a.t_hi; t >= a.t_lo; --t) {
+                                hipLaunchKernelGGL(kernel, dim3(L.grid), dim3(kThreads), lds, stream, a, L, t, t, ks_wave);
+                                hipError_t le = hipGetLastError();
+                                if (le != hipSuccess) return le;
+                            }
+                            return hipSuccess;
+                        });
 }
 
-hipError_t launch_rec_bwd(const RecLayout& L, const RecBwdArgs& a, hipStream_t stream) {
+hipError_t launch_rec_bwd(const RecLayout& L, const RecBwdArgs& a, hipStream_t stream, StepGraphCache* graphs) {
     if (a.T <= 0 || a.B <= 0 || a.t_hi < a.t_lo) return hipSuccess;
     if (a.Hp % 32 != 0 || a.Hp % L.jb != 0 || a.t_lo < -1 || a.t_hi >= a.T) return hipErrorInvalidValue;
-    if (!L.resident) return run_bwd<2, 1, false, 0, 2>(L, a, stream);
-    if (L.nt == 2) return L.mt == 1 ? run_bwd<2, 32, true, 8, 1>(L, a, stream) : run_bwd<2, 32, true, 8, 2>(L, a, stream);
-    if (L.nt == 1) return L.mt == 1 ? run_bwd<1, 64, true, 24, 1>(L, a, stream) : run_bwd<1, 64, true, 24, 2>(L, a, stream);
+    if (!L.resident) return run_bwd<2, 1, false, 0, 2>(L, a, stream, graphs);
+    if (L.nt == 2) return L.mt == 1 ? run_bwd<2, 32, true, 8, 1>(L, a, stream, graphs) : run_bwd<2, 32, true, 8, 2>(L, a, stream, graphs);
+    if (L.nt == 1) return L.mt == 1 ? run_bwd<1, 64, true, 24, 1>(L, a, stream, graphs) : run_bwd<1, 64, true, 24, 2>(L, a, stream, graphs);
     return hipErrorInvalidValue;
 }
 

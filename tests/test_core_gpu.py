@@ -169,6 +169,50 @@ def test_give_up_demotes_for_a_few_passes_and_then_the_persistent_kernel_returns
     core.close()
 
 
+@pytest.mark.parametrize("shape", [(24, 40, 64, 256), (12, 8, 32, 3072)])
+def test_stepwise_launches_replay_from_a_captured_graph(shape):
+    # Where a pass is one launch per time step (here: forced; H = 3072: weights that do not fit on chip) the launches
+    # of a range are captured into a hipGraph once and replayed afterwards.  Every replay is checked against the
+    # first (eager-equivalent) results, with the program's own eager work and synchronisations between the replays.
+    from flashlstm_poc_amd import LstmCore
+    T, B, I, H = shape
+    p = make_problem(T, B, I, H, seed=8)
+    dev = {k: v.cuda() for k, v in p.items()}
+    x, h0, c0, dy = dev["x"].half(), dev["h0"].half(), dev["c0"].half(), dev["dy"].half()
+    side = torch.cuda.Stream()      # the legacy default stream cannot be captured
+    with torch.cuda.stream(side):
+        plain = LstmCore(B, I, H)
+        plain.pack(dev["w_ih"], dev["w_hh"], dev["b_ih"], dev["b_hh"])
+        plain.set_option("stepwise", 1)
+        plain.set_option("step_graphs", 0)
+        y_ref, hy_ref, cy_ref = plain.forward(x, h0, c0)
+        g_ref = plain.backward(x, dy)
+        assert plain.info("graph_captures") == 0 and plain.info("persistent_fwd") == 0
+        core = LstmCore(B, I, H)
+        core.pack(dev["w_ih"], dev["w_hh"], dev["b_ih"], dev["b_hh"])
+        core.set_option("stepwise", 1)
+        for rep in range(4):
+            y, hy, cy = core.forward(x, h0, c0)
+            g = core.backward(x, dy)
+            side.synchronize()
+            assert torch.equal(y, y_ref) and torch.equal(cy, cy_ref), rep
+            for a, b_, name in zip(g, g_ref, ("dx", "dW_ih", "dW_hh", "db", "dh0", "dc0")):
+                assert torch.equal(a, b_), (rep, name)
+            junk = (torch.randn(256, 256, device="cuda") @ torch.randn(256, 256, device="cuda")).sum().item()   # eager work between replays
+            assert junk == junk
+        assert core.info("graphs_disabled") == 0
+        assert core.info("graph_captures") == 2 and core.info("graph_replays") == 6     # one graph per direction, 3 replays each
+        # a different sequence length is a different graph; the old ones stay usable
+        y2, _, _ = core.forward(x[:T - 2].contiguous(), h0, c0)
+        assert torch.equal(y2, y_ref[:T - 2]) and core.info("graph_captures") == 3
+        y3, _, _ = core.forward(x, h0, c0)
+        assert torch.equal(y3, y_ref) and core.info("graph_captures") == 3
+        plain.close(); core.close()
+    ref, _ = oracle_reference(p, state_grads=False)
+    check_against(ref, dict(y=to_np(y_ref), hn=to_np(hy_ref), cn=to_np(cy_ref), dx=to_np(g_ref[0]), dw_ih=to_np(g_ref[1]),
+                            dw_hh=to_np(g_ref[2]), db=to_np(g_ref[3]), dh0=to_np(g_ref[4]), dc0=to_np(g_ref[5])))
+
+
 def test_projection_chunk_size_does_not_change_results():
     p = make_problem(17, 6, 48, 40, seed=9)
     base, _ = run_core(p, proj_chunk=0)
