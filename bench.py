@@ -5,7 +5,7 @@ A "step" is one forward + backward pass of the hot path over one synthetic batch
 already resident in HBM (fp16 x / dY, packed fp16 weights); weight packing and plan creation happen
 before the timed region.  Prints ONE JSON line.
 
-  python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload config3|config2|config4]
+  python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload config3|config2|config4|config5|config5_layer]
                   [--no-cpu-baseline] [--no-parity]
 """
 import argparse
@@ -25,6 +25,8 @@ WORKLOADS = {
     "config2": (512, 64, 1024, 1024, False),
     "config3": (1024, 256, 1024, 1024, True),
     "config4": (2048, 16, 2048, 2048, True),
+    # one upper layer of the config-5 stack on its own (layers 1-3: I = H = 2048, B = 128, T = 4096), for profiles
+    "config5_layer": (4096, 128, 2048, 2048, True),
 }
 # 4-layer stack (no reference counterpart: the layer loop of flashlstm_poc_amd.LstmStack): T, B, I, H, layers
 STACKS = {"config5": (4096, 128, 512, 2048, 4)}

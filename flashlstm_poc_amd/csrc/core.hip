@@ -104,6 +104,7 @@ struct flstm_core_plan {
     int opt_mt_f = 0, opt_mt_b = 0;
     int eff_mt_f = 0, eff_mt_b = 0, eff_step_f = 0, eff_step_b = 0, eff_dw = 0;
     size_t eff_T = 0;
+    int opt_cooperative = 1;
     StepGraphCache graphs_f, graphs_b;   // captured step-wise launches (only used where the persistent kernels are not)
     int opt_graphs = 1;
     int* status_host = nullptr;   // pinned: the device status word lands here with the end-of-pass copy
@@ -141,6 +142,7 @@ void replan(flstm_core_plan* p) {
                          p->opt_mt_f ? p->opt_mt_f : p->eff_mt_f);
     p->Lb = plan_rec_bwd(p->d.B, p->d.Hp, p->num_cus, p->opt_stepwise || p->hold_bwd > 0 || p->eff_step_b,
                          p->opt_mt_b ? p->opt_mt_b : p->eff_mt_b);
+    p->Lf.cooperative = p->Lb.cooperative = p->opt_cooperative;
     p->ks_f = rec_fwd_ks(p->Lf, p->d.Hp);
     p->ks_b = rec_bwd_ks(p->Lb, p->d.Hp);
 }
@@ -238,6 +240,19 @@ extern "C" int flstm_core_create(size_t batch, size_t input_size, size_t hidden_
     p->d.H = int(hidden_size);
     p->d.Ip = int(round_up(input_size, 64));
     p->d.Hp = int(round_up(hidden_size, 32));
+    // Persistent launches are cooperative launches (co-residency of the whole grid is then a condition of the launch
+    // instead of an assumption) -- except under a rocprofiler-sdk tool: with rocprofv3 attached, a process that has
+    // made a cooperative launch takes a segmentation fault inside the tool when it exits (results and traces are
+    // complete by then; seen with ROCm 7.2), so plain launches are used there.  FLASHLSTM_COOPERATIVE_LAUNCH=0/1
+    // or the option "cooperative" decides explicitly.
+    {
+        const char* preload = getenv("LD_PRELOAD");
+        const bool profiled = (preload && strstr(preload, "rocprofiler")) || getenv("ROCPROFILER_REGISTER_LIBRARY") ||
+                              getenv("ROCP_TOOL_LIBRARIES") || getenv("ROCPROF_OUTPUT_PATH");
+        p->opt_cooperative = profiled ? 0 : 1;
+        if (const char* v = getenv("FLASHLSTM_COOPERATIVE_LAUNCH")) p->opt_cooperative = atoi(v) != 0;
+        if (const char* v = getenv("FLASHLSTM_STEP_GRAPHS")) p->opt_graphs = atoi(v) != 0;
+    }
     replan(p);
     e = p->status.reserve(64);
     if (e == hipSuccess) e = hipMemset(p->status.p, 0, 64);
@@ -281,6 +296,7 @@ extern "C" int flstm_core_set_option(flstm_core_plan* p, const char* name, long 
         return 0;
     }
     if (!strcmp(name, "clear_tuned")) { p->tuned.clear(); use_tuned(p, 1); return 0; }
+    if (!strcmp(name, "cooperative")) { p->opt_cooperative = value != 0; replan(p); return 0; }
     if (!strcmp(name, "step_graphs")) { p->opt_graphs = value != 0; return 0; }
     if (!strcmp(name, "inject_stall")) { if (value < 0) return FLSTM_E_INVALID; p->inject_stall = int(value); return 0; }
     if (!strcmp(name, "dw_splits")) { if (value < 0) return FLSTM_E_INVALID; p->opt_dw_splits = int(value); return 0; }
@@ -299,6 +315,7 @@ extern "C" long flstm_core_get_info(const flstm_core_plan* p, const char* name) 
     if (!strcmp(name, "row_tiles")) return p->Lf.mt;
     if (!strcmp(name, "row_tiles_fwd")) return p->Lf.mt;
     if (!strcmp(name, "row_tiles_bwd")) return p->Lb.mt;
+    if (!strcmp(name, "cooperative")) return p->opt_cooperative;
     if (!strcmp(name, "graph_captures")) return p->graphs_f.captures + p->graphs_b.captures;
     if (!strcmp(name, "graph_replays")) return p->graphs_f.replays + p->graphs_b.replays;
     if (!strcmp(name, "graphs_disabled")) return (p->graphs_f.disabled ? 1 : 0) + (p->graphs_b.disabled ? 2 : 0);

@@ -20,6 +20,7 @@ struct RecLayout {
     int persistent;  // 1: one launch walks all steps, 0: one launch per step
     int resident;    // 1: weight fragments live in registers for the whole launch
     int grid;        // workgroups per launch
+    int cooperative; // host side: 1 = persistent launches go through hipLaunchCooperativeKernel (set by the plan)
 };
 
 struct RecFwdArgs {

@@ -1037,11 +1037,13 @@ hipError_t raise_lds(K kernel, size_t bytes) {
 template <typename K, typename A>
 hipError_t launch_persistent(K kernel, int grid, size_t lds, hipStream_t stream, A a, RecLayout L, int t_a, int t_b,
                              int ks_wave) {
-    void* params[] = {&a, &L, &t_a, &t_b, &ks_wave};
-    hipError_t e = hipLaunchCooperativeKernel(reinterpret_cast<const void*>(kernel), dim3(grid), dim3(kThreads), params,
-                                              unsigned(lds), stream);
-    if (e == hipSuccess) return hipSuccess;
-    (void)hipGetLastError();
+    if (L.cooperative) {
+        void* params[] = {&a, &L, &t_a, &t_b, &ks_wave};
+        hipError_t e = hipLaunchCooperativeKernel(reinterpret_cast<const void*>(kernel), dim3(grid), dim3(kThreads), params,
+                                                  unsigned(lds), stream);
+        if (e == hipSuccess) return hipSuccess;
+        (void)hipGetLastError();
+    }
     hipLaunchKernelGGL(kernel, dim3(grid), dim3(kThreads), lds, stream, a, L, t_a, t_b, ks_wave);
     return hipGetLastError();
 }

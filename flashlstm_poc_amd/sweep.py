@@ -192,6 +192,8 @@ def main(argv: Optional[Sequence[str]] = None) -> int:
     ap.add_argument("--tune-stepwise", action="store_true", help="with --tune: also time one launch per step")
     ap.add_argument("--dw-splits-table", action="store_true", help="print the weight-gradient time for every "
                     "split-K count instead of sweeping")
+    ap.add_argument("--side-stream", action="store_true", help="run on a stream of its own instead of the default "
+                    "stream (step-wise launches can only be captured into a hipGraph off the default stream)")
     ap.add_argument("--csv", type=str, default=None)
     ap.add_argument("--json", type=str, default=None)
     args = ap.parse_args(argv)
@@ -205,6 +207,9 @@ def main(argv: Optional[Sequence[str]] = None) -> int:
         while t <= args.seq_len_max:
             lens.append(t)
             t *= 2
+    if args.side_stream:
+        side = torch.cuda.Stream()
+        torch.cuda.set_stream(side)
     if args.dw_splits_table:
         results = [tune_dw_splits(args.batch, args.input_size, args.hidden_size, T, seed=args.seed) for T in lens]
         for r in results:

@@ -48,9 +48,12 @@ int flstm_core_destroy(flstm_core_plan* plan);
  * and db_hh to what the caller's buffers hold instead of overwriting them: a sequence processed as several
  * consecutive segments, last segment first, each segment's dh0 / dc0 fed to the next call as d_hn / d_cn),
  * "row_tiles_fwd" / "row_tiles_bwd" (16-row tiles per row block of that recurrence: 1, 2, or 0 = automatic),
+ * "cooperative" (1: persistent launches are cooperative launches, so that co-residency of the whole grid is a
+ * condition of the launch; 0: plain launches; default 1, but 0 when a rocprofiler-sdk tool is attached -- a process
+ * that made a cooperative launch faults inside that tool at exit -- and FLASHLSTM_COOPERATIVE_LAUNCH overrides),
  * "step_graphs" (1, the default: where a pass runs as one launch per time step -- weights that do not fit on chip, a
  * demoted direction, "stepwise" -- the launches of a range of steps are captured into a hipGraph on first use and
- * replayed afterwards, when the stream allows capture; 0 = plain launches),
+ * replayed afterwards, when the stream allows capture; 0 = plain launches; FLASHLSTM_STEP_GRAPHS sets the default),
  * "inject_stall" (test hook: the next N passes that use a persistent kernel are treated as if that launch had
  * given up, which exercises the step-wise repeat and the demotion rule without making any kernel wait). */
 int flstm_core_set_option(flstm_core_plan* plan, const char* name, long value);
