@@ -4,6 +4,6 @@
 the drop-in `flashlstm` Python package of the streaming surface lives in `flashlstm_poc_amd/python`.
 """
 from .core import LstmCore, load_library, library_path, LibraryMissing, add_flashlstm_to_path
-from .stack import LstmStack
+from .stack import LstmStack, StackedLSTM
 
-__all__ = ["LstmCore", "LstmStack", "load_library", "library_path", "LibraryMissing", "add_flashlstm_to_path"]
+__all__ = ["LstmCore", "LstmStack", "StackedLSTM", "load_library", "library_path", "LibraryMissing", "add_flashlstm_to_path"]

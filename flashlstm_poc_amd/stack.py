@@ -4,6 +4,8 @@ pass layer l+1's input gradient is layer l's upstream gradient.  The reference i
 needs, with everything resident on the GPU in fp16 between layers."""
 from typing import List, Optional, Sequence, Tuple
 
+import torch
+
 from .core import LstmCore
 
 
@@ -87,3 +89,107 @@ class LstmStack:
         if cur is not None and S != 1.0:
             cur = cur.float() * (1.0 / S)   # fp32: the unscaled values may lie below the fp16 range
         return cur, grads, dh0s, dc0s
+
+
+class _StackFunction(torch.autograd.Function):
+    """Autograd node around LstmStack: inputs (x, h0 (L,B,H) or None, c0 or None, 4 * L parameters)."""
+
+    @staticmethod
+    def forward(ctx, module, x, h0, c0, y_dtype, loss_scale, *params):
+        L = module.num_layers
+        stack = module._stack_for(x.shape[1])
+        stack.pack([tuple(p.detach() for p in params[4 * l:4 * l + 4]) for l in range(L)])
+        y, hys, cys = stack.forward(x.detach(), None if h0 is None else list(h0.detach().half()),
+                                    None if c0 is None else list(c0.detach().half()))
+        module._generation += 1
+        ctx.module, ctx.stack, ctx.generation, ctx.loss_scale = module, stack, module._generation, loss_scale
+        ctx.has_state = (h0 is not None, c0 is not None)
+        ctx.x_dtype = x.dtype
+        if y_dtype != y.dtype:
+            y = y.to(y_dtype)
+        return y, torch.stack(hys), torch.stack(cys)
+
+    @staticmethod
+    def backward(ctx, dy, dhn, dcn):
+        if ctx.generation != ctx.module._generation:
+            raise RuntimeError("StackedLSTM keeps the caches of its most recent forward pass only: call backward "
+                               "before the next forward pass of the same module")
+        L = ctx.module.num_layers
+        zero_state = lambda g: None if g is None else list(g)
+        if dy is None:
+            dy = torch.zeros((ctx.stack._inputs[0].shape[0], ctx.stack.B, ctx.stack.H), device=dhn.device, dtype=torch.float16)
+        dx, grads, dh0s, dc0s = ctx.stack.backward(dy, loss_scale=ctx.loss_scale, d_hn=zero_state(dhn), d_cn=zero_state(dcn),
+                                                   want_dx=ctx.needs_input_grad[1])
+        flat = []
+        for l in range(L):
+            dW_ih, dW_hh, db = grads[l]
+            flat += [dW_ih, dW_hh, db, db.clone()]
+        gx = None if dx is None else dx.to(ctx.x_dtype)
+        gh0 = torch.stack(dh0s).half() if ctx.has_state[0] and ctx.needs_input_grad[2] else None
+        gc0 = torch.stack(dc0s).half() if ctx.has_state[1] and ctx.needs_input_grad[3] else None
+        return (None, gx, gh0, gc0, None, None, *flat)
+
+
+class StackedLSTM(torch.nn.Module):
+    """Multi-layer LSTM as an nn.Module with autograd, on the device-resident core: the training surface for a
+    stacked workload (BASELINE config 5).  The reference's module is single-layer and host-streaming
+    (flashlstm_v2/python/flashlstm/streaming_lstm.py:380-430, mirrored by flashlstm.StreamingLSTM); this one keeps
+    every sequence on the GPU.  Parameters carry torch.nn.LSTM's names (weight_ih_l0, weight_hh_l0, bias_ih_l0,
+    bias_hh_l0, ...), layout and initialisation (U(-1/sqrt(H), 1/sqrt(H)), fp32, on the GPU), so a state_dict moves
+    between the two.
+
+    forward(x, (h0, c0)=None) -> (y, (h_n, c_n)):  x (T,B,I) fp16 CUDA; h0 / c0 (L,B,H) fp16 or None (zeros);
+    y (T,B,H) in `output_dtype` (fp16, or fp32 for losses whose gradient per element lies below the fp16 range: the
+    gradient arrives in y's dtype); h_n, c_n (L,B,H) fp16.  Differentiable in x, h0, c0 and all parameters.  Inside,
+    gradients pass from layer to layer in fp16 under a power-of-two loss scale (`loss_scale`, default "auto").
+    The module keeps the caches of its MOST RECENT forward pass only; backward must run before the next forward."""
+
+    def __init__(self, input_size: int, hidden_size: int, num_layers: int = 1, *, output_dtype=torch.float16,
+                 loss_scale="auto", device="cuda"):
+        super().__init__()
+        if num_layers < 1:
+            raise ValueError("num_layers must be >= 1")
+        self.input_size, self.hidden_size, self.num_layers = int(input_size), int(hidden_size), int(num_layers)
+        self.output_dtype, self.loss_scale = output_dtype, loss_scale
+        H = self.hidden_size
+        for l in range(self.num_layers):
+            I = self.input_size if l == 0 else H
+            for name, shape in ((f"weight_ih_l{l}", (4 * H, I)), (f"weight_hh_l{l}", (4 * H, H)),
+                                (f"bias_ih_l{l}", (4 * H,)), (f"bias_hh_l{l}", (4 * H,))):
+                self.register_parameter(name, torch.nn.Parameter(torch.empty(shape, device=device, dtype=torch.float32)))
+        self.reset_parameters()
+        self._stacks = {}       # batch size -> LstmStack
+        self._generation = 0
+
+    def reset_parameters(self) -> None:
+        k = 1.0 / self.hidden_size ** 0.5
+        for p in self.parameters():     # same order as torch.nn.LSTM.reset_parameters
+            torch.nn.init.uniform_(p, -k, k)
+
+    def _stack_for(self, batch: int) -> LstmStack:
+        st = self._stacks.get(batch)
+        if st is None:
+            for old in self._stacks.values():   # one batch size at a time: the caches are large
+                old.close()
+            self._stacks = {}
+            st = self._stacks[batch] = LstmStack(batch, self.input_size, self.hidden_size, self.num_layers)
+        return st
+
+    def forward(self, x, state=None):
+        if not x.is_cuda or x.dtype != torch.float16 or x.dim() != 3 or x.shape[2] != self.input_size:
+            raise ValueError(f"x must be a CUDA float16 tensor of shape (T, B, {self.input_size})")
+        h0 = c0 = None
+        if state is not None:
+            h0, c0 = state
+            for name, t in (("h0", h0), ("c0", c0)):
+                if t is not None and (not t.is_cuda or tuple(t.shape) != (self.num_layers, x.shape[1], self.hidden_size)):
+                    raise ValueError(f"{name} must be a CUDA tensor of shape ({self.num_layers}, {x.shape[1]}, {self.hidden_size})")
+        params = [getattr(self, f"{n}_l{l}") for l in range(self.num_layers) for n in ("weight_ih", "weight_hh", "bias_ih", "bias_hh")]
+        y, h_n, c_n = _StackFunction.apply(self, x.contiguous(), h0, c0, self.output_dtype, self.loss_scale, *params)
+        return y, (h_n, c_n)
+
+    def release(self) -> None:
+        """Frees the device caches (plans are rebuilt on the next forward pass)."""
+        for st in self._stacks.values():
+            st.close()
+        self._stacks = {}

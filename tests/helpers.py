@@ -62,16 +62,26 @@ def torch_reference(p, dtype=torch.float64, device="cpu", fp16_weights=True, wit
 
 
 def check_against(ref, got, label=""):
-    """got: dict with a subset of the reference keys. Asserts the parity contract and returns the errors."""
+    """got: dict with a subset of the reference keys. Asserts the parity contract and returns the errors.
+
+    Beside the contract's norms (which are dominated by the large entries) every element is held to an absolute +
+    relative band, the kind of check the reference's own tests make (python/test_lstm.py:370-381: atol 1e-3, rtol
+    5e-2 on outputs; flashlstm_v2/python/tests/test_streaming_lstm.py: atol 2e-3 / 5e-3): outputs and states
+    |err| <= 3e-3 + 5e-2 |ref|, gradients |err| <= 5e-3 max|ref| + 5e-2 |ref|."""
     errs = {}
     for k in ("y", "hn", "cn"):
         if k in got and got[k] is not None:
             errs[k] = relmax(got[k], ref[k])
             assert errs[k] <= TOL_OUT, f"{label} {k}: max rel err {errs[k]:.3e} > {TOL_OUT}"
+            np.testing.assert_allclose(np.asarray(got[k], dtype=np.float64), ref[k], atol=3e-3, rtol=5e-2,
+                                       err_msg=f"{label} {k}")
     for k in ("dx", "dw_ih", "dw_hh", "db", "dh0", "dc0"):
         if k in got and got[k] is not None:
             errs[k] = rell2(got[k], ref[k])
             assert errs[k] <= TOL_GRAD, f"{label} {k}: rel L2 err {errs[k]:.3e} > {TOL_GRAD}"
+            scale = float(np.abs(ref[k]).max())
+            np.testing.assert_allclose(np.asarray(got[k], dtype=np.float64), ref[k], atol=5e-3 * scale + 1e-30, rtol=5e-2,
+                                       err_msg=f"{label} {k}")
     return errs
 
 

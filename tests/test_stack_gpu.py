@@ -99,3 +99,50 @@ def test_config5_stack_full_size_against_fp32_torch_lstm():
     errs = _run(4096, 128, 512, 2048, 4, loss_scale="auto", seed=7, safe_reference=True)
     print("\nconfig5 stack: " + ", ".join(f"{k}={v:.2e}" for k, v in errs.items()))
     assert max(errs.values()) <= 1e-2, errs
+
+
+def test_stacked_module_trains_like_torch_lstm():
+    # StackedLSTM as an nn.Module under autograd, the way the reference's pytest drives its single-layer module
+    # (flashlstm_v2/python/tests/test_streaming_lstm.py:15-64): same state_dict as nn.LSTM(num_layers=2), loss on
+    # y, h_n and c_n, gradients of x, h0, c0 and every parameter.
+    from flashlstm_poc_amd import StackedLSTM
+    T, B, I, H, L = 10, 6, 20, 32, 2
+    torch.manual_seed(1234)
+    ref = torch.nn.LSTM(I, H, num_layers=L, device="cuda")
+    mod = StackedLSTM(I, H, L, output_dtype=torch.float32)
+    with torch.no_grad():
+        for name, prm in ref.named_parameters():
+            if name.startswith("weight"):
+                prm.copy_(prm.half().float())
+    mod.load_state_dict(ref.state_dict())       # same parameter names and layouts
+    x = torch.randn(T, B, I, device="cuda").half()
+    h0 = (torch.randn(L, B, H, device="cuda") * 0.3).half()
+    c0 = (torch.randn(L, B, H, device="cuda") * 0.3).half()
+    xa, ha, ca = (t.clone().requires_grad_(True) for t in (x, h0, c0))
+    xb, hb, cb = (t.float().clone().requires_grad_(True) for t in (x, h0, c0))
+    ya, (hna, cna) = mod(xa, (ha, ca))
+    yb, (hnb, cnb) = ref(xb, (hb, cb))
+    assert ya.dtype == torch.float32 and relmax(to_np(ya), to_np(yb)) <= 1e-2
+    assert relmax(to_np(hna), to_np(hnb)) <= 1e-2 and relmax(to_np(cna), to_np(cnb)) <= 1e-2
+    loss = lambda y, hn, cn: (y.float() ** 2).mean() + (hn.float() ** 2).mean() + (cn.float() ** 2).mean()
+    loss(ya, hna, cna).backward()
+    loss(yb, hnb, cnb).backward()
+    assert rell2(to_np(xa.grad), to_np(xb.grad)) <= 1e-2 and xa.grad.dtype == torch.float16
+    assert rell2(to_np(ha.grad), to_np(hb.grad)) <= 1e-2 and rell2(to_np(ca.grad), to_np(cb.grad)) <= 1e-2
+    for name, prm in ref.named_parameters():
+        got = getattr(mod, name).grad
+        assert got is not None and rell2(to_np(got), to_np(prm.grad)) <= 1e-2, name
+    # one optimiser step on both, then a second forward/backward: repacking follows the updated weights
+    with torch.no_grad():
+        for name, prm in ref.named_parameters():
+            prm -= 0.1 * prm.grad
+            getattr(mod, name).copy_(prm)
+    ya2, _ = mod(x)
+    yb2, _ = ref(x.float())
+    assert relmax(to_np(ya2), to_np(yb2)) <= 1e-2
+    # the caches belong to the latest forward pass only
+    y_old, _ = mod(xa)
+    mod(xa)
+    with pytest.raises(RuntimeError, match="most recent forward"):
+        y_old.sum().backward()
+    mod.release()
