@@ -184,6 +184,44 @@ def cpu_baseline(B, I, H, backward, budget_s=15.0):
                         "fwd_bwd_batch_timesteps_per_s": round(512 / c1fb, 1)}}
 
 
+def stack_parity(params, x, target, y, grads):
+    """The timed stack problem through fp32 torch.nn.LSTM on the GPU: one single-layer module per layer, the bias as
+    the weight of an extra all-ones input column, every call on at most 131072 rows with (h, c) carried between the
+    time segments (beyond that size PyTorch-ROCm's nn.LSTM itself goes wrong: its bias gradient from 262144 rows,
+    its outputs from 524288).  `y`, `grads` = what the last timed step produced."""
+    import torch
+    T, B, _ = x.shape
+    mods = []
+    for w_ih, w_hh, b_ih, b_hh in params:
+        m = torch.nn.LSTM(w_ih.shape[1] + 1, w_hh.shape[1], bias=False, device="cuda")
+        with torch.no_grad():
+            m.weight_ih_l0[:, :-1].copy_(w_ih.half().float()); m.weight_ih_l0[:, -1].copy_(b_ih + b_hh)
+            m.weight_hh_l0.copy_(w_hh.half().float())
+        mods.append(m)
+    seg = max(1, 131072 // B)
+    cur = x.float()
+    for m in mods:
+        h = c = cur.new_zeros(1, B, m.hidden_size)
+        outs = []
+        for t0 in range(0, T, seg):
+            xs = cur[t0:t0 + seg]
+            ys, (h, c) = m(torch.cat([xs, torch.ones_like(xs[:, :, :1])], dim=2), (h, c))
+            outs.append(ys)
+        cur = outs[0] if len(outs) == 1 else torch.cat(outs, dim=0)
+    relmax = lambda a, b: ((a.float() - b.float()).abs().max() / b.float().abs().max()).item()
+    rell2 = lambda a, b: ((a.double() - b.double()).norm() / b.double().norm()).item()
+    errs = {"y": relmax(y, cur), "y_last_step": relmax(y[-1], cur[-1])}
+    torch.nn.functional.mse_loss(cur, target.float()).backward()
+    for l, (m, (dW_ih, dW_hh, db)) in enumerate(zip(mods, grads)):
+        g = m.weight_ih_l0.grad
+        errs[f"dW_ih{l}"] = rell2(dW_ih, g[:, :-1]); errs[f"dW_hh{l}"] = rell2(dW_hh, m.weight_hh_l0.grad)
+        errs[f"db{l}"] = rell2(db, g[:, -1])
+    worst = max(errs.values())
+    return {"on": "the timed tensors", "T": T, "reference": "torch.nn.LSTM fp32 on the GPU per layer, fp16-rounded weights, "
+            "calls of at most 131072 rows", "errors": {k: float(f"{v:.3e}") for k, v in errs.items()},
+            "max_err": float(f"{worst:.3e}"), "tolerance": 1e-2, "ok": bool(worst <= 1e-2)}
+
+
 def bench_stack(args, device):
     """fwd+bwd of a stack of layers with MSE on the top layer's outputs (automatic power-of-two loss scale)."""
     import torch
@@ -193,14 +231,17 @@ def bench_stack(args, device):
     k = 1.0 / H ** 0.5
     u = lambda *s: (torch.rand(*s, generator=g, device="cuda") * 2 - 1) * k
     stack = LstmStack(B, I, H, L)
-    stack.pack([(u(4 * H, I if l == 0 else H), u(4 * H, H), u(4 * H), u(4 * H)) for l in range(L)])
+    params = [(u(4 * H, I if l == 0 else H), u(4 * H, H), u(4 * H), u(4 * H)) for l in range(L)]
+    stack.pack(params)
     x = torch.randn(T, B, I, generator=g, device="cuda").half()
     target = torch.randn(T, B, H, generator=g, device="cuda").half()
+    last = {}
 
     def step():
         y, _, _ = stack.forward(x)
         dy = (y.float() - target.float()).mul_(2.0 / y.numel())
-        stack.backward(dy, want_dx=False)   # loss scale: automatic (a power of two from the largest |dy|)
+        _, grads, _, _ = stack.backward(dy, want_dx=False)   # loss scale: automatic (a power of two from the largest |dy|)
+        last["y"], last["grads"] = y, grads
 
     for _ in range(args.warmup):
         step()
@@ -232,8 +273,11 @@ def bench_stack(args, device):
                         "peak": PEAK_FP16_TFLOPS, "unit": "TFLOP/s", "frac": round(tf / PEAK_FP16_TFLOPS, 4), "traffic": None},
            "us_per_timestep": {"fwd_rec": round(phases["fwd_rec"] * 1e3 / (T * L), 3),
                                "bwd_rec": round(phases["bwd_rec"] * 1e3 / (T * L), 3)},
-           "device": device, "cpu_baseline": None}
+           "loss_scale": stack.last_loss_scale, "device": device, "cpu_baseline": None}
     stack.close()
+    torch.cuda.empty_cache()
+    if not args.no_parity:
+        out["parity"] = stack_parity(params, x, target, last["y"], last["grads"])
     return out
 
 
