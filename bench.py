@@ -59,7 +59,14 @@ def parity_check(p, outputs, grads):
     want_grads = grads is not None
     xr = torch.cat([p["x"].float(), torch.ones(T, B, 1, device="cuda")], dim=2).requires_grad_(want_grads)
     hr = p["h0"].float().requires_grad_(want_grads); cr = p["c0"].float().requires_grad_(want_grads)
-    yr, (hn, cn) = m(xr, (hr[None], cr[None]))
+    # (and one call of more than 131072 rows returns wrong outputs at H = 2048: the sequence goes through in
+    # segments, the state carried from one call to the next inside the same autograd graph)
+    seg = max(1, 131072 // B)
+    ys, state = [], (hr[None], cr[None])
+    for t0 in range(0, T, seg):
+        y_seg, state = m(xr[t0:t0 + seg], state)
+        ys.append(y_seg)
+    yr, (hn, cn) = (ys[0] if len(ys) == 1 else torch.cat(ys)), state
     relmax = lambda a, b: ((a.float() - b.float()).abs().max() / b.float().abs().max()).item()
     rell2 = lambda a, b: ((a.double() - b.double()).norm() / b.double().norm()).item()
     y, hy, cy = outputs
@@ -72,7 +79,7 @@ def parity_check(p, outputs, grads):
                      "dW_hh": rell2(dW_hh, m.weight_hh_l0.grad), "db": rell2(db, gw[:, I]),
                      "dh0": rell2(dh0, hr.grad), "dc0": rell2(dc0, cr.grad)})
     worst = max(errs.values())
-    return {"on": "the timed tensors", "T": T, "reference": "torch.nn.LSTM fp32 on the GPU, fp16-rounded weights",
+    return {"on": "the timed tensors", "T": T, "reference": "torch.nn.LSTM fp32 on the GPU, fp16-rounded weights, calls of at most 131072 rows",
             "errors": {k: float(f"{v:.3e}") for k, v in errs.items()}, "max_err": float(f"{worst:.3e}"),
             "tolerance": 1e-2, "ok": bool(worst <= 1e-2)}
 
@@ -351,7 +358,8 @@ def main():
               "bwd_rec": 2.0 * T * B * 4 * H * H, "bwd_dx": 2.0 * T * B * 4 * H * I,
               "bwd_dw": 2.0 * T * B * 4 * H * (I + H)}
     kname = {"fwd_proj": "gemm_nt_stream (X*W_ih^T + bias)", "fwd_rec": "rec_fwd_kernel (persistent recurrence)",
-             "bwd_rec": "rec_bwd_kernel (persistent BPTT)", "bwd_dx": "gemm_nt_stream (dG*W_ih)",
+             "bwd_rec": ("rec_bwd2d_kernel (persistent BPTT, product split over columns and contraction)"
+                         if core.info("bwd_two_d") == 1 else "rec_bwd_kernel (persistent BPTT)"), "bwd_dx": "gemm_nt_stream (dG*W_ih)",
              "bwd_dw": "gemm_tn_256x256 split-K x2 (dG^T*X, dG^T*H) + reduce_dw"}
     kernels = []
     for k in phases:
@@ -382,7 +390,7 @@ def main():
         "mfu_target": 0.40, "tflops": round(flops / (ms * 1e-3) / 1e12, 1), "flops_per_step": flops,
         "persistent": {"fwd": core.info("persistent_fwd"), "bwd": core.info("persistent_bwd"),
                        "xcd_local_fwd": core.info("xcd_local_fwd"), "xcd_local_bwd": core.info("xcd_local_bwd"),
-                       "fallbacks": core.info("fallbacks")},
+                       "bwd_two_d": core.info("bwd_two_d"), "fallbacks": core.info("fallbacks")},
         "roofline": roofline, "kernels": kernels, "device": device,
         "us_per_timestep": {"fwd_rec": round(phase_ms["fwd_rec"] * 1e3 / T, 3),
                             **({"bwd_rec": round(phase_ms["bwd_rec"] * 1e3 / T, 3)} if backward else {})},
@@ -398,6 +406,11 @@ def main():
         slices = Hp // core.info("slice_" + d)
         l2_bytes = rows * slices * k_cols * 2
         lds_bytes = 2 * 4 * rows * slices * core.info("slice_" + d) * gate_cols * 4
+        if d == "bwd" and core.info("bwd_two_d") == 1:
+            # 256 workgroups, each fetches an eighth of dG_{t+1} of every row; the fp32 partial products
+            # [rows][64 columns] of each go through LDS (4 waves) and, 7/8 of them, once through the L2 to the slice's peers
+            l2_bytes = rows * 256 * (k_cols // 8) * 2 + 2 * rows * 256 * 64 * 4
+            lds_bytes = 2 * 4 * rows * 256 * 64 * 4
         xch[d] = {"l2_fetch_bytes_per_step": l2_bytes, "l2_fetch_gb_per_s": round(l2_bytes / us / 1e3, 1),
                   "lds_bytes_per_step": lds_bytes, "lds_gb_per_s": round(lds_bytes / us / 1e3, 1)}
     out["exchange_per_step"] = xch

@@ -107,10 +107,11 @@ struct flstm_core_plan {
     int opt_cooperative = 1;
     StepGraphCache graphs_f, graphs_b;   // captured step-wise launches (only used where the persistent kernels are not)
     int opt_graphs = 1;
+    int opt_two_d = 1;   // backward recurrence for 2048 hidden units, two-way split: 0 never, 1 where it is faster, 2 wherever it can run
     int* status_host = nullptr;   // pinned: the device status word lands here with the end-of-pass copy
     int inject_stall = 0;         // test hook: treat the next N persistent passes as if their launch had given up
     // weights
-    DevBuf wih_p, wih_t, wfrag_f, wfrag_b, bias_p;
+    DevBuf wih_p, wih_t, wfrag_f, wfrag_b, wfrag_b2, bias_p;
     bool weights_packed = false, bias_packed = false;
     // forward state / caches
     DevBuf X16, G, Y, C, status, xch_f, xch_b;
@@ -122,7 +123,7 @@ struct flstm_core_plan {
     struct { size_t T = 0; const half_t* dYk = nullptr; const void* dY = nullptr; flstm_dtype dy_dtype = FLSTM_F16;
              float S = 1.f, dy_scale = 1.f; void* dx = nullptr; flstm_dtype dx_dtype = FLSTM_F16; bool open = false; } bw;
     // backward scratch
-    DevBuf dYp, dG, dHn, dC, dH0, db_part, dw_part, prof;
+    DevBuf dYp, dG, dHn, dC, dH0, db_part, dw_part, prof, part_b;
     int opt_profile = 0, wall_khz = 100000;
     long long prof_f[8] = {}, prof_b[8] = {};
     PhaseTimer tm;
@@ -141,7 +142,7 @@ void replan(flstm_core_plan* p) {
     p->Lf = plan_rec_fwd(p->d.B, p->d.Hp, p->num_cus, p->opt_stepwise || p->hold_fwd > 0 || p->eff_step_f,
                          p->opt_mt_f ? p->opt_mt_f : p->eff_mt_f);
     p->Lb = plan_rec_bwd(p->d.B, p->d.Hp, p->num_cus, p->opt_stepwise || p->hold_bwd > 0 || p->eff_step_b,
-                         p->opt_mt_b ? p->opt_mt_b : p->eff_mt_b);
+                         p->opt_mt_b ? p->opt_mt_b : p->eff_mt_b, p->opt_two_d);
     p->Lf.cooperative = p->Lb.cooperative = p->opt_cooperative;
     p->ks_f = rec_fwd_ks(p->Lf, p->d.Hp);
     p->ks_b = rec_bwd_ks(p->Lb, p->d.Hp);
@@ -252,6 +253,7 @@ extern "C" int flstm_core_create(size_t batch, size_t input_size, size_t hidden_
         p->opt_cooperative = profiled ? 0 : 1;
         if (const char* v = getenv("FLASHLSTM_COOPERATIVE_LAUNCH")) p->opt_cooperative = atoi(v) != 0;
         if (const char* v = getenv("FLASHLSTM_STEP_GRAPHS")) p->opt_graphs = atoi(v) != 0;
+        if (const char* v = getenv("FLASHLSTM_BWD_TWO_D")) p->opt_two_d = atoi(v) < 0 ? 0 : (atoi(v) > 2 ? 2 : atoi(v));
     }
     replan(p);
     e = p->status.reserve(64);
@@ -266,7 +268,7 @@ extern "C" int flstm_core_create(size_t batch, size_t input_size, size_t hidden_
 
 extern "C" int flstm_core_destroy(flstm_core_plan* p) {
     if (!p) return FLSTM_E_INVALID;
-    for (DevBuf* b : {&p->wih_p, &p->wih_t, &p->wfrag_f, &p->wfrag_b, &p->bias_p, &p->X16, &p->G, &p->Y, &p->C,
+    for (DevBuf* b : {&p->wih_p, &p->wih_t, &p->wfrag_f, &p->wfrag_b, &p->wfrag_b2, &p->part_b, &p->bias_p, &p->X16, &p->G, &p->Y, &p->C,
                       &p->status, &p->xch_f, &p->xch_b, &p->dYp, &p->dG, &p->dHn, &p->dC,
                       &p->dH0, &p->db_part, &p->dw_part, &p->prof})
         b->release();
@@ -280,7 +282,7 @@ extern "C" int flstm_core_set_option(flstm_core_plan* p, const char* name, long 
     if (!p || !name) return FLSTM_E_INVALID;
     if (!strcmp(name, "stepwise")) { p->opt_stepwise = value != 0; replan(p); return 0; }
     if (!strcmp(name, "proj_chunk")) { p->opt_proj_chunk = int(value); return 0; }
-    if (!strcmp(name, "spin_limit")) { if (value < 1) return FLSTM_E_INVALID; p->opt_spin_limit = int(value); return 0; }
+    if (!strcmp(name, "spin_limit")) { if (value < 0) return FLSTM_E_INVALID; p->opt_spin_limit = int(value); return 0; }
     if (!strcmp(name, "spin_ms")) { if (value < 1 || value > 60000) return FLSTM_E_INVALID; p->opt_spin_ms = int(value); return 0; }
     if (!strcmp(name, "profile")) {
         p->opt_profile = value != 0;
@@ -298,6 +300,7 @@ extern "C" int flstm_core_set_option(flstm_core_plan* p, const char* name, long 
     if (!strcmp(name, "clear_tuned")) { p->tuned.clear(); use_tuned(p, 1); return 0; }
     if (!strcmp(name, "cooperative")) { p->opt_cooperative = value != 0; replan(p); return 0; }
     if (!strcmp(name, "step_graphs")) { p->opt_graphs = value != 0; return 0; }
+    if (!strcmp(name, "bwd_two_d")) { if (value < 0 || value > 2) return FLSTM_E_INVALID; p->opt_two_d = int(value); replan(p); return 0; }
     if (!strcmp(name, "inject_stall")) { if (value < 0) return FLSTM_E_INVALID; p->inject_stall = int(value); return 0; }
     if (!strcmp(name, "dw_splits")) { if (value < 0) return FLSTM_E_INVALID; p->opt_dw_splits = int(value); return 0; }
     if (!strcmp(name, "accumulate_grads")) { p->opt_accumulate = value != 0; return 0; }
@@ -316,6 +319,7 @@ extern "C" long flstm_core_get_info(const flstm_core_plan* p, const char* name) 
     if (!strcmp(name, "row_tiles_fwd")) return p->Lf.mt;
     if (!strcmp(name, "row_tiles_bwd")) return p->Lb.mt;
     if (!strcmp(name, "cooperative")) return p->opt_cooperative;
+    if (!strcmp(name, "bwd_two_d")) return p->Lb.two_d;
     if (!strcmp(name, "graph_captures")) return p->graphs_f.captures + p->graphs_b.captures;
     if (!strcmp(name, "graph_replays")) return p->graphs_f.replays + p->graphs_b.replays;
     if (!strcmp(name, "graphs_disabled")) return (p->graphs_f.disabled ? 1 : 0) + (p->graphs_b.disabled ? 2 : 0);
@@ -328,7 +332,7 @@ extern "C" long flstm_core_get_info(const flstm_core_plan* p, const char* name) 
     if (!strcmp(name, "tuned_dw_splits")) return p->eff_dw;
     if (!strcmp(name, "device_bytes")) {
         size_t sum = 0;
-        for (const DevBuf* b : {&p->wih_p, &p->wih_t, &p->wfrag_f, &p->wfrag_b, &p->bias_p, &p->X16, &p->G, &p->Y, &p->C,
+        for (const DevBuf* b : {&p->wih_p, &p->wih_t, &p->wfrag_f, &p->wfrag_b, &p->wfrag_b2, &p->part_b, &p->bias_p, &p->X16, &p->G, &p->Y, &p->C,
                                 &p->status, &p->xch_f, &p->xch_b, &p->dYp, &p->dG, &p->dHn, &p->dC, &p->dH0, &p->db_part,
                                 &p->dw_part, &p->prof})
             sum += b->bytes;
@@ -361,6 +365,10 @@ extern "C" int flstm_core_pack_weights(flstm_core_plan* p, const float* w_ih, co
     FL_TRY(p->wfrag_b.reserve(size_t(p->Lb.nh) * 4 * p->ks_b * p->Lb.nt * kWave * sizeof(half8)));
     FL_TRY(pack_weights(d, w_ih, w_hh, p->wih_p.as<half_t>(), p->wih_t.as<half_t>(), p->wfrag_f.as<half8>(),
                         p->ks_f, p->Lf.nt, p->wfrag_b.as<half8>(), p->ks_b, p->Lb.nt, s));
+    if (rec_bwd_two_d_possible(d.Hp, p->num_cus)) {   // whether or not the current layout uses them
+        FL_TRY(p->wfrag_b2.reserve(rec_bwd_two_d_wfrag_bytes(d.Hp)));
+        FL_TRY(pack_wfrag_bwd2d(d, w_hh, p->wfrag_b2.as<half8>(), s));
+    }
     FL_TRY(hipStreamSynchronize(s));
     p->weights_packed = true;
     return 0;
@@ -610,8 +618,15 @@ int backward_setup(flstm_core_plan* p, size_t T, const void* dY, flstm_dtype dy_
     FL_TRY(p->dG.reserve(TB * 4 * d.Hp * sizeof(half_t)));
     FL_TRY(p->db_part.reserve(size_t(p->Lb.ng) * 4 * d.Hp * sizeof(float)));
     const size_t xslot = exchange_slot_halfs(d.B, 4 * d.Hp);
-    FL_TRY(p->xch_b.reserve(4 * xslot * sizeof(half_t)));
-    FL_TRY(fill_words(p->xch_b.p, 4 * xslot * sizeof(half_t), 0xFFFFFFFFu, s));
+    const size_t dg_slots = size_t(rec_bwd_dg_slots(p->Lb));
+    FL_TRY(p->xch_b.reserve(dg_slots * xslot * sizeof(half_t)));
+    FL_TRY(fill_words(p->xch_b.p, dg_slots * xslot * sizeof(half_t), 0xFFFFFFFFu, s));
+    if (p->Lb.two_d) {
+        const size_t pslot = rec_bwd_part_slot_floats(p->Lb) * sizeof(float);
+        FL_TRY(p->part_b.reserve(kRecBwdPartSlots * pslot));
+        for (int k = 0; k < kRecBwdPartSlots; ++k)
+            FL_TRY(fill_words(static_cast<char*>(p->part_b.p) + size_t(k) * pslot, pslot, rec_bwd_part_fill(k, int(T)), s));
+    }
     FL_TRY(convert_pad_f32(d_hn, dstate_dtype == FLSTM_F32, size_t(d.B), d.H, S, p->dHn.as<float>(), size_t(d.Hp), s));
     FL_TRY(convert_pad_f32(d_cn, dstate_dtype == FLSTM_F32, size_t(d.B), d.H, S, p->dC.as<float>(), size_t(d.Hp), s));
     FL_TRY(fill_zero(p->db_part.p, size_t(p->Lb.ng) * 4 * d.Hp * sizeof(float), s));
@@ -636,6 +651,11 @@ int backward_recur(flstm_core_plan* p, long t_hi, long t_lo, hipStream_t s) {
     a.G = p->G.as<half_t>(); a.C = p->C.as<float>(); a.dY = p->bw.dYk; a.dG = p->dG.as<half_t>();
     a.dHn = p->dHn.as<float>(); a.dC = p->dC.as<float>(); a.dH0 = p->dH0.as<float>();
     a.X = p->xch_b.as<half_t>(); a.x_slot = exchange_slot_halfs(d.B, 4 * d.Hp);
+    if (p->Lb.two_d) {
+        a.wfrag2 = p->wfrag_b2.as<half8>();
+        a.P = p->part_b.as<float>();
+        a.p_slot = rec_bwd_part_slot_floats(p->Lb);
+    }
     a.db_part = p->db_part.as<float>();
     a.status = p->status.as<int>();
     a.seats = p->status.as<unsigned>() + 8;

@@ -21,6 +21,9 @@ struct RecLayout {
     int resident;    // 1: weight fragments live in registers for the whole launch
     int grid;        // workgroups per launch
     int cooperative; // host side: 1 = persistent launches go through hipLaunchCooperativeKernel (set by the plan)
+    int two_d;       // backward, 2048 hidden units: workgroups split the product over output columns AND the contraction
+                     // (32 column slices x 8 contraction slices, partial sums exchanged inside an XCD); nt, jb, nh
+                     // still describe the one-dimensional layout, whose weight fragments the step-wise fallback uses
 };
 
 struct RecFwdArgs {
@@ -51,7 +54,13 @@ struct RecBwdArgs {
     half_t* dG;          // [T*B][4Hp] pre-activation gradients (scaled), row-major, for the GEMMs
     half_t* X;           // exchange ring, 4 slots of x_slot halfs, fragment-major; step t writes slot t%4 (dG_t);
                          // before the first step all four hold the 0xFFFF 'unwritten' pattern
+                         // (two-dimensional layout: rec_bwd_dg_slots() = 8 slots, step t writes slot t%8)
     size_t x_slot;
+    const half8* wfrag2; // two-dimensional layout: [32 column slices][8 contraction slices][4 waves][8 k-steps][4 tiles][64]
+    float* P;            // two-dimensional layout: ring of 3 slots of p_slot floats for the partial sums; before the first
+                         // step the lowest bit of every word of slot (t+3)%3 is the opposite of t&1 for the first step t
+                         // that uses the slot (rec_bwd_part_fill)
+    size_t p_slot;
     float* dHn;          // [B][Hp] scaled gradient wrt final h (zeros when absent)
     float* dC;           // [B][Hp] running scaled dc; in: gradient wrt final c, out: dc0
     float* dH0;          // [B][Hp] out: scaled gradient wrt h0
@@ -94,7 +103,18 @@ constexpr size_t kGraphCacheEntries = 4;
 // thumb (16-row blocks whenever all of them can run side by side), 1 / 2 = that many 16-row tiles per row block
 // (1 only where it fits).  The choice does not change the weight-fragment layout.
 RecLayout plan_rec_fwd(int B, int Hp, int num_cus, bool force_stepwise, int force_mt = 0);
-RecLayout plan_rec_bwd(int B, int Hp, int num_cus, bool force_stepwise, int force_mt = 0);
+// two_d: 0 = never the two-way split, 1 = where it is the faster layout, 2 = wherever it can run
+RecLayout plan_rec_bwd(int B, int Hp, int num_cus, bool force_stepwise, int force_mt = 0, int two_d = 1);
+
+// The two-dimensional backward layout: whether a device/size can use it at all (decides whether its weight fragments
+// are packed), slots of its dG ring, floats per slot of its partial ring and bytes of its weight fragments.
+bool rec_bwd_two_d_possible(int Hp, int num_cus);
+int rec_bwd_dg_slots(const RecLayout& L);
+size_t rec_bwd_part_slot_floats(const RecLayout& L);
+constexpr int kRecBwdPartSlots = 3;
+size_t rec_bwd_two_d_wfrag_bytes(int Hp);
+// Word to fill slot `slot` of the partial ring with before a pass over T steps (see RecBwdArgs::P).
+unsigned rec_bwd_part_fill(int slot, int T);
 
 // Halfs in one slot of an exchange ring for a [rows][cols] operand (rows padded to 32).
 size_t exchange_slot_halfs(int rows, int cols);

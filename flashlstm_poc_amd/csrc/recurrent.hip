@@ -1014,6 +1014,375 @@ __global__ __launch_bounds__(kThreads) void rec_bwd_kernel(RecBwdArgs p, RecLayo
     }
 }
 
+// --------------------------------------------------------------- backward, two-dimensional split
+// For 2048 hidden units the product dG_{t+1} * W_hh^T has 32 MiB of weights: spread over the 256 compute units without
+// replication, every workgroup holds 128 KiB, and what it fetches per step depends on how its block is shaped.  The
+// kernel above gives a workgroup 16 output columns and the whole contraction (8192 packed gate columns), so every
+// workgroup pulls all of dG_{t+1} through its vector-memory path each step (512 KiB for a 32-row block).  Here a
+// workgroup owns a 64-column slice `s` (32 of them) and one EIGHTH `q` of the contraction: it fetches an eighth of
+// dG_{t+1}, forms a partial product [rows][64], and the eight workgroups of a slice -- seated in one XCD -- sum
+// their partials through a small ring in that XCD's L2: workgroup q sends columns 8q'..8q'+7 of its partial to
+// workgroup q' of the slice and finishes the 8 hidden units 64s + 8q .. +7 for all rows (one cell per thread).
+//
+// Two rings carry a step:
+//  * dG ring (p.X): 8 slots, fragment-major, written with device-scope stores and validated through the 'unwritten'
+//    pattern like the rings above.  A workgroup that has its product of step t knows that every workgroup has stored
+//    dG_{t+2} (its 32 producers stored dG_{t+1}, and each of those needed partials from a full slice, which together
+//    read all of dG_{t+2}), i.e. nobody reads dG_{t+3} any more: that slot is marked, five steps before it is reused.
+//  * partial ring (p.P): 3 slots of fp32 partial sums, [slice][receiver][row block][sender][row][8].  Plain stores,
+//    XCD-local.  It needs no marks: the lowest mantissa bit of every word carries the parity of the step, and a slot
+//    is reused every third step, so what a slot held before always shows the other parity (the bit costs 2^-24
+//    relative precision).  A sender overwrites the partials of step t+3 after its product of step t, when all
+//    workgroups are past step t+2.
+// A row block's partials are collected one product later (row block i-1 after the product of row block i), which
+// hides the trip through the L2 except for the last row block of a step.
+constexpr int kKQ = 8;          // contraction slices = workgroups per column slice
+constexpr int kDgSlots = 8;     // dG ring
+static_assert(kRecBwdPartSlots % 2 == 1, "consecutive uses of a partial-ring slot must differ in step parity");
+
+// Every global load of this kernel is a buffer load the compiler knows about (cache policy in the builtin's last
+// argument: 16 = device scope, served by the L2 and beyond; 2 = non-temporal), so the compiler places the
+// vector-memory waits itself and counts them exactly -- fragments requested a whole row block ahead stay in flight
+// across loop iterations as ordinary values.  order_here() keeps it from moving, merging or hoisting them: the
+// order of issue is part of the design (loads return in order), and a poll has to load again.
+typedef __amdgpu_buffer_rsrc_t rsrc_t;
+__device__ __forceinline__ rsrc_t make_rsrc(const void* p, size_t bytes) {
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(p), 0, int(unsigned(bytes < 0xFFFFFFFFull ? bytes : 0xFFFFFFFFull)),
+                                             0x00020000);
+}
+__device__ __forceinline__ void order_here() { asm volatile("" ::: "memory"); }
+constexpr int kDeviceScope = 16, kNonTemporal = 2;
+
+template <int MT>
+__global__ __launch_bounds__(kThreads) void rec_bwd2d_kernel(RecBwdArgs p, RecLayout L, int t_first, int t_last, int) {
+    constexpr int NT = 4;    // 64 output columns
+    constexpr int KS = 8;    // k-steps per wave: 4 waves * 8 * 32 = 1024 packed gate columns
+    constexpr int PLD = 16 * NT + kPartPad;
+    constexpr int RB = 16 * MT;
+    extern __shared__ __attribute__((aligned(16))) float part_all[];  // [2][4][32][PLD] partial sums | [nrb][256] running dc
+    __shared__ int lds_abort;
+    __shared__ int lds_role[2];
+    const int tid = threadIdx.x, wave = tid / kWave, lane = tid % kWave;
+    if (tid == 0) {
+        lds_abort = 0;
+        const int xcd = int(xcc_id()) & 7;
+        const unsigned seat = __hip_atomic_fetch_add(p.seats + xcd, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (seat >= 32u) __hip_atomic_store(p.status, 2, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        lds_role[0] = xcd;
+        lds_role[1] = int(seat);
+    }
+    __syncthreads();
+    if (lds_role[1] >= 32) return;
+    const int seat = __builtin_amdgcn_readfirstlane(lds_role[1]);
+    const int s = __builtin_amdgcn_readfirstlane(lds_role[0]) * 4 + seat / kKQ;   // column slice (its 8 workgroups share the XCD)
+    const int q = seat % kKQ;                            // contraction slice; also: which 8 columns of the slice end here
+    const int wave_u = __builtin_amdgcn_readfirstlane(wave);
+    const int nks = p.Hp / 8;                            // k-steps of the whole contraction
+    const int nrb = L.nrb;
+    const Poll poll{true, p.spin_limit, p.spin_ticks, p.status, &lds_abort};
+    const float S = p.dy_scale;
+    PhaseClock clk{(blockIdx.x == 0) ? p.prof : nullptr, 0};
+
+    half8 wreg[KS][NT];
+    {
+        const half8* wf = p.wfrag2 + ((size_t(s) * kKQ + q) * 4 + wave) * size_t(KS) * NT * kWave;
+#pragma unroll
+        for (int k = 0; k < KS; ++k)
+#pragma unroll
+            for (int n = 0; n < NT; ++n) wreg[k][n] = wf[(k * NT + n) * kWave + lane];
+    }
+
+    // this thread's cell: row pr of a row block, hidden unit j; as a sender: row pr, columns 8*pj.. of the partial
+    const int pr = tid / 8, pj = tid % 8;
+    const bool row_used = pr < RB;
+    const int j = s * 64 + q * 8 + pj;
+    const size_t pq = size_t(4) * j;
+    const size_t gld = size_t(4) * p.Hp;
+    float* dcl = part_all + 2 * 4 * kRows * PLD;
+    for (int rb = 0; rb < nrb; ++rb) {
+        const int b = rb * RB + pr;
+        dcl[rb * kThreads + tid] = (row_used && b < p.B) ? p.dC[size_t(b) * p.Hp + j] : 0.f;
+    }
+    float dbacc[4] = {};
+    int item = 0;
+
+    // poll bookkeeping shared by the two kinds of waits; true = give up
+    auto spin_out = [&](int& spins, long long& spin_start) -> bool {
+        ++spins;
+        if (spins == 1) spin_start = wall_clock64();
+        if (spins > poll.limit || *reinterpret_cast<volatile int*>(poll.lds_abort) != 0 ||
+            ((spins & 255) == 0 &&
+             (wall_clock64() - spin_start > poll.ticks ||
+              __hip_atomic_load(poll.status, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0))) {
+            if (lane == 0) {
+                __hip_atomic_store(poll.status, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                *reinterpret_cast<volatile int*>(poll.lds_abort) = 1;
+            }
+            return true;   // results are garbage from here on; the workgroup leaves at its next barrier
+        }
+        return false;
+    };
+
+    // Per-cell operands of a row block (activated gates, c_{t-1}, c_t, dY): requested while the block's product runs,
+    // used one product later; two sets, by the parity of the row block.
+    uintx2 og[2];
+    unsigned ocp[2], occ[2];
+    unsigned short ody[2];
+    auto load_ops = [&](int t, int rb, uintx2& g, unsigned& cp, unsigned& cc, unsigned short& dy) {
+        const int b = min(rb * RB + pr, p.B - 1);
+        const size_t tt = size_t(max(t, 0));
+        // (a descriptor per step: the arrays of a long sequence are larger than a 32-bit offset reaches)
+        const rsrc_t rg = make_rsrc(p.G + tt * p.B * gld, size_t(p.B) * gld * 2);
+        const rsrc_t rc = make_rsrc(p.C + tt * p.B * p.Hp, size_t(2) * p.B * p.Hp * 4);
+        const rsrc_t ry = make_rsrc(p.dY + tt * p.B * p.Hp, size_t(p.B) * p.Hp * 2);
+        const unsigned cell_idx = unsigned(b) * unsigned(p.Hp) + unsigned(j);
+        g = __builtin_amdgcn_raw_buffer_load_b64(rg, (unsigned(b) * unsigned(gld) + unsigned(pq)) * 2u, 0, kNonTemporal);
+        cp = __builtin_amdgcn_raw_buffer_load_b32(rc, cell_idx * 4u, 0, kNonTemporal);
+        cc = __builtin_amdgcn_raw_buffer_load_b32(rc, (cell_idx + unsigned(p.B) * unsigned(p.Hp)) * 4u, 0, kNonTemporal);
+        dy = __builtin_amdgcn_raw_buffer_load_b16(ry, cell_idx * 2u, 0, kNonTemporal);
+        order_here();
+    };
+    // the cell update of (t, rb) given dh from the product (or dHn), and everything it stores
+    auto cell = [&](int t, int rb, float dh, uintx2 g, unsigned cpb, unsigned ccb, unsigned short dyb) {
+        const int b = rb * RB + pr;
+        const bool live = row_used && b < p.B;
+        const size_t sidx = size_t(b) * p.Hp + j;
+        if (t < 0) {   // closing pass: gradient wrt h0; dc0 is the running dc
+            if (live) {
+                p.dH0[sidx] = dh;
+                p.dC[sidx] = dcl[rb * kThreads + tid];
+            }
+            return;
+        }
+        half_t* xout = p.X + size_t((t + 8) & (kDgSlots - 1)) * p.x_slot;     // dG_t for everybody
+        half_t* xmark = p.X + size_t((t + 11) & (kDgSlots - 1)) * p.x_slot;   // dG_{t+3}: read by nobody any more
+        unsigned off = 0;
+        if (row_used) {
+            off = unsigned(xch_offset(b, int(pq), nks));
+            store_xch(xmark + off, Pack<4>{uintx2{kUnwritten, kUnwritten}}, true);
+        }
+        Pack<4> out{uintx2{0u, 0u}};   // batch rows past B travel as zeros
+        if (live) {
+            float gate[4];
+            unpack(Pack<4>{g}, gate);
+            float dyl, dyh;
+            unpack_h2(unsigned(dyb), dyl, dyh);
+            const float pcp = __builtin_bit_cast(float, cpb), pcc = __builtin_bit_cast(float, ccb);
+            const float ig = gate[0], fg = gate[1], gg = gate[2], og_ = gate[3];
+            const float dhu = dh + S * dyl;
+            const float tc = tanhf_dev(pcc);
+            const float dov = dhu * tc;
+            const float dc = dcl[rb * kThreads + tid] + dhu * og_ * (1.f - tc * tc);
+            float da[4];
+            da[0] = dc * gg * ig * (1.f - ig);
+            da[1] = dc * pcp * fg * (1.f - fg);
+            da[2] = dc * ig * (1.f - gg * gg);
+            da[3] = dov * og_ * (1.f - og_);
+            dcl[rb * kThreads + tid] = dc * fg;
+            out = pack(da);
+            float r[4];   // db sums the values the weight-gradient GEMMs will see (fp16-rounded)
+            unpack(out, r);
+#pragma unroll
+            for (int gt = 0; gt < 4; ++gt) dbacc[gt] += r[gt];
+        }
+        if (row_used) store_xch(xout + off, out, true);
+        clk.lap(2);
+        if (live) st_pack(p.dG + (size_t(t) * p.B + b) * gld + pq, out);
+        clk.lap(3);
+    };
+
+    // Fragments of dG_{t+1} for one row block: this wave's 8 k-steps of the workgroup's contraction slice, requested
+    // together; two sets, so the next row block's fetch runs under this one's MFMAs and the partial exchange (and the
+    // first row block of the next step is requested while the last one of this step is being finished).
+    const rsrc_t rx = make_rsrc(p.X, size_t(kDgSlots) * p.x_slot * 2);
+    const rsrc_t rp = make_rsrc(p.P, size_t(kRecBwdPartSlots) * p.p_slot * 4);
+    uintx4 fr[2][KS][MT];
+    unsigned voff[KS];   // byte offset of this lane's 16 bytes in k-step k of the wave (k-steps of a wave are 4 apart)
+#pragma unroll
+    for (int k = 0; k < KS; ++k) voff[k] = unsigned(lane) * 16u + unsigned(k) * 4096u;
+    auto load_set = [&](uintx4 (&f)[KS][MT], int slot, int rb) {
+        const unsigned base = unsigned((size_t(slot) * p.x_slot + (size_t(MT * rb) * nks + size_t(q) * 32 + wave_u) * 512) * 2);
+#pragma unroll
+        for (int k = 0; k < KS; ++k)
+#pragma unroll
+            for (int m = 0; m < MT; ++m)
+                f[k][m] = __builtin_amdgcn_raw_buffer_load_b128(rx, voff[k], base + unsigned(m) * unsigned(nks) * 1024u, kDeviceScope);
+        order_here();
+    };
+    bool pending0 = false;   // set 0 already holds (or awaits) the first row block of the step that comes next
+
+    __syncthreads();
+    clk.start();
+    for (int t = t_first; t >= t_last; --t) {
+        if (t >= p.T - 1) {   // the last step of the sequence: dh comes from the caller
+            for (int rb = 0; rb < nrb; ++rb) {
+                load_ops(t, rb, og[0], ocp[0], occ[0], ody[0]);
+                const int b = min(rb * RB + pr, p.B - 1);
+                const float dh = p.dHn[size_t(b) * p.Hp + j];
+                cell(t, rb, dh, og[0], ocp[0], occ[0], ody[0]);
+            }
+            continue;
+        }
+        const int slot_in = (t + 9) & (kDgSlots - 1);   // dG_{t+1}
+        const unsigned pbase = unsigned((t + 3) % kRecBwdPartSlots) * unsigned(p.p_slot);   // in floats
+        float* pslot = p.P + size_t(pbase);
+        const unsigned par = unsigned(t) & 1u;
+        if (!pending0) load_set(fr[0], slot_in, 0);
+        // One pass of the loop below for row block i (parity BUF): request the partials of block i-1, the fragments of
+        // block i+1 and the cell operands of block i, multiply block i, send its partials, then finish block i-1.
+        auto pass = [&](int i, auto buf_tag) -> bool {
+            constexpr int BUF = decltype(buf_tag)::value;
+            const bool product = i < nrb, finish = i >= 1, more = i + 1 < nrb;
+            uintx4 in0 = {0u, 0u, 0u, 0u}, in1 = {0u, 0u, 0u, 0u};
+            // partials of block i-1: sender pj, row pr (byte offset into the ring)
+            const unsigned src = (pbase + unsigned(((((s * kKQ + q) * nrb + max(i - 1, 0)) * kKQ + pj) * RB + min(pr, RB - 1)) * 8)) * 4u;
+            if (finish) {
+                in0 = __builtin_amdgcn_raw_buffer_load_b128(rp, src, 0, kDeviceScope);
+                in1 = __builtin_amdgcn_raw_buffer_load_b128(rp, src + 16u, 0, kDeviceScope);
+                order_here();
+            }
+            if (product) {
+                float* part = part_all + size_t(item & 1) * 4 * kRows * PLD;
+                if (more) load_set(fr[BUF ^ 1], slot_in, i + 1);
+                load_ops(t, i, og[BUF], ocp[BUF], occ[BUF], ody[BUF]);
+                // A word that still shows the pattern has not been written yet: fetch the block again.  (The first check
+                // stands outside the loop: the compiler then waits for exactly this set there, not for everything a
+                // path through the loop might have requested.)
+                auto stale = [&]() -> bool {
+                    unsigned mx = 0u;
+#pragma unroll
+                    for (int k = 0; k < KS; ++k)
+#pragma unroll
+                        for (int mm = 0; mm < MT; ++mm) {
+                            const uintx4 u = fr[BUF][k][mm];
+                            mx = max(mx, max(max(u.x, u.y), max(u.z, u.w)));
+                        }
+                    return __any(mx == kUnwritten) != 0;
+                };
+                if (stale()) {
+                    int spins = 0;
+                    long long spin_start = 0;
+                    do {
+                        if (spin_out(spins, spin_start)) break;
+                        order_here();
+                        load_set(fr[BUF], slot_in, i);
+                    } while (stale());
+                }
+                floatx4 acc[2][NT];
+#pragma unroll
+                for (int m = 0; m < 2; ++m)
+#pragma unroll
+                    for (int n = 0; n < NT; ++n) acc[m][n] = floatx4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int k = 0; k < KS; ++k)
+#pragma unroll
+                    for (int n = 0; n < NT; ++n)
+#pragma unroll
+                        for (int m = 0; m < MT; ++m)
+                            acc[m][n] = __builtin_amdgcn_mfma_f32_16x16x32_f16(wreg[k][n], __builtin_bit_cast(half8, fr[BUF][k][m]),
+                                                                               acc[m][n], 0, 0, 0);
+                clk.lap(0);
+                spill_partials<NT, MT>(part, acc, wave, lane, PLD);
+                ++item;
+                __syncthreads();
+                if (lds_abort != 0) return false;
+                if (row_used) {   // sum the four waves' k-slices and send 8 columns to workgroup pj of the slice
+                    floatx4 v0 = {0.f, 0.f, 0.f, 0.f}, v1 = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                    for (int w = 0; w < 4; ++w) {
+                        const float* src_l = part + (size_t(w) * kRows + pr) * PLD + 8 * pj;
+                        v0 += *reinterpret_cast<const floatx4*>(src_l);
+                        v1 += *reinterpret_cast<const floatx4*>(src_l + 4);
+                    }
+                    uintx4 u0 = __builtin_bit_cast(uintx4, v0), u1 = __builtin_bit_cast(uintx4, v1);
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        u0[e] = (u0[e] & ~1u) | par;
+                        u1[e] = (u1[e] & ~1u) | par;
+                    }
+                    float* dst = pslot + ((((size_t(s) * kKQ + pj) * nrb + i) * kKQ + q) * RB + pr) * 8;
+                    *reinterpret_cast<uintx4*>(dst) = u0;
+                    *reinterpret_cast<uintx4*>(dst + 4) = u1;
+                }
+                clk.lap(1);
+            } else if (nrb >= 2 && t - 1 >= t_last) {
+                // The first row block of the next step (dG_t, block 0: stored by everyone a pass ago or more) is requested
+                // while the last block of this step is being finished.  (With one row block per step everyone's dG_t is
+                // being stored right now: the request goes out after this workgroup's own cell update, below.)
+                load_set(fr[0], (t + 8) & (kDgSlots - 1), 0);
+            }
+            if (finish) {
+                auto tags_bad = [&]() -> bool {
+                    const unsigned all1 = in0.x & in0.y & in0.z & in0.w & in1.x & in1.y & in1.z & in1.w;
+                    const unsigned any1 = in0.x | in0.y | in0.z | in0.w | in1.x | in1.y | in1.z | in1.w;
+                    const bool ok = par ? ((all1 & 1u) != 0u) : ((any1 & 1u) == 0u);
+                    return __any(row_used && !ok) != 0;
+                };
+                if (tags_bad()) {
+                    int spins = 0;
+                    long long spin_start = 0;
+                    do {
+                        if (spin_out(spins, spin_start)) break;
+                        order_here();
+                        in0 = __builtin_amdgcn_raw_buffer_load_b128(rp, src, 0, kDeviceScope);
+                        in1 = __builtin_amdgcn_raw_buffer_load_b128(rp, src + 16u, 0, kDeviceScope);
+                        order_here();
+                    } while (tags_bad());
+                }
+                clk.lap(4);
+                // sum over the 8 senders (lanes that differ in their low three bits): lane pj keeps column pj
+                const floatx4 f0 = __builtin_bit_cast(floatx4, in0), f1 = __builtin_bit_cast(floatx4, in1);
+                float a4[4], a2[2];
+                {
+                    const bool hi = (lane & 4) != 0;
+#pragma unroll
+                    for (int k = 0; k < 4; ++k) {
+                        const float keep = hi ? f1[k] : f0[k], send = hi ? f0[k] : f1[k];
+                        a4[k] = keep + __shfl_xor(send, 4);
+                    }
+                }
+                {
+                    const bool hi = (lane & 2) != 0;
+#pragma unroll
+                    for (int k = 0; k < 2; ++k) {
+                        const float keep = hi ? a4[2 + k] : a4[k], send = hi ? a4[k] : a4[2 + k];
+                        a2[k] = keep + __shfl_xor(send, 2);
+                    }
+                }
+                const bool hi = (lane & 1) != 0;
+                const float dh = (hi ? a2[1] : a2[0]) + __shfl_xor(hi ? a2[0] : a2[1], 1);
+                cell(t, i - 1, dh, og[BUF ^ 1], ocp[BUF ^ 1], occ[BUF ^ 1], ody[BUF ^ 1]);
+            }
+            return true;
+        };
+        for (int i = 0; i <= nrb; i += 2) {
+            if (!pass(i, std::integral_constant<int, 0>{})) return;
+            if (i + 1 <= nrb && !pass(i + 1, std::integral_constant<int, 1>{})) return;
+        }
+        pending0 = (t - 1 >= t_last);
+        if (pending0 && nrb == 1) load_set(fr[0], (t + 8) & (kDgSlots - 1), 0);
+    }
+    clk.flush();
+    if (t_last >= 0) {   // a launch that stops before the closing pass leaves dc in memory for the next one
+        for (int rb = 0; rb < nrb; ++rb) {
+            const int b = rb * RB + pr;
+            if (row_used && b < p.B) p.dC[size_t(b) * p.Hp + j] = dcl[rb * kThreads + tid];
+        }
+    }
+    // Bias gradient: fold this launch's sums over the 32 rows (fixed order).
+    __syncthreads();
+    float* red = part_all;   // [256][4]
+#pragma unroll
+    for (int gt = 0; gt < 4; ++gt) red[tid * 4 + gt] = dbacc[gt];
+    __syncthreads();
+    if (tid < 32) {
+        const int uj = tid / 4, gt = tid % 4;
+        float sum = 0.f;
+        for (int r = 0; r < kThreads / 8; ++r) sum += red[(r * 8 + uj) * 4 + gt];
+        p.db_part[size_t(4) * (s * 64 + q * 8 + uj) + gt] += sum;
+    }
+}
+
 // rows x cols row-major (ld) -> fragment-major exchange layout (one thread per pair of halfs)
 __global__ void to_exchange_layout_kernel(const half_t* __restrict__ in, int rows, int cols, size_t ld,
                                           half_t* __restrict__ out, int nks) {
@@ -1107,7 +1476,7 @@ RecLayout plan_rec_fwd(int B, int Hp, int num_cus, bool force_stepwise, int forc
     return L;
 }
 
-RecLayout plan_rec_bwd(int B, int Hp, int num_cus, bool force_stepwise, int force_mt) {
+RecLayout plan_rec_bwd(int B, int Hp, int num_cus, bool force_stepwise, int force_mt, int two_d) {
     RecLayout L{};
     bool fits = true;
     if (Hp <= 1024) L.nt = 2;
@@ -1115,7 +1484,38 @@ RecLayout plan_rec_bwd(int B, int Hp, int num_cus, bool force_stepwise, int forc
     else { L.nt = 2; fits = false; }
     L.jb = 16 * L.nt;
     finish_layout(L, B, Hp, num_cus, force_stepwise, fits, force_mt);
+    if (two_d > 0 && L.persistent && rec_bwd_two_d_possible(Hp, num_cus)) {
+        const int mt = (B <= 16 && force_mt != 2) ? 1 : 2;
+        const int nrb = int(ceil_div(size_t(B), size_t(16 * mt)));
+        // Every workgroup walks all row blocks (its running dc for them sits in LDS: at most 8).  Measured on MI355X
+        // the two-way split wins where a step is one row block (batches up to 32 rows: 4.0 against 6.5 us per step at
+        // 16 rows) and only ties with the one-way layout at four (13.4 us either way at 128 rows: what it saves on
+        // the fetch it spends on the second exchange, every row block paying both in turn), so it is chosen by itself
+        // only for one row block; two_d = 2 forces it wherever it can run.
+        if (nrb <= (two_d >= 2 ? 8 : 1)) {
+            L.two_d = 1;
+            L.mt = mt;
+            L.nrb = nrb;
+            L.ng = 1;
+            L.xcd_local = 0;
+            L.gpx = 0;
+            L.grid = 256;
+        }
+    }
     return L;
+}
+
+bool rec_bwd_two_d_possible(int Hp, int num_cus) { return Hp == 2048 && num_cus == 256; }
+int rec_bwd_dg_slots(const RecLayout& L) { return L.two_d ? kDgSlots : 4; }
+size_t rec_bwd_part_slot_floats(const RecLayout& L) {
+    return L.two_d ? size_t(256) * L.nrb * kKQ * (16 * L.mt) * 8 : 0;
+}
+size_t rec_bwd_two_d_wfrag_bytes(int Hp) { return size_t(Hp) * 4 * Hp * sizeof(half_t); }
+unsigned rec_bwd_part_fill(int slot, int T) {
+    // the first product step of a pass is T-2; going down from there, the first step that lands in `slot`
+    for (int t = T - 2; t >= -1 && t > T - 2 - kRecBwdPartSlots; --t)
+        if ((t + 3) % kRecBwdPartSlots == slot) return (unsigned(t) & 1u) ^ 1u;
+    return 0u;
 }
 
 void StepGraphCache::clear() {
@@ -1232,9 +1632,25 @@ static hipError_t run_bwd(const RecLayout& L, const RecBwdArgs& a, hipStream_t s
                         });
 }
 
+template <int MT>
+static hipError_t run_bwd2d(const RecLayout& L, const RecBwdArgs& a, hipStream_t stream) {
+    auto kernel = rec_bwd2d_kernel<MT>;
+    const size_t lds = (size_t(2) * 4 * kRows * (64 + kPartPad) + size_t(L.nrb) * kThreads) * sizeof(float);
+    hipError_t e = raise_lds(kernel, lds);
+    if (e != hipSuccess) return e;
+    return launch_persistent(kernel, L.grid, lds, stream, a, L, a.t_hi, a.t_lo, 0);
+}
+
 hipError_t launch_rec_bwd(const RecLayout& L, const RecBwdArgs& a, hipStream_t stream, StepGraphCache* graphs) {
     if (a.T <= 0 || a.B <= 0 || a.t_hi < a.t_lo) return hipSuccess;
     if (a.Hp % 32 != 0 || a.Hp % L.jb != 0 || a.t_lo < -1 || a.t_hi >= a.T) return hipErrorInvalidValue;
+    if (L.two_d) {
+        // what the kernel's indexing assumes
+        if (!L.persistent || a.Hp != 2048 || L.grid != 256 || L.nrb < 1 || L.nrb > 8 || !a.wfrag2 || !a.P ||
+            L.nrb * 16 * L.mt < a.B || a.p_slot != rec_bwd_part_slot_floats(L))
+            return hipErrorInvalidValue;
+        return L.mt == 1 ? run_bwd2d<1>(L, a, stream) : run_bwd2d<2>(L, a, stream);
+    }
     if (!L.resident) return run_bwd<2, 1, false, 0, 2>(L, a, stream, graphs);
     if (L.nt == 2) return L.mt == 1 ? run_bwd<2, 32, true, 8, 1>(L, a, stream, graphs) : run_bwd<2, 32, true, 8, 2>(L, a, stream, graphs);
     if (L.nt == 1) return L.mt == 1 ? run_bwd<1, 64, true, 24, 1>(L, a, stream, graphs) : run_bwd<1, 64, true, 24, 2>(L, a, stream, graphs);

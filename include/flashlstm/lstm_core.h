@@ -43,7 +43,8 @@ int flstm_core_destroy(flstm_core_plan* plan);
 /* Options: "stepwise" (1 = one launch per time step instead of the persistent kernels),
  * "proj_chunk" (time steps per input-projection GEMM, <=0 = whole sequence; results do not depend
  * on it), "spin_limit" / "spin_ms" (reloads of a not-yet-written operand, and milliseconds spent on them, before a
- * waiting workgroup of a persistent launch gives up; default 2^30 reloads / 250 ms), "dw_splits" (split-K slices of
+ * waiting workgroup of a persistent launch gives up; default 2^30 reloads / 250 ms; 0 reloads = give up at the first
+ * operand found unwritten), "dw_splits" (split-K slices of
  * the weight-gradient GEMM, 0 = automatic), "accumulate_grads" (1 = the backward pass adds dW_ih, dW_hh, db_ih
  * and db_hh to what the caller's buffers hold instead of overwriting them: a sequence processed as several
  * consecutive segments, last segment first, each segment's dh0 / dc0 fed to the next call as d_hn / d_cn),
@@ -54,6 +55,10 @@ int flstm_core_destroy(flstm_core_plan* plan);
  * "step_graphs" (1, the default: where a pass runs as one launch per time step -- weights that do not fit on chip, a
  * demoted direction, "stepwise" -- the launches of a range of steps are captured into a hipGraph on first use and
  * replayed afterwards, when the stream allows capture; 0 = plain launches; FLASHLSTM_STEP_GRAPHS sets the default),
+ * "bwd_two_d" (backward recurrence at 2048 padded hidden units on a 256-CU device: the layout that splits the product
+ * over output columns and over the contraction and sums partial products through a second ring; 0 = never, 1 = where
+ * it is the faster layout (batches of at most 32 rows), 2 = wherever it can run (at most 256 rows); default 1,
+ * FLASHLSTM_BWD_TWO_D sets the default),
  * "inject_stall" (test hook: the next N passes that use a persistent kernel are treated as if that launch had
  * given up, which exercises the step-wise repeat and the demotion rule without making any kernel wait). */
 int flstm_core_set_option(flstm_core_plan* plan, const char* name, long value);

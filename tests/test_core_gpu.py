@@ -32,7 +32,7 @@ def run_core(p, *, half=True, stepwise=False, proj_chunk=0, grad_scale=1.0, stat
     torch.cuda.synchronize()
     out = dict(y=to_np(y), hn=to_np(hy), cn=to_np(cy), dx=to_np(dx), dw_ih=to_np(dW_ih), dw_hh=to_np(dW_hh),
                db=to_np(db), dh0=to_np(dh0), dc0=to_np(dc0))
-    info = {k: core.info(k) for k in ("persistent_fwd", "persistent_bwd", "xcd_local_fwd", "fallbacks")}
+    info = {k: core.info(k) for k in ("persistent_fwd", "persistent_bwd", "xcd_local_fwd", "fallbacks", "bwd_two_d")}
     if own:
         core.close()
     return out, info
@@ -110,8 +110,46 @@ def test_persistent_and_stepwise_agree(shape):
     assert ia["persistent_fwd"] == 1 and ib["persistent_fwd"] == 0
     for k in ("y", "hn", "cn"):
         np.testing.assert_array_equal(a[k], b[k])       # same arithmetic, same order
+    # the backward kernels sum a product in the same order either way -- except the persistent kernel for 2048 hidden
+    # units, which splits the contraction over eight workgroups (other fp32 summation order, then fp16 rounding of dG)
+    tol = 2e-4 if ia["bwd_two_d"] == 1 else 1e-5
+    assert ib["bwd_two_d"] == 0
     for k in ("dx", "dh0", "dc0", "dw_hh", "db"):
-        assert rell2(a[k], b[k]) < 1e-5, k
+        assert rell2(a[k], b[k]) < tol, k
+
+
+@pytest.mark.parametrize("shape", [(7, 256, 32, 2048), (6, 40, 32, 2048), (9, 5, 64, 2040), (4, 17, 32, 2048),
+                                   (1, 16, 32, 2048), (2, 33, 32, 2017)])
+def test_two_way_split_backward_for_2048_units(shape):
+    # 2048 (padded) hidden units: the persistent backward kernel splits its product over column slices AND over the
+    # contraction, and sums the partial products through a second ring.  One to eight row blocks, ragged batches,
+    # padded hidden sizes, a single step; against torch, against the one-way layout, and through the give-up path.
+    from flashlstm_poc_amd import LstmCore
+    T, B, I, H = shape
+    p = make_problem(*shape, seed=11)
+    ref = torch_reference(p, dtype=torch.float32, device="cuda")
+    core = LstmCore(B, I, H)
+    core.pack(*(p[k].cuda() for k in ("w_ih", "w_hh", "b_ih", "b_hh")))
+    assert core.info("bwd_two_d") == (1 if B <= 32 else 0)   # by itself the plan takes it for one row block per step
+    core.set_option("bwd_two_d", 2)                           # here: wherever it can run
+    got, info = run_core(p, core=core)
+    assert info["persistent_bwd"] == 1 and info["bwd_two_d"] == 1 and info["fallbacks"] == 0
+    check_against(ref, got, label=f"two-way {shape}")
+    again, _ = run_core(p, core=core)
+    for k in got:
+        np.testing.assert_array_equal(again[k], got[k], err_msg=k)   # fixed summation order: run-to-run identical
+    core.set_option("bwd_two_d", 0)
+    one_way, info1 = run_core(p, core=core)
+    assert info1["persistent_bwd"] == 1 and info1["bwd_two_d"] == 0
+    for k in ("dx", "dh0", "dc0", "dw_ih", "dw_hh", "db"):
+        assert rell2(got[k], one_way[k]) < 2e-4, k
+    core.set_option("bwd_two_d", 2)
+    core.set_option("spin_limit", 0)   # the first operand found unwritten makes the launch give up; the pass is repeated step-wise
+    repaired, info2 = run_core(p, core=core)
+    if T > 1 and B <= 32:   # one row block per step: the next step's operand is always requested before it is complete
+        assert info2["fallbacks"] >= 1
+    check_against(ref, repaired, label=f"two-way, repaired {shape}")
+    core.close()
 
 
 def test_retry_limit_hit_is_repaired_by_stepwise_pass():

@@ -128,7 +128,8 @@ def test_backward_without_device_cache_recomputes_the_forward_pass():
         np.testing.assert_array_equal(a[k], b[k], err_msg=k)
 
 
-@pytest.mark.parametrize("shape", [(10, 3, 12, 20), (70, 5, 16, 24), (37, 40, 64, 256), (9, 1, 3, 5), (33, 2, 63, 257)])
+@pytest.mark.parametrize("shape", [(10, 3, 12, 20), (70, 5, 16, 24), (37, 40, 64, 256), (9, 1, 3, 5), (33, 2, 63, 257),
+                                   (7, 20, 32, 2048)])
 def test_chunked_streaming_gives_the_whole_sequence_results(shape, monkeypatch):
     # FLASHLSTM_V2_CHUNK_STEPS cuts the sequence into chunks that are uploaded, processed and downloaded on the three
     # streams (counterpart of the 32-step pipeline of lstm_forward.cu:646-940); the arithmetic must not depend on it
