@@ -246,8 +246,8 @@ def bench_stack(args, device):
 
     def step():
         y, _, _ = stack.forward(x)
-        dy = (y.float() - target.float()).mul_(2.0 / y.numel())
-        _, grads, _, _ = stack.backward(dy, want_dx=False)   # loss scale: automatic (a power of two from the largest |dy|)
+        # d/dy of mean((y - target)^2); loss scale: automatic (a power of two from the largest |dy|)
+        _, grads, _, _ = stack.backward_mse(y, target, want_dx=False)
         last["y"], last["grads"] = y, grads
 
     for _ in range(args.warmup):

@@ -48,8 +48,10 @@ class LstmStack:
         return cur, hys, cys
 
     def backward(self, dy_top, *, loss_scale="auto", d_hn: Optional[Sequence] = None,
-                 d_cn: Optional[Sequence] = None, want_dx: bool = True):
-        """dy_top (T,B,H): gradient wrt the top layer's outputs.  loss_scale (a power of two) multiplies it before
+                 d_cn: Optional[Sequence] = None, want_dx: bool = True, dy_factor: float = 1.0):
+        """dy_top (T,B,H): gradient wrt the top layer's outputs, times 1 / dy_factor: the gradient is dy_factor * dy_top
+        (a loss that averages over many elements has a gradient of the form tiny_constant * tensor_of_order_one; handing
+        the two over apart keeps the tensor in fp16 range and saves the fp32 passes that would form their product).  loss_scale (a power of two) multiplies it before
         it is rounded to fp16 and stays on every inter-layer gradient, so that small gradients survive the fp16
         hand-over between layers; it is divided out of everything returned.  "auto" (the default) picks the power
         of two that brings the largest |dy_top| to about 64: far enough from the fp16 maximum (65504) for the
@@ -65,12 +67,17 @@ class LstmStack:
         if isinstance(loss_scale, str):
             if loss_scale != "auto":
                 raise ValueError("loss_scale must be a positive number or 'auto'")
-            amax = float(dy_top.abs().max())
+            lo, hi = torch.aminmax(dy_top)
+            amax = max(-float(lo), float(hi)) * abs(float(dy_factor))
             S = 2.0 ** min(60, max(-14, math.floor(math.log2(64.0 / amax)))) if 0.0 < amax < float("inf") else 1.0
         else:
             S = float(loss_scale) if loss_scale and loss_scale > 0 else 1.0
         self.last_loss_scale = S
-        cur = (dy_top.float() * S).half() if S != 1.0 else dy_top.half()
+        k = S * float(dy_factor)
+        if dy_top.dtype == torch.float16:
+            cur = dy_top * k if k != 1.0 else dy_top     # one pass: the product is formed in fp32 and rounded once
+        else:
+            cur = (dy_top.float() * k).half()
         grads: List = [None] * self.L
         dh0s: List = [None] * self.L
         dc0s: List = [None] * self.L
@@ -89,6 +96,14 @@ class LstmStack:
         if cur is not None and S != 1.0:
             cur = cur.float() * (1.0 / S)   # fp32: the unscaled values may lie below the fp16 range
         return cur, grads, dh0s, dc0s
+
+    def backward_mse(self, y_top, target, **kwargs):
+        """backward() for the loss mean((y_top - target)^2) over all elements: its gradient 2 / N * (y_top - target) is
+        handed over as the fp16 difference and the factor 2 / N (see dy_factor).  y_top: what forward() returned."""
+        import torch
+        if y_top.dtype != torch.float16 or target.dtype != torch.float16:
+            return self.backward((y_top.float() - target.float()), dy_factor=2.0 / y_top.numel(), **kwargs)
+        return self.backward(torch.sub(y_top, target), dy_factor=2.0 / y_top.numel(), **kwargs)
 
 
 class _StackFunction(torch.autograd.Function):

@@ -10,7 +10,7 @@ from helpers import SafeTorchLstm, rell2, relmax, to_np
 pytestmark = pytest.mark.gpu
 
 
-def _run(T, B, I, H, L, loss_scale, seed=5, safe_reference=False, max_rows=131072):
+def _run(T, B, I, H, L, loss_scale, seed=5, safe_reference=False, max_rows=131072, mse_helper=False):
     """Our stack first (forward, MSE gradient, backward), then -- after its device memory has been given back -- the
     fp32 reference on the same inputs: nn.LSTM(num_layers=L) itself, or (safe_reference) the same function built
     from nn.LSTM calls of bounded size, helpers.SafeTorchLstm.  Returns the error of every output and gradient."""
@@ -23,14 +23,19 @@ def _run(T, B, I, H, L, loss_scale, seed=5, safe_reference=False, max_rows=13107
                 prm.copy_(prm.half().float())
     x = torch.randn(T, B, I, device="cuda").half()
     target = torch.randn(T, B, H, device="cuda")
+    if mse_helper:
+        target = target.half().float()   # the helper takes an fp16 target: give the reference the same values
     stack = LstmStack(B, I, H, L)
     stack.pack([tuple(getattr(ref, f"{n}_l{l}").detach() for n in ("weight_ih", "weight_hh", "bias_ih", "bias_hh"))
                 for l in range(L)])
     y, hys, cys = stack.forward(x)
     # MSE(y_top, target): d loss / d y = 2 (y - target) / numel
-    dy = 2.0 * (y.float() - target) / y.numel()
-    dx, grads, dh0s, dc0s = stack.backward(dy, loss_scale=loss_scale)
-    del dy
+    if mse_helper:   # the same gradient handed over as fp16 difference and factor 2 / numel
+        dx, grads, dh0s, dc0s = stack.backward_mse(y, target.half(), loss_scale=loss_scale)
+    else:
+        dy = 2.0 * (y.float() - target) / y.numel()
+        dx, grads, dh0s, dc0s = stack.backward(dy, loss_scale=loss_scale)
+        del dy
     stack.close()
     torch.cuda.empty_cache()
 
@@ -88,6 +93,12 @@ def test_loss_scale_is_what_keeps_small_gradients():
     auto = _run(12, 5, 16, 24, 3, loss_scale="auto")
     assert max(scaled.values()) <= 1e-2 and max(auto.values()) <= 1e-2
     assert max(errs.values()) > max(scaled.values())   # unscaled: fp16 underflow costs accuracy
+
+
+def test_mse_helper_gives_the_gradients_of_the_mse_loss():
+    a = _run(12, 5, 16, 24, 3, loss_scale="auto", mse_helper=True)
+    b = _run(33, 40, 64, 256, 2, loss_scale="auto", mse_helper=True)
+    assert max(a.values()) <= 1e-2 and max(b.values()) <= 1e-2, (a, b)
 
 
 def test_config5_stack_full_size_against_fp32_torch_lstm():
