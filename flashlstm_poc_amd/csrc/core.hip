@@ -364,7 +364,7 @@ extern "C" int flstm_core_pack_weights(flstm_core_plan* p, const float* w_ih, co
     FL_TRY(p->wfrag_f.reserve(size_t(p->Lf.nh) * 4 * p->ks_f * p->Lf.nt * kWave * sizeof(half8)));
     FL_TRY(p->wfrag_b.reserve(size_t(p->Lb.nh) * 4 * p->ks_b * p->Lb.nt * kWave * sizeof(half8)));
     FL_TRY(pack_weights(d, w_ih, w_hh, p->wih_p.as<half_t>(), p->wih_t.as<half_t>(), p->wfrag_f.as<half8>(),
-                        p->ks_f, p->Lf.nt, p->wfrag_b.as<half8>(), p->ks_b, p->Lb.nt, s));
+                        p->ks_f, p->Lf.nt, p->Lf.rot_div, p->wfrag_b.as<half8>(), p->ks_b, p->Lb.nt, p->Lb.rot_div, s));
     if (rec_bwd_two_d_possible(d.Hp, p->num_cus)) {   // whether or not the current layout uses them
         FL_TRY(p->wfrag_b2.reserve(rec_bwd_two_d_wfrag_bytes(d.Hp)));
         FL_TRY(pack_wfrag_bwd2d(d, w_hh, p->wfrag_b2.as<half8>(), s));

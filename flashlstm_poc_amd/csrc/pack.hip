@@ -1,6 +1,7 @@
 // Layout kernels: weight packing, padded dtype conversion, transposes and output reductions.
 // All are pure HBM-bandwidth work; each thread moves a few elements with coalesced accesses.
 #include "pack.h"
+#include "recurrent.h"
 
 namespace flstm_hip {
 namespace {
@@ -36,7 +37,7 @@ __global__ void pack_wih_kernel(Dims d, const float* __restrict__ w_ih, half_t* 
 // fragment (hs, wave, ks, n): lane l holds column c = n*16 + l%16 of slice hs,
 // k = (ks*4 + wave)*32 + 8*(l/16) + e, e = 0..7.
 __global__ void pack_wfrag_fwd_kernel(Dims d, const float* __restrict__ w_hh, half_t* __restrict__ out,
-                                      int ks_wave, int nt) {
+                                      int ks_wave, int nt, int rot_div) {
     const size_t idx = size_t(blockIdx.x) * kT + threadIdx.x;  // one half element
     const int nh = d.Hp / (4 * nt);
     const size_t total = size_t(nh) * 4 * ks_wave * nt * kWave * 8;
@@ -50,7 +51,9 @@ __global__ void pack_wfrag_fwd_kernel(Dims d, const float* __restrict__ w_hh, ha
     const int hs = int(r);
     const int jb = 4 * nt, c = n * 16 + lane % 16;
     const int gate = c / jb, unit = hs * jb + c % jb;
-    const int k = (ks * 4 + wave) * 32 + 8 * (lane / 16) + e;
+    // (slot ks of slice hs holds a rotated k-step: recurrent.h, rec_kstep_rotation)
+    const int kstep = rec_kstep_of_slot(ks, rec_kstep_rotation(hs, nh, ks_wave, rot_div), ks_wave);
+    const int k = (kstep * 4 + wave) * 32 + 8 * (lane / 16) + e;
     out[idx] = (half_t)((unit < d.H && k < d.H) ? w_hh[size_t(gate * d.H + unit) * d.H + k] : 0.f);
 }
 
@@ -58,7 +61,7 @@ __global__ void pack_wfrag_fwd_kernel(Dims d, const float* __restrict__ w_hh, ha
 // fragment (hs, wave, ks, n): lane l holds output column k = hs*16*NT + n*16 + l%16,
 // contraction index q = (ks*4 + wave)*32 + 8*(l/16) + e.
 __global__ void pack_wfrag_bwd_kernel(Dims d, const float* __restrict__ w_hh, half_t* __restrict__ out,
-                                      int ks_wave, int nt) {
+                                      int ks_wave, int nt, int rot_div) {
     const size_t idx = size_t(blockIdx.x) * kT + threadIdx.x;
     const int nh = d.Hp / (16 * nt);
     const size_t total = size_t(nh) * 4 * ks_wave * nt * kWave * 8;
@@ -71,7 +74,8 @@ __global__ void pack_wfrag_bwd_kernel(Dims d, const float* __restrict__ w_hh, ha
     const int wave = int(r % 4); r /= 4;
     const int hs = int(r);
     const int k = hs * 16 * nt + n * 16 + lane % 16;
-    const int q = (ks * 4 + wave) * 32 + 8 * (lane / 16) + e;
+    const int kstep = rec_kstep_of_slot(ks, rec_kstep_rotation(hs, nh, ks_wave, rot_div), ks_wave);
+    const int q = (kstep * 4 + wave) * 32 + 8 * (lane / 16) + e;
     float v = 0.f;
     if (q < 4 * d.Hp && k < d.H) {
         const int row = torch_row(q, d.H);
@@ -215,16 +219,16 @@ __global__ void fill_words_kernel(unsigned* p, size_t words, unsigned value) {
 }  // namespace
 
 hipError_t pack_weights(const Dims& d, const float* w_ih, const float* w_hh, half_t* wih_p, half_t* wih_t,
-                        half8* wfrag_fwd, int ks_fwd, int nt_fwd, half8* wfrag_bwd, int ks_bwd, int nt_bwd,
-                        hipStream_t s) {
+                        half8* wfrag_fwd, int ks_fwd, int nt_fwd, int rot_div_fwd, half8* wfrag_bwd, int ks_bwd,
+                        int nt_bwd, int rot_div_bwd, hipStream_t s) {
     const size_t n1 = size_t(4) * d.Hp * d.Ip;
     hipLaunchKernelGGL(pack_wih_kernel, dim3(grid_for(n1)), dim3(kT), 0, s, d, w_ih, wih_p, wih_t);
     const size_t n2 = size_t(d.Hp / (4 * nt_fwd)) * 4 * ks_fwd * nt_fwd * kWave * 8;
     hipLaunchKernelGGL(pack_wfrag_fwd_kernel, dim3(grid_for(n2)), dim3(kT), 0, s, d, w_hh,
-                       reinterpret_cast<half_t*>(wfrag_fwd), ks_fwd, nt_fwd);
+                       reinterpret_cast<half_t*>(wfrag_fwd), ks_fwd, nt_fwd, rot_div_fwd);
     const size_t n3 = size_t(d.Hp / (16 * nt_bwd)) * 4 * ks_bwd * nt_bwd * kWave * 8;
     hipLaunchKernelGGL(pack_wfrag_bwd_kernel, dim3(grid_for(n3)), dim3(kT), 0, s, d, w_hh,
-                       reinterpret_cast<half_t*>(wfrag_bwd), ks_bwd, nt_bwd);
+                       reinterpret_cast<half_t*>(wfrag_bwd), ks_bwd, nt_bwd, rot_div_bwd);
     return hipGetLastError();
 }
 

@@ -21,6 +21,7 @@ struct RecLayout {
     int resident;    // 1: weight fragments live in registers for the whole launch
     int grid;        // workgroups per launch
     int cooperative; // host side: 1 = persistent launches go through hipLaunchCooperativeKernel (set by the plan)
+    int rot_div;     // k-step rotation (rec_kstep_rotation): slices rot_div apart run on the same XCD
     int two_d;       // backward, 2048 hidden units: workgroups split the product over output columns AND the contraction
                      // (32 column slices x 8 contraction slices, partial sums exchanged inside an XCD); nt, jb, nh
                      // still describe the one-dimensional layout, whose weight fragments the step-wise fallback uses
@@ -74,6 +75,25 @@ struct RecBwdArgs {
     long long spin_ticks;
     long long* prof;     // optional [8] cycle counters of workgroup 0 per phase (null = off)
 };
+
+// Which k-step a wave's register slot holds.  The workgroups of one XCD that belong to the same group fetch the same
+// exchanged operand every step, and walking its k-steps in the same order they ask for the same lines at the same
+// moment.  Where that operand is large and comes through memory from the other XCDs, spreading the requests pays
+// (rot_div > 0; 0 = no rotation): slice `hs` starts `rotation` k-steps further on and wraps round: slot ks of a wave holds the weights of (and fetches) k-step
+// 4 * ((ks + rotation) % ks_wave) + wave.  Slices that share an XCD are `rot_div` apart (1 where a group sits inside
+// one XCD, 8 where the workgroups of a group are dealt round-robin over the 8 XCDs), and their rotations are spread
+// evenly over the ks_wave positions.  The weight packing and the kernels use the same function.
+__host__ __device__ inline int rec_kstep_rotation(int hs, int nh, int ks_wave, int rot_div) {
+    if (ks_wave <= 1 || rot_div <= 0) return 0;
+    const int mates = nh / rot_div > 0 ? nh / rot_div : 1;   // slices of a group on one XCD
+    const int r = hs / rot_div;
+    return (ks_wave >= mates ? r * (ks_wave / mates) : r) % ks_wave;
+}
+__host__ __device__ inline int rec_kstep_of_slot(int ks, int rotation, int ks_wave) {
+    if (ks >= ks_wave) return ks;   // slots past the real contraction hold zero weights
+    const int k = ks + rotation;
+    return k >= ks_wave ? k - ks_wave : k;
+}
 
 // Step-wise launches as hipGraphs.  Where the persistent kernels cannot be used (weights that do not fit on chip,
 // a plan demoted after a give-up, "stepwise" forced) a pass is one launch per time step; the launches of a range of

@@ -172,7 +172,8 @@ __device__ __forceinline__ void wait_frags(half8 (&a)[8]) {
 template <int NT, int KS, int KL, int NPF, int NBUF, typename Prefetch>
 __device__ __forceinline__ void wave_product_tiles(floatx4 (&acc)[2][NT], const half8 (&wreg)[KS - KL][NT],
                                                    const half8* wlds, const half_t* a0, const half_t* a1, int wave,
-                                                   int lane, int nks_total, const Poll& poll, Prefetch&& prefetch) {
+                                                   int lane, int nks_total, int ks_wave, int rotation, const Poll& poll,
+                                                   Prefetch&& prefetch) {
     static_assert(KS % 8 == 0, "whole chunks");
     constexpr int CKT = (KS >= 16) ? 8 : 4;
     constexpr int NCHK = KS / CKT;      // chunks per tile
@@ -183,7 +184,7 @@ __device__ __forceinline__ void wave_product_tiles(floatx4 (&acc)[2][NT], const 
         const half_t* base = (c / NCHK) ? a1 : a0;
 #pragma unroll
         for (int k = 0; k < CKT; ++k) {
-            const int kg = min(((c % NCHK) * CKT + k) * 4 + wave, nks_total - 1);
+            const int kg = min(rec_kstep_of_slot((c % NCHK) * CKT + k, rotation, ks_wave) * 4 + wave, nks_total - 1);
             ld_frag_async(f[c % NBUF][k], base + size_t(kg) * 512);
         }
     };
@@ -261,7 +262,7 @@ template <int NT, int KS, bool RESIDENT, int KL, int NPF, int MT, typename Prefe
 __device__ __forceinline__ void wave_product(floatx4 (&acc)[2][NT], const half8 (&wreg)[KS - KL][NT],
                                              const half8* wlds, const half8* wfrag_wave, const half_t* a0,
                                              const half_t* a1, int wave, int lane, int nks_total,
-                                             int ks_wave, const Poll& poll, Prefetch&& prefetch) {
+                                             int ks_wave, int rotation, const Poll& poll, Prefetch&& prefetch) {
     if constexpr (RESIDENT && (KS % 8 == 0)) {
         // Loads and MFMAs are unconditional: k-steps beyond the real contraction length fetch a
         // clamped (finite) address and meet all-zero weight fragments.  Chunks of CK k-steps (2*CK
@@ -273,7 +274,7 @@ __device__ __forceinline__ void wave_product(floatx4 (&acc)[2][NT], const half8 
         auto issue = [&](int c, int buf) {
 #pragma unroll
             for (int k = 0; k < CK; ++k) {
-                const int kg = min((c * CK + k) * 4 + wave, nks_total - 1);
+                const int kg = min(rec_kstep_of_slot(c * CK + k, rotation, ks_wave) * 4 + wave, nks_total - 1);
                 ld_frag_async(fa[buf][k], a0 + size_t(kg) * 512);
                 if constexpr (MT == 2) ld_frag_async(fb[buf][k], a1 + size_t(kg) * 512);
             }
@@ -350,8 +351,8 @@ __device__ __forceinline__ void wave_product(floatx4 (&acc)[2][NT], const half8 
         }
     } else {
         for (int k = 0; k < ks_wave; ++k) {
-            const int kg = k * 4 + wave;
-            if (kg >= nks_total) break;
+            const int kg = rec_kstep_of_slot(k, rotation, ks_wave) * 4 + wave;
+            if (kg >= nks_total) continue;
             const half8 fa = ld_frag(a0 + size_t(kg) * 512);
             half8 fb{};
             if constexpr (MT == 2) fb = ld_frag(a1 + size_t(kg) * 512);
@@ -623,6 +624,7 @@ __global__ __launch_bounds__(kThreads) void rec_fwd_kernel(RecFwdArgs p, RecLayo
     if (!role.active) return;
     const int tid = threadIdx.x, wave = tid / kWave, lane = tid % kWave;
     const int hs = role.hs, g = role.g;
+    const int rotation = __builtin_amdgcn_readfirstlane(rec_kstep_rotation(hs, L.nh, ks_wave, L.rot_div));
     const int nks_total = p.Hp / 32;
     const bool device_scope = (L.persistent != 0) && (L.xcd_local == 0);
     const Poll poll{L.persistent != 0, p.spin_limit, p.spin_ticks, p.status, &lds_abort};
@@ -686,11 +688,11 @@ __global__ __launch_bounds__(kThreads) void rec_fwd_kernel(RecFwdArgs p, RecLayo
 #pragma unroll
                 for (int n = 0; n < NT; ++n) acc[m][n] = floatx4{0.f, 0.f, 0.f, 0.f};
             if constexpr (SPLIT)
-                wave_product_tiles<NT, KS, 0, NPH * UPT / 2, kFwdBufs>(acc, wreg, nullptr, a0, a1, wave, lane, nks_total, poll,
+                wave_product_tiles<NT, KS, 0, NPH * UPT / 2, kFwdBufs>(acc, wreg, nullptr, a0, a1, wave, lane, nks_total, ks_wave, rotation, poll,
                                                              [&]() { prefetch(t, rb); });
             else
                 wave_product<NT, KS, RESIDENT, 0, UPT / 2, MT>(acc, wreg, nullptr, wfrag_wave, a0, a1, wave, lane, nks_total,
-                                                               ks_wave, poll, [&]() { prefetch(t, rb); });
+                                                               ks_wave, rotation, poll, [&]() { prefetch(t, rb); });
             clk.lap(0);
             spill_partials<NT, MT>(part, acc, wave, lane, PLD);
             __syncthreads();
@@ -801,6 +803,7 @@ __global__ __launch_bounds__(kThreads) void rec_bwd_kernel(RecBwdArgs p, RecLayo
     if (!role.active) return;
     const int tid = threadIdx.x, wave = tid / kWave, lane = tid % kWave;
     const int hs = role.hs, g = role.g;
+    const int rotation = __builtin_amdgcn_readfirstlane(rec_kstep_rotation(hs, L.nh, ks_wave, L.rot_div));
     const int nks_total = p.Hp / 8;  // contraction over 4Hp packed gate columns
     const bool device_scope = (L.persistent != 0) && (L.xcd_local == 0);
     const Poll poll{L.persistent != 0, p.spin_limit, p.spin_ticks, p.status, &lds_abort};
@@ -879,7 +882,7 @@ __global__ __launch_bounds__(kThreads) void rec_bwd_kernel(RecBwdArgs p, RecLayo
 #pragma unroll
                     for (int n = 0; n < NT; ++n) acc[m][n] = floatx4{0.f, 0.f, 0.f, 0.f};
                 wave_product<NT, KS, RESIDENT, KL, NPF, MT>(acc, wreg, wlds, wfrag_wave, a0, a1, wave, lane, nks_total,
-                                                          ks_wave, poll, [&]() { prefetch(t, rb); });
+                                                          ks_wave, rotation, poll, [&]() { prefetch(t, rb); });
                 clk.lap(0);
                 spill_partials<NT, MT>(part, acc, wave, lane, PLD);
                 __syncthreads();
@@ -1436,6 +1439,7 @@ int rec_bwd_ks(const RecLayout&, int Hp) { return int(ceil_div(size_t(Hp) / 8, 4
 static void finish_layout(RecLayout& L, int B, int Hp, int num_cus, bool force_stepwise, bool fits, int force_mt) {
     L.nh = Hp / L.jb;
     L.resident = fits ? 1 : 0;
+    L.rot_div = 0;   // no k-step rotation (plan_rec_bwd turns it on where it pays)
     // Row blocks of 16 rows (one MFMA row tile) when all of them can run side by side: twice the workgroups
     // of 32-row blocks, each with half the product, fetch and cell-update work per step.
     const bool xcd_mode = (num_cus == 256 && L.nh <= 32);
@@ -1484,6 +1488,12 @@ RecLayout plan_rec_bwd(int B, int Hp, int num_cus, bool force_stepwise, int forc
     else { L.nt = 2; fits = false; }
     L.jb = 16 * L.nt;
     finish_layout(L, B, Hp, num_cus, force_stepwise, fits, force_mt);
+    // k-step rotation (recurrent.h): measured, it pays where a group spans the XCDs and a step fetches a lot -- the
+    // backward pass at 2048 hidden units, 13.4 -> 12.4 us per step at 128 rows -- and costs a little where the
+    // workgroups of an XCD read the same lines in step out of their own L2 (5.33 -> 5.42 us at 1024 units, where
+    // reading in step is what lets the L2 serve one line to many).  A function of the sizes alone: the packed
+    // weights depend on it.
+    L.rot_div = (L.nh > 32) ? 8 : 0;
     if (two_d > 0 && L.persistent && rec_bwd_two_d_possible(Hp, num_cus)) {
         const int mt = (B <= 16 && force_mt != 2) ? 1 : 2;
         const int nrb = int(ceil_div(size_t(B), size_t(16 * mt)));
