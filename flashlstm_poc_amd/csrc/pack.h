@@ -18,8 +18,9 @@ struct Dims {
 hipError_t pack_weights(const Dims& d, const float* w_ih, const float* w_hh, half_t* wih_p /*[4Hp][Ip]*/,
                         half_t* wih_t /*[Ip][4Hp]*/, half8* wfrag_fwd, int ks_fwd, int nt_fwd, int rot_div_fwd,
                         half8* wfrag_bwd, int ks_bwd, int nt_bwd, int rot_div_bwd, hipStream_t s);
-// W_hh in the layout of the backward recurrence that splits its product two ways (2048 padded hidden units only).
-hipError_t pack_wfrag_bwd2d(const Dims& d, const float* w_hh, half8* out, hipStream_t s);
+// W_hh in the layout of the backward recurrence that splits its product two ways (2048 padded hidden units only);
+// kq = 8 or 4 contraction slices.
+hipError_t pack_wfrag_bwd2d(const Dims& d, const float* w_hh, half8* out, int kq, hipStream_t s);
 hipError_t pack_bias(const Dims& d, const float* b_ih, const float* b_hh, float* bias_p, hipStream_t s);
 
 // rows x cols (ld_in, fp32 when in_f32 else fp16) -> fp16 [rows_out][ld_out], zero padded.

@@ -84,23 +84,24 @@ __global__ void pack_wfrag_bwd_kernel(Dims d, const float* __restrict__ w_hh, ha
     out[idx] = (half_t)v;
 }
 
-// Two-dimensional backward layout: [32 column slices s][8 contraction slices q][4 waves][8 k-steps][4 tiles][64 lanes][8]:
-// lane l of tile n holds column 64 s + 16 n + l % 16 of W_hh (hidden unit k of dh = dG * W_hh^T-packed) and the eight
-// packed gate rows 1024 q + 32 (4 ks + wave) + 8 (l / 16) .. +7.
-__global__ void pack_wfrag_bwd2d_kernel(Dims d, const float* __restrict__ w_hh, half_t* __restrict__ out) {
+// Two-dimensional backward layout: [32 column slices s][kq contraction slices q][4 waves][ks k-steps][4 tiles][64 lanes][8],
+// ks = 64 / kq: lane l of tile n holds column 64 s + 16 n + l % 16 of W_hh (hidden unit k of dh = dG * W_hh^T-packed) and
+// the eight packed gate rows (8192 / kq) q + 32 (4 ks + wave) + 8 (l / 16) .. +7.
+__global__ void pack_wfrag_bwd2d_kernel(Dims d, const float* __restrict__ w_hh, half_t* __restrict__ out, int kq) {
     const size_t idx = size_t(blockIdx.x) * kT + threadIdx.x;
     const size_t total = size_t(4) * d.Hp * d.Hp;
     if (idx >= total) return;
+    const int ksn = 64 / kq;
     size_t r = idx;
     const int e = int(r % 8); r /= 8;
     const int lane = int(r % kWave); r /= kWave;
     const int n = int(r % 4); r /= 4;
-    const int ks = int(r % 8); r /= 8;
+    const int ks = int(r % ksn); r /= ksn;
     const int wave = int(r % 4); r /= 4;
-    const int qs = int(r % 8); r /= 8;
+    const int qs = int(r % kq); r /= kq;
     const int sl = int(r);
     const int k = sl * 64 + n * 16 + lane % 16;
-    const int q = qs * 1024 + (ks * 4 + wave) * 32 + 8 * (lane / 16) + e;
+    const int q = qs * (8192 / kq) + (ks * 4 + wave) * 32 + 8 * (lane / 16) + e;
     float v = 0.f;
     if (q < 4 * d.Hp && k < d.H) {
         const int row = torch_row(q, d.H);
@@ -232,10 +233,10 @@ hipError_t pack_weights(const Dims& d, const float* w_ih, const float* w_hh, hal
     return hipGetLastError();
 }
 
-hipError_t pack_wfrag_bwd2d(const Dims& d, const float* w_hh, half8* out, hipStream_t s) {
-    if (d.Hp != 2048) return hipErrorInvalidValue;   // 32 slices of 64 columns, 8 slices of 1024 packed gate rows
+hipError_t pack_wfrag_bwd2d(const Dims& d, const float* w_hh, half8* out, int kq, hipStream_t s) {
+    if (d.Hp != 2048 || (kq != 4 && kq != 8)) return hipErrorInvalidValue;   // 32 slices of 64 columns, kq slices of 8192 / kq packed gate rows
     const size_t n = size_t(4) * d.Hp * d.Hp;
-    hipLaunchKernelGGL(pack_wfrag_bwd2d_kernel, dim3(grid_for(n)), dim3(kT), 0, s, d, w_hh, reinterpret_cast<half_t*>(out));
+    hipLaunchKernelGGL(pack_wfrag_bwd2d_kernel, dim3(grid_for(n)), dim3(kT), 0, s, d, w_hh, reinterpret_cast<half_t*>(out), kq);
     return hipGetLastError();
 }
 

@@ -23,8 +23,10 @@ struct RecLayout {
     int cooperative; // host side: 1 = persistent launches go through hipLaunchCooperativeKernel (set by the plan)
     int rot_div;     // k-step rotation (rec_kstep_rotation): slices rot_div apart run on the same XCD
     int two_d;       // backward, 2048 hidden units: workgroups split the product over output columns AND the contraction
-                     // (32 column slices x 8 contraction slices, partial sums exchanged inside an XCD); nt, jb, nh
+                     // (32 column slices x kq contraction slices, partial sums exchanged inside an XCD); nt, jb, nh
                      // still describe the one-dimensional layout, whose weight fragments the step-wise fallback uses
+    int kq;          // two_d: contraction slices, 8 (one group of 256 workgroups) or 4 (two groups of 128)
+    int nm;          // two_d: passes per step the kernel is built for (row blocks per workgroup, rounded up to 1, 2, 4)
 };
 
 struct RecFwdArgs {
@@ -57,7 +59,7 @@ struct RecBwdArgs {
                          // before the first step all four hold the 0xFFFF 'unwritten' pattern
                          // (two-dimensional layout: rec_bwd_dg_slots() = 8 slots, step t writes slot t%8)
     size_t x_slot;
-    const half8* wfrag2; // two-dimensional layout: [32 column slices][8 contraction slices][4 waves][8 k-steps][4 tiles][64]
+    const half8* wfrag2; // two-dimensional layout: [32 column slices][kq contraction slices][4 waves][64/kq k-steps][4 tiles][64]
     float* P;            // two-dimensional layout: ring of 3 slots of p_slot floats for the partial sums; before the first
                          // step the lowest bit of every word of slot (t+3)%3 is the opposite of t&1 for the first step t
                          // that uses the slot (rec_bwd_part_fill)
@@ -127,8 +129,11 @@ RecLayout plan_rec_fwd(int B, int Hp, int num_cus, bool force_stepwise, int forc
 RecLayout plan_rec_bwd(int B, int Hp, int num_cus, bool force_stepwise, int force_mt = 0, int two_d = 1);
 
 // The two-dimensional backward layout: whether a device/size can use it at all (decides whether its weight fragments
-// are packed), slots of its dG ring, floats per slot of its partial ring and bytes of its weight fragments.
+// are packed) and with how many contraction slices (a function of the sizes alone, so that the packed weights fit
+// whatever the options say later), slots of its dG ring, floats per slot of its partial ring and bytes of its weight
+// fragments.
 bool rec_bwd_two_d_possible(int Hp, int num_cus);
+int rec_bwd_two_d_kq(int B);
 int rec_bwd_dg_slots(const RecLayout& L);
 size_t rec_bwd_part_slot_floats(const RecLayout& L);
 constexpr int kRecBwdPartSlots = 3;

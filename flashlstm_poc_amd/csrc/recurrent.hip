@@ -157,6 +157,14 @@ __device__ __forceinline__ void wait_frags(half8 (&a)[2], half8 (&b)[2]) {
 }
 
 template <int N>
+__device__ __forceinline__ void wait_frags(half8 (&a)[8], half8 (&b)[8]) {
+    asm volatile("s_waitcnt vmcnt(%16)"
+                 : "+v"(a[0]), "+v"(a[1]), "+v"(a[2]), "+v"(a[3]), "+v"(a[4]), "+v"(a[5]), "+v"(a[6]), "+v"(a[7]), "+v"(b[0]),
+                   "+v"(b[1]), "+v"(b[2]), "+v"(b[3]), "+v"(b[4]), "+v"(b[5]), "+v"(b[6]), "+v"(b[7])
+                 : "n"(N)
+                 : "memory");
+}
+template <int N>
 __device__ __forceinline__ void wait_frags(half8 (&a)[8]) {
     asm volatile("s_waitcnt vmcnt(%8)"
                  : "+v"(a[0]), "+v"(a[1]), "+v"(a[2]), "+v"(a[3]), "+v"(a[4]), "+v"(a[5]), "+v"(a[6]), "+v"(a[7])
@@ -258,7 +266,7 @@ __device__ __forceinline__ void wave_product_tiles(floatx4 (&acc)[2][NT], const 
 // 4*KL*NT registers for fragments in flight.
 // `prefetch` issues exactly NPF vector loads (for every wave, whatever its lanes need) behind the last
 // fragment load.
-template <int NT, int KS, bool RESIDENT, int KL, int NPF, int MT, typename Prefetch>
+template <int NT, int KS, bool RESIDENT, int KL, int NPF, int MT, int NBUF = 2, int CKO = 0, typename Prefetch>
 __device__ __forceinline__ void wave_product(floatx4 (&acc)[2][NT], const half8 (&wreg)[KS - KL][NT],
                                              const half8* wlds, const half8* wfrag_wave, const half_t* a0,
                                              const half_t* a1, int wave, int lane, int nks_total,
@@ -268,9 +276,13 @@ __device__ __forceinline__ void wave_product(floatx4 (&acc)[2][NT], const half8 
         // clamped (finite) address and meet all-zero weight fragments.  Chunks of CK k-steps (2*CK
         // fragments) alternate between two register sets: one is in flight while the other feeds the
         // MFMAs.  (Short contractions take small chunks: their kernels have no registers to spare.)
-        constexpr int CK = (KS >= 16) ? 4 : 2;
+        // Chunks rotate through NBUF register sets: one feeds the MFMAs, the others are in flight (two by default; a
+        // kernel that waits on a trip through memory takes more, of shorter chunks (CKO) where registers are short:
+        // five sets of 2 k-steps keep as much in flight as three sets of 4 and take 5/6 of the registers).
+        constexpr int CK = CKO ? CKO : ((KS >= 16) ? 4 : 2);
         constexpr int NCH = KS / CK;
-        half8 fa[2][CK], fb[2][CK];
+        constexpr int D = NBUF - 1;   // chunks requested ahead of the one being multiplied
+        half8 fa[NBUF][CK], fb[NBUF][CK];
         auto issue = [&](int c, int buf) {
 #pragma unroll
             for (int k = 0; k < CK; ++k) {
@@ -284,21 +296,33 @@ __device__ __forceinline__ void wave_product(floatx4 (&acc)[2][NT], const half8 
             if constexpr (MT == 2) wait_frags<N>(fa[buf], fb[buf]);
             else wait_frags<N>(fa[buf]);
         };
-        issue(0, 0);
-        if (NCH == 1) prefetch();
+#pragma unroll
+        for (int j = 0; j < (D < NCH ? D : NCH); ++j) issue(j, j % NBUF);
+        if (D >= NCH) prefetch();
 #pragma unroll
         for (int c = 0; c < NCH; ++c) {
-            const int buf = c & 1;
-            if (c + 2 < NCH) {
-                issue(c + 1, buf ^ 1);
-                wait(std::integral_constant<int, MT * CK>{}, buf);
-            } else if (c + 2 == NCH) {
-                issue(c + 1, buf ^ 1);
-                prefetch();
-                wait(std::integral_constant<int, MT * CK + NPF>{}, buf);
-            } else {
-                wait(std::integral_constant<int, NPF>{}, buf);
+            const int buf = c % NBUF;
+            if (c + D < NCH) {
+                issue(c + D, (c + D) % NBUF);
+                if (c + D == NCH - 1) prefetch();
             }
+            // requested after chunk c by now: the chunks up to c + D (or the last one), and the prefetch once the last
+            // chunk is out (c, D, NCH are compile-time constants: the switch folds)
+            const int last_now = (c + D < NCH - 1) ? c + D : NCH - 1;
+            const bool prefetched = (c + D >= NCH - 1);
+            switch ((last_now - c) * 2 + (prefetched ? 1 : 0)) {
+                case 0: wait(std::integral_constant<int, 0>{}, buf); break;
+                case 1: wait(std::integral_constant<int, NPF>{}, buf); break;
+                case 2: wait(std::integral_constant<int, MT * CK>{}, buf); break;
+                case 3: wait(std::integral_constant<int, MT * CK + NPF>{}, buf); break;
+                case 4: wait(std::integral_constant<int, 2 * MT * CK>{}, buf); break;
+                case 5: wait(std::integral_constant<int, 2 * MT * CK + NPF>{}, buf); break;
+                case 6: wait(std::integral_constant<int, 3 * MT * CK>{}, buf); break;
+                case 7: wait(std::integral_constant<int, 3 * MT * CK + NPF>{}, buf); break;
+                case 8: wait(std::integral_constant<int, 4 * MT * CK>{}, buf); break;
+                default: wait(std::integral_constant<int, 4 * MT * CK + NPF>{}, buf); break;
+            }
+            static_assert(NBUF <= 5, "the switch above knows up to four chunks ahead");
             if (poll.on) {
                 // A pair of halfs that still holds the pattern has not been written yet by its producer:
                 // fetch the chunk again (the chunk in flight behind it has to land first, loads return
@@ -1018,51 +1042,63 @@ __global__ __launch_bounds__(kThreads) void rec_bwd_kernel(RecBwdArgs p, RecLayo
 }
 
 // --------------------------------------------------------------- backward, two-dimensional split
-// For 2048 hidden units the product dG_{t+1} * W_hh^T has 32 MiB of weights: spread over the 256 compute units without
-// replication, every workgroup holds 128 KiB, and what it fetches per step depends on how its block is shaped.  The
-// kernel above gives a workgroup 16 output columns and the whole contraction (8192 packed gate columns), so every
-// workgroup pulls all of dG_{t+1} through its vector-memory path each step (512 KiB for a 32-row block).  Here a
-// workgroup owns a 64-column slice `s` (32 of them) and one EIGHTH `q` of the contraction: it fetches an eighth of
-// dG_{t+1}, forms a partial product [rows][64], and the eight workgroups of a slice -- seated in one XCD -- sum
-// their partials through a small ring in that XCD's L2: workgroup q sends columns 8q'..8q'+7 of its partial to
-// workgroup q' of the slice and finishes the 8 hidden units 64s + 8q .. +7 for all rows (one cell per thread).
+// For 2048 hidden units the product dG_{t+1} * W_hh^T has 32 MiB of weights.  The kernel above gives a workgroup 16
+// output columns and the whole contraction (8192 packed gate columns), so every workgroup pulls all of dG_{t+1}
+// of its rows through its XCD's L2 each step (512 KiB for a 32-row block); with 32 workgroups per XCD doing that,
+// the step is bound by the bandwidth of the L2 (measured: 1.1 KiB per clock and XCD, 5.8 us per row block).  Here a
+// workgroup owns a 64-column slice `s` (32 of them) and one of KQ slices `q` of the contraction: it fetches 1/KQ of
+// dG_{t+1}, forms a partial product [rows][64], and the KQ workgroups of a column slice -- seated in one XCD -- sum
+// their partials through a small ring in that XCD's L2: workgroup q sends columns (64/KQ)q' .. of its partial to
+// workgroup q' of the slice and finishes the 64/KQ hidden units 64s + (64/KQ)q .. for all rows of the block.
+//   KQ = 8, one group:  256 workgroups hold the weights once (128 KiB each); every workgroup takes every row block.
+//                       For batches of one row block.
+//   KQ = 4, two groups: a workgroup holds 256 KiB, the weights are held twice, and the groups take alternate row
+//                       blocks (a workgroup makes half as many passes per step, each with a quarter of the fetch).
 //
 // Two rings carry a step:
 //  * dG ring (p.X): 8 slots, fragment-major, written with device-scope stores and validated through the 'unwritten'
-//    pattern like the rings above.  A workgroup that has its product of step t knows that every workgroup has stored
-//    dG_{t+2} (its 32 producers stored dG_{t+1}, and each of those needed partials from a full slice, which together
-//    read all of dG_{t+2}), i.e. nobody reads dG_{t+3} any more: that slot is marked, five steps before it is reused.
-//  * partial ring (p.P): 3 slots of fp32 partial sums, [slice][receiver][row block][sender][row][8].  Plain stores,
+//    pattern like the rings above.  A workgroup that has its product of (step t, row block r) knows that every
+//    workgroup of its group has stored dG_{t+2} of r (its producers stored dG_{t+1}, and each of those needed partials
+//    from a full column slice, which together read all of dG_{t+2}), i.e. nobody reads dG_{t+3} of r any more: that
+//    region is marked, five steps before it is reused.
+//  * partial ring (p.P): 3 slots of fp32 partial sums, [workgroup][pass][sender][row][columns].  Plain stores,
 //    XCD-local.  It needs no marks: the lowest mantissa bit of every word carries the parity of the step, and a slot
 //    is reused every third step, so what a slot held before always shows the other parity (the bit costs 2^-24
 //    relative precision).  A sender overwrites the partials of step t+3 after its product of step t, when all
-//    workgroups are past step t+2.
-// A row block's partials are collected one product later (row block i-1 after the product of row block i), which
-// hides the trip through the L2 except for the last row block of a step.
-constexpr int kKQ = 8;          // contraction slices = workgroups per column slice
+//    workgroups of its group are past step t+2.
+// A row block's partials are collected one product later (block i-1 after the product of block i), which hides the
+// trip through the L2 except for the last block of a step.  The fragments are fetched as in the kernels above
+// (hand-issued, counted waits, all inside wave_product); every other load is a buffer load the compiler sees, used
+// in the same step it is issued in, so the compiler's own waits are exact and nothing stays in flight across the
+// step loop's back edge.
 constexpr int kDgSlots = 8;     // dG ring
 static_assert(kRecBwdPartSlots % 2 == 1, "consecutive uses of a partial-ring slot must differ in step parity");
 
-// Every global load of this kernel is a buffer load the compiler knows about (cache policy in the builtin's last
-// argument: 16 = device scope, served by the L2 and beyond; 2 = non-temporal), so the compiler places the
-// vector-memory waits itself and counts them exactly -- fragments requested a whole row block ahead stay in flight
-// across loop iterations as ordinary values.  order_here() keeps it from moving, merging or hoisting them: the
-// order of issue is part of the design (loads return in order), and a poll has to load again.
 typedef __amdgpu_buffer_rsrc_t rsrc_t;
 __device__ __forceinline__ rsrc_t make_rsrc(const void* p, size_t bytes) {
     return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(p), 0, int(unsigned(bytes < 0xFFFFFFFFull ? bytes : 0xFFFFFFFFull)),
                                              0x00020000);
 }
 __device__ __forceinline__ void order_here() { asm volatile("" ::: "memory"); }
-constexpr int kDeviceScope = 16, kNonTemporal = 2;
+constexpr int kDeviceScope = 16, kNonTemporal = 2;   // cache policy of a buffer load (last argument of the builtin)
 
-template <int MT>
+// MT: 16-row tiles per row block; KQ: contraction slices; NM: passes (row blocks) a workgroup makes per step at most
+template <int MT, int KQ, int NM>
 __global__ __launch_bounds__(kThreads) void rec_bwd2d_kernel(RecBwdArgs p, RecLayout L, int t_first, int t_last, int) {
-    constexpr int NT = 4;    // 64 output columns
-    constexpr int KS = 8;    // k-steps per wave: 4 waves * 8 * 32 = 1024 packed gate columns
+    constexpr int NT = 4;            // 64 output columns
+    constexpr int KS = 64 / KQ;      // k-steps per wave: 4 waves * KS * 32 = 8192 / KQ packed gate columns
+    constexpr int CPW = 64 / KQ;     // columns (hidden units) a workgroup finishes
+    constexpr int UPT = CPW / 8;     // ... per thread: 8 threads share a row
     constexpr int PLD = 16 * NT + kPartPad;
     constexpr int RB = 16 * MT;
-    extern __shared__ __attribute__((aligned(16))) float part_all[];  // [2][4][32][PLD] partial sums | [nrb][256] running dc
+    constexpr int NPF = 4;
+    // 256 KiB of weights per workgroup (KQ = 4) would take all 256 accumulation registers of a lane and leave the
+    // compiler nowhere to park what does not fit the ordinary ones: 5 of a wave's 16 k-steps live in LDS instead
+    // (80 KiB; with the partial sums 150 of the 160 KiB)
+    constexpr int KL = (KQ == 4) ? 5 : 0;
+    constexpr int KR = KS - KL;
+    static_assert(KQ == 4 || KQ == 8, "4 or 8 contraction slices");
+    extern __shared__ __attribute__((aligned(16))) float part_all[];  // [2][4][32][PLD] partial sums | weight fragments of the last KL k-steps
     __shared__ int lds_abort;
     __shared__ int lds_role[2];
     const int tid = threadIdx.x, wave = tid / kWave, lane = tid % kWave;
@@ -1076,40 +1112,54 @@ __global__ __launch_bounds__(kThreads) void rec_bwd2d_kernel(RecBwdArgs p, RecLa
     }
     __syncthreads();
     if (lds_role[1] >= 32) return;
+    // seats of an XCD: [group][4 column slices][KQ contraction slices]; the workgroups of a column slice share the XCD
     const int seat = __builtin_amdgcn_readfirstlane(lds_role[1]);
-    const int s = __builtin_amdgcn_readfirstlane(lds_role[0]) * 4 + seat / kKQ;   // column slice (its 8 workgroups share the XCD)
-    const int q = seat % kKQ;                            // contraction slice; also: which 8 columns of the slice end here
-    const int wave_u = __builtin_amdgcn_readfirstlane(wave);
-    const int nks = p.Hp / 8;                            // k-steps of the whole contraction
-    const int nrb = L.nrb;
+    const int g = seat / (4 * KQ);
+    const int s = __builtin_amdgcn_readfirstlane(lds_role[0]) * 4 + (seat % (4 * KQ)) / KQ;
+    const int q = seat % KQ;             // contraction slice; also: which CPW columns of the slice end here
+    if (g >= L.ng) return;               // (more seats than the layout uses: cannot happen with 256 workgroups)
+    const int nks = p.Hp / 8;            // k-steps of the whole contraction
+    const int nrb = L.nrb, ng = L.ng;
+    const int nmine = (nrb - g + ng - 1) / ng;   // row blocks g, g + ng, ...
     const Poll poll{true, p.spin_limit, p.spin_ticks, p.status, &lds_abort};
     const float S = p.dy_scale;
     PhaseClock clk{(blockIdx.x == 0) ? p.prof : nullptr, 0};
 
-    half8 wreg[KS][NT];
+    half8 wreg[KR][NT];
+    half8* wlds = reinterpret_cast<half8*>(part_all + 2 * 4 * kRows * PLD) + size_t(wave) * KL * NT * kWave;
     {
-        const half8* wf = p.wfrag2 + ((size_t(s) * kKQ + q) * 4 + wave) * size_t(KS) * NT * kWave;
+        const half8* wf = p.wfrag2 + ((size_t(s) * KQ + q) * 4 + wave) * size_t(KS) * NT * kWave;
 #pragma unroll
-        for (int k = 0; k < KS; ++k)
+        for (int k = 0; k < KR; ++k)
 #pragma unroll
             for (int n = 0; n < NT; ++n) wreg[k][n] = wf[(k * NT + n) * kWave + lane];
+#pragma unroll
+        for (int k = 0; k < KL; ++k)
+#pragma unroll
+            for (int n = 0; n < NT; ++n) wlds[(k * NT + n) * kWave + lane] = wf[((KR + k) * NT + n) * kWave + lane];
     }
 
-    // this thread's cell: row pr of a row block, hidden unit j; as a sender: row pr, columns 8*pj.. of the partial
+    // As a sender a thread sums row pr, columns 8*pj .. 8*pj+7 of the partial; as a receiver it collects the 8 columns
+    // 8*(pj / KQ) .. of sender pj % KQ for row pr and ends up with UPT of them: the cells (row pr, unit j .. j+UPT-1).
     const int pr = tid / 8, pj = tid % 8;
     const bool row_used = pr < RB;
-    const int j = s * 64 + q * 8 + pj;
+    const int j = s * 64 + q * CPW + (pj / KQ) * 8 + (pj % KQ) * UPT;
     const size_t pq = size_t(4) * j;
     const size_t gld = size_t(4) * p.Hp;
-    float* dcl = part_all + 2 * 4 * kRows * PLD;
-    for (int rb = 0; rb < nrb; ++rb) {
-        const int b = rb * RB + pr;
-        dcl[rb * kThreads + tid] = (row_used && b < p.B) ? p.dC[size_t(b) * p.Hp + j] : 0.f;
+    // the running dc of every row block this workgroup takes stays in registers
+    float dcreg[NM][UPT];
+#pragma unroll
+    for (int i = 0; i < NM; ++i) {
+        const int b = (g + i * ng) * RB + pr;
+#pragma unroll
+        for (int u = 0; u < UPT; ++u) dcreg[i][u] = (i < nmine && row_used && b < p.B) ? p.dC[size_t(b) * p.Hp + j + u] : 0.f;
     }
-    float dbacc[4] = {};
+    float dbacc[4][UPT] = {};
     int item = 0;
+    const rsrc_t rp = make_rsrc(p.P, size_t(kRecBwdPartSlots) * p.p_slot * 4);
+    const unsigned wg_id = unsigned((g * 32 + s) * KQ);   // + receiver's q: inbox index in the partial ring
 
-    // poll bookkeeping shared by the two kinds of waits; true = give up
+    // poll bookkeeping; true = give up
     auto spin_out = [&](int& spins, long long& spin_start) -> bool {
         ++spins;
         if (spins == 1) spin_start = wall_clock64();
@@ -1126,12 +1176,13 @@ __global__ __launch_bounds__(kThreads) void rec_bwd2d_kernel(RecBwdArgs p, RecLa
         return false;
     };
 
-    // Per-cell operands of a row block (activated gates, c_{t-1}, c_t, dY): requested while the block's product runs,
-    // used one product later; two sets, by the parity of the row block.
-    uintx2 og[2];
-    unsigned ocp[2], occ[2];
-    unsigned short ody[2];
-    auto load_ops = [&](int t, int rb, uintx2& g, unsigned& cp, unsigned& cc, unsigned short& dy) {
+    // Per-cell operands of a row block (activated gates, c_{t-1}, c_t, dY), NPF buffer loads.
+    struct Ops {
+        uintx4 g;        // UPT == 2: eight halfs; UPT == 1: .xy
+        uintx2 cp, cc;   // UPT == 1: .x
+        unsigned dy;     // UPT == 1: low half
+    };
+    auto load_ops = [&](int t, int rb, Ops& o) {
         const int b = min(rb * RB + pr, p.B - 1);
         const size_t tt = size_t(max(t, 0));
         // (a descriptor per step: the arrays of a long sequence are larger than a 32-bit offset reaches)
@@ -1139,21 +1190,33 @@ __global__ __launch_bounds__(kThreads) void rec_bwd2d_kernel(RecBwdArgs p, RecLa
         const rsrc_t rc = make_rsrc(p.C + tt * p.B * p.Hp, size_t(2) * p.B * p.Hp * 4);
         const rsrc_t ry = make_rsrc(p.dY + tt * p.B * p.Hp, size_t(p.B) * p.Hp * 2);
         const unsigned cell_idx = unsigned(b) * unsigned(p.Hp) + unsigned(j);
-        g = __builtin_amdgcn_raw_buffer_load_b64(rg, (unsigned(b) * unsigned(gld) + unsigned(pq)) * 2u, 0, kNonTemporal);
-        cp = __builtin_amdgcn_raw_buffer_load_b32(rc, cell_idx * 4u, 0, kNonTemporal);
-        cc = __builtin_amdgcn_raw_buffer_load_b32(rc, (cell_idx + unsigned(p.B) * unsigned(p.Hp)) * 4u, 0, kNonTemporal);
-        dy = __builtin_amdgcn_raw_buffer_load_b16(ry, cell_idx * 2u, 0, kNonTemporal);
-        order_here();
+        const unsigned goff = (unsigned(b) * unsigned(gld) + unsigned(pq)) * 2u;
+        const unsigned next = unsigned(p.B) * unsigned(p.Hp);
+        if constexpr (UPT == 2) {
+            o.g = __builtin_amdgcn_raw_buffer_load_b128(rg, goff, 0, kNonTemporal);
+            o.cp = __builtin_amdgcn_raw_buffer_load_b64(rc, cell_idx * 4u, 0, kNonTemporal);
+            o.cc = __builtin_amdgcn_raw_buffer_load_b64(rc, (cell_idx + next) * 4u, 0, kNonTemporal);
+            o.dy = __builtin_amdgcn_raw_buffer_load_b32(ry, cell_idx * 2u, 0, kNonTemporal);
+        } else {
+            const uintx2 g2 = __builtin_amdgcn_raw_buffer_load_b64(rg, goff, 0, kNonTemporal);
+            o.g = uintx4{g2.x, g2.y, 0u, 0u};
+            o.cp.x = __builtin_amdgcn_raw_buffer_load_b32(rc, cell_idx * 4u, 0, kNonTemporal);
+            o.cc.x = __builtin_amdgcn_raw_buffer_load_b32(rc, (cell_idx + next) * 4u, 0, kNonTemporal);
+            o.dy = __builtin_amdgcn_raw_buffer_load_b16(ry, cell_idx * 2u, 0, kNonTemporal);
+        }
     };
-    // the cell update of (t, rb) given dh from the product (or dHn), and everything it stores
-    auto cell = [&](int t, int rb, float dh, uintx2 g, unsigned cpb, unsigned ccb, unsigned short dyb) {
+    // the cell update of (t, pass i: row block rb) given dh from the product (or dHn), and everything it stores
+    auto cell = [&](int t, int rb, float (&dcr)[UPT], const float (&dh)[UPT], const Ops& o) {
         const int b = rb * RB + pr;
         const bool live = row_used && b < p.B;
         const size_t sidx = size_t(b) * p.Hp + j;
         if (t < 0) {   // closing pass: gradient wrt h0; dc0 is the running dc
             if (live) {
-                p.dH0[sidx] = dh;
-                p.dC[sidx] = dcl[rb * kThreads + tid];
+#pragma unroll
+                for (int u = 0; u < UPT; ++u) {
+                    p.dH0[sidx + u] = dh[u];
+                    p.dC[sidx + u] = dcr[u];
+                }
             }
             return;
         }
@@ -1161,84 +1224,88 @@ __global__ __launch_bounds__(kThreads) void rec_bwd2d_kernel(RecBwdArgs p, RecLa
         half_t* xmark = p.X + size_t((t + 11) & (kDgSlots - 1)) * p.x_slot;   // dG_{t+3}: read by nobody any more
         unsigned off = 0;
         if (row_used) {
-            off = unsigned(xch_offset(b, int(pq), nks));
-            store_xch(xmark + off, Pack<4>{uintx2{kUnwritten, kUnwritten}}, true);
-        }
-        Pack<4> out{uintx2{0u, 0u}};   // batch rows past B travel as zeros
-        if (live) {
-            float gate[4];
-            unpack(Pack<4>{g}, gate);
-            float dyl, dyh;
-            unpack_h2(unsigned(dyb), dyl, dyh);
-            const float pcp = __builtin_bit_cast(float, cpb), pcc = __builtin_bit_cast(float, ccb);
-            const float ig = gate[0], fg = gate[1], gg = gate[2], og_ = gate[3];
-            const float dhu = dh + S * dyl;
-            const float tc = tanhf_dev(pcc);
-            const float dov = dhu * tc;
-            const float dc = dcl[rb * kThreads + tid] + dhu * og_ * (1.f - tc * tc);
-            float da[4];
-            da[0] = dc * gg * ig * (1.f - ig);
-            da[1] = dc * pcp * fg * (1.f - fg);
-            da[2] = dc * ig * (1.f - gg * gg);
-            da[3] = dov * og_ * (1.f - og_);
-            dcl[rb * kThreads + tid] = dc * fg;
-            out = pack(da);
-            float r[4];   // db sums the values the weight-gradient GEMMs will see (fp16-rounded)
-            unpack(out, r);
+            off = unsigned(xch_offset(b, int(pq), nks));   // 4 * UPT consecutive halfs: one 8-byte group per unit
 #pragma unroll
-            for (int gt = 0; gt < 4; ++gt) dbacc[gt] += r[gt];
+            for (int u = 0; u < UPT; ++u) store_xch(xmark + off + 4 * u, Pack<4>{uintx2{kUnwritten, kUnwritten}}, true);
         }
-        if (row_used) store_xch(xout + off, out, true);
+        Pack<4> out[UPT];
+#pragma unroll
+        for (int u = 0; u < UPT; ++u) out[u] = Pack<4>{uintx2{0u, 0u}};   // batch rows past B travel as zeros
+        if (live) {
+#pragma unroll
+            for (int u = 0; u < UPT; ++u) {
+                float gate[4];
+                unpack(Pack<4>{u == 0 ? uintx2{o.g.x, o.g.y} : uintx2{o.g.z, o.g.w}}, gate);
+                float dyl, dyh;
+                unpack_h2(o.dy, dyl, dyh);
+                const float dyv = (u == 0) ? dyl : dyh;
+                const float pcp = __builtin_bit_cast(float, u == 0 ? o.cp.x : o.cp.y);
+                const float pcc = __builtin_bit_cast(float, u == 0 ? o.cc.x : o.cc.y);
+                const float ig = gate[0], fg = gate[1], gg = gate[2], og_ = gate[3];
+                const float dhu = dh[u] + S * dyv;
+                const float tc = tanhf_dev(pcc);
+                const float dov = dhu * tc;
+                const float dc = dcr[u] + dhu * og_ * (1.f - tc * tc);
+                float da[4];
+                da[0] = dc * gg * ig * (1.f - ig);
+                da[1] = dc * pcp * fg * (1.f - fg);
+                da[2] = dc * ig * (1.f - gg * gg);
+                da[3] = dov * og_ * (1.f - og_);
+                dcr[u] = dc * fg;
+                out[u] = pack(da);
+                float r[4];   // db sums the values the weight-gradient GEMMs will see (fp16-rounded)
+                unpack(out[u], r);
+#pragma unroll
+                for (int gt = 0; gt < 4; ++gt) dbacc[gt][u] += r[gt];
+            }
+        }
+        if (row_used) {
+#pragma unroll
+            for (int u = 0; u < UPT; ++u) store_xch(xout + off + 4 * u, out[u], true);
+        }
         clk.lap(2);
-        if (live) st_pack(p.dG + (size_t(t) * p.B + b) * gld + pq, out);
+        if (live) {
+            half_t* dst = p.dG + (size_t(t) * p.B + b) * gld + pq;
+            if constexpr (UPT == 2) __builtin_nontemporal_store(uintx4{out[0].v.x, out[0].v.y, out[1].v.x, out[1].v.y}, reinterpret_cast<uintx4*>(dst));
+            else st_pack(dst, out[0]);
+        }
         clk.lap(3);
     };
-
-    // Fragments of dG_{t+1} for one row block: this wave's 8 k-steps of the workgroup's contraction slice, requested
-    // together; two sets, so the next row block's fetch runs under this one's MFMAs and the partial exchange (and the
-    // first row block of the next step is requested while the last one of this step is being finished).
-    const rsrc_t rx = make_rsrc(p.X, size_t(kDgSlots) * p.x_slot * 2);
-    const rsrc_t rp = make_rsrc(p.P, size_t(kRecBwdPartSlots) * p.p_slot * 4);
-    uintx4 fr[2][KS][MT];
-    unsigned voff[KS];   // byte offset of this lane's 16 bytes in k-step k of the wave (k-steps of a wave are 4 apart)
-#pragma unroll
-    for (int k = 0; k < KS; ++k) voff[k] = unsigned(lane) * 16u + unsigned(k) * 4096u;
-    auto load_set = [&](uintx4 (&f)[KS][MT], int slot, int rb) {
-        const unsigned base = unsigned((size_t(slot) * p.x_slot + (size_t(MT * rb) * nks + size_t(q) * 32 + wave_u) * 512) * 2);
-#pragma unroll
-        for (int k = 0; k < KS; ++k)
-#pragma unroll
-            for (int m = 0; m < MT; ++m)
-                f[k][m] = __builtin_amdgcn_raw_buffer_load_b128(rx, voff[k], base + unsigned(m) * unsigned(nks) * 1024u, kDeviceScope);
-        order_here();
-    };
-    bool pending0 = false;   // set 0 already holds (or awaits) the first row block of the step that comes next
 
     __syncthreads();
     clk.start();
     for (int t = t_first; t >= t_last; --t) {
         if (t >= p.T - 1) {   // the last step of the sequence: dh comes from the caller
-            for (int rb = 0; rb < nrb; ++rb) {
-                load_ops(t, rb, og[0], ocp[0], occ[0], ody[0]);
+#pragma unroll
+            for (int i = 0; i < NM; ++i) {
+                if (i >= nmine) break;
+                const int rb = g + i * ng;
+                Ops o;
+                load_ops(t, rb, o);
                 const int b = min(rb * RB + pr, p.B - 1);
-                const float dh = p.dHn[size_t(b) * p.Hp + j];
-                cell(t, rb, dh, og[0], ocp[0], occ[0], ody[0]);
+                float dh[UPT];
+#pragma unroll
+                for (int u = 0; u < UPT; ++u) dh[u] = p.dHn[size_t(b) * p.Hp + j + u];
+                cell(t, rb, dcreg[i], dh, o);
             }
             continue;
         }
-        const int slot_in = (t + 9) & (kDgSlots - 1);   // dG_{t+1}
+        const half_t* xin = p.X + size_t((t + 9) & (kDgSlots - 1)) * p.x_slot;   // dG_{t+1}
         const unsigned pbase = unsigned((t + 3) % kRecBwdPartSlots) * unsigned(p.p_slot);   // in floats
         float* pslot = p.P + size_t(pbase);
         const unsigned par = unsigned(t) & 1u;
-        if (!pending0) load_set(fr[0], slot_in, 0);
-        // One pass of the loop below for row block i (parity BUF): request the partials of block i-1, the fragments of
-        // block i+1 and the cell operands of block i, multiply block i, send its partials, then finish block i-1.
-        auto pass = [&](int i, auto buf_tag) -> bool {
-            constexpr int BUF = decltype(buf_tag)::value;
-            const bool product = i < nrb, finish = i >= 1, more = i + 1 < nrb;
+        Ops ops[2];
+        // Pass i (unrolled): request the partials of block i-1, multiply block i (its cell operands are requested
+        // behind the last fragment load), send its partials, then finish block i-1.
+#pragma unroll
+        for (int i = 0; i <= NM; ++i) {
+            if (i > nmine) break;
+            const bool product = i < nmine, finish = i >= 1;
+            const int rb = g + i * ng, rb_prev = g + (i - 1) * ng;
             uintx4 in0 = {0u, 0u, 0u, 0u}, in1 = {0u, 0u, 0u, 0u};
-            // partials of block i-1: sender pj, row pr (byte offset into the ring)
-            const unsigned src = (pbase + unsigned(((((s * kKQ + q) * nrb + max(i - 1, 0)) * kKQ + pj) * RB + min(pr, RB - 1)) * 8)) * 4u;
+            // partials of block i-1 in this workgroup's inbox: sender pj % KQ, row pr, 8 columns from 8 * (pj / KQ)
+            const unsigned src = (pbase + ((((wg_id + unsigned(q)) * NM + unsigned(max(i - 1, 0))) * KQ + unsigned(pj % KQ)) * RB +
+                                           unsigned(min(pr, RB - 1))) * CPW + unsigned(pj / KQ) * 8u) * 4u;
             if (finish) {
                 in0 = __builtin_amdgcn_raw_buffer_load_b128(rp, src, 0, kDeviceScope);
                 in1 = __builtin_amdgcn_raw_buffer_load_b128(rp, src + 16u, 0, kDeviceScope);
@@ -1246,50 +1313,21 @@ __global__ __launch_bounds__(kThreads) void rec_bwd2d_kernel(RecBwdArgs p, RecLa
             }
             if (product) {
                 float* part = part_all + size_t(item & 1) * 4 * kRows * PLD;
-                if (more) load_set(fr[BUF ^ 1], slot_in, i + 1);
-                load_ops(t, i, og[BUF], ocp[BUF], occ[BUF], ody[BUF]);
-                // A word that still shows the pattern has not been written yet: fetch the block again.  (The first check
-                // stands outside the loop: the compiler then waits for exactly this set there, not for everything a
-                // path through the loop might have requested.)
-                auto stale = [&]() -> bool {
-                    unsigned mx = 0u;
-#pragma unroll
-                    for (int k = 0; k < KS; ++k)
-#pragma unroll
-                        for (int mm = 0; mm < MT; ++mm) {
-                            const uintx4 u = fr[BUF][k][mm];
-                            mx = max(mx, max(max(u.x, u.y), max(u.z, u.w)));
-                        }
-                    return __any(mx == kUnwritten) != 0;
-                };
-                if (stale()) {
-                    int spins = 0;
-                    long long spin_start = 0;
-                    do {
-                        if (spin_out(spins, spin_start)) break;
-                        order_here();
-                        load_set(fr[BUF], slot_in, i);
-                    } while (stale());
-                }
                 floatx4 acc[2][NT];
 #pragma unroll
                 for (int m = 0; m < 2; ++m)
 #pragma unroll
                     for (int n = 0; n < NT; ++n) acc[m][n] = floatx4{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-                for (int k = 0; k < KS; ++k)
-#pragma unroll
-                    for (int n = 0; n < NT; ++n)
-#pragma unroll
-                        for (int m = 0; m < MT; ++m)
-                            acc[m][n] = __builtin_amdgcn_mfma_f32_16x16x32_f16(wreg[k][n], __builtin_bit_cast(half8, fr[BUF][k][m]),
-                                                                               acc[m][n], 0, 0, 0);
+                const half_t* a0 = xin + (size_t(MT * rb) * nks + size_t(q) * (KS * 4)) * 512 + lane * 8;
+                const half_t* a1 = a0 + size_t(nks) * 512;
+                wave_product<NT, KS, true, KL, NPF, MT, (KS >= 16 ? 5 : 2), (KS >= 16 ? 2 : 0)>(acc, wreg, wlds, nullptr, a0, a1, wave, lane, KS * 4, KS, 0, poll,
+                                                       [&]() { load_ops(t, rb, ops[i & 1]); });
                 clk.lap(0);
                 spill_partials<NT, MT>(part, acc, wave, lane, PLD);
                 ++item;
                 __syncthreads();
-                if (lds_abort != 0) return false;
-                if (row_used) {   // sum the four waves' k-slices and send 8 columns to workgroup pj of the slice
+                if (lds_abort != 0) return;
+                if (row_used) {   // sum the four waves' k-slices and send 8 columns to their receiver in the slice
                     floatx4 v0 = {0.f, 0.f, 0.f, 0.f}, v1 = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
                     for (int w = 0; w < 4; ++w) {
@@ -1303,18 +1341,16 @@ __global__ __launch_bounds__(kThreads) void rec_bwd2d_kernel(RecBwdArgs p, RecLa
                         u0[e] = (u0[e] & ~1u) | par;
                         u1[e] = (u1[e] & ~1u) | par;
                     }
-                    float* dst = pslot + ((((size_t(s) * kKQ + pj) * nrb + i) * kKQ + q) * RB + pr) * 8;
+                    // columns 8*pj .. belong to receiver (8*pj) / CPW, at column (8*pj) % CPW of its block
+                    const unsigned recv = unsigned(8 * pj) / CPW, col = unsigned(8 * pj) % CPW;
+                    float* dst = pslot + ((((size_t(wg_id) + recv) * NM + i) * KQ + q) * RB + pr) * CPW + col;
                     *reinterpret_cast<uintx4*>(dst) = u0;
                     *reinterpret_cast<uintx4*>(dst + 4) = u1;
                 }
                 clk.lap(1);
-            } else if (nrb >= 2 && t - 1 >= t_last) {
-                // The first row block of the next step (dG_t, block 0: stored by everyone a pass ago or more) is requested
-                // while the last block of this step is being finished.  (With one row block per step everyone's dG_t is
-                // being stored right now: the request goes out after this workgroup's own cell update, below.)
-                load_set(fr[0], (t + 8) & (kDgSlots - 1), 0);
             }
             if (finish) {
+                // (the first check stands outside the loop: the compiler then waits for exactly these two loads there)
                 auto tags_bad = [&]() -> bool {
                     const unsigned all1 = in0.x & in0.y & in0.z & in0.w & in1.x & in1.y & in1.z & in1.w;
                     const unsigned any1 = in0.x | in0.y | in0.z | in0.w | in1.x | in1.y | in1.z | in1.w;
@@ -1333,56 +1369,70 @@ __global__ __launch_bounds__(kThreads) void rec_bwd2d_kernel(RecBwdArgs p, RecLa
                     } while (tags_bad());
                 }
                 clk.lap(4);
-                // sum over the 8 senders (lanes that differ in their low three bits): lane pj keeps column pj
+                // Sum over the KQ senders (lanes that differ in their low bits): each halving step keeps half of the
+                // columns, so lane pj ends up with columns UPT * (pj % KQ) .. of its 8.
                 const floatx4 f0 = __builtin_bit_cast(floatx4, in0), f1 = __builtin_bit_cast(floatx4, in1);
-                float a4[4], a2[2];
-                {
+                float a4[4], a2[2], dh[UPT];
+                if constexpr (KQ == 8) {
                     const bool hi = (lane & 4) != 0;
 #pragma unroll
                     for (int k = 0; k < 4; ++k) {
                         const float keep = hi ? f1[k] : f0[k], send = hi ? f0[k] : f1[k];
                         a4[k] = keep + __shfl_xor(send, 4);
                     }
-                }
-                {
-                    const bool hi = (lane & 2) != 0;
+                    const bool hi2 = (lane & 2) != 0;
 #pragma unroll
                     for (int k = 0; k < 2; ++k) {
-                        const float keep = hi ? a4[2 + k] : a4[k], send = hi ? a4[k] : a4[2 + k];
+                        const float keep = hi2 ? a4[2 + k] : a4[k], send = hi2 ? a4[k] : a4[2 + k];
                         a2[k] = keep + __shfl_xor(send, 2);
                     }
+                    const bool hi1 = (lane & 1) != 0;
+                    dh[0] = (hi1 ? a2[1] : a2[0]) + __shfl_xor(hi1 ? a2[0] : a2[1], 1);
+                } else {
+                    const bool hi2 = (lane & 2) != 0;
+#pragma unroll
+                    for (int k = 0; k < 4; ++k) {
+                        const float keep = hi2 ? f1[k] : f0[k], send = hi2 ? f0[k] : f1[k];
+                        a4[k] = keep + __shfl_xor(send, 2);
+                    }
+                    const bool hi1 = (lane & 1) != 0;
+#pragma unroll
+                    for (int k = 0; k < 2; ++k) {
+                        const float keep = hi1 ? a4[2 + k] : a4[k], send = hi1 ? a4[k] : a4[2 + k];
+                        dh[k] = keep + __shfl_xor(send, 1);
+                    }
+                    (void)a2;
                 }
-                const bool hi = (lane & 1) != 0;
-                const float dh = (hi ? a2[1] : a2[0]) + __shfl_xor(hi ? a2[0] : a2[1], 1);
-                cell(t, i - 1, dh, og[BUF ^ 1], ocp[BUF ^ 1], occ[BUF ^ 1], ody[BUF ^ 1]);
+                cell(t, rb_prev, dcreg[i >= 1 ? i - 1 : 0], dh, ops[(i + 1) & 1]);
             }
-            return true;
-        };
-        for (int i = 0; i <= nrb; i += 2) {
-            if (!pass(i, std::integral_constant<int, 0>{})) return;
-            if (i + 1 <= nrb && !pass(i + 1, std::integral_constant<int, 1>{})) return;
         }
-        pending0 = (t - 1 >= t_last);
-        if (pending0 && nrb == 1) load_set(fr[0], (t + 8) & (kDgSlots - 1), 0);
     }
     clk.flush();
     if (t_last >= 0) {   // a launch that stops before the closing pass leaves dc in memory for the next one
-        for (int rb = 0; rb < nrb; ++rb) {
-            const int b = rb * RB + pr;
-            if (row_used && b < p.B) p.dC[size_t(b) * p.Hp + j] = dcl[rb * kThreads + tid];
+#pragma unroll
+        for (int i = 0; i < NM; ++i) {
+            const int b = (g + i * ng) * RB + pr;
+            if (i < nmine && row_used && b < p.B) {
+#pragma unroll
+                for (int u = 0; u < UPT; ++u) p.dC[size_t(b) * p.Hp + j + u] = dcreg[i][u];
+            }
         }
     }
     // Bias gradient: fold this launch's sums over the 32 rows (fixed order).
     __syncthreads();
-    float* red = part_all;   // [256][4]
+    float* red = part_all;   // [256][4 * UPT]
 #pragma unroll
-    for (int gt = 0; gt < 4; ++gt) red[tid * 4 + gt] = dbacc[gt];
+    for (int gt = 0; gt < 4; ++gt)
+#pragma unroll
+        for (int u = 0; u < UPT; ++u) red[tid * (4 * UPT) + gt * UPT + u] = dbacc[gt][u];
     __syncthreads();
-    if (tid < 32) {
-        const int uj = tid / 4, gt = tid % 4;
+    if (tid < 8 * 4 * UPT) {
+        const int cpos = tid / (4 * UPT), e = tid % (4 * UPT);   // thread column pj, (gate, unit)
         float sum = 0.f;
-        for (int r = 0; r < kThreads / 8; ++r) sum += red[(r * 8 + uj) * 4 + gt];
-        p.db_part[size_t(4) * (s * 64 + q * 8 + uj) + gt] += sum;
+        for (int r = 0; r < kThreads / 8; ++r) sum += red[(r * 8 + cpos) * (4 * UPT) + e];
+        const int gt = e / UPT, u = e % UPT;
+        const int ju = s * 64 + q * CPW + (cpos / KQ) * 8 + (cpos % KQ) * UPT + u;
+        p.db_part[size_t(g) * gld + size_t(4) * ju + gt] += sum;
     }
 }
 
@@ -1497,16 +1547,23 @@ RecLayout plan_rec_bwd(int B, int Hp, int num_cus, bool force_stepwise, int forc
     if (two_d > 0 && L.persistent && rec_bwd_two_d_possible(Hp, num_cus)) {
         const int mt = (B <= 16 && force_mt != 2) ? 1 : 2;
         const int nrb = int(ceil_div(size_t(B), size_t(16 * mt)));
-        // Every workgroup walks all row blocks (its running dc for them sits in LDS: at most 8).  Measured on MI355X
-        // the two-way split wins where a step is one row block (batches up to 32 rows: 4.0 against 6.5 us per step at
-        // 16 rows) and only ties with the one-way layout at four (13.4 us either way at 128 rows: what it saves on
-        // the fetch it spends on the second exchange, every row block paying both in turn), so it is chosen by itself
-        // only for one row block; two_d = 2 forces it wherever it can run.
-        if (nrb <= (two_d >= 2 ? 8 : 1)) {
+        const int kq = rec_bwd_two_d_kq(B);
+        const int ng = kq == 8 ? 1 : 2;
+        const int per_wg = int(ceil_div(size_t(nrb), size_t(ng)));   // passes per step and workgroup
+        // One row block per step: 8 contraction slices, every workgroup on that block (4.0 against 6.5 us per step at
+        // 16 rows).  More: 4 slices and two groups that take alternate row blocks.  two_d = 1 takes the layout where
+        // it measured faster than the one-way layout, two_d = 2 wherever it can run (at most 2 passes per workgroup,
+        // i.e. 128 rows: a kernel unrolled for 4 passes does not fit the registers).
+        // Measured, us per backward step, one-way -> two-way: 16 rows 5.4 -> 4.0, 32 rows 5.8 -> 4.2, 64 rows 7.5 -> 7.6,
+        // 128 rows 12.4 -> 9.8.
+        const bool faster = (nrb != 2);
+        if (per_wg <= 2 && (two_d >= 2 || faster)) {
             L.two_d = 1;
+            L.kq = kq;
+            L.nm = per_wg;
             L.mt = mt;
             L.nrb = nrb;
-            L.ng = 1;
+            L.ng = ng;
             L.xcd_local = 0;
             L.gpx = 0;
             L.grid = 256;
@@ -1516,9 +1573,14 @@ RecLayout plan_rec_bwd(int B, int Hp, int num_cus, bool force_stepwise, int forc
 }
 
 bool rec_bwd_two_d_possible(int Hp, int num_cus) { return Hp == 2048 && num_cus == 256; }
+// Up to two row blocks: 8 slices and one group (with two blocks every workgroup makes two passes per step, and one
+// block's trip through memory hides behind the other's product: 7.0 us per step at 64 rows against 8.0 with 4 slices and
+// two groups of one pass each).  More: 4 slices, two groups.
+int rec_bwd_two_d_kq(int B) { return B <= 64 ? 8 : 4; }
 int rec_bwd_dg_slots(const RecLayout& L) { return L.two_d ? kDgSlots : 4; }
 size_t rec_bwd_part_slot_floats(const RecLayout& L) {
-    return L.two_d ? size_t(256) * L.nrb * kKQ * (16 * L.mt) * 8 : 0;
+    // [256 workgroups][nm passes][kq senders][rows][64 / kq columns]
+    return L.two_d ? size_t(256) * L.nm * 64 * (16 * L.mt) : 0;
 }
 size_t rec_bwd_two_d_wfrag_bytes(int Hp) { return size_t(Hp) * 4 * Hp * sizeof(half_t); }
 unsigned rec_bwd_part_fill(int slot, int T) {
@@ -1642,10 +1704,11 @@ static hipError_t run_bwd(const RecLayout& L, const RecBwdArgs& a, hipStream_t s
                         });
 }
 
-template <int MT>
+template <int MT, int KQ, int NM>
 static hipError_t run_bwd2d(const RecLayout& L, const RecBwdArgs& a, hipStream_t stream) {
-    auto kernel = rec_bwd2d_kernel<MT>;
-    const size_t lds = (size_t(2) * 4 * kRows * (64 + kPartPad) + size_t(L.nrb) * kThreads) * sizeof(float);
+    auto kernel = rec_bwd2d_kernel<MT, KQ, NM>;
+    constexpr int KL = (KQ == 4) ? 5 : 0;   // k-steps per wave whose weights live in LDS (as in the kernel)
+    const size_t lds = size_t(2) * 4 * kRows * (64 + kPartPad) * sizeof(float) + size_t(4) * KL * 4 * kWave * sizeof(half8);
     hipError_t e = raise_lds(kernel, lds);
     if (e != hipSuccess) return e;
     return launch_persistent(kernel, L.grid, lds, stream, a, L, a.t_hi, a.t_lo, 0);
@@ -1656,10 +1719,18 @@ hipError_t launch_rec_bwd(const RecLayout& L, const RecBwdArgs& a, hipStream_t s
     if (a.Hp % 32 != 0 || a.Hp % L.jb != 0 || a.t_lo < -1 || a.t_hi >= a.T) return hipErrorInvalidValue;
     if (L.two_d) {
         // what the kernel's indexing assumes
-        if (!L.persistent || a.Hp != 2048 || L.grid != 256 || L.nrb < 1 || L.nrb > 8 || !a.wfrag2 || !a.P ||
-            L.nrb * 16 * L.mt < a.B || a.p_slot != rec_bwd_part_slot_floats(L))
+        const int ng = L.kq == 8 ? 1 : 2;
+        if (!L.persistent || a.Hp != 2048 || L.grid != 256 || (L.kq != 4 && L.kq != 8) || L.ng != ng || L.nrb < 1 ||
+            (L.nrb + ng - 1) / ng > L.nm || !a.wfrag2 || !a.P || L.nrb * 16 * L.mt < a.B ||
+            a.p_slot != rec_bwd_part_slot_floats(L))
             return hipErrorInvalidValue;
-        return L.mt == 1 ? run_bwd2d<1>(L, a, stream) : run_bwd2d<2>(L, a, stream);
+        if (L.kq == 8 && L.nm == 1) return L.mt == 1 ? run_bwd2d<1, 8, 1>(L, a, stream) : run_bwd2d<2, 8, 1>(L, a, stream);
+        if (L.kq == 8 && L.nm == 2 && L.mt == 2) return run_bwd2d<2, 8, 2>(L, a, stream);
+        if (L.kq == 4 && L.mt == 2) {
+            if (L.nm == 1) return run_bwd2d<2, 4, 1>(L, a, stream);
+            if (L.nm == 2) return run_bwd2d<2, 4, 2>(L, a, stream);
+        }
+        return hipErrorInvalidValue;
     }
     if (!L.resident) return run_bwd<2, 1, false, 0, 2>(L, a, stream, graphs);
     if (L.nt == 2) return L.mt == 1 ? run_bwd<2, 32, true, 8, 1>(L, a, stream, graphs) : run_bwd<2, 32, true, 8, 2>(L, a, stream, graphs);

@@ -118,19 +118,20 @@ def test_persistent_and_stepwise_agree(shape):
         assert rell2(a[k], b[k]) < tol, k
 
 
-@pytest.mark.parametrize("shape", [(7, 256, 32, 2048), (6, 40, 32, 2048), (9, 5, 64, 2040), (4, 17, 32, 2048),
-                                   (1, 16, 32, 2048), (2, 33, 32, 2017)])
+@pytest.mark.parametrize("shape", [(7, 128, 32, 2048), (6, 40, 32, 2048), (9, 5, 64, 2040), (4, 17, 32, 2048),
+                                   (1, 16, 32, 2048), (2, 33, 32, 2017), (5, 96, 32, 2048), (3, 100, 64, 2048)])
 def test_two_way_split_backward_for_2048_units(shape):
     # 2048 (padded) hidden units: the persistent backward kernel splits its product over column slices AND over the
-    # contraction, and sums the partial products through a second ring.  One to eight row blocks, ragged batches,
-    # padded hidden sizes, a single step; against torch, against the one-way layout, and through the give-up path.
+    # contraction, and sums the partial products through a second ring.  One row block (8 contraction slices) and two
+    # to four (4 slices, two groups taking alternate blocks, one or two passes per workgroup), ragged batches, padded
+    # hidden sizes, a single step; against torch, against the one-way layout, and through the give-up path.
     from flashlstm_poc_amd import LstmCore
     T, B, I, H = shape
     p = make_problem(*shape, seed=11)
     ref = torch_reference(p, dtype=torch.float32, device="cuda")
     core = LstmCore(B, I, H)
     core.pack(*(p[k].cuda() for k in ("w_ih", "w_hh", "b_ih", "b_hh")))
-    assert core.info("bwd_two_d") == (1 if B <= 32 else 0)   # by itself the plan takes it for one row block per step
+    assert core.info("bwd_two_d") == (0 if 32 < B <= 64 else 1)   # (two row blocks per step: the layouts tie, the plan keeps the one-way one)
     core.set_option("bwd_two_d", 2)                           # here: wherever it can run
     got, info = run_core(p, core=core)
     assert info["persistent_bwd"] == 1 and info["bwd_two_d"] == 1 and info["fallbacks"] == 0
