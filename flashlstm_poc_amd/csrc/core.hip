@@ -367,7 +367,7 @@ extern "C" int flstm_core_pack_weights(flstm_core_plan* p, const float* w_ih, co
                         p->ks_f, p->Lf.nt, p->Lf.rot_div, p->wfrag_b.as<half8>(), p->ks_b, p->Lb.nt, p->Lb.rot_div, s));
     if (rec_bwd_two_d_possible(d.Hp, p->num_cus)) {   // whether or not the current layout uses them
         FL_TRY(p->wfrag_b2.reserve(rec_bwd_two_d_wfrag_bytes(d.Hp)));
-        FL_TRY(pack_wfrag_bwd2d(d, w_hh, p->wfrag_b2.as<half8>(), rec_bwd_two_d_kq(d.B), s));
+        FL_TRY(pack_wfrag_bwd2d(d, w_hh, p->wfrag_b2.as<half8>(), rec_bwd_two_d_kq(d.B, d.Hp), s));
     }
     FL_TRY(hipStreamSynchronize(s));
     p->weights_packed = true;

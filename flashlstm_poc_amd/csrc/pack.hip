@@ -84,14 +84,14 @@ __global__ void pack_wfrag_bwd_kernel(Dims d, const float* __restrict__ w_hh, ha
     out[idx] = (half_t)v;
 }
 
-// Two-dimensional backward layout: [32 column slices s][kq contraction slices q][4 waves][ks k-steps][4 tiles][64 lanes][8],
-// ks = 64 / kq: lane l of tile n holds column 64 s + 16 n + l % 16 of W_hh (hidden unit k of dh = dG * W_hh^T-packed) and
-// the eight packed gate rows (8192 / kq) q + 32 (4 ks + wave) + 8 (l / 16) .. +7.
+// Two-dimensional backward layout: [Hp / 64 column slices s][kq contraction slices q][4 waves][ks k-steps][4 tiles][64 lanes][8],
+// ks = Hp / (32 kq): lane l of tile n holds column 64 s + 16 n + l % 16 of W_hh (hidden unit k of dh = dG * W_hh^T-packed)
+// and the eight packed gate rows (4 Hp / kq) q + 32 (4 ks + wave) + 8 (l / 16) .. +7.
 __global__ void pack_wfrag_bwd2d_kernel(Dims d, const float* __restrict__ w_hh, half_t* __restrict__ out, int kq) {
     const size_t idx = size_t(blockIdx.x) * kT + threadIdx.x;
     const size_t total = size_t(4) * d.Hp * d.Hp;
     if (idx >= total) return;
-    const int ksn = 64 / kq;
+    const int ksn = d.Hp / (32 * kq);   // k-steps per wave: 4 waves * ksn * 32 = 4 Hp / kq packed gate rows
     size_t r = idx;
     const int e = int(r % 8); r /= 8;
     const int lane = int(r % kWave); r /= kWave;
@@ -101,7 +101,7 @@ __global__ void pack_wfrag_bwd2d_kernel(Dims d, const float* __restrict__ w_hh, 
     const int qs = int(r % kq); r /= kq;
     const int sl = int(r);
     const int k = sl * 64 + n * 16 + lane % 16;
-    const int q = qs * (8192 / kq) + (ks * 4 + wave) * 32 + 8 * (lane / 16) + e;
+    const int q = qs * (4 * d.Hp / kq) + (ks * 4 + wave) * 32 + 8 * (lane / 16) + e;
     float v = 0.f;
     if (q < 4 * d.Hp && k < d.H) {
         const int row = torch_row(q, d.H);
@@ -234,7 +234,8 @@ hipError_t pack_weights(const Dims& d, const float* w_ih, const float* w_hh, hal
 }
 
 hipError_t pack_wfrag_bwd2d(const Dims& d, const float* w_hh, half8* out, int kq, hipStream_t s) {
-    if (d.Hp != 2048 || (kq != 4 && kq != 8)) return hipErrorInvalidValue;   // 32 slices of 64 columns, kq slices of 8192 / kq packed gate rows
+    // Hp / 64 slices of 64 columns, kq slices of 4 Hp / kq packed gate rows, 8 or 16 k-steps per wave
+    if (!((d.Hp == 2048 && (kq == 4 || kq == 8)) || (d.Hp == 1024 && kq == 2))) return hipErrorInvalidValue;
     const size_t n = size_t(4) * d.Hp * d.Hp;
     hipLaunchKernelGGL(pack_wfrag_bwd2d_kernel, dim3(grid_for(n)), dim3(kT), 0, s, d, w_hh, reinterpret_cast<half_t*>(out), kq);
     return hipGetLastError();

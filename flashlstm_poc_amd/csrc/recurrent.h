@@ -133,7 +133,7 @@ RecLayout plan_rec_bwd(int B, int Hp, int num_cus, bool force_stepwise, int forc
 // whatever the options say later), slots of its dG ring, floats per slot of its partial ring and bytes of its weight
 // fragments.
 bool rec_bwd_two_d_possible(int Hp, int num_cus);
-int rec_bwd_two_d_kq(int B);
+int rec_bwd_two_d_kq(int B, int Hp);
 int rec_bwd_dg_slots(const RecLayout& L);
 size_t rec_bwd_part_slot_floats(const RecLayout& L);
 constexpr int kRecBwdPartSlots = 3;

@@ -1082,22 +1082,25 @@ __device__ __forceinline__ rsrc_t make_rsrc(const void* p, size_t bytes) {
 __device__ __forceinline__ void order_here() { asm volatile("" ::: "memory"); }
 constexpr int kDeviceScope = 16, kNonTemporal = 2;   // cache policy of a buffer load (last argument of the builtin)
 
-// MT: 16-row tiles per row block; KQ: contraction slices; NM: passes (row blocks) a workgroup makes per step at most
-template <int MT, int KQ, int NM>
+// MT: 16-row tiles per row block; KQ: contraction slices; NM: passes (row blocks) a workgroup makes per step at most;
+// KS: k-steps per wave (4 waves * KS * 32 = 4 Hp / KQ packed gate columns); LOCAL: every group sits inside one XCD
+// (1024 hidden units: 16 column slices x 2 contraction slices = the 32 workgroups of an XCD, group = XCD) -- else the
+// groups span the XCDs (2048 hidden units: 32 column slices, 4 per XCD).
+template <int MT, int KQ, int NM, int KS, bool LOCAL>
 __global__ __launch_bounds__(kThreads) void rec_bwd2d_kernel(RecBwdArgs p, RecLayout L, int t_first, int t_last, int) {
     constexpr int NT = 4;            // 64 output columns
-    constexpr int KS = 64 / KQ;      // k-steps per wave: 4 waves * KS * 32 = 8192 / KQ packed gate columns
     constexpr int CPW = 64 / KQ;     // columns (hidden units) a workgroup finishes
     constexpr int UPT = CPW / 8;     // ... per thread: 8 threads share a row
     constexpr int PLD = 16 * NT + kPartPad;
     constexpr int RB = 16 * MT;
-    constexpr int NPF = 4;
-    // 256 KiB of weights per workgroup (KQ = 4) would take all 256 accumulation registers of a lane and leave the
-    // compiler nowhere to park what does not fit the ordinary ones: 5 of a wave's 16 k-steps live in LDS instead
+    constexpr int NPF = (UPT == 4) ? 5 : 4;   // buffer loads of load_ops
+    // 256 KiB of weights per workgroup (16 k-steps per wave) would take all 256 accumulation registers of a lane and
+    // leave the compiler nowhere to park what does not fit the ordinary ones: 5 of the 16 k-steps live in LDS instead
     // (80 KiB; with the partial sums 150 of the 160 KiB)
-    constexpr int KL = (KQ == 4) ? 5 : 0;
+    constexpr int KL = (KS == 16) ? 5 : 0;
     constexpr int KR = KS - KL;
-    static_assert(KQ == 4 || KQ == 8, "4 or 8 contraction slices");
+    static_assert(KQ == 2 || KQ == 4 || KQ == 8, "2, 4 or 8 contraction slices");
+    static_assert(KS == 8 || KS == 16, "128 or 256 KiB of weights per workgroup");
     extern __shared__ __attribute__((aligned(16))) float part_all[];  // [2][4][32][PLD] partial sums | weight fragments of the last KL k-steps
     __shared__ int lds_abort;
     __shared__ int lds_role[2];
@@ -1112,12 +1115,15 @@ __global__ __launch_bounds__(kThreads) void rec_bwd2d_kernel(RecBwdArgs p, RecLa
     }
     __syncthreads();
     if (lds_role[1] >= 32) return;
-    // seats of an XCD: [group][4 column slices][KQ contraction slices]; the workgroups of a column slice share the XCD
+    // Seats of an XCD.  LOCAL: [column slice][KQ contraction slices], the XCD is the group.  Else [group][4 column
+    // slices][KQ contraction slices].  Either way the workgroups of a column slice share the XCD.
     const int seat = __builtin_amdgcn_readfirstlane(lds_role[1]);
-    const int g = seat / (4 * KQ);
-    const int s = __builtin_amdgcn_readfirstlane(lds_role[0]) * 4 + (seat % (4 * KQ)) / KQ;
+    const int xcd_u = __builtin_amdgcn_readfirstlane(lds_role[0]);
+    const int g = LOCAL ? xcd_u : seat / (4 * KQ);
+    const int s = LOCAL ? seat / KQ : xcd_u * 4 + (seat % (4 * KQ)) / KQ;
     const int q = seat % KQ;             // contraction slice; also: which CPW columns of the slice end here
-    if (g >= L.ng) return;               // (more seats than the layout uses: cannot happen with 256 workgroups)
+    if (g >= L.ng || s * 64 >= p.Hp) return;   // (more seats than the layout uses: a group without row blocks)
+    constexpr bool device_scope = !LOCAL;      // the dG ring: plain stores reach every reader inside an XCD
     const int nks = p.Hp / 8;            // k-steps of the whole contraction
     const int nrb = L.nrb, ng = L.ng;
     const int nmine = (nrb - g + ng - 1) / ng;   // row blocks g, g + ng, ...
@@ -1157,7 +1163,7 @@ __global__ __launch_bounds__(kThreads) void rec_bwd2d_kernel(RecBwdArgs p, RecLa
     float dbacc[4][UPT] = {};
     int item = 0;
     const rsrc_t rp = make_rsrc(p.P, size_t(kRecBwdPartSlots) * p.p_slot * 4);
-    const unsigned wg_id = unsigned((g * 32 + s) * KQ);   // + receiver's q: inbox index in the partial ring
+    const unsigned wg_id = unsigned((g * (p.Hp / 64) + s) * KQ);   // + receiver's q: inbox index in the partial ring
 
     // poll bookkeeping; true = give up
     auto spin_out = [&](int& spins, long long& spin_start) -> bool {
@@ -1178,9 +1184,9 @@ __global__ __launch_bounds__(kThreads) void rec_bwd2d_kernel(RecBwdArgs p, RecLa
 
     // Per-cell operands of a row block (activated gates, c_{t-1}, c_t, dY), NPF buffer loads.
     struct Ops {
-        uintx4 g;        // UPT == 2: eight halfs; UPT == 1: .xy
-        uintx2 cp, cc;   // UPT == 1: .x
-        unsigned dy;     // UPT == 1: low half
+        uintx4 g[(UPT + 1) / 2];   // four halfs (i, f, g, o) per unit
+        uintx4 cp, cc;             // one fp32 per unit
+        uintx2 dy;                 // one half per unit
     };
     auto load_ops = [&](int t, int rb, Ops& o) {
         const int b = min(rb * RB + pr, p.B - 1);
@@ -1192,17 +1198,27 @@ __global__ __launch_bounds__(kThreads) void rec_bwd2d_kernel(RecBwdArgs p, RecLa
         const unsigned cell_idx = unsigned(b) * unsigned(p.Hp) + unsigned(j);
         const unsigned goff = (unsigned(b) * unsigned(gld) + unsigned(pq)) * 2u;
         const unsigned next = unsigned(p.B) * unsigned(p.Hp);
-        if constexpr (UPT == 2) {
-            o.g = __builtin_amdgcn_raw_buffer_load_b128(rg, goff, 0, kNonTemporal);
-            o.cp = __builtin_amdgcn_raw_buffer_load_b64(rc, cell_idx * 4u, 0, kNonTemporal);
-            o.cc = __builtin_amdgcn_raw_buffer_load_b64(rc, (cell_idx + next) * 4u, 0, kNonTemporal);
-            o.dy = __builtin_amdgcn_raw_buffer_load_b32(ry, cell_idx * 2u, 0, kNonTemporal);
+        if constexpr (UPT == 4) {
+            o.g[0] = __builtin_amdgcn_raw_buffer_load_b128(rg, goff, 0, kNonTemporal);
+            o.g[1] = __builtin_amdgcn_raw_buffer_load_b128(rg, goff + 16u, 0, kNonTemporal);
+            const uintx4 cp4 = __builtin_amdgcn_raw_buffer_load_b128(rc, cell_idx * 4u, 0, kNonTemporal);
+            const uintx4 cc4 = __builtin_amdgcn_raw_buffer_load_b128(rc, (cell_idx + next) * 4u, 0, kNonTemporal);
+            o.cp = uintx4{cp4.x, cp4.y, cp4.z, cp4.w};
+            o.cc = uintx4{cc4.x, cc4.y, cc4.z, cc4.w};
+            o.dy = __builtin_amdgcn_raw_buffer_load_b64(ry, cell_idx * 2u, 0, kNonTemporal);
+        } else if constexpr (UPT == 2) {
+            o.g[0] = __builtin_amdgcn_raw_buffer_load_b128(rg, goff, 0, kNonTemporal);
+            const uintx2 cp2 = __builtin_amdgcn_raw_buffer_load_b64(rc, cell_idx * 4u, 0, kNonTemporal);
+            const uintx2 cc2 = __builtin_amdgcn_raw_buffer_load_b64(rc, (cell_idx + next) * 4u, 0, kNonTemporal);
+            o.cp = uintx4{cp2.x, cp2.y, 0u, 0u};
+            o.cc = uintx4{cc2.x, cc2.y, 0u, 0u};
+            o.dy = uintx2{__builtin_amdgcn_raw_buffer_load_b32(ry, cell_idx * 2u, 0, kNonTemporal), 0u};
         } else {
             const uintx2 g2 = __builtin_amdgcn_raw_buffer_load_b64(rg, goff, 0, kNonTemporal);
-            o.g = uintx4{g2.x, g2.y, 0u, 0u};
-            o.cp.x = __builtin_amdgcn_raw_buffer_load_b32(rc, cell_idx * 4u, 0, kNonTemporal);
-            o.cc.x = __builtin_amdgcn_raw_buffer_load_b32(rc, (cell_idx + next) * 4u, 0, kNonTemporal);
-            o.dy = __builtin_amdgcn_raw_buffer_load_b16(ry, cell_idx * 2u, 0, kNonTemporal);
+            o.g[0] = uintx4{g2.x, g2.y, 0u, 0u};
+            o.cp = uintx4{__builtin_amdgcn_raw_buffer_load_b32(rc, cell_idx * 4u, 0, kNonTemporal), 0u, 0u, 0u};
+            o.cc = uintx4{__builtin_amdgcn_raw_buffer_load_b32(rc, (cell_idx + next) * 4u, 0, kNonTemporal), 0u, 0u, 0u};
+            o.dy = uintx2{unsigned(__builtin_amdgcn_raw_buffer_load_b16(ry, cell_idx * 2u, 0, kNonTemporal)), 0u};
         }
     };
     // the cell update of (t, pass i: row block rb) given dh from the product (or dHn), and everything it stores
@@ -1222,11 +1238,14 @@ __global__ __launch_bounds__(kThreads) void rec_bwd2d_kernel(RecBwdArgs p, RecLa
         }
         half_t* xout = p.X + size_t((t + 8) & (kDgSlots - 1)) * p.x_slot;     // dG_t for everybody
         half_t* xmark = p.X + size_t((t + 11) & (kDgSlots - 1)) * p.x_slot;   // dG_{t+3}: read by nobody any more
-        unsigned off = 0;
+        // position of every unit's four gate columns in the fragment-major ring: eight columns (two units) are
+        // contiguous, the next eight belong to another lane of the fragment
+        unsigned off[UPT] = {};
         if (row_used) {
-            off = unsigned(xch_offset(b, int(pq), nks));   // 4 * UPT consecutive halfs: one 8-byte group per unit
 #pragma unroll
-            for (int u = 0; u < UPT; ++u) store_xch(xmark + off + 4 * u, Pack<4>{uintx2{kUnwritten, kUnwritten}}, true);
+            for (int u = 0; u < UPT; ++u) off[u] = unsigned(xch_offset(b, int(pq) + 4 * u, nks));
+#pragma unroll
+            for (int u = 0; u < UPT; ++u) store_xch(xmark + off[u], Pack<4>{uintx2{kUnwritten, kUnwritten}}, device_scope);
         }
         Pack<4> out[UPT];
 #pragma unroll
@@ -1235,12 +1254,16 @@ __global__ __launch_bounds__(kThreads) void rec_bwd2d_kernel(RecBwdArgs p, RecLa
 #pragma unroll
             for (int u = 0; u < UPT; ++u) {
                 float gate[4];
-                unpack(Pack<4>{u == 0 ? uintx2{o.g.x, o.g.y} : uintx2{o.g.z, o.g.w}}, gate);
+                const uintx4 gw = o.g[u / 2];
+                unpack(Pack<4>{(u % 2) == 0 ? uintx2{gw.x, gw.y} : uintx2{gw.z, gw.w}}, gate);
                 float dyl, dyh;
-                unpack_h2(o.dy, dyl, dyh);
-                const float dyv = (u == 0) ? dyl : dyh;
-                const float pcp = __builtin_bit_cast(float, u == 0 ? o.cp.x : o.cp.y);
-                const float pcc = __builtin_bit_cast(float, u == 0 ? o.cc.x : o.cc.y);
+                unpack_h2((u / 2) == 0 ? o.dy.x : o.dy.y, dyl, dyh);
+                const float dyv = (u % 2) == 0 ? dyl : dyh;
+                // (components picked by name: indexing a vector member through the reference gave wrong lanes)
+                const unsigned cpw = (u == 0) ? o.cp.x : (u == 1) ? o.cp.y : (u == 2) ? o.cp.z : o.cp.w;
+                const unsigned ccw = (u == 0) ? o.cc.x : (u == 1) ? o.cc.y : (u == 2) ? o.cc.z : o.cc.w;
+                const float pcp = __builtin_bit_cast(float, cpw);
+                const float pcc = __builtin_bit_cast(float, ccw);
                 const float ig = gate[0], fg = gate[1], gg = gate[2], og_ = gate[3];
                 const float dhu = dh[u] + S * dyv;
                 const float tc = tanhf_dev(pcc);
@@ -1261,13 +1284,19 @@ __global__ __launch_bounds__(kThreads) void rec_bwd2d_kernel(RecBwdArgs p, RecLa
         }
         if (row_used) {
 #pragma unroll
-            for (int u = 0; u < UPT; ++u) store_xch(xout + off + 4 * u, out[u], true);
+            for (int u = 0; u < UPT; ++u) store_xch(xout + off[u], out[u], device_scope);
         }
         clk.lap(2);
         if (live) {
             half_t* dst = p.dG + (size_t(t) * p.B + b) * gld + pq;
-            if constexpr (UPT == 2) __builtin_nontemporal_store(uintx4{out[0].v.x, out[0].v.y, out[1].v.x, out[1].v.y}, reinterpret_cast<uintx4*>(dst));
-            else st_pack(dst, out[0]);
+            if constexpr (UPT == 1) {
+                st_pack(dst, out[0]);
+            } else {
+#pragma unroll
+                for (int u = 0; u < UPT; u += 2)
+                    __builtin_nontemporal_store(uintx4{out[u].v.x, out[u].v.y, out[u + 1].v.x, out[u + 1].v.y},
+                                                reinterpret_cast<uintx4*>(dst + 4 * u));
+            }
         }
         clk.lap(3);
     };
@@ -1320,7 +1349,9 @@ __global__ __launch_bounds__(kThreads) void rec_bwd2d_kernel(RecBwdArgs p, RecLa
                     for (int n = 0; n < NT; ++n) acc[m][n] = floatx4{0.f, 0.f, 0.f, 0.f};
                 const half_t* a0 = xin + (size_t(MT * rb) * nks + size_t(q) * (KS * 4)) * 512 + lane * 8;
                 const half_t* a1 = a0 + size_t(nks) * 512;
-                wave_product<NT, KS, true, KL, NPF, MT, (KS >= 16 ? 5 : 2), (KS >= 16 ? 2 : 0)>(acc, wreg, wlds, nullptr, a0, a1, wave, lane, KS * 4, KS, 0, poll,
+                // (where the operand comes through memory -- groups that span XCDs -- and the contraction is long, five
+                // short fragment sets keep the fetch running over that trip)
+                wave_product<NT, KS, true, KL, NPF, MT, ((KS >= 16 && !LOCAL) ? 5 : 2), ((KS >= 16 && !LOCAL) ? 2 : 0)>(acc, wreg, wlds, nullptr, a0, a1, wave, lane, KS * 4, KS, 0, poll,
                                                        [&]() { load_ops(t, rb, ops[i & 1]); });
                 clk.lap(0);
                 spill_partials<NT, MT>(part, acc, wave, lane, PLD);
@@ -1388,7 +1419,7 @@ __global__ __launch_bounds__(kThreads) void rec_bwd2d_kernel(RecBwdArgs p, RecLa
                     }
                     const bool hi1 = (lane & 1) != 0;
                     dh[0] = (hi1 ? a2[1] : a2[0]) + __shfl_xor(hi1 ? a2[0] : a2[1], 1);
-                } else {
+                } else if constexpr (KQ == 4) {
                     const bool hi2 = (lane & 2) != 0;
 #pragma unroll
                     for (int k = 0; k < 4; ++k) {
@@ -1402,6 +1433,14 @@ __global__ __launch_bounds__(kThreads) void rec_bwd2d_kernel(RecBwdArgs p, RecLa
                         dh[k] = keep + __shfl_xor(send, 1);
                     }
                     (void)a2;
+                } else {
+                    const bool hi1 = (lane & 1) != 0;
+#pragma unroll
+                    for (int k = 0; k < 4; ++k) {
+                        const float keep = hi1 ? f1[k] : f0[k], send = hi1 ? f0[k] : f1[k];
+                        dh[k] = keep + __shfl_xor(send, 1);
+                    }
+                    (void)a4; (void)a2;
                 }
                 cell(t, rb_prev, dcreg[i >= 1 ? i - 1 : 0], dh, ops[(i + 1) & 1]);
             }
@@ -1545,18 +1584,20 @@ RecLayout plan_rec_bwd(int B, int Hp, int num_cus, bool force_stepwise, int forc
     // weights depend on it.
     L.rot_div = (L.nh > 32) ? 8 : 0;
     if (two_d > 0 && L.persistent && rec_bwd_two_d_possible(Hp, num_cus)) {
-        const int mt = (B <= 16 && force_mt != 2) ? 1 : 2;
+        const int mt = (B <= 16 && force_mt != 2 && Hp == 2048) ? 1 : 2;
         const int nrb = int(ceil_div(size_t(B), size_t(16 * mt)));
-        const int kq = rec_bwd_two_d_kq(B);
-        const int ng = kq == 8 ? 1 : 2;
+        const int kq = rec_bwd_two_d_kq(B, Hp);
+        const int ng = Hp == 1024 ? 8 : (kq == 8 ? 1 : 2);
         const int per_wg = int(ceil_div(size_t(nrb), size_t(ng)));   // passes per step and workgroup
-        // One row block per step: 8 contraction slices, every workgroup on that block (4.0 against 6.5 us per step at
-        // 16 rows).  More: 4 slices and two groups that take alternate row blocks.  two_d = 1 takes the layout where
-        // it measured faster than the one-way layout, two_d = 2 wherever it can run (at most 2 passes per workgroup,
-        // i.e. 128 rows: a kernel unrolled for 4 passes does not fit the registers).
-        // Measured, us per backward step, one-way -> two-way: 16 rows 5.4 -> 4.0, 32 rows 5.8 -> 4.2, 64 rows 7.5 -> 7.6,
-        // 128 rows 12.4 -> 9.8.
-        const bool faster = (nrb != 2);
+        // 2048 units.  One row block per step: 8 contraction slices, every workgroup on that block.  More: 4 slices and
+        // two groups that take alternate row blocks.  Measured, us per backward step, one-way -> two-way: 16 rows
+        // 5.4 -> 4.0, 32 rows 5.8 -> 4.2, 64 rows 7.5 -> 7.6, 128 rows 12.4 -> 9.8.
+        // 1024 units: 16 column slices x 2 contraction slices inside every XCD, the XCD's row blocks in turn.  Measured
+        // slower than the one-way layout (256 rows: 5.3 -> 5.9 us per step; 512 rows: 10.7 -> 11.2): inside an XCD the
+        // step waits on the trips through the L2, not on the amount fetched, and the second exchange adds one.
+        // two_d = 1 takes the layout where it measured faster than the one-way layout, two_d = 2 wherever it can run
+        // (at most 2 passes per workgroup: a kernel unrolled for 4 does not fit the registers).
+        const bool faster = Hp == 2048 && nrb != 2;
         if (per_wg <= 2 && (two_d >= 2 || faster)) {
             L.two_d = 1;
             L.kq = kq;
@@ -1572,11 +1613,11 @@ RecLayout plan_rec_bwd(int B, int Hp, int num_cus, bool force_stepwise, int forc
     return L;
 }
 
-bool rec_bwd_two_d_possible(int Hp, int num_cus) { return Hp == 2048 && num_cus == 256; }
+bool rec_bwd_two_d_possible(int Hp, int num_cus) { return (Hp == 2048 || Hp == 1024) && num_cus == 256; }
 // Up to two row blocks: 8 slices and one group (with two blocks every workgroup makes two passes per step, and one
 // block's trip through memory hides behind the other's product: 7.0 us per step at 64 rows against 8.0 with 4 slices and
 // two groups of one pass each).  More: 4 slices, two groups.
-int rec_bwd_two_d_kq(int B) { return B <= 64 ? 8 : 4; }
+int rec_bwd_two_d_kq(int B, int Hp) { return Hp == 1024 ? 2 : (B <= 64 ? 8 : 4); }
 int rec_bwd_dg_slots(const RecLayout& L) { return L.two_d ? kDgSlots : 4; }
 size_t rec_bwd_part_slot_floats(const RecLayout& L) {
     // [256 workgroups][nm passes][kq senders][rows][64 / kq columns]
@@ -1704,10 +1745,10 @@ static hipError_t run_bwd(const RecLayout& L, const RecBwdArgs& a, hipStream_t s
                         });
 }
 
-template <int MT, int KQ, int NM>
+template <int MT, int KQ, int NM, int KS, bool LOCAL>
 static hipError_t run_bwd2d(const RecLayout& L, const RecBwdArgs& a, hipStream_t stream) {
-    auto kernel = rec_bwd2d_kernel<MT, KQ, NM>;
-    constexpr int KL = (KQ == 4) ? 5 : 0;   // k-steps per wave whose weights live in LDS (as in the kernel)
+    auto kernel = rec_bwd2d_kernel<MT, KQ, NM, KS, LOCAL>;
+    constexpr int KL = (KS == 16) ? 5 : 0;   // k-steps per wave whose weights live in LDS (as in the kernel)
     const size_t lds = size_t(2) * 4 * kRows * (64 + kPartPad) * sizeof(float) + size_t(4) * KL * 4 * kWave * sizeof(half8);
     hipError_t e = raise_lds(kernel, lds);
     if (e != hipSuccess) return e;
@@ -1719,16 +1760,23 @@ hipError_t launch_rec_bwd(const RecLayout& L, const RecBwdArgs& a, hipStream_t s
     if (a.Hp % 32 != 0 || a.Hp % L.jb != 0 || a.t_lo < -1 || a.t_hi >= a.T) return hipErrorInvalidValue;
     if (L.two_d) {
         // what the kernel's indexing assumes
-        const int ng = L.kq == 8 ? 1 : 2;
-        if (!L.persistent || a.Hp != 2048 || L.grid != 256 || (L.kq != 4 && L.kq != 8) || L.ng != ng || L.nrb < 1 ||
+        const bool local = a.Hp == 1024;
+        const int ng = local ? 8 : (L.kq == 8 ? 1 : 2);
+        if (!L.persistent || (a.Hp != 2048 && a.Hp != 1024) || L.grid != 256 || L.ng != ng || L.nrb < 1 ||
             (L.nrb + ng - 1) / ng > L.nm || !a.wfrag2 || !a.P || L.nrb * 16 * L.mt < a.B ||
-            a.p_slot != rec_bwd_part_slot_floats(L))
+            a.p_slot != rec_bwd_part_slot_floats(L) || (a.Hp / 64) * L.kq * ng != 256)
             return hipErrorInvalidValue;
-        if (L.kq == 8 && L.nm == 1) return L.mt == 1 ? run_bwd2d<1, 8, 1>(L, a, stream) : run_bwd2d<2, 8, 1>(L, a, stream);
-        if (L.kq == 8 && L.nm == 2 && L.mt == 2) return run_bwd2d<2, 8, 2>(L, a, stream);
+        if (local) {
+            if (L.kq == 2 && L.mt == 2 && L.nm == 1) return run_bwd2d<2, 2, 1, 16, true>(L, a, stream);
+            if (L.kq == 2 && L.mt == 2 && L.nm == 2) return run_bwd2d<2, 2, 2, 16, true>(L, a, stream);
+            return hipErrorInvalidValue;
+        }
+        if (L.kq == 8 && L.nm == 1)
+            return L.mt == 1 ? run_bwd2d<1, 8, 1, 8, false>(L, a, stream) : run_bwd2d<2, 8, 1, 8, false>(L, a, stream);
+        if (L.kq == 8 && L.nm == 2 && L.mt == 2) return run_bwd2d<2, 8, 2, 8, false>(L, a, stream);
         if (L.kq == 4 && L.mt == 2) {
-            if (L.nm == 1) return run_bwd2d<2, 4, 1>(L, a, stream);
-            if (L.nm == 2) return run_bwd2d<2, 4, 2>(L, a, stream);
+            if (L.nm == 1) return run_bwd2d<2, 4, 1, 16, false>(L, a, stream);
+            if (L.nm == 2) return run_bwd2d<2, 4, 2, 16, false>(L, a, stream);
         }
         return hipErrorInvalidValue;
     }
