@@ -147,6 +147,21 @@ def test_chunked_streaming_gives_the_whole_sequence_results(shape, monkeypatch):
             assert rell2(out["db"], whole["db"]) < 1e-6   # summed per launch, then over launches
 
 
+def test_chunked_streaming_with_the_grouped_two_way_backward_layout(monkeypatch):
+    # 2048 hidden units and 96 batch rows: the backward recurrence runs in two groups of workgroups that take alternate
+    # row blocks (one group makes two passes per step, the other one), fed here in ranges of 1, 2 and 5 steps.  The
+    # rings, the running dc and the bias sums have to carry over from launch to launch exactly.
+    p = make_problem(6, 96, 32, 2048, seed=12)
+    monkeypatch.setenv("FLASHLSTM_V2_CHUNK_STEPS", "0")
+    whole = run_v2(p, R=3)
+    for chunk in ("1", "2", "5"):
+        monkeypatch.setenv("FLASHLSTM_V2_CHUNK_STEPS", chunk)
+        out = run_v2(p, R=3, fresh_backward=(chunk == "2"))
+        for k in ("y", "hn", "cn", "ck_h", "ck_c", "dx", "dh0", "dc0", "dw_ih", "dw_hh"):
+            np.testing.assert_array_equal(out[k], whole[k], err_msg=f"chunk {chunk} {k}")
+        assert rell2(out["db"], whole["db"]) < 1e-6
+
+
 @pytest.mark.parametrize("shape,R,window", [((23, 3, 12, 20), 4, 5), ((23, 3, 12, 20), 7, 8), ((23, 3, 12, 20), 50, 6),
                                             ((70, 40, 64, 256), 16, 32), ((33, 5, 16, 24), 1, 11)])
 def test_windows_smaller_than_the_sequence_give_the_whole_sequence_results(shape, R, window, monkeypatch):
