@@ -1593,12 +1593,13 @@ RecLayout plan_rec_bwd(int B, int Hp, int num_cus, bool force_stepwise, int forc
         // two groups that take alternate row blocks.  Measured, us per backward step, one-way -> two-way: 16 rows
         // 5.4 -> 4.0, 32 rows 5.8 -> 4.2, 64 rows 7.5 -> 7.6, 128 rows 12.4 -> 9.8.
         // 1024 units: 16 column slices x 2 contraction slices inside every XCD, the XCD's row blocks in turn.  Measured
-        // slower than the one-way layout (256 rows: 5.3 -> 5.9 us per step; 512 rows: 10.7 -> 11.2): inside an XCD the
+        // slower than the one-way layout (256 rows: 5.3 -> 5.9 us per step; 512 rows: with two passes 10.7 -> 11.2): inside an XCD the
         // step waits on the trips through the L2, not on the amount fetched, and the second exchange adds one.
         // two_d = 1 takes the layout where it measured faster than the one-way layout, two_d = 2 wherever it can run
-        // (at most 2 passes per workgroup: a kernel unrolled for 4 does not fit the registers).
+        // (2048 units: at most 2 passes per workgroup, a kernel unrolled for 4 does not fit the registers; 1024 units,
+        // four cells per thread: one pass, i.e. 256 rows).
         const bool faster = Hp == 2048 && nrb != 2;
-        if (per_wg <= 2 && (two_d >= 2 || faster)) {
+        if (per_wg <= (Hp == 2048 ? 2 : 1) && (two_d >= 2 || faster)) {
             L.two_d = 1;
             L.kq = kq;
             L.nm = per_wg;
@@ -1768,7 +1769,6 @@ hipError_t launch_rec_bwd(const RecLayout& L, const RecBwdArgs& a, hipStream_t s
             return hipErrorInvalidValue;
         if (local) {
             if (L.kq == 2 && L.mt == 2 && L.nm == 1) return run_bwd2d<2, 2, 1, 16, true>(L, a, stream);
-            if (L.kq == 2 && L.mt == 2 && L.nm == 2) return run_bwd2d<2, 2, 2, 16, true>(L, a, stream);
             return hipErrorInvalidValue;
         }
         if (L.kq == 8 && L.nm == 1)

@@ -56,8 +56,8 @@ int flstm_core_destroy(flstm_core_plan* plan);
  * demoted direction, "stepwise" -- the launches of a range of steps are captured into a hipGraph on first use and
  * replayed afterwards, when the stream allows capture; 0 = plain launches; FLASHLSTM_STEP_GRAPHS sets the default),
  * "bwd_two_d" (backward recurrence on a 256-CU device: the layout that splits the product over output columns and
- * over the contraction and sums partial products through a second ring, for 2048 or 1024 padded hidden units and at most
- * two row blocks of 32 rows per workgroup and step; 0 = never, 1 = where it measured faster than the one-way layout
+ * over the contraction and sums partial products through a second ring, for 2048 padded hidden units and at most 128
+ * batch rows or 1024 and at most 256; 0 = never, 1 = where it measured faster than the one-way layout
  * (2048 units with at most 32 or with 65..128 batch rows), 2 = wherever it can run; default 1, FLASHLSTM_BWD_TWO_D sets
  * the default),
  * "inject_stall" (test hook: the next N passes that use a persistent kernel are treated as if that launch had
