@@ -172,6 +172,12 @@ __device__ __forceinline__ void wait_frags(half8 (&a)[8]) {
                  : "memory");
 }
 
+// Which of a wave's KS k-steps keep their weight fragments in LDS (KL of them, spread evenly) and where the others sit
+// in the register array.
+__host__ __device__ constexpr int wlds_before(int ks, int KS, int KL) { return ks * KL / KS; }          // LDS k-steps below ks
+__host__ __device__ constexpr bool wlds_has(int ks, int KS, int KL) { return wlds_before(ks + 1, KS, KL) > wlds_before(ks, KS, KL); }
+__host__ __device__ constexpr int wreg_slot(int ks, int KS, int KL) { return ks - wlds_before(ks, KS, KL); }
+
 // The same product for row blocks of two 16-row tiles whose producers publish the tiles one after the other (the
 // pointwise stage of a step handles rows 0..15 first, stores them, then rows 16..31): all k-steps of tile 0 are
 // fetched and multiplied before tile 1 is touched, so the first half of a step's product runs while the peers are
@@ -245,13 +251,12 @@ __device__ __forceinline__ void wave_product_tiles(floatx4 (&acc)[2][NT], const 
         }
 #pragma unroll
         for (int k = 0; k < CKT; ++k) {
-            constexpr int KR = KS - KL;
             const int ks = (c % NCHK) * CKT + k;
 #pragma unroll
             for (int n = 0; n < NT; ++n) {
                 half8 w;
-                if (ks < KR) w = wreg[ks < KR ? ks : 0][n];
-                else w = wlds[((ks - KR) * NT + n) * kWave + lane];
+                if (!wlds_has(ks, KS, KL)) w = wreg[wreg_slot(ks, KS, KL)][n];
+                else w = wlds[(wlds_before(ks, KS, KL) * NT + n) * kWave + lane];
                 acc[c / NCHK][n] = __builtin_amdgcn_mfma_f32_16x16x32_f16(w, f[buf][k], acc[c / NCHK][n], 0, 0, 0);
             }
         }
@@ -261,9 +266,12 @@ __device__ __forceinline__ void wave_product_tiles(floatx4 (&acc)[2][NT], const 
 // acc[mt][nt] += (A(16*MT rows x K) * Wslice)^T, this wave's interleaved k-steps only.
 // a0/a1: fragment (row tile, k-step 0) of the two 16-row tiles, already offset by lane*8 halfs; with MT = 1
 // (batches of at most 16 rows) the second tile is neither fetched nor multiplied.
-// The last KL of a wave's KS k-steps keep their weight fragments in LDS instead of registers (wlds:
-// this wave's [KL][NT][64 lanes] block); reading them back costs a few ds_read_b128 per step and frees
-// 4*KL*NT registers for fragments in flight.
+// KL of a wave's KS k-steps keep their weight fragments in LDS instead of registers (wlds: this wave's [KL][NT][64
+// lanes] block), which frees 4*KL*NT registers for fragments in flight.  They are spread evenly over the k-steps
+// (wlds_has), so that every chunk holds at most its share of them and their ds_read_b128 can be issued before the
+// chunk's wait for its fragments: read just in time, in front of the MFMA that needs them, each costs an LDS round
+// trip (~100 clocks) of a wave that has nothing else to run.
+
 // `prefetch` issues exactly NPF vector loads (for every wave, whatever its lanes need) behind the last
 // fragment load.
 template <int NT, int KS, bool RESIDENT, int KL, int NPF, int MT, int NBUF = 2, int CKO = 0, typename Prefetch>
@@ -306,6 +314,15 @@ __device__ __forceinline__ void wave_product(floatx4 (&acc)[2][NT], const half8 
                 issue(c + D, (c + D) % NBUF);
                 if (c + D == NCH - 1) prefetch();
             }
+            // this chunk's weight fragments that live in LDS: requested now, they arrive while the wave waits for the
+            // chunk's operand fragments
+            half8 wl[CK][NT];
+#pragma unroll
+            for (int k = 0; k < CK; ++k)
+                if (wlds_has(c * CK + k, KS, KL)) {
+#pragma unroll
+                    for (int n = 0; n < NT; ++n) wl[k][n] = wlds[(wlds_before(c * CK + k, KS, KL) * NT + n) * kWave + lane];
+                }
             // requested after chunk c by now: the chunks up to c + D (or the last one), and the prefetch once the last
             // chunk is out (c, D, NCH are compile-time constants: the switch folds)
             const int last_now = (c + D < NCH - 1) ? c + D : NCH - 1;
@@ -360,13 +377,12 @@ __device__ __forceinline__ void wave_product(floatx4 (&acc)[2][NT], const half8 
             }
 #pragma unroll
             for (int k = 0; k < CK; ++k) {
-                constexpr int KR = KS - KL;
                 const int ks = c * CK + k;
 #pragma unroll
                 for (int n = 0; n < NT; ++n) {
                     half8 w;
-                    if (ks < KR) w = wreg[ks < KR ? ks : 0][n];
-                    else w = wlds[((ks - KR) * NT + n) * kWave + lane];
+                    if (wlds_has(ks, KS, KL)) w = wl[k][n];
+                    else w = wreg[wreg_slot(ks, KS, KL)][n];
                     acc[0][n] = __builtin_amdgcn_mfma_f32_16x16x32_f16(w, fa[buf][k], acc[0][n], 0, 0, 0);
                     if constexpr (MT == 2)
                         acc[1][n] = __builtin_amdgcn_mfma_f32_16x16x32_f16(w, fb[buf][k], acc[1][n], 0, 0, 0);
@@ -837,20 +853,17 @@ __global__ __launch_bounds__(kThreads) void rec_bwd_kernel(RecBwdArgs p, RecLayo
 
     const half8* wfrag_wave = p.wfrag + (size_t(hs) * 4 + wave) * size_t(ks_wave) * NT * kWave;
     half8 wreg[KR][NT];
-    // LDS: [partials 2*4*32*PLD floats | weight fragments of the last KL k-steps, one block per wave]
+    // LDS: [partials 2*4*32*PLD floats | weight fragments of KL k-steps (wlds_has), one block per wave]
     half8* wlds = reinterpret_cast<half8*>(part_all + 2 * 4 * kRows * PLD) + size_t(wave) * KL * NT * kWave;
     if constexpr (RESIDENT) {
 #pragma unroll
-        for (int k = 0; k < KR; ++k)
+        for (int k = 0; k < KS; ++k)
 #pragma unroll
-            for (int n = 0; n < NT; ++n)
-                wreg[k][n] = (k < ks_wave) ? wfrag_wave[(size_t(k) * NT + n) * kWave + lane] : half8{};
-#pragma unroll
-        for (int k = 0; k < KL; ++k)
-#pragma unroll
-            for (int n = 0; n < NT; ++n)
-                wlds[(k * NT + n) * kWave + lane] =
-                    (KR + k < ks_wave) ? wfrag_wave[(size_t(KR + k) * NT + n) * kWave + lane] : half8{};
+            for (int n = 0; n < NT; ++n) {
+                const half8 w = (k < ks_wave) ? wfrag_wave[(size_t(k) * NT + n) * kWave + lane] : half8{};
+                if (wlds_has(k, KS, KL)) wlds[(wlds_before(k, KS, KL) * NT + n) * kWave + lane] = w;
+                else wreg[wreg_slot(k, KS, KL)][n] = w;
+            }
     }
 
     const size_t gld = size_t(4) * p.Hp;
@@ -1136,13 +1149,13 @@ __global__ __launch_bounds__(kThreads) void rec_bwd2d_kernel(RecBwdArgs p, RecLa
     {
         const half8* wf = p.wfrag2 + ((size_t(s) * KQ + q) * 4 + wave) * size_t(KS) * NT * kWave;
 #pragma unroll
-        for (int k = 0; k < KR; ++k)
+        for (int k = 0; k < KS; ++k)
 #pragma unroll
-            for (int n = 0; n < NT; ++n) wreg[k][n] = wf[(k * NT + n) * kWave + lane];
-#pragma unroll
-        for (int k = 0; k < KL; ++k)
-#pragma unroll
-            for (int n = 0; n < NT; ++n) wlds[(k * NT + n) * kWave + lane] = wf[((KR + k) * NT + n) * kWave + lane];
+            for (int n = 0; n < NT; ++n) {
+                const half8 w = wf[(k * NT + n) * kWave + lane];
+                if (wlds_has(k, KS, KL)) wlds[(wlds_before(k, KS, KL) * NT + n) * kWave + lane] = w;
+                else wreg[wreg_slot(k, KS, KL)][n] = w;
+            }
     }
 
     // As a sender a thread sums row pr, columns 8*pj .. 8*pj+7 of the partial; as a receiver it collects the 8 columns
