@@ -1156,6 +1156,16 @@ __global__ __launch_bounds__(kThreads) void rec_bwd2d_kernel(RecBwdArgs p, RecLa
                 if (wlds_has(k, KS, KL)) wlds[(wlds_before(k, KS, KL) * NT + n) * kWave + lane] = w;
                 else wreg[wreg_slot(k, KS, KL)][n] = w;
             }
+        // The weights belong in accumulation registers for the whole launch (an MFMA reads its operands from either
+        // file).  Said outright: left to itself the register allocator keeps them in ordinary registers, runs out,
+        // parks them in accumulation registers as spilled values and copies each back in front of every MFMA that
+        // uses it (4 copies per 2 MFMAs, a fifth of a pass's vector instructions).
+        if constexpr (KS >= 16) {
+#pragma unroll
+            for (int k = 0; k < KR; ++k)
+#pragma unroll
+                for (int n = 0; n < NT; ++n) asm volatile("" : "+a"(wreg[k][n]));
+        }
     }
 
     // As a sender a thread sums row pr, columns 8*pj .. 8*pj+7 of the partial; as a receiver it collects the 8 columns
