@@ -96,6 +96,12 @@ __device__ __forceinline__ Role make_role(int nh, int ng, int gpx, int xcd_local
 // Pattern that marks a not-yet-written pair of halfs in the exchange ring.
 constexpr unsigned kUnwritten = 0xFFFFFFFFu;
 
+// The abort flag of a workgroup is addressed as LDS, not through a generic pointer: a generic access is a FLAT
+// instruction, which may complete out of order with the vector-memory loads, so with one anywhere in a reload loop the
+// compiler ends the loop with a wait for ALL outstanding loads -- the chunk requested ahead included -- and the
+// prefetch distance of the products collapses to nothing.
+typedef __attribute__((address_space(3))) int lds_int_t;
+
 // How a persistent launch validates what it fetches (off for step-wise launches, where the kernel
 // boundary orders memory).
 struct Poll {
@@ -103,8 +109,32 @@ struct Poll {
     int limit;        // reloads of one fragment chunk before the launch gives up ...
     long long ticks;  // ... or this many ticks of the constant-rate wall clock spent reloading it, whichever comes first
     int* status;      // global: 1 = gave up
-    int* lds_abort;   // workgroup: some wave gave up
+    lds_int_t* lds_abort;   // workgroup: some wave gave up
 };
+
+// Said before a step loop: every load issued so far (the weight fragments, the state) has landed.  As an instruction
+// the compiler knows, not inline assembly: otherwise it meets the loop with loads it believes outstanding and puts
+// its own wait for ALL loads in front of the first MFMA of every step, behind the fragments requested ahead.
+__device__ __forceinline__ void loads_landed() { __builtin_amdgcn_s_waitcnt(0x0F70); }   // vmcnt(0), the other counters left alone
+
+// Bookkeeping of one more reload of something that has not arrived; true = give up (the caller leaves its reload
+// loop with garbage, and the workgroup leaves the kernel at its next barrier).  The clock and the global status word
+// are looked at every 256th reload only.
+__device__ __forceinline__ bool poll_give_up(const Poll& poll, int& spins, long long& spin_start, int lane) {
+    ++spins;
+    if (spins == 1) spin_start = wall_clock64();
+    if (spins > poll.limit || *static_cast<volatile lds_int_t*>(poll.lds_abort) != 0 ||
+        ((spins & 255) == 0 &&
+         (wall_clock64() - spin_start > poll.ticks ||
+          __hip_atomic_load(poll.status, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0))) {
+        if (lane == 0) {
+            __hip_atomic_store(poll.status, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            *static_cast<volatile lds_int_t*>(poll.lds_abort) = 1;
+        }
+        return true;
+    }
+    return false;
+}
 
 // Exchange layout ("fragment-major").  The operand a step fetches from its peers -- h_{t-1} in the
 // forward pass, dG_{t+1} in the backward pass -- is stored as ready-made MFMA A-fragments so that
@@ -222,32 +252,27 @@ __device__ __forceinline__ void wave_product_tiles(floatx4 (&acc)[2][NT], const 
             case 2 * CKT: wait_frags<2 * CKT>(f[buf]); break;
             default: wait_frags<0>(f[buf]); break;
         }
-        if (poll.on) {
+        // A pair of halfs that still holds the pattern has not been written yet by its producer: fetch the chunk
+        // again (whatever was in flight behind it lands first, loads return in order).  The decision is wave-uniform.
+        // The check is peeled out of the reload loop: a chunk that is complete -- nearly all of them -- then costs the
+        // comparison and ONE branch that is not taken; every taken branch stalls a wave that has its SIMD to itself.
+        auto unwritten = [&]() -> bool {
+            unsigned m = 0u;
+#pragma unroll
+            for (int k = 0; k < CKT; ++k) {
+                const uint4 ua = __builtin_bit_cast(uint4, f[buf][k]);
+                m = max(m, max(max(ua.x, ua.y), max(ua.z, ua.w)));
+            }
+            return __any(m == kUnwritten) != 0;
+        };
+        if (__builtin_expect(unwritten() && poll.on, 0)) {
             int spins = 0;
             long long spin_start = 0;
-            for (;;) {
-                unsigned m = 0u;
-#pragma unroll
-                for (int k = 0; k < CKT; ++k) {
-                    const uint4 ua = __builtin_bit_cast(uint4, f[buf][k]);
-                    m = max(m, max(max(ua.x, ua.y), max(ua.z, ua.w)));
-                }
-                if (!__any(m == kUnwritten)) break;
-                ++spins;
-                if (spins == 1) spin_start = wall_clock64();
-                if (spins > poll.limit || *reinterpret_cast<volatile int*>(poll.lds_abort) != 0 ||
-                    ((spins & 255) == 0 &&
-                     (wall_clock64() - spin_start > poll.ticks ||
-                      __hip_atomic_load(poll.status, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0))) {
-                    if (lane == 0) {
-                        __hip_atomic_store(poll.status, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                        *reinterpret_cast<volatile int*>(poll.lds_abort) = 1;
-                    }
-                    break;   // results are garbage from here on; the workgroup leaves at its next barrier
-                }
+            do {
+                if (poll_give_up(poll, spins, spin_start, lane)) break;   // results are garbage from here on; the workgroup leaves at its next barrier
                 issue(c);
                 wait_frags<0>(f[buf]);   // (whatever was in flight behind this chunk has landed as well)
-            }
+            } while (unwritten());
         }
 #pragma unroll
         for (int k = 0; k < CKT; ++k) {
@@ -340,40 +365,27 @@ __device__ __forceinline__ void wave_product(floatx4 (&acc)[2][NT], const half8 
                 default: wait(std::integral_constant<int, 4 * MT * CK + NPF>{}, buf); break;
             }
             static_assert(NBUF <= 5, "the switch above knows up to four chunks ahead");
-            if (poll.on) {
-                // A pair of halfs that still holds the pattern has not been written yet by its producer:
-                // fetch the chunk again (the chunk in flight behind it has to land first, loads return
-                // in order).  The decision is wave-uniform.
+            auto unwritten = [&]() -> bool {
+                unsigned m = 0u;
+#pragma unroll
+                for (int k = 0; k < CK; ++k) {
+                    const uint4 ua = __builtin_bit_cast(uint4, fa[buf][k]);
+                    m = max(m, max(max(ua.x, ua.y), max(ua.z, ua.w)));
+                    if constexpr (MT == 2) {
+                        const uint4 ub = __builtin_bit_cast(uint4, fb[buf][k]);
+                        m = max(m, max(max(ub.x, ub.y), max(ub.z, ub.w)));
+                    }
+                }
+                return __any(m == kUnwritten) != 0;
+            };
+            if (__builtin_expect(unwritten() && poll.on, 0)) {   // (peeled, as in wave_product_tiles)
                 int spins = 0;
                 long long spin_start = 0;
-                for (;;) {
-                    unsigned m = 0u;
-#pragma unroll
-                    for (int k = 0; k < CK; ++k) {
-                        const uint4 ua = __builtin_bit_cast(uint4, fa[buf][k]);
-                        m = max(m, max(max(ua.x, ua.y), max(ua.z, ua.w)));
-                        if constexpr (MT == 2) {
-                            const uint4 ub = __builtin_bit_cast(uint4, fb[buf][k]);
-                            m = max(m, max(max(ub.x, ub.y), max(ub.z, ub.w)));
-                        }
-                    }
-                    if (!__any(m == kUnwritten)) break;
-                    ++spins;
-                    if (spins == 1) spin_start = wall_clock64();
-                    // (the clock and the global status word are looked at every 256th reload only)
-                    if (spins > poll.limit || *reinterpret_cast<volatile int*>(poll.lds_abort) != 0 ||
-                        ((spins & 255) == 0 &&
-                         (wall_clock64() - spin_start > poll.ticks ||
-                          __hip_atomic_load(poll.status, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0))) {
-                        if (lane == 0) {
-                            __hip_atomic_store(poll.status, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                            *reinterpret_cast<volatile int*>(poll.lds_abort) = 1;
-                        }
-                        break;   // results are garbage from here on; the workgroup leaves at its next barrier
-                    }
+                do {
+                    if (poll_give_up(poll, spins, spin_start, lane)) break;
                     issue(c, buf);
                     wait(std::integral_constant<int, 0>{}, buf);   // (also what was issued after this chunk the first time)
-                }
+                } while (unwritten());
             }
 #pragma unroll
             for (int k = 0; k < CK; ++k) {
@@ -566,10 +578,16 @@ __device__ __forceinline__ void ld_f32_coherent(const float* p, float (&f)[4]) {
     f[0] = v.x; f[1] = v.y; f[2] = v.z; f[3] = v.w;
 }
 
-// Thread -> (row, group): the 8 (or 16) groups of a row go to consecutive lanes, and the rows are taken in the
-// order 0, 8, 1, 9, ...: the lanes that the LDS serves together then read the partial sums of rows
-// r and r + 8, which are 32 banks apart for every row pitch in use (132, 68, 36, 20 floats).
-__device__ __forceinline__ int group_row(int idx) { return (idx % 2) * 8 + (idx / 2) % 8 + (idx / 16) * 16; }
+// Thread -> (row, group): the 8 (or 16) groups of a row go to consecutive lanes.  The LDS serves 256 bytes per clock,
+// i.e. the lanes of TOGETHER rows at once (2 rows of 128 bytes, or 4 rows of 64 bytes where 8 threads read 8 bytes
+// each), so the rows are taken in the order 0, 8, 1, 9, ... (rows r and r + 8 are 32 banks apart for every row pitch
+// in use: 132, 68, 36, 20 floats) or 0, 4, 8, 12, 1, 5, ... (r, r + 4, r + 8, r + 12 are 16 banks apart).
+template <int TOGETHER>
+__device__ __forceinline__ int group_row(int idx) {
+    static_assert(TOGETHER == 2 || TOGETHER == 4, "rows whose lanes the LDS serves in one clock");
+    if constexpr (TOGETHER == 4) return (idx % 4) * 4 + (idx / 4) % 4 + (idx / 16) * 16;
+    return (idx % 2) * 8 + (idx / 2) % 8 + (idx / 16) * 16;
+}
 
 // Asynchronous loads of the per-step operands that come from HBM (x-projection, gate and cell caches, dY).
 // They are issued by hand, right after the LAST fragment load of a step's product: loads return in issue
@@ -637,11 +655,16 @@ struct PhaseClock {
 // off that path.
 // MT = 16-row tiles per row block: 2, or 1 for batches of at most 16 rows (the threads of rows 16..31 then only
 // keep the barriers company).
+// DEEP (2048 hidden units, 32-row blocks, several row blocks per workgroup and step): the operand comes through memory
+// from the other XCDs, and a workgroup finds a block's operand complete when it gets there (it was published a block
+// ago), so the product runs at the rate the fetch sustains: four sets of 2 k-steps in flight instead of two sets of 4
+// (measured at 128 rows: 6.9 -> 6.4 us per step).  With one block per step the product waits for its producers
+// anyway and the longer sets are the better ones (64 rows: 4.5 against 4.65 us).
 // Slices of 32 units with two row tiles run the pointwise stage in two PHASES: all 256 threads update rows 0..15
 // of the block (two units each) and store that half of h_t, then rows 16..31.  The consumers fetch and multiply
 // tile by tile (wave_product_tiles), so the second phase of a step overlaps the first half of the peers' next
 // product instead of sitting on the path from one step to the next.
-template <int NT, int KS, bool RESIDENT, int MT>
+template <int NT, int KS, bool RESIDENT, int MT, bool DEEP = false>
 __global__ __launch_bounds__(kThreads) void rec_fwd_kernel(RecFwdArgs p, RecLayout L, int t_begin,
                                                            int t_end, int ks_wave) {
     constexpr int JB = 4 * NT;    // hidden units of this slice
@@ -667,7 +690,7 @@ __global__ __launch_bounds__(kThreads) void rec_fwd_kernel(RecFwdArgs p, RecLayo
     const int rotation = __builtin_amdgcn_readfirstlane(rec_kstep_rotation(hs, L.nh, ks_wave, L.rot_div));
     const int nks_total = p.Hp / 32;
     const bool device_scope = (L.persistent != 0) && (L.xcd_local == 0);
-    const Poll poll{L.persistent != 0, p.spin_limit, p.spin_ticks, p.status, &lds_abort};
+    const Poll poll{L.persistent != 0, p.spin_limit, p.spin_ticks, p.status, (lds_int_t*)&lds_abort};
     PhaseClock clk{(blockIdx.x == 0) ? p.prof : nullptr, 0};
     int item = 0;   // work items done: selects the partial-sum buffer
 
@@ -684,7 +707,7 @@ __global__ __launch_bounds__(kThreads) void rec_fwd_kernel(RecFwdArgs p, RecLayo
     const size_t gld = size_t(4) * p.Hp;
     // this thread's groups: row pr (+ 16 in the second phase) of the row block, units pj .. pj+UPT-1 of the slice
     constexpr int RB = 16 * MT;   // batch rows of a row block
-    const int pr = group_row(tid / GPR);
+    const int pr = group_row<(GPR * UPT == 16) ? 4 : 2>(tid / GPR);
     const bool row_used = pr + 16 * (NPH - 1) < RB;   // with one row tile per block the threads of rows 16..31 only keep the barriers company
     const int pj = (tid % GPR) * UPT;
     const int j = hs * JB + pj;   // first hidden unit of the group
@@ -711,6 +734,7 @@ __global__ __launch_bounds__(kThreads) void rec_fwd_kernel(RecFwdArgs p, RecLayo
         }
     }
     __syncthreads();
+    loads_landed();
     clk.start();
 
     for (int t = t_begin; t < t_end; ++t) {
@@ -731,7 +755,7 @@ __global__ __launch_bounds__(kThreads) void rec_fwd_kernel(RecFwdArgs p, RecLayo
                 wave_product_tiles<NT, KS, 0, NPH * UPT / 2, kFwdBufs>(acc, wreg, nullptr, a0, a1, wave, lane, nks_total, ks_wave, rotation, poll,
                                                              [&]() { prefetch(t, rb); });
             else
-                wave_product<NT, KS, RESIDENT, 0, UPT / 2, MT>(acc, wreg, nullptr, wfrag_wave, a0, a1, wave, lane, nks_total,
+                wave_product<NT, KS, RESIDENT, 0, UPT / 2, MT, DEEP ? 4 : 2, DEEP ? 2 : 0>(acc, wreg, nullptr, wfrag_wave, a0, a1, wave, lane, nks_total,
                                                                ks_wave, rotation, poll, [&]() { prefetch(t, rb); });
             clk.lap(0);
             spill_partials<NT, MT>(part, acc, wave, lane, PLD);
@@ -846,7 +870,7 @@ __global__ __launch_bounds__(kThreads) void rec_bwd_kernel(RecBwdArgs p, RecLayo
     const int rotation = __builtin_amdgcn_readfirstlane(rec_kstep_rotation(hs, L.nh, ks_wave, L.rot_div));
     const int nks_total = p.Hp / 8;  // contraction over 4Hp packed gate columns
     const bool device_scope = (L.persistent != 0) && (L.xcd_local == 0);
-    const Poll poll{L.persistent != 0, p.spin_limit, p.spin_ticks, p.status, &lds_abort};
+    const Poll poll{L.persistent != 0, p.spin_limit, p.spin_ticks, p.status, (lds_int_t*)&lds_abort};
     const float S = p.dy_scale;
     PhaseClock clk{(blockIdx.x == 0) ? p.prof : nullptr, 0};
     int item = 0;   // work items done: selects the partial-sum buffer
@@ -869,7 +893,7 @@ __global__ __launch_bounds__(kThreads) void rec_bwd_kernel(RecBwdArgs p, RecLayo
     const size_t gld = size_t(4) * p.Hp;
     // this thread's group: row pr of the row block, units pj .. pj+UPT-1 of the slice
     constexpr int RB = 16 * MT;   // batch rows of a row block
-    const int pr = group_row(tid / GPR);
+    const int pr = group_row<(GPR * UPT == 16) ? 4 : 2>(tid / GPR);
     const bool row_used = pr < RB;   // with one row tile per block the threads of rows 16..31 only keep the barriers company
     const int pj = (tid % GPR) * UPT;
     const int j = hs * JB + pj;
@@ -900,6 +924,7 @@ __global__ __launch_bounds__(kThreads) void rec_bwd_kernel(RecBwdArgs p, RecLayo
     };
     __syncthreads();
     float dbacc[4][UPT] = {};
+    loads_landed();
     clk.start();
 
     for (int t = t_first; t >= t_last; --t) {
@@ -1140,7 +1165,7 @@ __global__ __launch_bounds__(kThreads) void rec_bwd2d_kernel(RecBwdArgs p, RecLa
     const int nks = p.Hp / 8;            // k-steps of the whole contraction
     const int nrb = L.nrb, ng = L.ng;
     const int nmine = (nrb - g + ng - 1) / ng;   // row blocks g, g + ng, ...
-    const Poll poll{true, p.spin_limit, p.spin_ticks, p.status, &lds_abort};
+    const Poll poll{true, p.spin_limit, p.spin_ticks, p.status, (lds_int_t*)&lds_abort};
     const float S = p.dy_scale;
     PhaseClock clk{(blockIdx.x == 0) ? p.prof : nullptr, 0};
 
@@ -1188,22 +1213,7 @@ __global__ __launch_bounds__(kThreads) void rec_bwd2d_kernel(RecBwdArgs p, RecLa
     const rsrc_t rp = make_rsrc(p.P, size_t(kRecBwdPartSlots) * p.p_slot * 4);
     const unsigned wg_id = unsigned((g * (p.Hp / 64) + s) * KQ);   // + receiver's q: inbox index in the partial ring
 
-    // poll bookkeeping; true = give up
-    auto spin_out = [&](int& spins, long long& spin_start) -> bool {
-        ++spins;
-        if (spins == 1) spin_start = wall_clock64();
-        if (spins > poll.limit || *reinterpret_cast<volatile int*>(poll.lds_abort) != 0 ||
-            ((spins & 255) == 0 &&
-             (wall_clock64() - spin_start > poll.ticks ||
-              __hip_atomic_load(poll.status, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0))) {
-            if (lane == 0) {
-                __hip_atomic_store(poll.status, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                *reinterpret_cast<volatile int*>(poll.lds_abort) = 1;
-            }
-            return true;   // results are garbage from here on; the workgroup leaves at its next barrier
-        }
-        return false;
-    };
+    auto spin_out = [&](int& spins, long long& spin_start) -> bool { return poll_give_up(poll, spins, spin_start, lane); };
 
     // Per-cell operands of a row block (activated gates, c_{t-1}, c_t, dY), NPF buffer loads.
     struct Ops {
@@ -1325,6 +1335,7 @@ __global__ __launch_bounds__(kThreads) void rec_bwd2d_kernel(RecBwdArgs p, RecLa
     };
 
     __syncthreads();
+    loads_landed();
     clk.start();
     for (int t = t_first; t >= t_last; --t) {
         if (t >= p.T - 1) {   // the last step of the sequence: dh comes from the caller
@@ -1721,9 +1732,9 @@ static hipError_t launch_steps(StepGraphCache* graphs, const void* kernel, const
     return hipGraphLaunch(exec, stream);
 }
 
-template <int NT, int KS, bool RES, int MT>
+template <int NT, int KS, bool RES, int MT, bool DEEP = false>
 static hipError_t run_fwd(const RecLayout& L, const RecFwdArgs& a, hipStream_t stream, StepGraphCache* graphs) {
-    auto kernel = rec_fwd_kernel<NT, KS, RES, MT>;
+    auto kernel = rec_fwd_kernel<NT, KS, RES, MT, DEEP>;
     const size_t lds = size_t(2) * 4 * kRows * (16 * NT + kPartPad) * sizeof(float);
     hipError_t e = raise_lds(kernel, lds);
     if (e != hipSuccess) return e;
@@ -1745,7 +1756,11 @@ hipError_t launch_rec_fwd(const RecLayout& L, const RecFwdArgs& a, hipStream_t s
     if (a.Hp % 32 != 0 || a.Hp % L.jb != 0 || a.t0 < 0 || a.t1 > a.T) return hipErrorInvalidValue;
     if (!L.resident) return run_fwd<8, 1, false, 2>(L, a, stream, graphs);
     if (L.nt == 8) return L.mt == 1 ? run_fwd<8, 8, true, 1>(L, a, stream, graphs) : run_fwd<8, 8, true, 2>(L, a, stream, graphs);
-    if (L.nt == 4) return L.mt == 1 ? run_fwd<4, 16, true, 1>(L, a, stream, graphs) : run_fwd<4, 16, true, 2>(L, a, stream, graphs);
+    if (L.nt == 4) {
+        if (L.mt == 1) return run_fwd<4, 16, true, 1>(L, a, stream, graphs);
+        const bool several_blocks = L.persistent && L.nrb >= 2 * L.ng;   // every workgroup takes at least two row blocks per step
+        return several_blocks ? run_fwd<4, 16, true, 2, true>(L, a, stream, graphs) : run_fwd<4, 16, true, 2>(L, a, stream, graphs);
+    }
     return hipErrorInvalidValue;
 }
 
