@@ -208,12 +208,35 @@ __host__ __device__ constexpr int wlds_before(int ks, int KS, int KL) { return k
 __host__ __device__ constexpr bool wlds_has(int ks, int KS, int KL) { return wlds_before(ks + 1, KS, KL) > wlds_before(ks, KS, KL); }
 __host__ __device__ constexpr int wreg_slot(int ks, int KS, int KL) { return ks - wlds_before(ks, KS, KL); }
 
+// Validation by effect.  A word of the ring that still holds the 'unwritten' pattern is a pair of fp16 NaNs, and a NaN
+// anywhere in row r of the fetched operand makes EVERY column of row r of the product NaN (NaN times anything, a zero
+// weight included, is NaN, and sums keep it).  With the operands swapped a lane holds row lane % 16 of each row tile
+// in every one of its accumulation registers, so one register per row tile tells whether the wave multiplied
+// something its producers had not written yet: two instructions per product instead of a maximum over every
+// fetched word (10 vector instructions per chunk of 4 fragments, a fifth of a step's instructions in the backward
+// kernel).  A wave still checks the FIRST chunk of a product word by word -- that is where it waits for its producers,
+// and they finish within a fraction of a microsecond of each other; if it did have to wait there, also the chunks it
+// had requested ahead by then -- multiplies the rest as it lands, and repeats
+// its part of the product with every chunk checked if the result says so (LAZY = false: checked from the start).
+// Measured, it pays only where a wave finds its operand complete when it gets there (several row blocks per workgroup
+// and step: forward at 2048 units and 128 rows 6.7 -> 6.2 us per step).  A wave that arrives ahead of its producers
+// -- one row block per step, every configuration of 1024 units -- runs into words that were fetched too early often
+// enough for the repeated products to cost more than the checks (256 rows at 1024 units, backward: 4.9 -> 5.3 us
+// per step; 64 rows at 2048 units: 7.3 -> 11.3), so those kernels keep the check of every chunk.  Values that are NaN in
+// their own right (or sums of opposite infinities) take that second pass too and come out as what they are.
+template <int MT, int NT>
+__device__ __forceinline__ bool product_poisoned(const floatx4 (&acc)[2][NT]) {
+    float probe = acc[0][0][0];
+    if constexpr (MT == 2) probe += acc[1][0][0];
+    return __any(probe != probe) != 0;
+}
+
 // The same product for row blocks of two 16-row tiles whose producers publish the tiles one after the other (the
 // pointwise stage of a step handles rows 0..15 first, stores them, then rows 16..31): all k-steps of tile 0 are
 // fetched and multiplied before tile 1 is touched, so the first half of a step's product runs while the peers are
 // still busy with the second half of their cell updates.  Chunks of CKT k-steps of ONE tile alternate between two
 // register sets (as many registers as the two-tile chunks of wave_product).  Resident weights only.
-template <int NT, int KS, int KL, int NPF, int NBUF, typename Prefetch>
+template <int NT, int KS, int KL, int NPF, int NBUF, bool LAZY = false, typename Prefetch>
 __device__ __forceinline__ void wave_product_tiles(floatx4 (&acc)[2][NT], const half8 (&wreg)[KS - KL][NT],
                                                    const half8* wlds, const half_t* a0, const half_t* a1, int wave,
                                                    int lane, int nks_total, int ks_wave, int rotation, const Poll& poll,
@@ -224,8 +247,15 @@ __device__ __forceinline__ void wave_product_tiles(floatx4 (&acc)[2][NT], const 
     constexpr int NCH = 2 * NCHK;
     static_assert(NBUF >= 2 && NBUF <= NCH, "register sets: one feeds the MFMAs, the others are in flight");
     half8 f[NBUF][CKT];
+    bool check_all = !LAZY;   // second pass: every chunk is checked word by word
+    bool early = false;
+    for (;;) {
+    // (the operand's address as a value the compiler cannot see through: the fragment addresses are then computed
+    // where they are used in every pass instead of all of them ahead of this loop, in registers that are not there)
+    const half_t *p0 = a0, *p1 = a1;
+    if constexpr (LAZY) asm volatile("" : "+v"(p0), "+v"(p1));
     auto issue = [&](int c) {
-        const half_t* base = (c / NCHK) ? a1 : a0;
+        const half_t* base = (c / NCHK) ? p1 : p0;
 #pragma unroll
         for (int k = 0; k < CKT; ++k) {
             const int kg = min(rec_kstep_of_slot((c % NCHK) * CKT + k, rotation, ks_wave) * 4 + wave, nks_total - 1);
@@ -265,14 +295,23 @@ __device__ __forceinline__ void wave_product_tiles(floatx4 (&acc)[2][NT], const 
             }
             return __any(m == kUnwritten) != 0;
         };
-        if (__builtin_expect(unwritten() && poll.on, 0)) {
-            int spins = 0;
-            long long spin_start = 0;
-            do {
-                if (poll_give_up(poll, spins, spin_start, lane)) break;   // results are garbage from here on; the workgroup leaves at its next barrier
-                issue(c);
-                wait_frags<0>(f[buf]);   // (whatever was in flight behind this chunk has landed as well)
-            } while (unwritten());
+        // LAZY: only the first chunk of a tile is checked here -- the wave waits there for its producers -- and the
+        // rest by their effect on the result (product_poisoned)
+        // (early: this tile's first chunk had to be fetched again, i.e. the wave got here before its producers; the
+        // chunks requested ahead of that moment are then checked as well)
+        const bool ahead = (c % NCHK) >= 1 && (c % NCHK) <= NBUF - 1;
+        if (c % NCHK == 0) early = false;
+        if (c % NCHK == 0 || (ahead && early) || __builtin_expect(check_all, 0)) {
+            if (__builtin_expect(unwritten() && poll.on, 0)) {
+                if (c % NCHK == 0) early = true;
+                int spins = 0;
+                long long spin_start = 0;
+                do {
+                    if (poll_give_up(poll, spins, spin_start, lane)) break;   // results are garbage from here on; the workgroup leaves at its next barrier
+                    issue(c);
+                    wait_frags<0>(f[buf]);   // (whatever was in flight behind this chunk has landed as well)
+                } while (unwritten());
+            }
         }
 #pragma unroll
         for (int k = 0; k < CKT; ++k) {
@@ -285,6 +324,20 @@ __device__ __forceinline__ void wave_product_tiles(floatx4 (&acc)[2][NT], const 
                 acc[c / NCHK][n] = __builtin_amdgcn_mfma_f32_16x16x32_f16(w, f[buf][k], acc[c / NCHK][n], 0, 0, 0);
             }
         }
+        // (chunks stay apart: without the checks between them the product is one long block, and a scheduler free to
+        // move the address arithmetic of later chunks up runs out of registers)
+        if constexpr (LAZY) __builtin_amdgcn_sched_barrier(0);
+    }
+    if (__builtin_expect(check_all || !poll.on || !product_poisoned<2>(acc), 1)) break;
+    check_all = true;
+    // Whatever this pass left in flight (the loads of `prefetch`) lands before the next one starts: that pass issues
+    // them again into registers of its own, the compiler takes the old ones for dead and hands them out -- as address
+    // registers, for one -- while the hardware still writes them.
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+#pragma unroll
+    for (int m = 0; m < 2; ++m)
+#pragma unroll
+        for (int n = 0; n < NT; ++n) acc[m][n] = floatx4{0.f, 0.f, 0.f, 0.f};
     }
 }
 
@@ -299,7 +352,7 @@ __device__ __forceinline__ void wave_product_tiles(floatx4 (&acc)[2][NT], const 
 
 // `prefetch` issues exactly NPF vector loads (for every wave, whatever its lanes need) behind the last
 // fragment load.
-template <int NT, int KS, bool RESIDENT, int KL, int NPF, int MT, int NBUF = 2, int CKO = 0, typename Prefetch>
+template <int NT, int KS, bool RESIDENT, int KL, int NPF, int MT, int NBUF = 2, int CKO = 0, bool LAZY = false, typename Prefetch>
 __device__ __forceinline__ void wave_product(floatx4 (&acc)[2][NT], const half8 (&wreg)[KS - KL][NT],
                                              const half8* wlds, const half8* wfrag_wave, const half_t* a0,
                                              const half_t* a1, int wave, int lane, int nks_total,
@@ -316,12 +369,17 @@ __device__ __forceinline__ void wave_product(floatx4 (&acc)[2][NT], const half8 
         constexpr int NCH = KS / CK;
         constexpr int D = NBUF - 1;   // chunks requested ahead of the one being multiplied
         half8 fa[NBUF][CK], fb[NBUF][CK];
+        bool check_all = !LAZY;   // second pass: every chunk is checked word by word
+        bool early = false;               // the first chunk had to be fetched again: what was requested ahead of it is checked too
+        for (;;) {
+        const half_t *p0 = a0, *p1 = a1;   // (opaque copies, as in wave_product_tiles)
+        if constexpr (LAZY) asm volatile("" : "+v"(p0), "+v"(p1));
         auto issue = [&](int c, int buf) {
 #pragma unroll
             for (int k = 0; k < CK; ++k) {
                 const int kg = min(rec_kstep_of_slot(c * CK + k, rotation, ks_wave) * 4 + wave, nks_total - 1);
-                ld_frag_async(fa[buf][k], a0 + size_t(kg) * 512);
-                if constexpr (MT == 2) ld_frag_async(fb[buf][k], a1 + size_t(kg) * 512);
+                ld_frag_async(fa[buf][k], p0 + size_t(kg) * 512);
+                if constexpr (MT == 2) ld_frag_async(fb[buf][k], p1 + size_t(kg) * 512);
             }
         };
         auto wait = [&](auto younger, int buf) {   // until at most `younger` loads issued later are outstanding
@@ -378,14 +436,17 @@ __device__ __forceinline__ void wave_product(floatx4 (&acc)[2][NT], const half8 
                 }
                 return __any(m == kUnwritten) != 0;
             };
-            if (__builtin_expect(unwritten() && poll.on, 0)) {   // (peeled, as in wave_product_tiles)
-                int spins = 0;
-                long long spin_start = 0;
-                do {
-                    if (poll_give_up(poll, spins, spin_start, lane)) break;
-                    issue(c, buf);
-                    wait(std::integral_constant<int, 0>{}, buf);   // (also what was issued after this chunk the first time)
-                } while (unwritten());
+            if (c == 0 || (c <= D && early) || __builtin_expect(check_all, 0)) {   // (peeled; first pass: as in wave_product_tiles)
+                if (__builtin_expect(unwritten() && poll.on, 0)) {
+                    if (c == 0) early = true;
+                    int spins = 0;
+                    long long spin_start = 0;
+                    do {
+                        if (poll_give_up(poll, spins, spin_start, lane)) break;
+                        issue(c, buf);
+                        wait(std::integral_constant<int, 0>{}, buf);   // (also what was issued after this chunk the first time)
+                    } while (unwritten());
+                }
             }
 #pragma unroll
             for (int k = 0; k < CK; ++k) {
@@ -400,6 +461,15 @@ __device__ __forceinline__ void wave_product(floatx4 (&acc)[2][NT], const half8 
                         acc[1][n] = __builtin_amdgcn_mfma_f32_16x16x32_f16(w, fb[buf][k], acc[1][n], 0, 0, 0);
                 }
             }
+            if constexpr (LAZY) __builtin_amdgcn_sched_barrier(0);   // (chunks stay apart, as in wave_product_tiles)
+        }
+        if (__builtin_expect(check_all || !poll.on || !product_poisoned<MT>(acc), 1)) break;
+        check_all = true;
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // (as in wave_product_tiles: nothing in flight into registers the next pass reuses)
+#pragma unroll
+        for (int m = 0; m < 2; ++m)
+#pragma unroll
+            for (int n = 0; n < NT; ++n) acc[m][n] = floatx4{0.f, 0.f, 0.f, 0.f};
         }
     } else {
         for (int k = 0; k < ks_wave; ++k) {
@@ -635,10 +705,14 @@ struct PhaseClock {
         }
     }
     __device__ __forceinline__ void lap(int slot) {
-        if (out && threadIdx.x == 0) {
-            const long long now = wall_clock64();
-            acc()[slot] += now - last;
-            last = now;
+        // (the pointer is the same for the whole workgroup: tested on its own and marked unlikely, a launch without
+        // counters falls through one scalar branch instead of jumping over a masked block)
+        if (__builtin_expect(out != nullptr, 0)) {
+            if (threadIdx.x == 0) {
+                const long long now = wall_clock64();
+                acc()[slot] += now - last;
+                last = now;
+            }
         }
     }
     __device__ __forceinline__ void flush() {
@@ -658,13 +732,13 @@ struct PhaseClock {
 // DEEP (2048 hidden units, 32-row blocks, several row blocks per workgroup and step): the operand comes through memory
 // from the other XCDs, and a workgroup finds a block's operand complete when it gets there (it was published a block
 // ago), so the product runs at the rate the fetch sustains: four sets of 2 k-steps in flight instead of two sets of 4
-// (measured at 128 rows: 6.9 -> 6.4 us per step).  With one block per step the product waits for its producers
+// (measured at 128 rows: 6.9 -> 6.4 us per step), validated by their effect on the result (product_poisoned).  With one block per step the product waits for its producers
 // anyway and the longer sets are the better ones (64 rows: 4.5 against 4.65 us).
 // Slices of 32 units with two row tiles run the pointwise stage in two PHASES: all 256 threads update rows 0..15
 // of the block (two units each) and store that half of h_t, then rows 16..31.  The consumers fetch and multiply
 // tile by tile (wave_product_tiles), so the second phase of a step overlaps the first half of the peers' next
 // product instead of sitting on the path from one step to the next.
-template <int NT, int KS, bool RESIDENT, int MT, bool DEEP = false>
+template <int NT, int KS, bool RESIDENT, int MT, bool DS, bool DEEP = false>
 __global__ __launch_bounds__(kThreads) void rec_fwd_kernel(RecFwdArgs p, RecLayout L, int t_begin,
                                                            int t_end, int ks_wave) {
     constexpr int JB = 4 * NT;    // hidden units of this slice
@@ -689,7 +763,7 @@ __global__ __launch_bounds__(kThreads) void rec_fwd_kernel(RecFwdArgs p, RecLayo
     const int hs = role.hs, g = role.g;
     const int rotation = __builtin_amdgcn_readfirstlane(rec_kstep_rotation(hs, L.nh, ks_wave, L.rot_div));
     const int nks_total = p.Hp / 32;
-    const bool device_scope = (L.persistent != 0) && (L.xcd_local == 0);
+    constexpr bool device_scope = DS;   // a persistent launch whose groups span XCDs (chosen by the host: no branch per store)
     const Poll poll{L.persistent != 0, p.spin_limit, p.spin_ticks, p.status, (lds_int_t*)&lds_abort};
     PhaseClock clk{(blockIdx.x == 0) ? p.prof : nullptr, 0};
     int item = 0;   // work items done: selects the partial-sum buffer
@@ -755,7 +829,7 @@ __global__ __launch_bounds__(kThreads) void rec_fwd_kernel(RecFwdArgs p, RecLayo
                 wave_product_tiles<NT, KS, 0, NPH * UPT / 2, kFwdBufs>(acc, wreg, nullptr, a0, a1, wave, lane, nks_total, ks_wave, rotation, poll,
                                                              [&]() { prefetch(t, rb); });
             else
-                wave_product<NT, KS, RESIDENT, 0, UPT / 2, MT, DEEP ? 4 : 2, DEEP ? 2 : 0>(acc, wreg, nullptr, wfrag_wave, a0, a1, wave, lane, nks_total,
+                wave_product<NT, KS, RESIDENT, 0, UPT / 2, MT, DEEP ? 4 : 2, DEEP ? 2 : 0, DEEP>(acc, wreg, nullptr, wfrag_wave, a0, a1, wave, lane, nks_total,
                                                                ks_wave, rotation, poll, [&]() { prefetch(t, rb); });
             clk.lap(0);
             spill_partials<NT, MT>(part, acc, wave, lane, PLD);
@@ -848,7 +922,7 @@ __global__ __launch_bounds__(kThreads) void rec_fwd_kernel(RecFwdArgs p, RecLayo
 // ----------------------------------------------------------------------------------- backward
 // Gate order and the pointwise derivative follow flashlstm_v2/src/lstm_backward.cu:199-211, except
 // that c_{t-1}, c_t come from the cell-state cache instead of being rebuilt through atanh.
-template <int NT, int KS, bool RESIDENT, int KL, int MT>
+template <int NT, int KS, bool RESIDENT, int KL, int MT, bool DS>
 __global__ __launch_bounds__(kThreads) void rec_bwd_kernel(RecBwdArgs p, RecLayout L, int t_first,
                                                            int t_last, int ks_wave) {
     constexpr int JB = 16 * NT;  // hidden units (= output columns of dG*W_hh) of this slice
@@ -869,7 +943,7 @@ __global__ __launch_bounds__(kThreads) void rec_bwd_kernel(RecBwdArgs p, RecLayo
     const int hs = role.hs, g = role.g;
     const int rotation = __builtin_amdgcn_readfirstlane(rec_kstep_rotation(hs, L.nh, ks_wave, L.rot_div));
     const int nks_total = p.Hp / 8;  // contraction over 4Hp packed gate columns
-    const bool device_scope = (L.persistent != 0) && (L.xcd_local == 0);
+    constexpr bool device_scope = DS;   // a persistent launch whose groups span XCDs (chosen by the host: no branch per store)
     const Poll poll{L.persistent != 0, p.spin_limit, p.spin_ticks, p.status, (lds_int_t*)&lds_abort};
     const float S = p.dy_scale;
     PhaseClock clk{(blockIdx.x == 0) ? p.prof : nullptr, 0};
@@ -1732,9 +1806,9 @@ static hipError_t launch_steps(StepGraphCache* graphs, const void* kernel, const
     return hipGraphLaunch(exec, stream);
 }
 
-template <int NT, int KS, bool RES, int MT, bool DEEP = false>
+template <int NT, int KS, bool RES, int MT, bool DS, bool DEEP = false>
 static hipError_t run_fwd(const RecLayout& L, const RecFwdArgs& a, hipStream_t stream, StepGraphCache* graphs) {
-    auto kernel = rec_fwd_kernel<NT, KS, RES, MT, DEEP>;
+    auto kernel = rec_fwd_kernel<NT, KS, RES, MT, DS, DEEP>;
     const size_t lds = size_t(2) * 4 * kRows * (16 * NT + kPartPad) * sizeof(float);
     hipError_t e = raise_lds(kernel, lds);
     if (e != hipSuccess) return e;
@@ -1754,19 +1828,25 @@ static hipError_t run_fwd(const RecLayout& L, const RecFwdArgs& a, hipStream_t s
 hipError_t launch_rec_fwd(const RecLayout& L, const RecFwdArgs& a, hipStream_t stream, StepGraphCache* graphs) {
     if (a.T <= 0 || a.B <= 0 || a.t1 <= a.t0) return hipSuccess;
     if (a.Hp % 32 != 0 || a.Hp % L.jb != 0 || a.t0 < 0 || a.t1 > a.T) return hipErrorInvalidValue;
-    if (!L.resident) return run_fwd<8, 1, false, 2>(L, a, stream, graphs);
-    if (L.nt == 8) return L.mt == 1 ? run_fwd<8, 8, true, 1>(L, a, stream, graphs) : run_fwd<8, 8, true, 2>(L, a, stream, graphs);
+    // device-scope stores into the exchange ring: a persistent launch whose groups span XCDs
+    const bool ds = L.persistent && !L.xcd_local;
+    if (!L.resident) return run_fwd<8, 1, false, 2, false>(L, a, stream, graphs);
+    if (L.nt == 8) {
+        if (L.mt == 1) return ds ? run_fwd<8, 8, true, 1, true>(L, a, stream, graphs) : run_fwd<8, 8, true, 1, false>(L, a, stream, graphs);
+        return ds ? run_fwd<8, 8, true, 2, true>(L, a, stream, graphs) : run_fwd<8, 8, true, 2, false>(L, a, stream, graphs);
+    }
     if (L.nt == 4) {
-        if (L.mt == 1) return run_fwd<4, 16, true, 1>(L, a, stream, graphs);
-        const bool several_blocks = L.persistent && L.nrb >= 2 * L.ng;   // every workgroup takes at least two row blocks per step
-        return several_blocks ? run_fwd<4, 16, true, 2, true>(L, a, stream, graphs) : run_fwd<4, 16, true, 2>(L, a, stream, graphs);
+        if (L.mt == 1) return ds ? run_fwd<4, 16, true, 1, true>(L, a, stream, graphs) : run_fwd<4, 16, true, 1, false>(L, a, stream, graphs);
+        if (!ds) return run_fwd<4, 16, true, 2, false>(L, a, stream, graphs);
+        const bool several_blocks = L.nrb >= 2 * L.ng;   // every workgroup takes at least two row blocks per step
+        return several_blocks ? run_fwd<4, 16, true, 2, true, true>(L, a, stream, graphs) : run_fwd<4, 16, true, 2, true>(L, a, stream, graphs);
     }
     return hipErrorInvalidValue;
 }
 
-template <int NT, int KS, bool RES, int KL, int MT>
+template <int NT, int KS, bool RES, int KL, int MT, bool DS>
 static hipError_t run_bwd(const RecLayout& L, const RecBwdArgs& a, hipStream_t stream, StepGraphCache* graphs) {
-    auto kernel = rec_bwd_kernel<NT, KS, RES, KL, MT>;
+    auto kernel = rec_bwd_kernel<NT, KS, RES, KL, MT, DS>;
     static_assert(size_t(2) * 4 * kRows * (16 * NT + kPartPad) >= size_t(kThreads) * 8 * NT, "db reduction reuses the partial-sum area");
     const size_t lds = size_t(2) * 4 * kRows * (16 * NT + kPartPad) * sizeof(float) + size_t(4) * KL * NT * kWave * sizeof(half8);
     hipError_t e = raise_lds(kernel, lds);
@@ -1818,9 +1898,16 @@ hipError_t launch_rec_bwd(const RecLayout& L, const RecBwdArgs& a, hipStream_t s
         }
         return hipErrorInvalidValue;
     }
-    if (!L.resident) return run_bwd<2, 1, false, 0, 2>(L, a, stream, graphs);
-    if (L.nt == 2) return L.mt == 1 ? run_bwd<2, 32, true, 8, 1>(L, a, stream, graphs) : run_bwd<2, 32, true, 8, 2>(L, a, stream, graphs);
-    if (L.nt == 1) return L.mt == 1 ? run_bwd<1, 64, true, 24, 1>(L, a, stream, graphs) : run_bwd<1, 64, true, 24, 2>(L, a, stream, graphs);
+    const bool ds = L.persistent && !L.xcd_local;   // (as in launch_rec_fwd)
+    if (!L.resident) return run_bwd<2, 1, false, 0, 2, false>(L, a, stream, graphs);
+    if (L.nt == 2) {
+        if (L.mt == 1) return ds ? run_bwd<2, 32, true, 8, 1, true>(L, a, stream, graphs) : run_bwd<2, 32, true, 8, 1, false>(L, a, stream, graphs);
+        return ds ? run_bwd<2, 32, true, 8, 2, true>(L, a, stream, graphs) : run_bwd<2, 32, true, 8, 2, false>(L, a, stream, graphs);
+    }
+    if (L.nt == 1) {
+        if (L.mt == 1) return ds ? run_bwd<1, 64, true, 24, 1, true>(L, a, stream, graphs) : run_bwd<1, 64, true, 24, 1, false>(L, a, stream, graphs);
+        return ds ? run_bwd<1, 64, true, 24, 2, true>(L, a, stream, graphs) : run_bwd<1, 64, true, 24, 2, false>(L, a, stream, graphs);
+    }
     return hipErrorInvalidValue;
 }
 

@@ -158,6 +158,37 @@ def test_two_way_split_backward_for_2048_units(shape):
     core.close()
 
 
+@pytest.mark.parametrize("shape", [(6, 128, 32, 2048), (6, 40, 32, 1024), (5, 33, 16, 256)])
+def test_a_batch_row_of_nans_stays_in_its_row(shape):
+    """Values that are NaN in their own right must travel through the exchange like any others.  The forward kernel
+    for 2048 units with several row blocks per workgroup validates what it fetched by its effect on the product (a
+    NaN in the result sends the wave through a second, word-by-word checked pass): a NaN row takes that second pass at
+    every step, must not be mistaken for unwritten data (no give-up, no fallback), and must leave every other batch
+    row bit-identical to a run without it."""
+    from flashlstm_poc_amd import LstmCore
+    T, B, I, H = shape
+    p = make_problem(T, B, I, H, seed=11)
+    core = LstmCore(B, I, H)
+    core.pack(p["w_ih"].cuda(), p["w_hh"].cuda(), p["b_ih"].cuda(), p["b_hh"].cuda())
+    x = p["x"].cuda().half()
+    h0, c0 = p["h0"].cuda().half(), p["c0"].cuda().half()
+    y_clean, hn_clean, cn_clean = (t.clone() for t in core.forward(x, h0, c0))
+    bad = 5
+    x_bad = x.clone()
+    x_bad[1:, bad, :] = float("nan")
+    y, hn, cn = core.forward(x_bad, h0, c0)
+    dy = p["dy"].cuda().half()
+    grads = core.backward(x_bad, dy, None, None)
+    torch.cuda.synchronize()
+    assert core.info("fallbacks") == 0 and core.info("persistent_fwd") == 1
+    keep = [b for b in range(B) if b != bad]
+    assert torch.equal(y[:, keep], y_clean[:, keep]) and torch.equal(hn[keep], hn_clean[keep]) and torch.equal(cn[keep], cn_clean[keep])
+    assert torch.equal(y[0, bad], y_clean[0, bad]) and bool(torch.isnan(y[1:, bad]).all())
+    dx = grads[0]
+    assert bool(torch.isfinite(dx[:, keep]).all()) and bool(torch.isnan(dx[1:, bad]).all())
+    core.close()
+
+
 def test_retry_limit_hit_is_repaired_by_stepwise_pass():
     # Failure handling of the persistent kernels, forced from the host: with a retry limit of 1 a workgroup
     # that finds an operand not yet written gives up at once, every kernel still exits normally, and the
