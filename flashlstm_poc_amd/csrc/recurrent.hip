@@ -208,22 +208,23 @@ __host__ __device__ constexpr int wlds_before(int ks, int KS, int KL) { return k
 __host__ __device__ constexpr bool wlds_has(int ks, int KS, int KL) { return wlds_before(ks + 1, KS, KL) > wlds_before(ks, KS, KL); }
 __host__ __device__ constexpr int wreg_slot(int ks, int KS, int KL) { return ks - wlds_before(ks, KS, KL); }
 
-// Validation by effect.  A word of the ring that still holds the 'unwritten' pattern is a pair of fp16 NaNs, and a NaN
-// anywhere in row r of the fetched operand makes EVERY column of row r of the product NaN (NaN times anything, a zero
-// weight included, is NaN, and sums keep it).  With the operands swapped a lane holds row lane % 16 of each row tile
-// in every one of its accumulation registers, so one register per row tile tells whether the wave multiplied
-// something its producers had not written yet: two instructions per product instead of a maximum over every
-// fetched word (10 vector instructions per chunk of 4 fragments, a fifth of a step's instructions in the backward
-// kernel).  A wave still checks the FIRST chunk of a product word by word -- that is where it waits for its producers,
-// and they finish within a fraction of a microsecond of each other; if it did have to wait there, also the chunks it
-// had requested ahead by then -- multiplies the rest as it lands, and repeats
-// its part of the product with every chunk checked if the result says so (LAZY = false: checked from the start).
-// Measured, it pays only where a wave finds its operand complete when it gets there (several row blocks per workgroup
-// and step: forward at 2048 units and 128 rows 6.7 -> 6.2 us per step).  A wave that arrives ahead of its producers
-// -- one row block per step, every configuration of 1024 units -- runs into words that were fetched too early often
-// enough for the repeated products to cost more than the checks (256 rows at 1024 units, backward: 4.9 -> 5.3 us
-// per step; 64 rows at 2048 units: 7.3 -> 11.3), so those kernels keep the check of every chunk.  Values that are NaN in
+// Validation by effect (LAZY).  A word of the ring that still holds the 'unwritten' pattern is a pair of fp16 NaNs, and
+// a NaN anywhere in row r of the fetched operand makes EVERY column of row r of the product NaN (NaN times anything, a
+// zero weight included, is NaN, and sums keep it).  With the operands swapped a lane holds row lane % 16 of each row
+// tile in every one of its accumulation registers, so one register per row tile tells whether the wave multiplied
+// something its producers had not written yet: two instructions per product instead of a maximum over every fetched
+// word (10 vector instructions per chunk of 4 fragments).  A LAZY product checks its FIRST chunk word by word -- that
+// is where a wave waits for its producers, and they finish within a fraction of a microsecond of each other -- and,
+// if it did have to wait there, the chunks it had requested ahead by then; it multiplies the rest as it lands and
+// repeats the wave's part of the product with every chunk checked if the result says so.  Values that are NaN in
 // their own right (or sums of opposite infinities) take that second pass too and come out as what they are.
+// Measured, this pays only where a wave finds its operand complete when it gets there (several row blocks per
+// workgroup and step: forward at 2048 units and 128 rows 6.7 -> 6.2 us per step).  A wave that arrives ahead of its
+// producers -- one row block per step, every configuration of 1024 units -- runs into words that were fetched too
+// early often enough for the repeated products to cost more than the checks save (256 rows at 1024 units, backward:
+// 4.9 -> 5.3 us per step; 64 rows at 2048 units: 7.3 -> 11.3), so every other kernel checks every chunk (LAZY = false).
+// Checking one word per 16-byte fragment lane instead of four, with the same probe as safety net, was measured too:
+// 120 vector instructions fewer per backward step and no change in time (the checks run in the shadow of the MFMAs).
 template <int MT, int NT>
 __device__ __forceinline__ bool product_poisoned(const floatx4 (&acc)[2][NT]) {
     float probe = acc[0][0][0];
