@@ -166,3 +166,42 @@ def test_error_codes_follow_the_reference():
     assert forward(lib, buf, p, T, ACC32)[0] == 0
     assert lib.lstm_destroy_buffers(ctypes.byref(buf)) == 0
     assert forward(lib, buf, p, T, ACC32)[0] == 1            # destroyed handle
+
+
+def test_entry_points_open_the_reference_s_range_names_when_a_tracing_library_is_there(tmp_path):
+    """The reference brackets its entry points with NVTX ranges (src/lstm.cu:1898, flashlstm_v2/src/nvtx_guard.hpp);
+    here they are roctx ranges, looked up at run time.  A stand-in library of that name, first on the loader's path
+    of a child process, records what is pushed and popped around one forward and one backward call."""
+    import os
+    import subprocess
+    import sys
+    stub = tmp_path / "stub.c"
+    stub.write_text(
+        '#include <stdio.h>\n#include <stdlib.h>\n'
+        'static void note(const char* what, const char* name) { FILE* f = fopen(getenv("FLSTM_RANGE_LOG"), "a");'
+        ' if (f) { fprintf(f, "%s %s\\n", what, name); fclose(f); } }\n'
+        'int roctxRangePushA(const char* name) { note("push", name); return 0; }\n'
+        'int roctxRangePop(void) { note("pop", "-"); return 0; }\n')
+    lib = tmp_path / "librocprofiler-sdk-roctx.so"
+    subprocess.run(["gcc", "-shared", "-fPIC", "-o", str(lib), str(stub)], check=True)
+    log = tmp_path / "ranges.log"
+    here = os.path.dirname(os.path.abspath(__file__))
+    child = (
+        "import ctypes, sys, torch\n"
+        f"sys.path.insert(0, {here!r}); sys.path.insert(0, {os.path.dirname(here)!r})\n"
+        "import test_v1_api_gpu as t\n"
+        "from helpers import make_problem\n"
+        "lib = t.bind(); p = make_problem(6, 2, 16, 24, seed=3, fp16_values=False); buf = t.Buffers()\n"
+        "assert lib.lstm_create_buffers(t.ACC16, 6, 2, 16, 24, 64, ctypes.byref(buf)) == 0\n"
+        "w_ih, w_hh = p['w_ih'].cuda().contiguous(), p['w_hh'].cuda().contiguous()\n"
+        "assert lib.lstm_pack_weights(t.ACC16, w_ih.data_ptr(), w_hh.data_ptr(), 16, 24, ctypes.byref(buf)) == 0\n"
+        "rc, out, hn, cn = t.forward(lib, buf, p, 6, t.ACC16); assert rc == 0\n"
+        "torch.cuda.synchronize(); assert lib.lstm_destroy_buffers(ctypes.byref(buf)) == 0\n")
+    env = dict(os.environ, FLSTM_RANGE_LOG=str(log),
+               LD_LIBRARY_PATH=str(tmp_path) + os.pathsep + os.environ.get("LD_LIBRARY_PATH", ""))
+    r = subprocess.run([sys.executable, "-c", child], env=env, capture_output=True, text=True, timeout=300)
+    assert r.returncode == 0, r.stderr[-2000:]
+    lines = log.read_text().split("\n")
+    pushed = [l.split(" ", 1)[1] for l in lines if l.startswith("push ")]
+    assert "FlashLSTM::lstm_forward" in pushed and "FlashLSTM::lstm_forward::compute" in pushed
+    assert sum(l.startswith("pop ") for l in lines) == len(pushed)   # every range is closed
