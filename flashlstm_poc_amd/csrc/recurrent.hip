@@ -202,6 +202,20 @@ __device__ __forceinline__ void wait_frags(half8 (&a)[8]) {
                  : "memory");
 }
 
+// The same with the count as a value: for callers whose count is a constant only after unrolling.
+template <int NF>
+__device__ __forceinline__ void wait_frags_upto(half8 (&a)[NF], int younger) {
+    switch (younger) {
+#define FLSTM_WAIT_CASE(n) case n: wait_frags<n>(a); break;
+        FLSTM_WAIT_CASE(1) FLSTM_WAIT_CASE(2) FLSTM_WAIT_CASE(3) FLSTM_WAIT_CASE(4) FLSTM_WAIT_CASE(5) FLSTM_WAIT_CASE(6)
+        FLSTM_WAIT_CASE(7) FLSTM_WAIT_CASE(8) FLSTM_WAIT_CASE(9) FLSTM_WAIT_CASE(10) FLSTM_WAIT_CASE(11) FLSTM_WAIT_CASE(12)
+        FLSTM_WAIT_CASE(13) FLSTM_WAIT_CASE(14) FLSTM_WAIT_CASE(15) FLSTM_WAIT_CASE(16) FLSTM_WAIT_CASE(17) FLSTM_WAIT_CASE(18)
+        FLSTM_WAIT_CASE(19) FLSTM_WAIT_CASE(20) FLSTM_WAIT_CASE(21) FLSTM_WAIT_CASE(22) FLSTM_WAIT_CASE(23) FLSTM_WAIT_CASE(24)
+#undef FLSTM_WAIT_CASE
+        default: wait_frags<0>(a); break;   // (0, and anything larger than listed: waiting for more is always safe)
+    }
+}
+
 // Which of a wave's KS k-steps keep their weight fragments in LDS (KL of them, spread evenly) and where the others sit
 // in the register array.
 __host__ __device__ constexpr int wlds_before(int ks, int KS, int KL) { return ks * KL / KS; }          // LDS k-steps below ks
@@ -273,16 +287,18 @@ __device__ __forceinline__ void wave_product_tiles(floatx4 (&acc)[2][NT], const 
             issue(c + NBUF - 1);
             if (c + NBUF - 1 == NCH - 1) prefetch();
         }
+        // this chunk's weight fragments that live in LDS: requested now, they arrive while the wave waits for the
+        // chunk's operand fragments (as in wave_product)
+        half8 wl[CKT][NT];
+#pragma unroll
+        for (int k = 0; k < CKT; ++k)
+            if (wlds_has((c % NCHK) * CKT + k, KS, KL)) {
+#pragma unroll
+                for (int n = 0; n < NT; ++n) wl[k][n] = wlds[(wlds_before((c % NCHK) * CKT + k, KS, KL) * NT + n) * kWave + lane];
+            }
         // loads return in issue order: chunk c has landed once at most the loads issued after it are outstanding
         const int younger = (last_issued - c) * CKT + ((last_issued == NCH - 1) ? NPF : 0);
-        switch (younger) {   // (a compile-time constant in every unrolled iteration)
-            case NPF: wait_frags<NPF>(f[buf]); break;
-            case CKT + NPF: wait_frags<CKT + NPF>(f[buf]); break;
-            case 2 * CKT + NPF: wait_frags<2 * CKT + NPF>(f[buf]); break;
-            case CKT: wait_frags<CKT>(f[buf]); break;
-            case 2 * CKT: wait_frags<2 * CKT>(f[buf]); break;
-            default: wait_frags<0>(f[buf]); break;
-        }
+        wait_frags_upto(f[buf], younger);   // (a compile-time constant in every unrolled iteration: the switch folds)
         // A pair of halfs that still holds the pattern has not been written yet by its producer: fetch the chunk
         // again (whatever was in flight behind it lands first, loads return in order).  The decision is wave-uniform.
         // The check is peeled out of the reload loop: a chunk that is complete -- nearly all of them -- then costs the
@@ -321,7 +337,7 @@ __device__ __forceinline__ void wave_product_tiles(floatx4 (&acc)[2][NT], const 
             for (int n = 0; n < NT; ++n) {
                 half8 w;
                 if (!wlds_has(ks, KS, KL)) w = wreg[wreg_slot(ks, KS, KL)][n];
-                else w = wlds[(wlds_before(ks, KS, KL) * NT + n) * kWave + lane];
+                else w = wl[k][n];
                 acc[c / NCHK][n] = __builtin_amdgcn_mfma_f32_16x16x32_f16(w, f[buf][k], acc[c / NCHK][n], 0, 0, 0);
             }
         }
@@ -929,8 +945,14 @@ __global__ __launch_bounds__(kThreads) void rec_bwd_kernel(RecBwdArgs p, RecLayo
     constexpr int JB = 16 * NT;  // hidden units (= output columns of dG*W_hh) of this slice
     constexpr int PLD = JB + kPartPad;
     constexpr int KR = KS - KL;  // k-steps whose weight fragments stay in registers
-    constexpr int GPR = (MT == 1 && JB >= 32) ? 16 : 8;   // threads per batch row (as in the forward kernel)
+    // As in the forward kernel: slices of 32 units with two row tiles update rows 0..15 first and publish that half of
+    // dG_t, then rows 16..31, and fetch and multiply tile by tile, so the second half of a step's cell updates and its
+    // cache stores run while the peers are already in the first half of their next product (measured at 1024 units
+    // and 256 rows: 4.85 -> 4.5 us per step; without waiting for producers at all the step takes 4.2).
+    constexpr bool SPLIT = RESIDENT && MT == 2 && JB >= 32 && (KS % 8 == 0);
+    constexpr int GPR = (SPLIT || (MT == 1 && JB >= 32)) ? 16 : 8;   // threads per batch row (as in the forward kernel)
     constexpr int UPT = JB / GPR;
+    constexpr int NPH = SPLIT ? 2 : 1;   // pointwise phases per step
     static_assert(UPT == 2 || UPT == 4, "2 or 4 hidden units per thread");
     typedef Pack<UPT> PackT;
     extern __shared__ __attribute__((aligned(16))) float part_all[];  // [2][4][32][PLD], reused for db
@@ -966,36 +988,42 @@ __global__ __launch_bounds__(kThreads) void rec_bwd_kernel(RecBwdArgs p, RecLayo
     }
 
     const size_t gld = size_t(4) * p.Hp;
-    // this thread's group: row pr of the row block, units pj .. pj+UPT-1 of the slice
+    // this thread's groups: row pr (+ 16 in the second phase) of the row block, units pj .. pj+UPT-1 of the slice
     constexpr int RB = 16 * MT;   // batch rows of a row block
     const int pr = group_row<(GPR * UPT == 16) ? 4 : 2>(tid / GPR);
-    const bool row_used = pr < RB;   // with one row tile per block the threads of rows 16..31 only keep the barriers company
+    const bool row_used = pr + 16 * (NPH - 1) < RB;   // with one row tile per block the threads of rows 16..31 only keep the barriers company
     const int pj = (tid % GPR) * UPT;
     const int j = hs * JB + pj;
     const size_t pq = size_t(4) * j;   // column of (unit j, gate 0) in the gate arrays
     const int rb_count = (L.nrb - g + L.ng - 1) / L.ng;
     // the running dc of the workgroup's first and second row block stays in registers for the whole launch
     const bool dc_in_regs = (rb_count <= 2) && (t_first - t_last > 0);
-    float dcreg[UPT] = {}, dcreg2[UPT] = {};
+    float dcreg[NPH][UPT] = {}, dcreg2[NPH][UPT] = {};
     if (dc_in_regs) {
-        const int b = g * RB + pr, b2 = (g + L.ng) * RB + pr;
-        if (row_used && b < p.B) ld_f32_now(p.dC + size_t(b) * p.Hp + j, dcreg);
-        if (rb_count == 2 && row_used && b2 < p.B) ld_f32_now(p.dC + size_t(b2) * p.Hp + j, dcreg2);
-    }
-    // prefetched per work item: activated gates, c_{t-1}, c_t, dY_t
-    GateRow<UPT> pg;
-    PackT pdy;
-    F32<UPT> pcp_r, pcc_r;
-    constexpr int NPF = UPT / 2 + 3;
-    auto prefetch = [&](int t, int rb) {   // NPF loads per wave; rows past B fetch row B-1, the closing pass step 0
-        const int b = min(rb * RB + pr, p.B - 1);
-        const int tt = max(t, 0);
-        const half_t* gsrc = p.G + (size_t(tt) * p.B + b) * gld + pq;
 #pragma unroll
-        for (int c = 0; c < UPT / 2; ++c) ld_stream(pg.v[c], gsrc + 8 * c);
-        ld_stream(pcp_r.v, p.C + (size_t(tt) * p.B + b) * p.Hp + j);
-        ld_stream(pcc_r.v, p.C + (size_t(tt + 1) * p.B + b) * p.Hp + j);
-        ld_stream(pdy.v, p.dY + (size_t(tt) * p.B + b) * p.Hp + j);
+        for (int ph = 0; ph < NPH; ++ph) {
+            const int b = g * RB + pr + 16 * ph, b2 = (g + L.ng) * RB + pr + 16 * ph;
+            if (row_used && b < p.B) ld_f32_now(p.dC + size_t(b) * p.Hp + j, dcreg[ph]);
+            if (rb_count == 2 && row_used && b2 < p.B) ld_f32_now(p.dC + size_t(b2) * p.Hp + j, dcreg2[ph]);
+        }
+    }
+    // prefetched per work item and phase: activated gates, c_{t-1}, c_t, dY_t
+    GateRow<UPT> pg[NPH];
+    PackT pdy[NPH];
+    F32<UPT> pcp_r[NPH], pcc_r[NPH];
+    constexpr int NPF = NPH * (UPT / 2 + 3);
+    auto prefetch = [&](int t, int rb) {   // NPF loads per wave; rows past B fetch row B-1, the closing pass step 0
+        const int tt = max(t, 0);
+#pragma unroll
+        for (int ph = 0; ph < NPH; ++ph) {
+            const int b = min(rb * RB + pr + 16 * ph, p.B - 1);
+            const half_t* gsrc = p.G + (size_t(tt) * p.B + b) * gld + pq;
+#pragma unroll
+            for (int c = 0; c < UPT / 2; ++c) ld_stream(pg[ph].v[c], gsrc + 8 * c);
+            ld_stream(pcp_r[ph].v, p.C + (size_t(tt) * p.B + b) * p.Hp + j);
+            ld_stream(pcc_r[ph].v, p.C + (size_t(tt + 1) * p.B + b) * p.Hp + j);
+            ld_stream(pdy[ph].v, p.dY + (size_t(tt) * p.B + b) * p.Hp + j);
+        }
     };
     __syncthreads();
     float dbacc[4][UPT] = {};
@@ -1018,8 +1046,12 @@ __global__ __launch_bounds__(kThreads) void rec_bwd_kernel(RecBwdArgs p, RecLayo
                 for (int m = 0; m < 2; ++m)
 #pragma unroll
                     for (int n = 0; n < NT; ++n) acc[m][n] = floatx4{0.f, 0.f, 0.f, 0.f};
-                wave_product<NT, KS, RESIDENT, KL, NPF, MT>(acc, wreg, wlds, wfrag_wave, a0, a1, wave, lane, nks_total,
-                                                          ks_wave, rotation, poll, [&]() { prefetch(t, rb); });
+                if constexpr (SPLIT)
+                    wave_product_tiles<NT, KS, KL, NPF, 2>(acc, wreg, wlds, a0, a1, wave, lane, nks_total, ks_wave, rotation, poll,
+                                                           [&]() { prefetch(t, rb); });
+                else
+                    wave_product<NT, KS, RESIDENT, KL, NPF, MT>(acc, wreg, wlds, wfrag_wave, a0, a1, wave, lane, nks_total,
+                                                              ks_wave, rotation, poll, [&]() { prefetch(t, rb); });
                 clk.lap(0);
                 spill_partials<NT, MT>(part, acc, wave, lane, PLD);
                 __syncthreads();
@@ -1030,99 +1062,113 @@ __global__ __launch_bounds__(kThreads) void rec_bwd_kernel(RecBwdArgs p, RecLayo
             }
             wait_all_vm();   // gates, cell states and dY of this step, issued during the product
 #pragma unroll
-            for (int c = 0; c < UPT / 2; ++c) settle(pg.v[c]);
-            settle(pdy.v);
-            settle(pcp_r.v);
-            settle(pcc_r.v);
+            for (int ph = 0; ph < NPH; ++ph) {
+#pragma unroll
+                for (int c = 0; c < UPT / 2; ++c) settle(pg[ph].v[c]);
+                settle(pdy[ph].v);
+                settle(pcp_r[ph].v);
+                settle(pcc_r[ph].v);
+            }
             clk.lap(4);
-            const int b = row0 + pr;
-            const bool live = row_used && b < p.B;
-            const size_t sidx = size_t(b) * p.Hp + j;
             half_t* xout = p.X + size_t((t + 8) & 3) * p.x_slot;    // dG_t for the peers
             half_t* xnext = p.X + size_t((t + 6) & 3) * p.x_slot;   // will take dG_{t-2}
-            unsigned xoff[UPT / 2];   // 32 bits: a slot is far below 4G halfs; 8 columns = 16 contiguous bytes
-            GateRow<UPT> dgnew = gates_fill<UPT>(0u);   // batch rows past B travel as zeros
-            float dcnew[UPT] = {};
+            unsigned xoff[NPH][UPT / 2];   // 32 bits: a slot is far below 4G halfs; 8 columns = 16 contiguous bytes
             if (t >= 0 && row_used) {
                 // every peer has delivered dG_{t+1}, so all of them are done reading dG_{t+2}: mark its slot
                 // (the wait above has drained the marks of the previous step)
 #pragma unroll
-                for (int c = 0; c < UPT / 2; ++c) {
-                    xoff[c] = unsigned(xch_offset(b, int(pq) + 8 * c, nks_total));
-                    store_xch16(xnext + xoff[c], uintx4{kUnwritten, kUnwritten, kUnwritten, kUnwritten}, device_scope);
-                }
+                for (int ph = 0; ph < NPH; ++ph)
+#pragma unroll
+                    for (int c = 0; c < UPT / 2; ++c) {
+                        xoff[ph][c] = unsigned(xch_offset(row0 + pr + 16 * ph, int(pq) + 8 * c, nks_total));
+                        store_xch16(xnext + xoff[ph][c], uintx4{kUnwritten, kUnwritten, kUnwritten, kUnwritten}, device_scope);
+                    }
             }
-            if (live) {
-                float pcp[UPT], pcc[UPT];
-                to_floats(pcp_r, pcp);
-                to_floats(pcc_r, pcc);
-                float dh[UPT];
-                if (from_product) {
+            GateRow<UPT> dgnew[NPH];
+            float dcnew[NPH][UPT] = {};
+            bool live[NPH];
+            const bool second = (rb != g);
 #pragma unroll
-                    for (int u = 0; u < UPT; ++u) dh[u] = 0.f;
+            for (int ph = 0; ph < NPH; ++ph) {
+                const int prow = pr + 16 * ph, b = row0 + prow;
+                live[ph] = row_used && b < p.B;
+                const size_t sidx = size_t(b) * p.Hp + j;
+                dgnew[ph] = gates_fill<UPT>(0u);   // batch rows past B travel as zeros
+                if (live[ph]) {
+                    float pcp[UPT], pcc[UPT];
+                    to_floats(pcp_r[ph], pcp);
+                    to_floats(pcc_r[ph], pcc);
+                    float dh[UPT];
+                    if (from_product) {
 #pragma unroll
-                    for (int w = 0; w < 4; ++w) {
-                        float v[UPT];
-                        ld_f32(part + (size_t(w) * kRows + pr) * PLD + pj, v);
+                        for (int u = 0; u < UPT; ++u) dh[u] = 0.f;
 #pragma unroll
-                        for (int u = 0; u < UPT; ++u) dh[u] += v[u];
-                    }
-                } else {
-                    ld_f32_now(p.dHn + sidx, dh);
-                }
-                const bool second = (rb != g);
-                if (t < 0) {  // closing pass: gradient wrt h0; dc0 is the running dc
-                    st_f32(p.dH0 + sidx, dh);
-                    if (dc_in_regs) {
-                        if (second) st_f32(p.dC + sidx, dcreg2);
-                        else st_f32(p.dC + sidx, dcreg);
-                    }
-                } else {
-                    float dy[UPT], dcin[UPT];
-                    unpack(pdy, dy);
-                    if (dc_in_regs) {
+                        for (int w = 0; w < 4; ++w) {
+                            float v[UPT];
+                            ld_f32(part + (size_t(w) * kRows + prow) * PLD + pj, v);
 #pragma unroll
-                        for (int u = 0; u < UPT; ++u) dcin[u] = second ? dcreg2[u] : dcreg[u];
+                            for (int u = 0; u < UPT; ++u) dh[u] += v[u];
+                        }
                     } else {
-                        ld_f32_coherent(p.dC + sidx, dcin);
+                        ld_f32_now(p.dHn + sidx, dh);
                     }
-                    float gate[4][UPT];
-                    unpack_gates(pg, gate);
-                    float da[4][UPT];
+                    if (t < 0) {  // closing pass: gradient wrt h0; dc0 is the running dc
+                        st_f32(p.dH0 + sidx, dh);
+                        if (dc_in_regs) {
+                            if (second) st_f32(p.dC + sidx, dcreg2[ph]);
+                            else st_f32(p.dC + sidx, dcreg[ph]);
+                        }
+                    } else {
+                        float dy[UPT], dcin[UPT];
+                        unpack(pdy[ph], dy);
+                        if (dc_in_regs) {
 #pragma unroll
-                    for (int u = 0; u < UPT; ++u) {
-                        const float ig = gate[0][u], fg = gate[1][u], gg = gate[2][u], og = gate[3][u];
-                        const float dhu = dh[u] + S * dy[u];
-                        const float tc = tanhf_dev(pcc[u]);
-                        const float dov = dhu * tc;
-                        const float dc = dcin[u] + dhu * og * (1.f - tc * tc);
-                        da[0][u] = dc * gg * ig * (1.f - ig);
-                        da[1][u] = dc * pcp[u] * fg * (1.f - fg);
-                        da[2][u] = dc * ig * (1.f - gg * gg);
-                        da[3][u] = dov * og * (1.f - og);
-                        dcnew[u] = dc * fg;
-                        if (second) dcreg2[u] = dcnew[u];
-                        else dcreg[u] = dcnew[u];
+                            for (int u = 0; u < UPT; ++u) dcin[u] = second ? dcreg2[ph][u] : dcreg[ph][u];
+                        } else {
+                            ld_f32_coherent(p.dC + sidx, dcin);
+                        }
+                        float gate[4][UPT];
+                        unpack_gates(pg[ph], gate);
+                        float da[4][UPT];
+#pragma unroll
+                        for (int u = 0; u < UPT; ++u) {
+                            const float ig = gate[0][u], fg = gate[1][u], gg = gate[2][u], og = gate[3][u];
+                            const float dhu = dh[u] + S * dy[u];
+                            const float tc = tanhf_dev(pcc[u]);
+                            const float dov = dhu * tc;
+                            const float dc = dcin[u] + dhu * og * (1.f - tc * tc);
+                            da[0][u] = dc * gg * ig * (1.f - ig);
+                            da[1][u] = dc * pcp[u] * fg * (1.f - fg);
+                            da[2][u] = dc * ig * (1.f - gg * gg);
+                            da[3][u] = dov * og * (1.f - og);
+                            dcnew[ph][u] = dc * fg;
+                            if (second) dcreg2[ph][u] = dcnew[ph][u];
+                            else dcreg[ph][u] = dcnew[ph][u];
+                        }
+                        // db sums the values the weight-gradient GEMMs will see (fp16-rounded)
+                        dgnew[ph] = pack_gates(da);
+                        float r[4][UPT];
+                        unpack_gates(dgnew[ph], r);
+#pragma unroll
+                        for (int gt = 0; gt < 4; ++gt)
+#pragma unroll
+                            for (int u = 0; u < UPT; ++u) dbacc[gt][u] += r[gt][u];
                     }
-                    // db sums the values the weight-gradient GEMMs will see (fp16-rounded)
-                    dgnew = pack_gates(da);
-                    float r[4][UPT];
-                    unpack_gates(dgnew, r);
-#pragma unroll
-                    for (int gt = 0; gt < 4; ++gt)
-#pragma unroll
-                        for (int u = 0; u < UPT; ++u) dbacc[gt][u] += r[gt][u];
                 }
-            }
-            if (t >= 0 && row_used) {
-                // the exchanged values go out first
+                if (t >= 0 && row_used) {
+                    // the exchanged values go out first (one row tile after the other)
 #pragma unroll
-                for (int c = 0; c < UPT / 2; ++c) store_xch16(xout + xoff[c], dgnew.v[c], device_scope);
+                    for (int c = 0; c < UPT / 2; ++c) store_xch16(xout + xoff[ph][c], dgnew[ph].v[c], device_scope);
+                }
             }
             clk.lap(2);
-            if (t >= 0 && live) {   // row-major dG for the GEMMs that follow; running dc when it lives in memory
-                st_gates(p.dG + (size_t(t) * p.B + b) * gld + pq, dgnew);
-                if (!dc_in_regs) st_f32(p.dC + sidx, dcnew);
+#pragma unroll
+            for (int ph = 0; ph < NPH; ++ph) {
+                if (t >= 0 && live[ph]) {   // row-major dG for the GEMMs that follow; running dc when it lives in memory
+                    const int b = row0 + pr + 16 * ph;
+                    st_gates(p.dG + (size_t(t) * p.B + b) * gld + pq, dgnew[ph]);
+                    if (!dc_in_regs) st_f32(p.dC + size_t(b) * p.Hp + j, dcnew[ph]);
+                }
             }
             clk.lap(3);
         }
@@ -1130,9 +1176,12 @@ __global__ __launch_bounds__(kThreads) void rec_bwd_kernel(RecBwdArgs p, RecLayo
     clk.flush();
     // single-step launches leave dc in memory for the next launch
     if (dc_in_regs && t_last >= 0) {
-        const int b = g * RB + pr, b2 = (g + L.ng) * RB + pr;
-        if (row_used && b < p.B) st_f32(p.dC + size_t(b) * p.Hp + j, dcreg);
-        if (rb_count == 2 && row_used && b2 < p.B) st_f32(p.dC + size_t(b2) * p.Hp + j, dcreg2);
+#pragma unroll
+        for (int ph = 0; ph < NPH; ++ph) {
+            const int b = g * RB + pr + 16 * ph, b2 = (g + L.ng) * RB + pr + 16 * ph;
+            if (row_used && b < p.B) st_f32(p.dC + size_t(b) * p.Hp + j, dcreg[ph]);
+            if (rb_count == 2 && row_used && b2 < p.B) st_f32(p.dC + size_t(b2) * p.Hp + j, dcreg2[ph]);
+        }
     }
 
     // Bias gradient: fold this launch's sums over the threads that share a group column (fixed order).
