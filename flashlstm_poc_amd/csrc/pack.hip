@@ -101,7 +101,9 @@ __global__ void pack_wfrag_bwd2d_kernel(Dims d, const float* __restrict__ w_hh, 
     const int qs = int(r % kq); r /= kq;
     const int sl = int(r);
     const int k = sl * 64 + n * 16 + lane % 16;
-    const int q = qs * (4 * d.Hp / kq) + (ks * 4 + wave) * 32 + 8 * (lane / 16) + e;
+    // (slot ks of a wave holds the k-step the kernel fetches there: rotated per column slice)
+    const int kstep = rec_kstep_of_slot(ks, rec_bwd2d_rotation(sl, ksn, kq), ksn);
+    const int q = qs * (4 * d.Hp / kq) + (kstep * 4 + wave) * 32 + 8 * (lane / 16) + e;
     float v = 0.f;
     if (q < 4 * d.Hp && k < d.H) {
         const int row = torch_row(q, d.H);

@@ -91,6 +91,14 @@ __host__ __device__ inline int rec_kstep_rotation(int hs, int nh, int ks_wave, i
     const int r = hs / rot_div;
     return (ks_wave >= mates ? r * (ks_wave / mates) : r) % ks_wave;
 }
+// The same idea in the two-way backward layout with 8 contraction slices (one group of 256 workgroups, batches of one
+// row block): the 4 column slices of an XCD that share a contraction slice fetch the same fragments, and slice s starts
+// a quarter of the way further round than slice s - 1.  Measured at 16 rows: 3.71 -> 3.50 us per step.  With 4
+// contraction slices and two passes per step it cost 2 % (9.0 -> 9.2 us at 128 rows) and is off, as it is at 1024 units.
+__host__ __device__ inline int rec_bwd2d_rotation(int s, int ks_wave, int kq) {
+    if (kq != 8 || ks_wave < 4) return 0;
+    return ((s % 4) * (ks_wave / 4)) % ks_wave;
+}
 __host__ __device__ inline int rec_kstep_of_slot(int ks, int rotation, int ks_wave) {
     if (ks >= ks_wave) return ks;   // slots past the real contraction hold zero weights
     const int k = ks + rotation;

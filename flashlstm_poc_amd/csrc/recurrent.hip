@@ -1289,6 +1289,7 @@ __global__ __launch_bounds__(kThreads) void rec_bwd2d_kernel(RecBwdArgs p, RecLa
     if (g >= L.ng || s * 64 >= p.Hp) return;   // (more seats than the layout uses: a group without row blocks)
     constexpr bool device_scope = !LOCAL;      // the dG ring: plain stores reach every reader inside an XCD
     const int nks = p.Hp / 8;            // k-steps of the whole contraction
+    const int rotation = __builtin_amdgcn_readfirstlane(rec_bwd2d_rotation(s, KS, KQ));   // (the weight fragments are packed to match)
     const int nrb = L.nrb, ng = L.ng;
     const int nmine = (nrb - g + ng - 1) / ng;   // row blocks g, g + ng, ...
     const Poll poll{true, p.spin_limit, p.spin_ticks, p.status, (lds_int_t*)&lds_abort};
@@ -1511,7 +1512,7 @@ __global__ __launch_bounds__(kThreads) void rec_bwd2d_kernel(RecBwdArgs p, RecLa
                 const half_t* a1 = a0 + size_t(nks) * 512;
                 // (where the operand comes through memory -- groups that span XCDs -- and the contraction is long, five
                 // short fragment sets keep the fetch running over that trip)
-                wave_product<NT, KS, true, KL, NPF, MT, ((KS >= 16 && !LOCAL) ? 5 : 2), ((KS >= 16 && !LOCAL) ? 2 : 0)>(acc, wreg, wlds, nullptr, a0, a1, wave, lane, KS * 4, KS, 0, poll,
+                wave_product<NT, KS, true, KL, NPF, MT, ((KS >= 16 && !LOCAL) ? 5 : 2), ((KS >= 16 && !LOCAL) ? 2 : 0)>(acc, wreg, wlds, nullptr, a0, a1, wave, lane, KS * 4, KS, rotation, poll,
                                                        [&]() { load_ops(t, rb, ops[i & 1]); });
                 clk.lap(0);
                 spill_partials<NT, MT>(part, acc, wave, lane, PLD);
