@@ -617,7 +617,7 @@ int backward_setup(flstm_core_plan* p, size_t T, const void* dY, flstm_dtype dy_
     FL_TRY(p->dH0.reserve(st_bytes));
     FL_TRY(p->dG.reserve(TB * 4 * d.Hp * sizeof(half_t)));
     FL_TRY(p->db_part.reserve(size_t(p->Lb.ng) * 4 * d.Hp * sizeof(float)));
-    const size_t xslot = exchange_slot_halfs(d.B, 4 * d.Hp);
+    const size_t xslot = exchange_slot_halfs(rec_bwd_ring_rows(p->Lb, d.B), 4 * d.Hp);
     const size_t dg_slots = size_t(rec_bwd_dg_slots(p->Lb));
     FL_TRY(p->xch_b.reserve(dg_slots * xslot * sizeof(half_t)));
     FL_TRY(fill_words(p->xch_b.p, dg_slots * xslot * sizeof(half_t), 0xFFFFFFFFu, s));
@@ -650,7 +650,7 @@ int backward_recur(flstm_core_plan* p, long t_hi, long t_lo, hipStream_t s) {
     a.wfrag = p->wfrag_b.as<half8>();
     a.G = p->G.as<half_t>(); a.C = p->C.as<float>(); a.dY = p->bw.dYk; a.dG = p->dG.as<half_t>();
     a.dHn = p->dHn.as<float>(); a.dC = p->dC.as<float>(); a.dH0 = p->dH0.as<float>();
-    a.X = p->xch_b.as<half_t>(); a.x_slot = exchange_slot_halfs(d.B, 4 * d.Hp);
+    a.X = p->xch_b.as<half_t>(); a.x_slot = exchange_slot_halfs(rec_bwd_ring_rows(p->Lb, d.B), 4 * d.Hp);
     if (p->Lb.two_d) {
         a.wfrag2 = p->wfrag_b2.as<half8>();
         a.P = p->part_b.as<float>();
@@ -659,13 +659,27 @@ int backward_recur(flstm_core_plan* p, long t_hi, long t_lo, hipStream_t s) {
     a.db_part = p->db_part.as<float>();
     a.status = p->status.as<int>();
     a.seats = p->status.as<unsigned>() + 8;
-    FL_TRY(fill_zero(a.seats, 8 * sizeof(unsigned), s));
     a.B = d.B; a.Hp = d.Hp; a.T = int(p->bw.T); a.dy_scale = p->bw.dy_scale;
     a.t_hi = int(t_hi); a.t_lo = int(t_lo);
     a.spin_limit = p->opt_spin_limit;
     a.spin_ticks = (long long)p->opt_spin_ms * p->wall_khz;
     a.prof = p->opt_profile ? p->prof.as<long long>() + 8 : nullptr;
-    FL_TRY(launch_rec_bwd(p->Lb, a, s, p->opt_graphs ? &p->graphs_b : nullptr));
+    // One launch, or one per window of batch rows (RecLayout::win_rows).  The windows share the ring of partial sums,
+    // so every launch of a windowed pass starts from a ring prepared for ITS first product step (a single window's
+    // launches continue each other's parities instead).
+    const int win = (p->Lb.two_d && p->Lb.win_rows) ? p->Lb.win_rows : d.B;
+    for (int b_lo = 0; b_lo < d.B; b_lo += win) {
+        a.b_lo = b_lo;
+        a.b_hi = b_lo + win < d.B ? b_lo + win : d.B;
+        FL_TRY(fill_zero(a.seats, 8 * sizeof(unsigned), s));
+        if (win < d.B) {
+            const size_t pslot = a.p_slot * sizeof(float);
+            const int first_T = t_hi >= long(p->bw.T) - 1 ? int(p->bw.T) : int(t_hi) + 2;   // (its first product step is first_T - 2)
+            for (int k = 0; k < kRecBwdPartSlots; ++k)
+                FL_TRY(fill_words(static_cast<char*>(p->part_b.p) + size_t(k) * pslot, pslot, rec_bwd_part_fill(k, first_T), s));
+        }
+        FL_TRY(launch_rec_bwd(p->Lb, a, s, p->opt_graphs ? &p->graphs_b : nullptr));
+    }
     return 0;
 }
 

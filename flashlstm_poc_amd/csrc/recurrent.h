@@ -27,6 +27,8 @@ struct RecLayout {
                      // still describe the one-dimensional layout, whose weight fragments the step-wise fallback uses
     int kq;          // two_d: contraction slices, 8 (one group of 256 workgroups) or 4 (two groups of 128)
     int nm;          // two_d: passes per step the kernel is built for (row blocks per workgroup, rounded up to 1, 2, 4)
+    int win_rows;    // two_d: 0, or the batch is walked in windows of this many rows, one persistent launch each (batch
+                     // rows are independent sequences); nrb, mt, ng, nm then describe one window
 };
 
 struct RecFwdArgs {
@@ -71,6 +73,8 @@ struct RecBwdArgs {
     unsigned* seats;     // [8] zeroed before every launch
     int* status;
     int B, Hp, T;
+    int b_lo, b_hi;      // two-dimensional layout: the launch works on batch rows [b_lo, b_hi) (b_lo a multiple of 32;
+                         // every array keeps its full-batch strides, the rings are indexed by the row in the batch)
     float dy_scale;      // factor applied to dY on load (the loss scale, or 1 when dY is pre-scaled)
     int t_hi, t_lo;      // steps t_hi down to t_lo are run by this call; t_lo = -1 adds the closing dh0 product
     int spin_limit;
@@ -148,6 +152,8 @@ constexpr int kRecBwdPartSlots = 3;
 size_t rec_bwd_two_d_wfrag_bytes(int Hp);
 // Word to fill slot `slot` of the partial ring with before a pass over T steps (see RecBwdArgs::P).
 unsigned rec_bwd_part_fill(int slot, int T);
+// Batch rows the rings of a backward layout are sized for (whole windows where the batch is walked in windows).
+int rec_bwd_ring_rows(const RecLayout& L, int B);
 
 // Halfs in one slot of an exchange ring for a [rows][cols] operand (rows padded to 32).
 size_t exchange_slot_halfs(int rows, int cols);

@@ -120,12 +120,14 @@ def test_persistent_and_stepwise_agree(shape):
 
 @pytest.mark.parametrize("shape", [(7, 128, 32, 2048), (6, 40, 32, 2048), (9, 5, 64, 2040), (4, 17, 32, 2048),
                                    (1, 16, 32, 2048), (2, 33, 32, 2017), (5, 96, 32, 2048), (3, 100, 64, 2048),
+                                   (4, 256, 32, 2048), (3, 200, 32, 2048), (3, 150, 32, 2040), (2, 300, 32, 2048),
                                    (6, 256, 32, 1024), (5, 200, 32, 1024), (4, 130, 64, 1000), (7, 40, 32, 1024)])
 def test_two_way_split_backward_for_2048_units(shape):
     # 2048 (padded) hidden units: the persistent backward kernel splits its product over column slices AND over the
     # contraction, and sums the partial products through a second ring.  One row block (8 contraction slices) and two
     # to four (4 slices, two groups taking alternate blocks, one or two passes per workgroup), ragged batches, padded
-    # hidden sizes, a single step; against torch, against the one-way layout, and through the give-up path.
+    # hidden sizes, a single step; against torch, against the one-way layout, and through the give-up path.  More than
+    # 128 rows: the batch is walked in windows of 128 rows, one persistent launch each (the last one short).
     # 1024 (padded) hidden units: 16 column slices x 2 contraction slices inside every XCD, one row block per XCD.
     from flashlstm_poc_amd import LstmCore
     T, B, I, H = shape

@@ -147,11 +147,13 @@ def test_chunked_streaming_gives_the_whole_sequence_results(shape, monkeypatch):
             assert rell2(out["db"], whole["db"]) < 1e-6   # summed per launch, then over launches
 
 
-def test_chunked_streaming_with_the_grouped_two_way_backward_layout(monkeypatch):
+@pytest.mark.parametrize("B", [96, 200])
+def test_chunked_streaming_with_the_grouped_two_way_backward_layout(B, monkeypatch):
     # 2048 hidden units and 96 batch rows: the backward recurrence runs in two groups of workgroups that take alternate
     # row blocks (one group makes two passes per step, the other one), fed here in ranges of 1, 2 and 5 steps.  The
-    # rings, the running dc and the bias sums have to carry over from launch to launch exactly.
-    p = make_problem(6, 96, 32, 2048, seed=12)
+    # rings, the running dc and the bias sums have to carry over from launch to launch exactly.  200 rows: every range
+    # of steps is two launches (windows of 128 and 72 batch rows) that share the ring of partial sums.
+    p = make_problem(6, B, 32, 2048, seed=12)
     monkeypatch.setenv("FLASHLSTM_V2_CHUNK_STEPS", "0")
     whole = run_v2(p, R=3)
     for chunk in ("1", "2", "5"):
