@@ -725,14 +725,12 @@ int backward_finish(flstm_core_plan* p, const void* x, flstm_dtype x_dtype, floa
     const half_t* Hop = p->Y.as<half_t>();
     const int n_ih = dW_ih ? d.Ip : 0, n_hh = dW_hh ? d.Hp : 0, ncols = n_ih + n_hh;
     if (ncols > 0) {
-        const int tiles = int(ceil_div(size_t(4) * d.Hp, 256) * (ceil_div(size_t(n_ih), 256) + ceil_div(size_t(n_hh), 256)));
-        // automatic: one work item (tile x split) per compute unit, at least four 64-row slabs per split
-        // (measured best or within a few percent of it from 4 to 256 tiles)
+        // automatic: what the kernel's own schedule makes fastest (gemm_tn_auto_splits), at least four 64-row slabs
+        // per split
         int want = p->opt_dw_splits > 0 ? p->opt_dw_splits : p->eff_dw;
         if (want <= 0) {
-            want = int(ceil_div(size_t(p->num_cus > 0 ? p->num_cus : 256), size_t(tiles)));
-            const int cap = int(TB / 256);
-            if (want > cap) want = cap;
+            const size_t cap = TB / 256 < 64 ? TB / 256 : 64;
+            want = gemm_tn_auto_splits(4 * d.Hp, n_ih ? n_ih : n_hh, n_ih ? n_hh : 0, int(TB), cap < 1 ? 1 : int(cap));
         }
         if (want > 64) want = 64;
         const int splits = gemm_effective_splits(int(TB), want);
@@ -1045,14 +1043,13 @@ extern "C" int flstm_core_tune(flstm_core_plan* p, size_t T, int repeats, int tr
             if (b_is && (best.ms_b < 0 || b_ms < best.ms_b)) { best.ms_b = b_ms; best.mt_b = mt; best.step_b = step; }
         }
     }
-    // 2) split-K count of the weight-gradient GEMM around the rule of thumb (one work item per compute unit)
+    // 2) split-K count of the weight-gradient GEMM around what the schedule model picks
     p->opt_stepwise = best.step_f && best.step_b; p->opt_mt_f = best.mt_f; p->opt_mt_b = best.mt_b;
     replan(p);
-    const int tiles = int(ceil_div(size_t(4) * d.Hp, 256) * (ceil_div(size_t(d.Ip), 256) + ceil_div(size_t(d.Hp), 256)));
-    int rule = int(ceil_div(size_t(p->num_cus > 0 ? p->num_cus : 256), size_t(tiles)));
-    if (rule < 1) rule = 1;
+    const size_t cap = TB / 256 < 64 ? TB / 256 : 64;
+    const int rule = gemm_tn_auto_splits(4 * d.Hp, d.Ip, d.Hp, int(TB), cap < 1 ? 1 : int(cap));
     int last_eff = -1;
-    for (int cand : {rule / 2, rule, rule * 2, rule * 4}) {
+    for (int cand : {rule / 2, rule, rule + 1, rule * 2, rule * 4}) {
         if (cand < 1 || cand > 64) continue;
         const int eff = gemm_effective_splits(int(TB), cand);
         if (eff == last_eff) continue;

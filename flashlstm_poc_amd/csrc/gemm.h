@@ -32,5 +32,8 @@ hipError_t launch_gemm_tn(const GemmNT& g, hipStream_t stream);
 // Number of K slices the launchers really produce when `wanted` are asked for (every slice gets a
 // whole number of 64-wide K slabs). Size split-K partial buffers with this.
 int gemm_effective_splits(int K, int wanted);
+// The split count launch_gemm_tn runs fastest with for fp32 partials of an M x (N1 + N2) product over K (two B operands
+// side by side when N2 > 0), at most max_splits.
+int gemm_tn_auto_splits(int M, int N1, int N2, int K, int max_splits);
 
 }  // namespace flstm_hip

@@ -580,6 +580,27 @@ hipError_t launch_gemm_tn(const GemmNT& g, hipStream_t stream) {
     return hipGetLastError();
 }
 
+// Split count for a TN product with fp32 partials, from the way the kernel schedules it: blocks of 32 tiles x splits
+// are dealt to the 8 XCDs in rounds, a round runs K / splits, and every work item costs about 16 slabs' worth of
+// prologue and partial-tile write on top.  (4096 x 2048 tiles at K = 262144: 2 splits, 4.6 ms against 8.2 at one;
+// 8192 x (512 + 2048): 10 blocks, 2 rounds at one split, 5 full ones at 4, 8.2 -> 6.05 ms at K = 131072.)
+int gemm_tn_auto_splits(int M, int N1, int N2, int K, int max_splits) {
+    const int tiles_m = (M + BM - 1) / BM;
+    const int tiles_n = (N1 + BN - 1) / BN + (N2 > 0 ? (N2 + BN - 1) / BN : 0);
+    const int nslab = (K + BK - 1) / BK;
+    const TileOrder o = make_order(tiles_m, tiles_n, 1);
+    const long blocks = long(o.nsm) * o.nsn;
+    int best_s = 1;
+    double best_cost = -1.0;
+    for (int sp = 1; sp <= max_splits && sp <= nslab; ++sp) {
+        if (gemm_effective_splits(K, sp) != sp) continue;
+        const long rounds = (blocks * sp + 7) / 8;
+        const double cost = double(rounds) * (double((nslab + sp - 1) / sp) + 16.0);
+        if (best_cost < 0 || cost < best_cost * (1.0 - 1e-9)) { best_cost = cost; best_s = sp; }
+    }
+    return best_s;
+}
+
 int gemm_effective_splits(int K, int wanted) {
     const int nslab = (K + BK - 1) / BK;
     if (wanted < 1) wanted = 1;
