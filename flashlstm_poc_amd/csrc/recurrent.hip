@@ -931,6 +931,12 @@ __global__ __launch_bounds__(kThreads) void rec_fwd_kernel(RecFwdArgs p, RecLayo
                 }
             }
             clk.lap(3);
+            // One row tile per block and 8 threads per row: the waves of rows 16..31 have no cells to update and would
+            // reach the next product ahead of its operand.  A wave that finds its first chunk unwritten polls, and a
+            // poll notices the data a full round trip to the L2 after it went out, whereas a wave that asks once the
+            // data is there has it after one trip: measured, the early waves finished their product 0.4 us AFTER the
+            // others (2048 units, 16 rows).  So all four waves start a product together.
+            if constexpr (MT == 1 && GPR == 8) __syncthreads();
         }
     }
     clk.flush();
@@ -1173,6 +1179,7 @@ __global__ __launch_bounds__(kThreads) void rec_bwd_kernel(RecBwdArgs p, RecLayo
                 }
             }
             clk.lap(3);
+            if constexpr (MT == 1 && GPR == 8) __syncthreads();   // (waves without cells to update: as in the forward kernel)
         }
     }
     clk.flush();
@@ -1607,6 +1614,9 @@ __global__ __launch_bounds__(kThreads) void rec_bwd2d_kernel(RecBwdArgs p, RecLa
                 cell(t, rb_prev, dcreg[i >= 1 ? i - 1 : 0], dh, ops[(i + 1) & 1]);
             }
         }
+        // (16-row blocks: the waves of rows 16..31 have no cells to update; all four waves start the next product
+        // together, as in the forward kernel)
+        if constexpr (MT == 1) __syncthreads();
     }
     clk.flush();
     if (t_last >= 0) {   // a launch that stops before the closing pass leaves dc in memory for the next one
