@@ -951,6 +951,11 @@ extern "C" size_t flstm_gemm_tn_workspace_bytes(size_t M, size_t N, size_t K, in
     return eff <= 1 ? 0 : size_t(eff) * M * N * sizeof(float);
 }
 
+extern "C" int flstm_gemm_tn_auto_splits(size_t M, size_t N, size_t K, int max_splits) {
+    if (M == 0 || N == 0 || K == 0 || M > (1u << 30) || N > (1u << 30) || K > (1u << 30)) return 1;
+    return gemm_tn_auto_splits(int(M), int(N), 0, int(K), max_splits < 1 ? 1 : (max_splits > 64 ? 64 : max_splits));
+}
+
 extern "C" int flstm_gemm_tn(const void* A, size_t lda, const void* B, size_t ldb, size_t M, size_t N, size_t K,
                              float* C, size_t ldc, float alpha, int splits, void* workspace, void* stream) {
     if (!A || !B || !C || M > (1u << 30) || N > (1u << 30) || K > (1u << 30)) return FLSTM_E_INVALID;

@@ -175,10 +175,13 @@ double flstm_core_tuned_ms(const flstm_core_plan* plan, size_t seq_len, const ch
  * flstm_gemm_tn:  C[M][N] = alpha * sum_k A[k][m] * B[k][n]; A is [K][lda], B is [K][ldb] fp16 (the weight gradients
  *   dG^T * X).  M and N must be multiples of 8, K is arbitrary; C is fp32, 16-byte aligned.  splits > 1 cuts K
  *   into that many slices (at most: every slice gets whole 64-row slabs) whose partial products go to `workspace`
- *   (flstm_gemm_tn_workspace_bytes() bytes of device memory, 16-byte aligned) and are then summed into C. */
+ *   (flstm_gemm_tn_workspace_bytes() bytes of device memory, 16-byte aligned) and are then summed into C.
+ * flstm_gemm_tn_auto_splits:  the split count flstm_gemm_tn runs fastest with on a 256-CU part, at most max_splits
+ *   (the rule flstm_core_backward applies to the weight gradients; a pure function of the sizes, no device needed). */
 int flstm_gemm_nt(const void* A, size_t lda, const void* B, size_t ldb, size_t M, size_t N, size_t K,
                   void* C, flstm_dtype c_dtype, size_t ldc, float alpha, const float* bias, void* stream);
 size_t flstm_gemm_tn_workspace_bytes(size_t M, size_t N, size_t K, int splits);
+int flstm_gemm_tn_auto_splits(size_t M, size_t N, size_t K, int max_splits);
 int flstm_gemm_tn(const void* A, size_t lda, const void* B, size_t ldb, size_t M, size_t N, size_t K,
                   float* C, size_t ldc, float alpha, int splits, void* workspace, void* stream);
 

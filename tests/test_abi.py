@@ -33,6 +33,23 @@ def test_library_exports_every_declared_symbol():
         assert hasattr(lib, name), f"{name} declared in a header but not exported"
 
 
+def test_split_count_rule_of_the_weight_gradient_gemm():
+    # A pure function of the sizes: blocks of 32 tiles x splits are dealt to the 8 XCDs in rounds, a round runs
+    # K / splits, every work item costs a fixed extra.  Pinned on cases whose answer follows from counting rounds.
+    from flashlstm_poc_amd import library_path
+    lib = ctypes.CDLL(library_path())
+    f = lib.flstm_gemm_tn_auto_splits
+    f.restype = ctypes.c_int
+    f.argtypes = [ctypes.c_size_t, ctypes.c_size_t, ctypes.c_size_t, ctypes.c_int]
+    assert f(4096, 2048, 262144, 64) == 2      # 128 tiles = 4 blocks: one split leaves half the XCDs idle, two fill them
+    assert f(8192, 4096, 524288, 64) == 1      # 512 tiles = 16 blocks: two full rounds already
+    assert f(8192, 2560, 524288, 64) == 4      # 320 tiles = 10 blocks: 2 rounds at one split, 5 full rounds at four
+    assert f(256, 256, 1 << 20, 64) == 8       # one block: a split per XCD, more only adds partial tiles
+    assert f(256, 256, 1 << 20, 3) == 3        # capped by the caller
+    assert f(4096, 2048, 64, 64) == 1          # a single 64-row slab cannot be split
+    assert f(0, 2048, 4096, 8) == 1 and f(4096, 2048, 4096, 0) == 1
+
+
 def test_v1_enum_values_and_handle_layout():
     text = open(os.path.join(ROOT, "include/flashlstm/lstm_api.h")).read()
     assert re.search(r"LSTM_COMPUTE_PRECISION_FP16_ACC32\s*=\s*0", text)
