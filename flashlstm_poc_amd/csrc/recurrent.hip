@@ -251,7 +251,7 @@ __device__ __forceinline__ bool product_poisoned(const floatx4 (&acc)[2][NT]) {
 // fetched and multiplied before tile 1 is touched, so the first half of a step's product runs while the peers are
 // still busy with the second half of their cell updates.  Chunks of CKT k-steps of ONE tile alternate between two
 // register sets (as many registers as the two-tile chunks of wave_product).  Resident weights only.
-template <int NT, int KS, int KL, int NPF, int NBUF, bool LAZY = false, int CKO = 0, typename Prefetch>
+template <int NT, int KS, int KL, int NPF, int NBUF, bool LAZY = false, int CKO = 0, bool REASK = false, typename Prefetch>
 __device__ __forceinline__ void wave_product_tiles(floatx4 (&acc)[2][NT], const half8 (&wreg)[KS - KL][NT],
                                                    const half8* wlds, const half_t* a0, const half_t* a1, int wave,
                                                    int lane, int nks_total, int ks_wave, int rotation, const Poll& poll,
@@ -325,8 +325,20 @@ __device__ __forceinline__ void wave_product_tiles(floatx4 (&acc)[2][NT], const 
                 long long spin_start = 0;
                 do {
                     if (poll_give_up(poll, spins, spin_start, lane)) break;   // results are garbage from here on; the workgroup leaves at its next barrier
+                    // The chunks requested ahead of this one went out at the same moment and are as stale: left alone,
+                    // each of them is found unwritten in its turn and costs a round trip of its own.  REASK requests
+                    // them again behind this chunk, so that the wave leaves this loop with fresh ones in flight.  That
+                    // pays where a round trip is long (groups that span XCDs: 2048 units and 16 rows, forward
+                    // 3.00 -> 2.85 us per step) and costs where it is short and the polls share one L2 (1024 units and
+                    // 256 rows, forward 3.56 -> 3.8: twice the poll traffic in front of the producers' stores).
                     issue(c);
-                    wait_frags<0>(f[buf]);   // (whatever was in flight behind this chunk has landed as well)
+                    if constexpr (REASK) {
+#pragma unroll
+                        for (int j = c + 1; j <= last_issued; ++j) issue(j);
+                        wait_frags_upto(f[buf], (last_issued - c) * CKT);   // (what was in flight before has landed as well)
+                    } else {
+                        wait_frags<0>(f[buf]);   // (whatever was in flight behind this chunk has landed as well)
+                    }
                 } while (unwritten());
             }
         }
@@ -369,7 +381,7 @@ __device__ __forceinline__ void wave_product_tiles(floatx4 (&acc)[2][NT], const 
 
 // `prefetch` issues exactly NPF vector loads (for every wave, whatever its lanes need) behind the last
 // fragment load.
-template <int NT, int KS, bool RESIDENT, int KL, int NPF, int MT, int NBUF = 2, int CKO = 0, bool LAZY = false, typename Prefetch>
+template <int NT, int KS, bool RESIDENT, int KL, int NPF, int MT, int NBUF = 2, int CKO = 0, bool LAZY = false, bool REASK = false, typename Prefetch>
 __device__ __forceinline__ void wave_product(floatx4 (&acc)[2][NT], const half8 (&wreg)[KS - KL][NT],
                                              const half8* wlds, const half8* wfrag_wave, const half_t* a0,
                                              const half_t* a1, int wave, int lane, int nks_total,
@@ -427,18 +439,21 @@ __device__ __forceinline__ void wave_product(floatx4 (&acc)[2][NT], const half8 
             // chunk is out (c, D, NCH are compile-time constants: the switch folds)
             const int last_now = (c + D < NCH - 1) ? c + D : NCH - 1;
             const bool prefetched = (c + D >= NCH - 1);
-            switch ((last_now - c) * 2 + (prefetched ? 1 : 0)) {
-                case 0: wait(std::integral_constant<int, 0>{}, buf); break;
-                case 1: wait(std::integral_constant<int, NPF>{}, buf); break;
-                case 2: wait(std::integral_constant<int, MT * CK>{}, buf); break;
-                case 3: wait(std::integral_constant<int, MT * CK + NPF>{}, buf); break;
-                case 4: wait(std::integral_constant<int, 2 * MT * CK>{}, buf); break;
-                case 5: wait(std::integral_constant<int, 2 * MT * CK + NPF>{}, buf); break;
-                case 6: wait(std::integral_constant<int, 3 * MT * CK>{}, buf); break;
-                case 7: wait(std::integral_constant<int, 3 * MT * CK + NPF>{}, buf); break;
-                case 8: wait(std::integral_constant<int, 4 * MT * CK>{}, buf); break;
-                default: wait(std::integral_constant<int, 4 * MT * CK + NPF>{}, buf); break;
-            }
+            auto wait_with = [&](int chunks_behind, bool prefetch_behind) {   // ... of chunk c; constants once unrolled
+                switch (chunks_behind * 2 + (prefetch_behind ? 1 : 0)) {
+                    case 0: wait(std::integral_constant<int, 0>{}, buf); break;
+                    case 1: wait(std::integral_constant<int, NPF>{}, buf); break;
+                    case 2: wait(std::integral_constant<int, MT * CK>{}, buf); break;
+                    case 3: wait(std::integral_constant<int, MT * CK + NPF>{}, buf); break;
+                    case 4: wait(std::integral_constant<int, 2 * MT * CK>{}, buf); break;
+                    case 5: wait(std::integral_constant<int, 2 * MT * CK + NPF>{}, buf); break;
+                    case 6: wait(std::integral_constant<int, 3 * MT * CK>{}, buf); break;
+                    case 7: wait(std::integral_constant<int, 3 * MT * CK + NPF>{}, buf); break;
+                    case 8: wait(std::integral_constant<int, 4 * MT * CK>{}, buf); break;
+                    default: wait(std::integral_constant<int, 4 * MT * CK + NPF>{}, buf); break;
+                }
+            };
+            wait_with(last_now - c, prefetched);
             static_assert(NBUF <= 5, "the switch above knows up to four chunks ahead");
             auto unwritten = [&]() -> bool {
                 unsigned m = 0u;
@@ -460,8 +475,17 @@ __device__ __forceinline__ void wave_product(floatx4 (&acc)[2][NT], const half8 
                     long long spin_start = 0;
                     do {
                         if (poll_give_up(poll, spins, spin_start, lane)) break;
+                        // (REASK: with the chunks that were requested ahead of it, which are as stale: see
+                        // wave_product_tiles; not where a wave holds 64 k-steps: that kernel has no registers left
+                        // for the addresses)
                         issue(c, buf);
-                        wait(std::integral_constant<int, 0>{}, buf);   // (also what was issued after this chunk the first time)
+                        if constexpr (REASK && KS < 64) {
+#pragma unroll
+                            for (int j = c + 1; j <= last_now; ++j) issue(j, j % NBUF);
+                            wait_with(last_now - c, false);   // (also what was issued after this chunk the first time)
+                        } else {
+                            wait(std::integral_constant<int, 0>{}, buf);
+                        }
                     } while (unwritten());
                 }
             }
@@ -843,10 +867,10 @@ __global__ __launch_bounds__(kThreads) void rec_fwd_kernel(RecFwdArgs p, RecLayo
 #pragma unroll
                 for (int n = 0; n < NT; ++n) acc[m][n] = floatx4{0.f, 0.f, 0.f, 0.f};
             if constexpr (SPLIT)
-                wave_product_tiles<NT, KS, 0, NPH * UPT / 2, kFwdBufs>(acc, wreg, nullptr, a0, a1, wave, lane, nks_total, ks_wave, rotation, poll,
+                wave_product_tiles<NT, KS, 0, NPH * UPT / 2, kFwdBufs, false, 0, DS>(acc, wreg, nullptr, a0, a1, wave, lane, nks_total, ks_wave, rotation, poll,
                                                              [&]() { prefetch(t, rb); });
             else
-                wave_product<NT, KS, RESIDENT, 0, UPT / 2, MT, DEEP ? 4 : 2, DEEP ? 2 : 0, DEEP>(acc, wreg, nullptr, wfrag_wave, a0, a1, wave, lane, nks_total,
+                wave_product<NT, KS, RESIDENT, 0, UPT / 2, MT, DEEP ? 4 : 2, DEEP ? 2 : 0, DEEP, DS && !DEEP>(acc, wreg, nullptr, wfrag_wave, a0, a1, wave, lane, nks_total,
                                                                ks_wave, rotation, poll, [&]() { prefetch(t, rb); });
             clk.lap(0);
             spill_partials<NT, MT>(part, acc, wave, lane, PLD);
@@ -1055,10 +1079,10 @@ __global__ __launch_bounds__(kThreads) void rec_bwd_kernel(RecBwdArgs p, RecLayo
                 if constexpr (SPLIT)
                     // (four sets of 4 k-steps: as many registers as two sets of 8, three quarters of them in flight
                     // instead of half; measured 4.59 -> 4.50 us per step, three sets of 8: 4.65)
-                    wave_product_tiles<NT, KS, KL, NPF, 4, false, 4>(acc, wreg, wlds, a0, a1, wave, lane, nks_total, ks_wave, rotation, poll,
+                    wave_product_tiles<NT, KS, KL, NPF, 4, false, 4, DS>(acc, wreg, wlds, a0, a1, wave, lane, nks_total, ks_wave, rotation, poll,
                                                            [&]() { prefetch(t, rb); });
                 else
-                    wave_product<NT, KS, RESIDENT, KL, NPF, MT>(acc, wreg, wlds, wfrag_wave, a0, a1, wave, lane, nks_total,
+                    wave_product<NT, KS, RESIDENT, KL, NPF, MT, 2, 0, false, DS>(acc, wreg, wlds, wfrag_wave, a0, a1, wave, lane, nks_total,
                                                               ks_wave, rotation, poll, [&]() { prefetch(t, rb); });
                 clk.lap(0);
                 spill_partials<NT, MT>(part, acc, wave, lane, PLD);
@@ -1520,7 +1544,7 @@ __global__ __launch_bounds__(kThreads) void rec_bwd2d_kernel(RecBwdArgs p, RecLa
                 const half_t* a1 = a0 + size_t(nks) * 512;
                 // (where the operand comes through memory -- groups that span XCDs -- and the contraction is long, five
                 // short fragment sets keep the fetch running over that trip)
-                wave_product<NT, KS, true, KL, NPF, MT, ((KS >= 16 && !LOCAL) ? 5 : 2), ((KS >= 16 && !LOCAL) ? 2 : 0)>(acc, wreg, wlds, nullptr, a0, a1, wave, lane, KS * 4, KS, rotation, poll,
+                wave_product<NT, KS, true, KL, NPF, MT, ((KS >= 16 && !LOCAL) ? 5 : 2), ((KS >= 16 && !LOCAL) ? 2 : 0), false, !LOCAL>(acc, wreg, wlds, nullptr, a0, a1, wave, lane, KS * 4, KS, rotation, poll,
                                                        [&]() { load_ops(t, rb, ops[i & 1]); });
                 clk.lap(0);
                 spill_partials<NT, MT>(part, acc, wave, lane, PLD);
