@@ -252,7 +252,7 @@ __device__ __forceinline__ bool product_poisoned(const floatx4 (&acc)[2][NT]) {
 // still busy with the second half of their cell updates.  Chunks of CKT k-steps of ONE tile alternate between two
 // register sets (as many registers as the two-tile chunks of wave_product).  Resident weights only.
 template <int NT, int KS, int KL, int NPF, int NBUF, bool LAZY = false, int CKO = 0, bool REASK = false, typename Prefetch>
-__device__ __forceinline__ void wave_product_tiles(floatx4 (&acc)[2][NT], const half8 (&wreg)[KS - KL][NT],
+__device__ __forceinline__ bool wave_product_tiles(floatx4 (&acc)[2][NT], const half8 (&wreg)[KS - KL][NT],
                                                    const half8* wlds, const half_t* a0, const half_t* a1, int wave,
                                                    int lane, int nks_total, int ks_wave, int rotation, const Poll& poll,
                                                    Prefetch&& prefetch) {
@@ -264,6 +264,7 @@ __device__ __forceinline__ void wave_product_tiles(floatx4 (&acc)[2][NT], const 
     half8 f[NBUF][CKT];
     bool check_all = !LAZY;   // second pass: every chunk is checked word by word
     bool early = false;
+    bool ahead_of_producers = false;   // the very first chunk was not there yet (returned: see FirstRequestDelay)
     for (;;) {
     // (the operand's address as a value the compiler cannot see through: the fragment addresses are then computed
     // where they are used in every pass instead of all of them ahead of this loop, in registers that are not there)
@@ -321,6 +322,7 @@ __device__ __forceinline__ void wave_product_tiles(floatx4 (&acc)[2][NT], const 
         if (c % NCHK == 0 || (ahead && early) || __builtin_expect(check_all, 0)) {
             if (__builtin_expect(unwritten() && poll.on, 0)) {
                 if (c % NCHK == 0) early = true;
+                if (c == 0) ahead_of_producers = true;
                 int spins = 0;
                 long long spin_start = 0;
                 do {
@@ -368,6 +370,7 @@ __device__ __forceinline__ void wave_product_tiles(floatx4 (&acc)[2][NT], const 
 #pragma unroll
         for (int n = 0; n < NT; ++n) acc[m][n] = floatx4{0.f, 0.f, 0.f, 0.f};
     }
+    return ahead_of_producers;
 }
 
 // acc[mt][nt] += (A(16*MT rows x K) * Wslice)^T, this wave's interleaved k-steps only.
@@ -382,7 +385,7 @@ __device__ __forceinline__ void wave_product_tiles(floatx4 (&acc)[2][NT], const 
 // `prefetch` issues exactly NPF vector loads (for every wave, whatever its lanes need) behind the last
 // fragment load.
 template <int NT, int KS, bool RESIDENT, int KL, int NPF, int MT, int NBUF = 2, int CKO = 0, bool LAZY = false, bool REASK = false, typename Prefetch>
-__device__ __forceinline__ void wave_product(floatx4 (&acc)[2][NT], const half8 (&wreg)[KS - KL][NT],
+__device__ __forceinline__ bool wave_product(floatx4 (&acc)[2][NT], const half8 (&wreg)[KS - KL][NT],
                                              const half8* wlds, const half8* wfrag_wave, const half_t* a0,
                                              const half_t* a1, int wave, int lane, int nks_total,
                                              int ks_wave, int rotation, const Poll& poll, Prefetch&& prefetch) {
@@ -400,6 +403,7 @@ __device__ __forceinline__ void wave_product(floatx4 (&acc)[2][NT], const half8 
         half8 fa[NBUF][CK], fb[NBUF][CK];
         bool check_all = !LAZY;   // second pass: every chunk is checked word by word
         bool early = false;               // the first chunk had to be fetched again: what was requested ahead of it is checked too
+        bool ahead_of_producers = false;  // ... on the first pass over the product (returned: see FirstRequestDelay)
         for (;;) {
         const half_t *p0 = a0, *p1 = a1;   // (opaque copies, as in wave_product_tiles)
         if constexpr (LAZY) asm volatile("" : "+v"(p0), "+v"(p1));
@@ -471,6 +475,7 @@ __device__ __forceinline__ void wave_product(floatx4 (&acc)[2][NT], const half8 
             if (c == 0 || (c <= D && early) || __builtin_expect(check_all, 0)) {   // (peeled; first pass: as in wave_product_tiles)
                 if (__builtin_expect(unwritten() && poll.on, 0)) {
                     if (c == 0) early = true;
+                    if (c == 0) ahead_of_producers = true;
                     int spins = 0;
                     long long spin_start = 0;
                     do {
@@ -512,6 +517,7 @@ __device__ __forceinline__ void wave_product(floatx4 (&acc)[2][NT], const half8 
 #pragma unroll
             for (int n = 0; n < NT; ++n) acc[m][n] = floatx4{0.f, 0.f, 0.f, 0.f};
         }
+        return ahead_of_producers;
     } else {
         for (int k = 0; k < ks_wave; ++k) {
             const int kg = rec_kstep_of_slot(k, rotation, ks_wave) * 4 + wave;
@@ -527,6 +533,7 @@ __device__ __forceinline__ void wave_product(floatx4 (&acc)[2][NT], const half8 
             }
         }
         prefetch();
+        return false;
     }
 }
 
@@ -762,6 +769,25 @@ struct PhaseClock {
     }
 };
 
+// When to send the first request of a product.  A wave that asks before its producers have published polls, and a poll
+// notices the data a full round trip after it went out; a wave that asks just after they have published has the data
+// after one trip.  Where the chain from step to step is exposed (one row block per group) every wave is ahead of its
+// producers at every step, by about the same time.  So a wave holds its first request back by a delay it regulates
+// itself: found the first chunk unwritten -> one unit (of 64 clocks) more, found it there -> a sixteenth of a unit
+// less.  It settles just behind the moment the data lands, with a miss every sixteenth step or so; where a wave is
+// not ahead of its producers (several row blocks per workgroup) it decays to nothing.  Measured, forward at 2048
+// units, us per step: 16 rows 2.89 -> 2.64 (the best fixed delay, 8 units: 2.56), 32 rows 3.23 -> 2.77, 64 rows
+// 4.43 -> 3.73; two units up and an eighth down: 2.73 / 2.83 / 3.81.
+struct FirstRequestDelay {
+    int sixteenths = 0;
+    __device__ __forceinline__ void hold() const {
+        for (int i = 0; i < (sixteenths >> 4); ++i) __builtin_amdgcn_s_sleep(1);
+    }
+    __device__ __forceinline__ void learn(bool ahead_of_producers) {
+        sixteenths = ahead_of_producers ? min(sixteenths + 16, 16 * 48) : max(sixteenths - 1, 0);
+    }
+};
+
 // ------------------------------------------------------------------------------------ forward
 // Per step and row block: K-split MFMA product on h_{t-1} as it arrives -> partial sums through LDS
 // (two buffers, one barrier per step) -> pointwise cell update -> store h_t -> store c_t and the
@@ -808,6 +834,7 @@ __global__ __launch_bounds__(kThreads) void rec_fwd_kernel(RecFwdArgs p, RecLayo
     const Poll poll{L.persistent != 0, p.spin_limit, p.spin_ticks, p.status, (lds_int_t*)&lds_abort};
     PhaseClock clk{(blockIdx.x == 0) ? p.prof : nullptr, 0};
     int item = 0;   // work items done: selects the partial-sum buffer
+    FirstRequestDelay first_request;
 
     const half8* wfrag_wave = p.wfrag + (size_t(hs) * 4 + wave) * size_t(ks_wave) * NT * kWave;
     half8 wreg[KS][NT];
@@ -866,12 +893,15 @@ __global__ __launch_bounds__(kThreads) void rec_fwd_kernel(RecFwdArgs p, RecLayo
             for (int m = 0; m < 2; ++m)
 #pragma unroll
                 for (int n = 0; n < NT; ++n) acc[m][n] = floatx4{0.f, 0.f, 0.f, 0.f};
+            if constexpr (DS) first_request.hold();
+            bool ahead;
             if constexpr (SPLIT)
-                wave_product_tiles<NT, KS, 0, NPH * UPT / 2, kFwdBufs, false, 0, DS>(acc, wreg, nullptr, a0, a1, wave, lane, nks_total, ks_wave, rotation, poll,
+                ahead = wave_product_tiles<NT, KS, 0, NPH * UPT / 2, kFwdBufs, false, 0, DS>(acc, wreg, nullptr, a0, a1, wave, lane, nks_total, ks_wave, rotation, poll,
                                                              [&]() { prefetch(t, rb); });
             else
-                wave_product<NT, KS, RESIDENT, 0, UPT / 2, MT, DEEP ? 4 : 2, DEEP ? 2 : 0, DEEP, DS && !DEEP>(acc, wreg, nullptr, wfrag_wave, a0, a1, wave, lane, nks_total,
+                ahead = wave_product<NT, KS, RESIDENT, 0, UPT / 2, MT, DEEP ? 4 : 2, DEEP ? 2 : 0, DEEP, DS && !DEEP>(acc, wreg, nullptr, wfrag_wave, a0, a1, wave, lane, nks_total,
                                                                ks_wave, rotation, poll, [&]() { prefetch(t, rb); });
+            if constexpr (DS) first_request.learn(ahead);
             clk.lap(0);
             spill_partials<NT, MT>(part, acc, wave, lane, PLD);
             __syncthreads();
