@@ -1031,6 +1031,7 @@ __global__ __launch_bounds__(kThreads) void rec_bwd_kernel(RecBwdArgs p, RecLayo
     const float S = p.dy_scale;
     PhaseClock clk{(blockIdx.x == 0) ? p.prof : nullptr, 0};
     int item = 0;   // work items done: selects the partial-sum buffer
+    FirstRequestDelay first_request;
 
     const half8* wfrag_wave = p.wfrag + (size_t(hs) * 4 + wave) * size_t(ks_wave) * NT * kWave;
     half8 wreg[KR][NT];
@@ -1106,14 +1107,17 @@ __global__ __launch_bounds__(kThreads) void rec_bwd_kernel(RecBwdArgs p, RecLayo
                 for (int m = 0; m < 2; ++m)
 #pragma unroll
                     for (int n = 0; n < NT; ++n) acc[m][n] = floatx4{0.f, 0.f, 0.f, 0.f};
+                if constexpr (DS) first_request.hold();   // (measured: 2048 units and 64 rows 7.37 -> 6.83 us per step; inside an XCD 1-6 % slower)
+                bool ahead;
                 if constexpr (SPLIT)
                     // (four sets of 4 k-steps: as many registers as two sets of 8, three quarters of them in flight
                     // instead of half; measured 4.59 -> 4.50 us per step, three sets of 8: 4.65)
-                    wave_product_tiles<NT, KS, KL, NPF, 4, false, 4, DS>(acc, wreg, wlds, a0, a1, wave, lane, nks_total, ks_wave, rotation, poll,
+                    ahead = wave_product_tiles<NT, KS, KL, NPF, 4, false, 4, DS>(acc, wreg, wlds, a0, a1, wave, lane, nks_total, ks_wave, rotation, poll,
                                                            [&]() { prefetch(t, rb); });
                 else
-                    wave_product<NT, KS, RESIDENT, KL, NPF, MT, 2, 0, false, DS>(acc, wreg, wlds, wfrag_wave, a0, a1, wave, lane, nks_total,
+                    ahead = wave_product<NT, KS, RESIDENT, KL, NPF, MT, 2, 0, false, DS>(acc, wreg, wlds, wfrag_wave, a0, a1, wave, lane, nks_total,
                                                               ks_wave, rotation, poll, [&]() { prefetch(t, rb); });
+                if constexpr (DS) first_request.learn(ahead);
                 clk.lap(0);
                 spill_partials<NT, MT>(part, acc, wave, lane, PLD);
                 __syncthreads();
