@@ -460,6 +460,7 @@ int forward_recur(flstm_core_plan* p, size_t t0, size_t n, hipStream_t s) {
     a.X = p->xch_f.as<half_t>(); a.x_slot = exchange_slot_halfs(d.B, d.Hp);
     a.status = p->status.as<int>();
     a.seats = p->status.as<unsigned>() + 8;
+    a.delay_hint = p->status.as<int>() + 1;   // (the status block: word 0 status, 1 / 2 delay hints, 8..15 seats)
     FL_TRY(fill_zero(a.seats, 8 * sizeof(unsigned), s));
     a.B = d.B; a.Hp = d.Hp; a.T = int(p->fw.T); a.t0 = int(t0); a.t1 = int(t0 + n);
     a.spin_limit = p->opt_spin_limit;
@@ -659,6 +660,7 @@ int backward_recur(flstm_core_plan* p, long t_hi, long t_lo, hipStream_t s) {
     a.db_part = p->db_part.as<float>();
     a.status = p->status.as<int>();
     a.seats = p->status.as<unsigned>() + 8;
+    a.delay_hint = p->status.as<int>() + 2;
     a.B = d.B; a.Hp = d.Hp; a.T = int(p->bw.T); a.dy_scale = p->bw.dy_scale;
     a.t_hi = int(t_hi); a.t_lo = int(t_lo);
     a.spin_limit = p->opt_spin_limit;

@@ -43,6 +43,8 @@ struct RecFwdArgs {
     half_t* G;           // [T*B][4Hp] packed gate order; in: x-projection + bias, out: activated i,f,g,o
     float* C;            // [(T+1)*B][Hp]; rows [0,B) = c0, rows [(t+1)B, ..) = c_t
     unsigned* seats;     // [8] zeroed before every launch: next free workgroup slot per XCD
+    int* delay_hint;     // may be null: where a launch that regulates its first requests finds the delay its predecessor
+                         // settled on, and leaves its own (a sequence fed in ranges of steps does not start over)
     int* status;         // 0 ok, 1 spin limit hit, 2 workgroup not on the expected XCD
     int B, Hp, T;
     int t0, t1;          // steps [t0, t1) of the sequence are run by this call (state and ring carry over)
@@ -71,6 +73,7 @@ struct RecBwdArgs {
     float* dH0;          // [B][Hp] out: scaled gradient wrt h0
     float* db_part;      // [ng][4Hp] scaled bias-gradient partial sums (accumulated into)
     unsigned* seats;     // [8] zeroed before every launch
+    int* delay_hint;     // as in RecFwdArgs
     int* status;
     int B, Hp, T;
     int b_lo, b_hi;      // two-dimensional layout: the launch works on batch rows [b_lo, b_hi) (b_lo a multiple of 32;

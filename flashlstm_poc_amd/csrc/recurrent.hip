@@ -779,12 +779,19 @@ struct PhaseClock {
 // units, us per step: 16 rows 2.89 -> 2.64 (the best fixed delay, 8 units: 2.56), 32 rows 3.23 -> 2.77, 64 rows
 // 4.43 -> 3.73; two units up and an eighth down: 2.73 / 2.83 / 3.81.
 struct FirstRequestDelay {
+    static constexpr int kMost = 16 * 48;
     int sixteenths = 0;
+    __device__ __forceinline__ void start_from(const int* hint) {
+        if (hint) sixteenths = __builtin_amdgcn_readfirstlane(min(max(*hint, 0), kMost));
+    }
+    __device__ __forceinline__ void leave(int* hint) const {
+        if (hint && blockIdx.x == 0 && threadIdx.x == 0) *hint = sixteenths;
+    }
     __device__ __forceinline__ void hold() const {
         for (int i = 0; i < (sixteenths >> 4); ++i) __builtin_amdgcn_s_sleep(1);
     }
     __device__ __forceinline__ void learn(bool ahead_of_producers) {
-        sixteenths = ahead_of_producers ? min(sixteenths + 16, 16 * 48) : max(sixteenths - 1, 0);
+        sixteenths = ahead_of_producers ? min(sixteenths + 16, kMost) : max(sixteenths - 1, 0);
     }
 };
 
@@ -835,6 +842,7 @@ __global__ __launch_bounds__(kThreads) void rec_fwd_kernel(RecFwdArgs p, RecLayo
     PhaseClock clk{(blockIdx.x == 0) ? p.prof : nullptr, 0};
     int item = 0;   // work items done: selects the partial-sum buffer
     FirstRequestDelay first_request;
+    if constexpr (DS) first_request.start_from(p.delay_hint);
 
     const half8* wfrag_wave = p.wfrag + (size_t(hs) * 4 + wave) * size_t(ks_wave) * NT * kWave;
     half8 wreg[KS][NT];
@@ -993,6 +1001,7 @@ __global__ __launch_bounds__(kThreads) void rec_fwd_kernel(RecFwdArgs p, RecLayo
             if constexpr (MT == 1 && GPR == 8) __syncthreads();
         }
     }
+    if constexpr (DS) first_request.leave(p.delay_hint);
     clk.flush();
 }
 
@@ -1032,6 +1041,7 @@ __global__ __launch_bounds__(kThreads) void rec_bwd_kernel(RecBwdArgs p, RecLayo
     PhaseClock clk{(blockIdx.x == 0) ? p.prof : nullptr, 0};
     int item = 0;   // work items done: selects the partial-sum buffer
     FirstRequestDelay first_request;
+    if constexpr (DS) first_request.start_from(p.delay_hint);
 
     const half8* wfrag_wave = p.wfrag + (size_t(hs) * 4 + wave) * size_t(ks_wave) * NT * kWave;
     half8 wreg[KR][NT];
@@ -1251,6 +1261,7 @@ __global__ __launch_bounds__(kThreads) void rec_bwd_kernel(RecBwdArgs p, RecLayo
         }
     }
 
+    if constexpr (DS) first_request.leave(p.delay_hint);
     // Bias gradient: fold this launch's sums over the threads that share a group column (fixed order).
     __syncthreads();
     float* red = part_all;  // [256][4 * UPT]
