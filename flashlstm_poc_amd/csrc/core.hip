@@ -108,6 +108,7 @@ struct flstm_core_plan {
     StepGraphCache graphs_f, graphs_b;   // captured step-wise launches (only used where the persistent kernels are not)
     int opt_graphs = 1;
     int opt_two_d = 1;   // backward recurrence for 2048 hidden units, two-way split: 0 never, 1 where it is faster, 2 wherever it can run
+    int opt_waves_f = 0, opt_waves_b = 0;   // wavefronts per workgroup of the recurrence kernels: 0 = by size, 4, 8 (the weights are packed for it)
     int* status_host = nullptr;   // pinned: the device status word lands here with the end-of-pass copy
     int inject_stall = 0;         // test hook: treat the next N persistent passes as if their launch had given up
     // weights
@@ -140,9 +141,9 @@ namespace {
 
 void replan(flstm_core_plan* p) {
     p->Lf = plan_rec_fwd(p->d.B, p->d.Hp, p->num_cus, p->opt_stepwise || p->hold_fwd > 0 || p->eff_step_f,
-                         p->opt_mt_f ? p->opt_mt_f : p->eff_mt_f);
+                         p->opt_mt_f ? p->opt_mt_f : p->eff_mt_f, p->opt_waves_f);
     p->Lb = plan_rec_bwd(p->d.B, p->d.Hp, p->num_cus, p->opt_stepwise || p->hold_bwd > 0 || p->eff_step_b,
-                         p->opt_mt_b ? p->opt_mt_b : p->eff_mt_b, p->opt_two_d);
+                         p->opt_mt_b ? p->opt_mt_b : p->eff_mt_b, p->opt_two_d, p->opt_waves_b);
     p->Lf.cooperative = p->Lb.cooperative = p->opt_cooperative;
     p->ks_f = rec_fwd_ks(p->Lf, p->d.Hp);
     p->ks_b = rec_bwd_ks(p->Lb, p->d.Hp);
@@ -254,6 +255,8 @@ extern "C" int flstm_core_create(size_t batch, size_t input_size, size_t hidden_
         if (const char* v = getenv("FLASHLSTM_COOPERATIVE_LAUNCH")) p->opt_cooperative = atoi(v) != 0;
         if (const char* v = getenv("FLASHLSTM_STEP_GRAPHS")) p->opt_graphs = atoi(v) != 0;
         if (const char* v = getenv("FLASHLSTM_BWD_TWO_D")) p->opt_two_d = atoi(v) < 0 ? 0 : (atoi(v) > 2 ? 2 : atoi(v));
+        if (const char* v = getenv("FLASHLSTM_WAVES_FWD")) p->opt_waves_f = (atoi(v) == 4 || atoi(v) == 8) ? atoi(v) : 0;
+        if (const char* v = getenv("FLASHLSTM_WAVES_BWD")) p->opt_waves_b = (atoi(v) == 4 || atoi(v) == 8) ? atoi(v) : 0;
     }
     replan(p);
     e = p->status.reserve(64);
@@ -301,6 +304,15 @@ extern "C" int flstm_core_set_option(flstm_core_plan* p, const char* name, long 
     if (!strcmp(name, "cooperative")) { p->opt_cooperative = value != 0; replan(p); return 0; }
     if (!strcmp(name, "step_graphs")) { p->opt_graphs = value != 0; return 0; }
     if (!strcmp(name, "bwd_two_d")) { if (value < 0 || value > 2) return FLSTM_E_INVALID; p->opt_two_d = int(value); replan(p); return 0; }
+    if (!strcmp(name, "waves_fwd") || !strcmp(name, "waves_bwd")) {
+        // wavefronts per workgroup of a recurrence: the weight fragments are packed for it, so a change un-packs them
+        if (value != 0 && value != 4 && value != 8) return FLSTM_E_INVALID;
+        const int before = name[6] == 'f' ? p->Lf.nw : p->Lb.nw;
+        (name[6] == 'f' ? p->opt_waves_f : p->opt_waves_b) = int(value);
+        replan(p);
+        if ((name[6] == 'f' ? p->Lf.nw : p->Lb.nw) != before) p->weights_packed = false;
+        return 0;
+    }
     if (!strcmp(name, "inject_stall")) { if (value < 0) return FLSTM_E_INVALID; p->inject_stall = int(value); return 0; }
     if (!strcmp(name, "dw_splits")) { if (value < 0) return FLSTM_E_INVALID; p->opt_dw_splits = int(value); return 0; }
     if (!strcmp(name, "accumulate_grads")) { p->opt_accumulate = value != 0; return 0; }
@@ -320,6 +332,8 @@ extern "C" long flstm_core_get_info(const flstm_core_plan* p, const char* name) 
     if (!strcmp(name, "row_tiles_bwd")) return p->Lb.mt;
     if (!strcmp(name, "cooperative")) return p->opt_cooperative;
     if (!strcmp(name, "bwd_two_d")) return p->Lb.two_d;
+    if (!strcmp(name, "waves_fwd")) return p->Lf.nw;
+    if (!strcmp(name, "waves_bwd")) return p->Lb.nw;
     if (!strcmp(name, "graph_captures")) return p->graphs_f.captures + p->graphs_b.captures;
     if (!strcmp(name, "graph_replays")) return p->graphs_f.replays + p->graphs_b.replays;
     if (!strcmp(name, "graphs_disabled")) return (p->graphs_f.disabled ? 1 : 0) + (p->graphs_b.disabled ? 2 : 0);
@@ -361,10 +375,11 @@ extern "C" int flstm_core_pack_weights(flstm_core_plan* p, const float* w_ih, co
     const Dims& d = p->d;
     FL_TRY(p->wih_p.reserve(size_t(4) * d.Hp * d.Ip * sizeof(half_t)));
     FL_TRY(p->wih_t.reserve(size_t(4) * d.Hp * d.Ip * sizeof(half_t)));
-    FL_TRY(p->wfrag_f.reserve(size_t(p->Lf.nh) * 4 * p->ks_f * p->Lf.nt * kWave * sizeof(half8)));
-    FL_TRY(p->wfrag_b.reserve(size_t(p->Lb.nh) * 4 * p->ks_b * p->Lb.nt * kWave * sizeof(half8)));
+    FL_TRY(p->wfrag_f.reserve(size_t(p->Lf.nh) * p->Lf.nw * p->ks_f * p->Lf.nt * kWave * sizeof(half8)));
+    FL_TRY(p->wfrag_b.reserve(size_t(p->Lb.nh) * p->Lb.nw * p->ks_b * p->Lb.nt * kWave * sizeof(half8)));
     FL_TRY(pack_weights(d, w_ih, w_hh, p->wih_p.as<half_t>(), p->wih_t.as<half_t>(), p->wfrag_f.as<half8>(),
-                        p->ks_f, p->Lf.nt, p->Lf.rot_div, p->wfrag_b.as<half8>(), p->ks_b, p->Lb.nt, p->Lb.rot_div, s));
+                        p->ks_f, p->Lf.nt, p->Lf.rot_div, p->Lf.nw, p->wfrag_b.as<half8>(), p->ks_b, p->Lb.nt,
+                        p->Lb.rot_div, p->Lb.nw, s));
     if (rec_bwd_two_d_possible(d.Hp, p->num_cus)) {   // whether or not the current layout uses them
         FL_TRY(p->wfrag_b2.reserve(rec_bwd_two_d_wfrag_bytes(d.Hp)));
         FL_TRY(pack_wfrag_bwd2d(d, w_hh, p->wfrag_b2.as<half8>(), rec_bwd_two_d_kq(d.B, d.Hp), s));

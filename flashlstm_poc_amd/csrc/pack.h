@@ -16,8 +16,8 @@ struct Dims {
 // Replaces src/kernels.cu:57-84 (pack_weights_kernel) and :45-55 (combine_bias_kernel): fp32
 // PyTorch-layout weights -> the fp16 operand layouts of the kernels in this library.
 hipError_t pack_weights(const Dims& d, const float* w_ih, const float* w_hh, half_t* wih_p /*[4Hp][Ip]*/,
-                        half_t* wih_t /*[Ip][4Hp]*/, half8* wfrag_fwd, int ks_fwd, int nt_fwd, int rot_div_fwd,
-                        half8* wfrag_bwd, int ks_bwd, int nt_bwd, int rot_div_bwd, hipStream_t s);
+                        half_t* wih_t /*[Ip][4Hp]*/, half8* wfrag_fwd, int ks_fwd, int nt_fwd, int rot_div_fwd, int nw_fwd,
+                        half8* wfrag_bwd, int ks_bwd, int nt_bwd, int rot_div_bwd, int nw_bwd, hipStream_t s);
 // W_hh in the layout of the backward recurrence that splits its product two ways (2048 padded hidden units only);
 // kq = 8 or 4 contraction slices.
 hipError_t pack_wfrag_bwd2d(const Dims& d, const float* w_hh, half8* out, int kq, hipStream_t s);

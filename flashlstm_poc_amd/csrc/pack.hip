@@ -35,47 +35,47 @@ __global__ void pack_wih_kernel(Dims d, const float* __restrict__ w_ih, half_t* 
 // a workgroup (they only meet the pointwise stage through LDS) and stay gate-major within the slice of JB = 4*NT
 // units: column c = gate * JB + unit.
 // fragment (hs, wave, ks, n): lane l holds column c = n*16 + l%16 of slice hs,
-// k = (ks*4 + wave)*32 + 8*(l/16) + e, e = 0..7.
+// k = (ks*nw + wave)*32 + 8*(l/16) + e, e = 0..7 (nw = wavefronts per workgroup, 4 or 8).
 __global__ void pack_wfrag_fwd_kernel(Dims d, const float* __restrict__ w_hh, half_t* __restrict__ out,
-                                      int ks_wave, int nt, int rot_div) {
+                                      int ks_wave, int nt, int rot_div, int nw) {
     const size_t idx = size_t(blockIdx.x) * kT + threadIdx.x;  // one half element
     const int nh = d.Hp / (4 * nt);
-    const size_t total = size_t(nh) * 4 * ks_wave * nt * kWave * 8;
+    const size_t total = size_t(nh) * nw * ks_wave * nt * kWave * 8;
     if (idx >= total) return;
     size_t r = idx;
     const int e = int(r % 8); r /= 8;
     const int lane = int(r % kWave); r /= kWave;
     const int n = int(r % nt); r /= nt;
     const int ks = int(r % ks_wave); r /= ks_wave;
-    const int wave = int(r % 4); r /= 4;
+    const int wave = int(r % nw); r /= nw;
     const int hs = int(r);
     const int jb = 4 * nt, c = n * 16 + lane % 16;
     const int gate = c / jb, unit = hs * jb + c % jb;
     // (slot ks of slice hs holds a rotated k-step: recurrent.h, rec_kstep_rotation)
     const int kstep = rec_kstep_of_slot(ks, rec_kstep_rotation(hs, nh, ks_wave, rot_div), ks_wave);
-    const int k = (kstep * 4 + wave) * 32 + 8 * (lane / 16) + e;
+    const int k = (kstep * nw + wave) * 32 + 8 * (lane / 16) + e;
     out[idx] = (half_t)((unit < d.H && k < d.H) ? w_hh[size_t(gate * d.H + unit) * d.H + k] : 0.f);
 }
 
 // Backward fragments: B operand of  dh[b][k] += dG[b][q] * W_hh[row(q)][k].
 // fragment (hs, wave, ks, n): lane l holds output column k = hs*16*NT + n*16 + l%16,
-// contraction index q = (ks*4 + wave)*32 + 8*(l/16) + e.
+// contraction index q = (ks*nw + wave)*32 + 8*(l/16) + e.
 __global__ void pack_wfrag_bwd_kernel(Dims d, const float* __restrict__ w_hh, half_t* __restrict__ out,
-                                      int ks_wave, int nt, int rot_div) {
+                                      int ks_wave, int nt, int rot_div, int nw) {
     const size_t idx = size_t(blockIdx.x) * kT + threadIdx.x;
     const int nh = d.Hp / (16 * nt);
-    const size_t total = size_t(nh) * 4 * ks_wave * nt * kWave * 8;
+    const size_t total = size_t(nh) * nw * ks_wave * nt * kWave * 8;
     if (idx >= total) return;
     size_t r = idx;
     const int e = int(r % 8); r /= 8;
     const int lane = int(r % kWave); r /= kWave;
     const int n = int(r % nt); r /= nt;
     const int ks = int(r % ks_wave); r /= ks_wave;
-    const int wave = int(r % 4); r /= 4;
+    const int wave = int(r % nw); r /= nw;
     const int hs = int(r);
     const int k = hs * 16 * nt + n * 16 + lane % 16;
     const int kstep = rec_kstep_of_slot(ks, rec_kstep_rotation(hs, nh, ks_wave, rot_div), ks_wave);
-    const int q = (kstep * 4 + wave) * 32 + 8 * (lane / 16) + e;
+    const int q = (kstep * nw + wave) * 32 + 8 * (lane / 16) + e;
     float v = 0.f;
     if (q < 4 * d.Hp && k < d.H) {
         const int row = torch_row(q, d.H);
@@ -222,16 +222,16 @@ __global__ void fill_words_kernel(unsigned* p, size_t words, unsigned value) {
 }  // namespace
 
 hipError_t pack_weights(const Dims& d, const float* w_ih, const float* w_hh, half_t* wih_p, half_t* wih_t,
-                        half8* wfrag_fwd, int ks_fwd, int nt_fwd, int rot_div_fwd, half8* wfrag_bwd, int ks_bwd,
-                        int nt_bwd, int rot_div_bwd, hipStream_t s) {
+                        half8* wfrag_fwd, int ks_fwd, int nt_fwd, int rot_div_fwd, int nw_fwd, half8* wfrag_bwd, int ks_bwd,
+                        int nt_bwd, int rot_div_bwd, int nw_bwd, hipStream_t s) {
     const size_t n1 = size_t(4) * d.Hp * d.Ip;
     hipLaunchKernelGGL(pack_wih_kernel, dim3(grid_for(n1)), dim3(kT), 0, s, d, w_ih, wih_p, wih_t);
-    const size_t n2 = size_t(d.Hp / (4 * nt_fwd)) * 4 * ks_fwd * nt_fwd * kWave * 8;
+    const size_t n2 = size_t(d.Hp / (4 * nt_fwd)) * nw_fwd * ks_fwd * nt_fwd * kWave * 8;
     hipLaunchKernelGGL(pack_wfrag_fwd_kernel, dim3(grid_for(n2)), dim3(kT), 0, s, d, w_hh,
-                       reinterpret_cast<half_t*>(wfrag_fwd), ks_fwd, nt_fwd, rot_div_fwd);
-    const size_t n3 = size_t(d.Hp / (16 * nt_bwd)) * 4 * ks_bwd * nt_bwd * kWave * 8;
+                       reinterpret_cast<half_t*>(wfrag_fwd), ks_fwd, nt_fwd, rot_div_fwd, nw_fwd);
+    const size_t n3 = size_t(d.Hp / (16 * nt_bwd)) * nw_bwd * ks_bwd * nt_bwd * kWave * 8;
     hipLaunchKernelGGL(pack_wfrag_bwd_kernel, dim3(grid_for(n3)), dim3(kT), 0, s, d, w_hh,
-                       reinterpret_cast<half_t*>(wfrag_bwd), ks_bwd, nt_bwd, rot_div_bwd);
+                       reinterpret_cast<half_t*>(wfrag_bwd), ks_bwd, nt_bwd, rot_div_bwd, nw_bwd);
     return hipGetLastError();
 }
 

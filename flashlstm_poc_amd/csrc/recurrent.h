@@ -29,10 +29,13 @@ struct RecLayout {
     int nm;          // two_d: passes per step the kernel is built for (row blocks per workgroup, rounded up to 1, 2, 4)
     int win_rows;    // two_d: 0, or the batch is walked in windows of this many rows, one persistent launch each (batch
                      // rows are independent sequences); nrb, mt, ng, nm then describe one window
+    int nw;          // wavefronts per workgroup of the one-way kernels, which split the contraction between them: 4, or 8
+                     // (two per SIMD).  The weight fragments are packed for this count, so it is a function of the
+                     // sizes alone and does not follow mt
 };
 
 struct RecFwdArgs {
-    const half8* wfrag;  // [nh][4 waves][ks][nt][64 lanes] MFMA B-fragments of W_hh (packed gate order)
+    const half8* wfrag;  // [nh][nw waves][ks][nt][64 lanes] MFMA B-fragments of W_hh (packed gate order)
     half_t* Y;           // [(T+1)*B][Hp]; rows [0,B) = h0, rows [(t+1)B, (t+2)B) = h_t (row-major, for later kernels)
     half_t* X;           // exchange ring, 4 slots of x_slot halfs, fragment-major; step t reads slot t%4 (h_{t-1}),
                          // writes slot (t+1)%4; before step 0 slot 0 holds h0 (padding rows zero) and the
@@ -54,7 +57,7 @@ struct RecFwdArgs {
 };
 
 struct RecBwdArgs {
-    const half8* wfrag;  // [nh][4 waves][ks][nt][64] B-fragments of W_hh^T (rows = hidden k, contraction = packed gate q)
+    const half8* wfrag;  // [nh][nw waves][ks][nt][64] B-fragments of W_hh^T (rows = hidden k, contraction = packed gate q)
     const half_t* G;     // activated gates cache [T*B][4Hp]
     const float* C;      // cell states [(T+1)*B][Hp]
     const half_t* dY;    // [T*B][Hp] upstream gradient
@@ -139,9 +142,12 @@ constexpr size_t kGraphCacheEntries = 4;
 // Picks tile shapes and the group structure for a problem size on the current device.  force_mt: 0 = the rule of
 // thumb (16-row blocks whenever all of them can run side by side), 1 / 2 = that many 16-row tiles per row block
 // (1 only where it fits).  The choice does not change the weight-fragment layout.
-RecLayout plan_rec_fwd(int B, int Hp, int num_cus, bool force_stepwise, int force_mt = 0);
+// waves: 0 = the rule of thumb (rec_waves), 4 or 8 = that many wavefronts per workgroup (8 only where it can run).
+RecLayout plan_rec_fwd(int B, int Hp, int num_cus, bool force_stepwise, int force_mt = 0, int waves = 0);
 // two_d: 0 = never the two-way split, 1 = where it is the faster layout, 2 = wherever it can run
-RecLayout plan_rec_bwd(int B, int Hp, int num_cus, bool force_stepwise, int force_mt = 0, int two_d = 1);
+RecLayout plan_rec_bwd(int B, int Hp, int num_cus, bool force_stepwise, int force_mt = 0, int two_d = 1, int waves = 0);
+// Wavefronts per workgroup the one-way kernels run with for these sizes (a function of the sizes alone).
+int rec_waves(int B, int Hp, int num_cus, int waves);
 
 // The two-dimensional backward layout: whether a device/size can use it at all (decides whether its weight fragments
 // are packed) and with how many contraction slices (a function of the sizes alone, so that the packed weights fit

@@ -166,6 +166,18 @@ __device__ __forceinline__ half8 ld_frag(const half_t* frag_lane) {
 __device__ __forceinline__ void ld_frag_async(half8& dst, const half_t* frag_lane) {
     asm volatile("global_load_dwordx4 %0, %1, off sc1" : "=v"(dst) : "v"(frag_lane) : "memory");
 }
+// The same with the address as scalar base (the same for the whole wave: ring slot, row tile and k-step) + a 32-bit
+// offset per lane: the k-step offsets then live in scalar registers and their arithmetic runs on the scalar unit.  For
+// the kernels with two waves per SIMD, which have 256 vector registers and none to spare for addresses.
+__device__ __forceinline__ void ld_frag_async_at(half8& dst, unsigned lane_off, const half_t* frag) {
+    asm volatile("global_load_dwordx4 %0, %1, %2 sc1" : "=v"(dst) : "v"(lane_off), "s"(frag) : "memory");
+}
+// (a pointer that is the same in every lane, as a value the compiler knows to be: it then lives in scalar registers)
+__device__ __forceinline__ const half_t* wave_uniform(const half_t* ptr) {
+    const unsigned long long v = reinterpret_cast<unsigned long long>(ptr);
+    const unsigned lo = __builtin_amdgcn_readfirstlane(unsigned(v)), hi = __builtin_amdgcn_readfirstlane(unsigned(v >> 32));
+    return reinterpret_cast<const half_t*>((static_cast<unsigned long long>(hi) << 32) | lo);
+}
 template <int N>
 __device__ __forceinline__ void wait_frags(half8 (&a)[4], half8 (&b)[4]) {
     asm volatile("s_waitcnt vmcnt(%8)"
@@ -251,7 +263,7 @@ __device__ __forceinline__ bool product_poisoned(const floatx4 (&acc)[2][NT]) {
 // fetched and multiplied before tile 1 is touched, so the first half of a step's product runs while the peers are
 // still busy with the second half of their cell updates.  Chunks of CKT k-steps of ONE tile alternate between two
 // register sets (as many registers as the two-tile chunks of wave_product).  Resident weights only.
-template <int NT, int KS, int KL, int NPF, int NBUF, bool LAZY = false, int CKO = 0, bool REASK = false, typename Prefetch>
+template <int NT, int KS, int KL, int NPF, int NBUF, bool LAZY = false, int CKO = 0, bool REASK = false, int NW = 4, typename Prefetch>
 __device__ __forceinline__ bool wave_product_tiles(floatx4 (&acc)[2][NT], const half8 (&wreg)[KS - KL][NT],
                                                    const half8* wlds, const half_t* a0, const half_t* a1, int wave,
                                                    int lane, int nks_total, int ks_wave, int rotation, const Poll& poll,
@@ -274,7 +286,7 @@ __device__ __forceinline__ bool wave_product_tiles(floatx4 (&acc)[2][NT], const 
         const half_t* base = (c / NCHK) ? p1 : p0;
 #pragma unroll
         for (int k = 0; k < CKT; ++k) {
-            const int kg = min(rec_kstep_of_slot((c % NCHK) * CKT + k, rotation, ks_wave) * 4 + wave, nks_total - 1);
+            const int kg = min(rec_kstep_of_slot((c % NCHK) * CKT + k, rotation, ks_wave) * NW + wave, nks_total - 1);
             ld_frag_async(f[c % NBUF][k], base + size_t(kg) * 512);
         }
     };
@@ -384,12 +396,12 @@ __device__ __forceinline__ bool wave_product_tiles(floatx4 (&acc)[2][NT], const 
 
 // `prefetch` issues exactly NPF vector loads (for every wave, whatever its lanes need) behind the last
 // fragment load.
-template <int NT, int KS, bool RESIDENT, int KL, int NPF, int MT, int NBUF = 2, int CKO = 0, bool LAZY = false, bool REASK = false, typename Prefetch>
+template <int NT, int KS, bool RESIDENT, int KL, int NPF, int MT, int NBUF = 2, int CKO = 0, bool LAZY = false, bool REASK = false, int NW = 4, typename Prefetch>
 __device__ __forceinline__ bool wave_product(floatx4 (&acc)[2][NT], const half8 (&wreg)[KS - KL][NT],
                                              const half8* wlds, const half8* wfrag_wave, const half_t* a0,
                                              const half_t* a1, int wave, int lane, int nks_total,
                                              int ks_wave, int rotation, const Poll& poll, Prefetch&& prefetch) {
-    if constexpr (RESIDENT && (KS % 8 == 0)) {
+    if constexpr (RESIDENT && (KS % 4 == 0)) {
         // Loads and MFMAs are unconditional: k-steps beyond the real contraction length fetch a
         // clamped (finite) address and meet all-zero weight fragments.  Chunks of CK k-steps (2*CK
         // fragments) alternate between two register sets: one is in flight while the other feeds the
@@ -407,12 +419,27 @@ __device__ __forceinline__ bool wave_product(floatx4 (&acc)[2][NT], const half8 
         for (;;) {
         const half_t *p0 = a0, *p1 = a1;   // (opaque copies, as in wave_product_tiles)
         if constexpr (LAZY) asm volatile("" : "+v"(p0), "+v"(p1));
+        // eight waves: scalar base + lane offset (ld_frag_async_at)
+        constexpr bool SADDR = (NW == 8);
+        const unsigned lane_off = unsigned(lane) * 16u;
+        const half_t *u0 = nullptr, *u1 = nullptr;
+        int wv = wave;
+        if constexpr (SADDR) {
+            u0 = wave_uniform(a0 - lane * 8);
+            u1 = wave_uniform(a1 - lane * 8);
+            wv = __builtin_amdgcn_readfirstlane(wave);
+        }
         auto issue = [&](int c, int buf) {
 #pragma unroll
             for (int k = 0; k < CK; ++k) {
-                const int kg = min(rec_kstep_of_slot(c * CK + k, rotation, ks_wave) * 4 + wave, nks_total - 1);
-                ld_frag_async(fa[buf][k], p0 + size_t(kg) * 512);
-                if constexpr (MT == 2) ld_frag_async(fb[buf][k], p1 + size_t(kg) * 512);
+                const int kg = min(rec_kstep_of_slot(c * CK + k, rotation, ks_wave) * NW + wv, nks_total - 1);
+                if constexpr (SADDR) {
+                    ld_frag_async_at(fa[buf][k], lane_off, u0 + size_t(kg) * 512);
+                    if constexpr (MT == 2) ld_frag_async_at(fb[buf][k], lane_off, u1 + size_t(kg) * 512);
+                } else {
+                    ld_frag_async(fa[buf][k], p0 + size_t(kg) * 512);
+                    if constexpr (MT == 2) ld_frag_async(fb[buf][k], p1 + size_t(kg) * 512);
+                }
             }
         };
         auto wait = [&](auto younger, int buf) {   // until at most `younger` loads issued later are outstanding
@@ -520,7 +547,7 @@ __device__ __forceinline__ bool wave_product(floatx4 (&acc)[2][NT], const half8 
         return ahead_of_producers;
     } else {
         for (int k = 0; k < ks_wave; ++k) {
-            const int kg = rec_kstep_of_slot(k, rotation, ks_wave) * 4 + wave;
+            const int kg = rec_kstep_of_slot(k, rotation, ks_wave) * NW + wave;
             if (kg >= nks_total) continue;
             const half8 fa = ld_frag(a0 + size_t(kg) * 512);
             half8 fb{};
@@ -812,21 +839,30 @@ struct FirstRequestDelay {
 // of the block (two units each) and store that half of h_t, then rows 16..31.  The consumers fetch and multiply
 // tile by tile (wave_product_tiles), so the second phase of a step overlaps the first half of the peers' next
 // product instead of sitting on the path from one step to the next.
-template <int NT, int KS, bool RESIDENT, int MT, bool DS, bool DEEP = false>
-__global__ __launch_bounds__(kThreads) void rec_fwd_kernel(RecFwdArgs p, RecLayout L, int t_begin,
-                                                           int t_end, int ks_wave) {
+// NW = wavefronts per workgroup.  8 (two per SIMD, at most 256 registers each; slices of 32 units): the contraction is
+// split eight ways, every wave holds half the weight fragments, fetches, checks and multiplies half as much and
+// updates half the cells, and the two waves of a SIMD fill each other's issue gaps -- a step of these kernels is
+// bound by the instructions one wave can issue, not by the matrix cores.  The eight partial sums of a step take the
+// whole LDS once, so there is one buffer and a second barrier (before the partials are written) instead of two
+// buffers; all 32 rows of a block are updated at once by the 512 threads (no phases).
+template <int NT, int KS, bool RESIDENT, int MT, bool DS, bool DEEP = false, int NW = 4>
+__global__ __launch_bounds__(NW * kWave) void rec_fwd_kernel(RecFwdArgs p, RecLayout L, int t_begin,
+                                                             int t_end, int ks_wave) {
     constexpr int JB = 4 * NT;    // hidden units of this slice
     constexpr int NC = 16 * NT;   // gate columns of this slice (i,f,g,o blocks of JB)
     constexpr int PLD = NC + kPartPad;
-    constexpr bool SPLIT = RESIDENT && MT == 2 && JB >= 32 && (KS % 8 == 0);
+    static_assert(NW == 4 || (NW == 8 && JB == 32 && !DEEP), "eight waves: slices of 32 units");
+    constexpr bool SPLIT = NW == 4 && RESIDENT && MT == 2 && JB >= 32 && (KS % 8 == 0);
+    constexpr int PBUFS = (NW == 8) ? 1 : 2;   // partial-sum buffers in LDS
+    constexpr bool SEQ = NW == 8 && MT == 2 && RESIDENT;   // the two row tiles of a block are multiplied one after the other
     // cell updates per thread: the slice's units of one batch row are shared by GPR threads; 32 rows x 8 threads,
     // or 16 rows x 16 threads (per phase, or when a block has one row tile) where the slice is wide enough for 2 units each
-    constexpr int GPR = (SPLIT || (MT == 1 && JB >= 32)) ? 16 : 8;
+    constexpr int GPR = (NW == 8 || SPLIT || (MT == 1 && JB >= 32)) ? 16 : 8;
     constexpr int UPT = JB / GPR;
     constexpr int NPH = SPLIT ? 2 : 1;   // pointwise phases per step
     static_assert(UPT == 2 || UPT == 4, "2 or 4 hidden units per thread");
     typedef Pack<UPT> PackT;
-    extern __shared__ __attribute__((aligned(16))) float part_all[];  // [2][4][32][PLD]
+    extern __shared__ __attribute__((aligned(16))) float part_all[];  // [PBUFS][NW][32][PLD]
     __shared__ int lds_abort;
     __shared__ int lds_role[2];
 
@@ -844,7 +880,7 @@ __global__ __launch_bounds__(kThreads) void rec_fwd_kernel(RecFwdArgs p, RecLayo
     FirstRequestDelay first_request;
     if constexpr (DS) first_request.start_from(p.delay_hint);
 
-    const half8* wfrag_wave = p.wfrag + (size_t(hs) * 4 + wave) * size_t(ks_wave) * NT * kWave;
+    const half8* wfrag_wave = p.wfrag + (size_t(hs) * NW + wave) * size_t(ks_wave) * NT * kWave;
     half8 wreg[KS][NT];
     if constexpr (RESIDENT) {
 #pragma unroll
@@ -890,7 +926,7 @@ __global__ __launch_bounds__(kThreads) void rec_fwd_kernel(RecFwdArgs p, RecLayo
     for (int t = t_begin; t < t_end; ++t) {
         for (int rb = g; rb < L.nrb; rb += L.ng, ++item) {
             const int row0 = rb * RB;
-            float* part = part_all + size_t(item & 1) * 4 * kRows * PLD;
+            float* part = part_all + size_t(item & (PBUFS - 1)) * NW * kRows * PLD;
             const half_t* xin = p.X + size_t(t & 3) * p.x_slot;          // h_{t-1}, fragment-major
             half_t* xout = p.X + size_t((t + 1) & 3) * p.x_slot;         // h_t
             half_t* xnext = p.X + size_t((t + 3) & 3) * p.x_slot;        // will take h_{t+2}: marked unwritten
@@ -903,15 +939,28 @@ __global__ __launch_bounds__(kThreads) void rec_fwd_kernel(RecFwdArgs p, RecLayo
                 for (int n = 0; n < NT; ++n) acc[m][n] = floatx4{0.f, 0.f, 0.f, 0.f};
             if constexpr (DS) first_request.hold();
             bool ahead;
-            if constexpr (SPLIT)
+            if constexpr (SEQ) {
+                // one row tile after the other through the same 32 accumulation registers: product, partial sums to
+                // LDS, product, partial sums
+                ahead = wave_product<NT, KS, RESIDENT, 0, 0, 1, 2, 0, false, DS, NW>(acc, wreg, nullptr, wfrag_wave, a0, a0, wave, lane, nks_total,
+                                                                                     ks_wave, rotation, poll, []() {});
+                __syncthreads();   // every thread has read the partial sums of the previous item
+                spill_partials<NT, 1>(part, acc, wave, lane, PLD);
+#pragma unroll
+                for (int n = 0; n < NT; ++n) acc[0][n] = floatx4{0.f, 0.f, 0.f, 0.f};
+                wave_product<NT, KS, RESIDENT, 0, UPT / 2, 1, 2, 0, false, DS, NW>(acc, wreg, nullptr, wfrag_wave, a1, a1, wave, lane, nks_total,
+                                                                                   ks_wave, rotation, poll, [&]() { prefetch(t, rb); });
+                spill_partials<NT, 1>(part + 16 * PLD, acc, wave, lane, PLD);
+            } else if constexpr (SPLIT)
                 ahead = wave_product_tiles<NT, KS, 0, NPH * UPT / 2, kFwdBufs, false, 0, DS>(acc, wreg, nullptr, a0, a1, wave, lane, nks_total, ks_wave, rotation, poll,
                                                              [&]() { prefetch(t, rb); });
             else
-                ahead = wave_product<NT, KS, RESIDENT, 0, UPT / 2, MT, DEEP ? 4 : 2, DEEP ? 2 : 0, DEEP, DS && !DEEP>(acc, wreg, nullptr, wfrag_wave, a0, a1, wave, lane, nks_total,
+                ahead = wave_product<NT, KS, RESIDENT, 0, UPT / 2, MT, DEEP ? 4 : 2, DEEP ? 2 : 0, DEEP, DS && !DEEP, NW>(acc, wreg, nullptr, wfrag_wave, a0, a1, wave, lane, nks_total,
                                                                ks_wave, rotation, poll, [&]() { prefetch(t, rb); });
             if constexpr (DS) first_request.learn(ahead);
             clk.lap(0);
-            spill_partials<NT, MT>(part, acc, wave, lane, PLD);
+            if constexpr (PBUFS == 1 && !SEQ) __syncthreads();   // every thread has read the partial sums of the previous item
+            if constexpr (!SEQ) spill_partials<NT, MT>(part, acc, wave, lane, PLD);
             __syncthreads();
             if (lds_abort != 0) return;
             clk.lap(1);
@@ -947,7 +996,7 @@ __global__ __launch_bounds__(kThreads) void rec_fwd_kernel(RecFwdArgs p, RecLayo
 #pragma unroll
                     for (int gt = 0; gt < 4; ++gt) {
 #pragma unroll
-                        for (int w = 0; w < 4; ++w) {
+                        for (int w = 0; w < NW; ++w) {
                             float v[UPT];
                             ld_f32(part + (size_t(w) * kRows + prow) * PLD + gt * JB + pj, v);
 #pragma unroll
@@ -1008,9 +1057,11 @@ __global__ __launch_bounds__(kThreads) void rec_fwd_kernel(RecFwdArgs p, RecLayo
 // ----------------------------------------------------------------------------------- backward
 // Gate order and the pointwise derivative follow flashlstm_v2/src/lstm_backward.cu:199-211, except
 // that c_{t-1}, c_t come from the cell-state cache instead of being rebuilt through atanh.
-template <int NT, int KS, bool RESIDENT, int KL, int MT, bool DS>
-__global__ __launch_bounds__(kThreads) void rec_bwd_kernel(RecBwdArgs p, RecLayout L, int t_first,
-                                                           int t_last, int ks_wave) {
+template <int NT, int KS, bool RESIDENT, int KL, int MT, bool DS, int NW = 4>
+__global__ __launch_bounds__(NW * kWave) void rec_bwd_kernel(RecBwdArgs p, RecLayout L, int t_first,
+                                                             int t_last, int ks_wave) {
+    static_assert(NW == 4 || (NW == 8 && NT == 2), "eight waves (see rec_fwd_kernel): slices of 32 units");
+    constexpr int THREADS = NW * kWave;
     constexpr int JB = 16 * NT;  // hidden units (= output columns of dG*W_hh) of this slice
     constexpr int PLD = JB + kPartPad;
     constexpr int KR = KS - KL;  // k-steps whose weight fragments stay in registers
@@ -1018,13 +1069,13 @@ __global__ __launch_bounds__(kThreads) void rec_bwd_kernel(RecBwdArgs p, RecLayo
     // dG_t, then rows 16..31, and fetch and multiply tile by tile, so the second half of a step's cell updates and its
     // cache stores run while the peers are already in the first half of their next product (measured at 1024 units
     // and 256 rows: 4.85 -> 4.5 us per step; without waiting for producers at all the step takes 4.2).
-    constexpr bool SPLIT = RESIDENT && MT == 2 && JB >= 32 && (KS % 8 == 0);
-    constexpr int GPR = (SPLIT || (MT == 1 && JB >= 32)) ? 16 : 8;   // threads per batch row (as in the forward kernel)
+    constexpr bool SPLIT = NW == 4 && RESIDENT && MT == 2 && JB >= 32 && (KS % 8 == 0);
+    constexpr int GPR = (NW == 8 || SPLIT || (MT == 1 && JB >= 32)) ? 16 : 8;   // threads per batch row (as in the forward kernel)
     constexpr int UPT = JB / GPR;
     constexpr int NPH = SPLIT ? 2 : 1;   // pointwise phases per step
     static_assert(UPT == 2 || UPT == 4, "2 or 4 hidden units per thread");
     typedef Pack<UPT> PackT;
-    extern __shared__ __attribute__((aligned(16))) float part_all[];  // [2][4][32][PLD], reused for db
+    extern __shared__ __attribute__((aligned(16))) float part_all[];  // [2][NW][32][PLD], reused for db
     __shared__ int lds_abort;
     __shared__ int lds_role[2];
 
@@ -1043,10 +1094,10 @@ __global__ __launch_bounds__(kThreads) void rec_bwd_kernel(RecBwdArgs p, RecLayo
     FirstRequestDelay first_request;
     if constexpr (DS) first_request.start_from(p.delay_hint);
 
-    const half8* wfrag_wave = p.wfrag + (size_t(hs) * 4 + wave) * size_t(ks_wave) * NT * kWave;
+    const half8* wfrag_wave = p.wfrag + (size_t(hs) * NW + wave) * size_t(ks_wave) * NT * kWave;
     half8 wreg[KR][NT];
-    // LDS: [partials 2*4*32*PLD floats | weight fragments of KL k-steps (wlds_has), one block per wave]
-    half8* wlds = reinterpret_cast<half8*>(part_all + 2 * 4 * kRows * PLD) + size_t(wave) * KL * NT * kWave;
+    // LDS: [partials 2*NW*32*PLD floats | weight fragments of KL k-steps (wlds_has), one block per wave]
+    half8* wlds = reinterpret_cast<half8*>(part_all + 2 * NW * kRows * PLD) + size_t(wave) * KL * NT * kWave;
     if constexpr (RESIDENT) {
 #pragma unroll
         for (int k = 0; k < KS; ++k)
@@ -1105,7 +1156,7 @@ __global__ __launch_bounds__(kThreads) void rec_bwd_kernel(RecBwdArgs p, RecLayo
         const bool from_product = (t < p.T - 1);
         for (int rb = g; rb < L.nrb; rb += L.ng, ++item) {
             const int row0 = rb * RB;
-            float* part = part_all + size_t(item & 1) * 4 * kRows * PLD;
+            float* part = part_all + size_t(item & 1) * NW * kRows * PLD;
             // ring slot of step u is (u + 8) & 3: this step reads dG_{t+1}, writes dG_t and marks the
             // slot of dG_{t-2} unwritten
             if (from_product) {
@@ -1125,7 +1176,7 @@ __global__ __launch_bounds__(kThreads) void rec_bwd_kernel(RecBwdArgs p, RecLayo
                     ahead = wave_product_tiles<NT, KS, KL, NPF, 4, false, 4, DS>(acc, wreg, wlds, a0, a1, wave, lane, nks_total, ks_wave, rotation, poll,
                                                            [&]() { prefetch(t, rb); });
                 else
-                    ahead = wave_product<NT, KS, RESIDENT, KL, NPF, MT, 2, 0, false, DS>(acc, wreg, wlds, wfrag_wave, a0, a1, wave, lane, nks_total,
+                    ahead = wave_product<NT, KS, RESIDENT, KL, NPF, MT, (NW == 8) ? 3 : 2, (NW == 8) ? 2 : 0, false, DS, NW>(acc, wreg, wlds, wfrag_wave, a0, a1, wave, lane, nks_total,
                                                               ks_wave, rotation, poll, [&]() { prefetch(t, rb); });
                 if constexpr (DS) first_request.learn(ahead);
                 clk.lap(0);
@@ -1179,7 +1230,7 @@ __global__ __launch_bounds__(kThreads) void rec_bwd_kernel(RecBwdArgs p, RecLayo
 #pragma unroll
                         for (int u = 0; u < UPT; ++u) dh[u] = 0.f;
 #pragma unroll
-                        for (int w = 0; w < 4; ++w) {
+                        for (int w = 0; w < NW; ++w) {
                             float v[UPT];
                             ld_f32(part + (size_t(w) * kRows + prow) * PLD + pj, v);
 #pragma unroll
@@ -1264,7 +1315,7 @@ __global__ __launch_bounds__(kThreads) void rec_bwd_kernel(RecBwdArgs p, RecLayo
     if constexpr (DS) first_request.leave(p.delay_hint);
     // Bias gradient: fold this launch's sums over the threads that share a group column (fixed order).
     __syncthreads();
-    float* red = part_all;  // [256][4 * UPT]
+    float* red = part_all;  // [THREADS][4 * UPT]
 #pragma unroll
     for (int gt = 0; gt < 4; ++gt)
 #pragma unroll
@@ -1273,7 +1324,7 @@ __global__ __launch_bounds__(kThreads) void rec_bwd_kernel(RecBwdArgs p, RecLayo
     if (tid < GPR * 4 * UPT) {
         const int gc = tid / (4 * UPT), e = tid % (4 * UPT);  // group column, (gate, unit)
         float sum = 0.f;
-        for (int k = gc; k < kThreads; k += GPR) sum += red[k * (4 * UPT) + e];
+        for (int k = gc; k < THREADS; k += GPR) sum += red[k * (4 * UPT) + e];
         const int gt = e / UPT, u = e % UPT;
         const int ju = hs * JB + gc * UPT + u;
         const size_t q = size_t(4) * ju + gt;
@@ -1738,15 +1789,15 @@ hipError_t raise_lds(K kernel, size_t bytes) {
 // bounded waits inside the kernel cover the case that some workgroup is late.
 template <typename K, typename A>
 hipError_t launch_persistent(K kernel, int grid, size_t lds, hipStream_t stream, A a, RecLayout L, int t_a, int t_b,
-                             int ks_wave) {
+                             int ks_wave, int threads = kThreads) {
     if (L.cooperative) {
         void* params[] = {&a, &L, &t_a, &t_b, &ks_wave};
-        hipError_t e = hipLaunchCooperativeKernel(reinterpret_cast<const void*>(kernel), dim3(grid), dim3(kThreads), params,
+        hipError_t e = hipLaunchCooperativeKernel(reinterpret_cast<const void*>(kernel), dim3(grid), dim3(threads), params,
                                                   unsigned(lds), stream);
         if (e == hipSuccess) return hipSuccess;
         (void)hipGetLastError();
     }
-    hipLaunchKernelGGL(kernel, dim3(grid), dim3(kThreads), lds, stream, a, L, t_a, t_b, ks_wave);
+    hipLaunchKernelGGL(kernel, dim3(grid), dim3(threads), lds, stream, a, L, t_a, t_b, ks_wave);
     return hipGetLastError();
 }
 
@@ -1763,8 +1814,20 @@ hipError_t to_exchange_layout(const half_t* in, int rows, int cols, size_t ld, h
 
 size_t exchange_slot_halfs(int rows, int cols) { return round_up(size_t(rows), 32) * size_t(cols); }
 
-int rec_fwd_ks(const RecLayout&, int Hp) { return int(ceil_div(size_t(Hp) / 32, 4)); }
-int rec_bwd_ks(const RecLayout&, int Hp) { return int(ceil_div(size_t(Hp) / 8, 4)); }
+int rec_fwd_ks(const RecLayout& L, int Hp) { return int(ceil_div(size_t(Hp) / 32, size_t(L.nw))); }
+int rec_bwd_ks(const RecLayout& L, int Hp) { return int(ceil_div(size_t(Hp) / 8, size_t(L.nw))); }
+
+// Eight waves per workgroup where a slice has 32 units (up to 1024 hidden units) and the default split gives every
+// workgroup 32-row blocks: measured there (1024 units, 256 rows).
+int rec_waves(int B, int Hp, int num_cus, int waves) {
+    if (Hp > 1024) return 4;
+    if (waves == 4 || waves == 8) return waves;
+    const int nh = Hp / 32;
+    const bool xcd_mode = (num_cus == 256 && nh <= 32);
+    const int side_by_side = nh > num_cus ? 0 : (xcd_mode ? 8 * (32 / nh) : num_cus / nh);
+    const bool can_16 = int(ceil_div(size_t(B), 16)) <= side_by_side;
+    return can_16 ? 4 : 8;
+}
 
 static void finish_layout(RecLayout& L, int B, int Hp, int num_cus, bool force_stepwise, bool fits, int force_mt) {
     L.nh = Hp / L.jb;
@@ -1799,23 +1862,25 @@ static void finish_layout(RecLayout& L, int B, int Hp, int num_cus, bool force_s
     }
 }
 
-RecLayout plan_rec_fwd(int B, int Hp, int num_cus, bool force_stepwise, int force_mt) {
+RecLayout plan_rec_fwd(int B, int Hp, int num_cus, bool force_stepwise, int force_mt, int waves) {
     RecLayout L{};
     bool fits = true;
     if (Hp <= 1024) L.nt = 8;
     else if (Hp <= 2048) L.nt = 4;
     else { L.nt = 8; fits = false; }
+    L.nw = fits ? rec_waves(B, Hp, num_cus, waves) : 4;
     L.jb = 4 * L.nt;
     finish_layout(L, B, Hp, num_cus, force_stepwise, fits, force_mt);
     return L;
 }
 
-RecLayout plan_rec_bwd(int B, int Hp, int num_cus, bool force_stepwise, int force_mt, int two_d) {
+RecLayout plan_rec_bwd(int B, int Hp, int num_cus, bool force_stepwise, int force_mt, int two_d, int waves) {
     RecLayout L{};
     bool fits = true;
     if (Hp <= 1024) L.nt = 2;
     else if (Hp <= 2048) L.nt = 1;
     else { L.nt = 2; fits = false; }
+    L.nw = fits ? rec_waves(B, Hp, num_cus, waves) : 4;
     L.jb = 16 * L.nt;
     finish_layout(L, B, Hp, num_cus, force_stepwise, fits, force_mt);
     // k-step rotation (recurrent.h): measured, it pays where a group spans the XCDs and a step fetches a lot -- the
@@ -1952,18 +2017,19 @@ static hipError_t launch_steps(StepGraphCache* graphs, const void* kernel, const
     return hipGraphLaunch(exec, stream);
 }
 
-template <int NT, int KS, bool RES, int MT, bool DS, bool DEEP = false>
+template <int NT, int KS, bool RES, int MT, bool DS, bool DEEP = false, int NW = 4>
 static hipError_t run_fwd(const RecLayout& L, const RecFwdArgs& a, hipStream_t stream, StepGraphCache* graphs) {
-    auto kernel = rec_fwd_kernel<NT, KS, RES, MT, DS, DEEP>;
-    const size_t lds = size_t(2) * 4 * kRows * (16 * NT + kPartPad) * sizeof(float);
+    auto kernel = rec_fwd_kernel<NT, KS, RES, MT, DS, DEEP, NW>;
+    if (L.nw != NW) return hipErrorInvalidValue;   // (the weight fragments are packed for L.nw waves)
+    const size_t lds = size_t(NW == 8 ? 1 : 2) * NW * kRows * (16 * NT + kPartPad) * sizeof(float);
     hipError_t e = raise_lds(kernel, lds);
     if (e != hipSuccess) return e;
     const int ks_wave = rec_fwd_ks(L, a.Hp);
-    if (L.persistent) return launch_persistent(kernel, L.grid, lds, stream, a, L, a.t0, a.t1, ks_wave);
+    if (L.persistent) return launch_persistent(kernel, L.grid, lds, stream, a, L, a.t0, a.t1, ks_wave, NW * kWave);
     return launch_steps(graphs, reinterpret_cast<const void*>(kernel), &a, sizeof(a), L, a.t0, a.t1, a.t1 - a.t0, stream,
                         [&]() -> hipError_t {
                             for (int t = a.t0; t < a.t1; ++t) {
-                                hipLaunchKernelGGL(kernel, dim3(L.grid), dim3(kThreads), lds, stream, a, L, t, t + 1, ks_wave);
+                                hipLaunchKernelGGL(kernel, dim3(L.grid), dim3(NW * kWave), lds, stream, a, L, t, t + 1, ks_wave);
                                 hipError_t le = hipGetLastError();
                                 if (le != hipSuccess) return le;
                             }
@@ -1977,6 +2043,10 @@ hipError_t launch_rec_fwd(const RecLayout& L, const RecFwdArgs& a, hipStream_t s
     // device-scope stores into the exchange ring: a persistent launch whose groups span XCDs
     const bool ds = L.persistent && !L.xcd_local;
     if (!L.resident) return run_fwd<8, 1, false, 2, false>(L, a, stream, graphs);
+    if (L.nt == 8 && L.nw == 8) {
+        if (L.mt == 1) return ds ? run_fwd<8, 4, true, 1, true, false, 8>(L, a, stream, graphs) : run_fwd<8, 4, true, 1, false, false, 8>(L, a, stream, graphs);
+        return ds ? run_fwd<8, 4, true, 2, true, false, 8>(L, a, stream, graphs) : run_fwd<8, 4, true, 2, false, false, 8>(L, a, stream, graphs);
+    }
     if (L.nt == 8) {
         if (L.mt == 1) return ds ? run_fwd<8, 8, true, 1, true>(L, a, stream, graphs) : run_fwd<8, 8, true, 1, false>(L, a, stream, graphs);
         return ds ? run_fwd<8, 8, true, 2, true>(L, a, stream, graphs) : run_fwd<8, 8, true, 2, false>(L, a, stream, graphs);
@@ -1990,19 +2060,20 @@ hipError_t launch_rec_fwd(const RecLayout& L, const RecFwdArgs& a, hipStream_t s
     return hipErrorInvalidValue;
 }
 
-template <int NT, int KS, bool RES, int KL, int MT, bool DS>
+template <int NT, int KS, bool RES, int KL, int MT, bool DS, int NW = 4>
 static hipError_t run_bwd(const RecLayout& L, const RecBwdArgs& a, hipStream_t stream, StepGraphCache* graphs) {
-    auto kernel = rec_bwd_kernel<NT, KS, RES, KL, MT, DS>;
-    static_assert(size_t(2) * 4 * kRows * (16 * NT + kPartPad) >= size_t(kThreads) * 8 * NT, "db reduction reuses the partial-sum area");
-    const size_t lds = size_t(2) * 4 * kRows * (16 * NT + kPartPad) * sizeof(float) + size_t(4) * KL * NT * kWave * sizeof(half8);
+    auto kernel = rec_bwd_kernel<NT, KS, RES, KL, MT, DS, NW>;
+    if (L.nw != NW) return hipErrorInvalidValue;   // (the weight fragments are packed for L.nw waves)
+    static_assert(size_t(2) * NW * kRows * (16 * NT + kPartPad) >= size_t(NW * kWave) * 8 * NT, "db reduction reuses the partial-sum area");
+    const size_t lds = size_t(2) * NW * kRows * (16 * NT + kPartPad) * sizeof(float) + size_t(NW) * KL * NT * kWave * sizeof(half8);
     hipError_t e = raise_lds(kernel, lds);
     if (e != hipSuccess) return e;
     const int ks_wave = rec_bwd_ks(L, a.Hp);
-    if (L.persistent) return launch_persistent(kernel, L.grid, lds, stream, a, L, a.t_hi, a.t_lo, ks_wave);
+    if (L.persistent) return launch_persistent(kernel, L.grid, lds, stream, a, L, a.t_hi, a.t_lo, ks_wave, NW * kWave);
     return launch_steps(graphs, reinterpret_cast<const void*>(kernel), &a, sizeof(a), L, a.t_hi, a.t_lo, a.t_hi - a.t_lo + 1,
                         stream, [&]() -> hipError_t {
                             for (int t = a.t_hi; t >= a.t_lo; --t) {
-                                hipLaunchKernelGGL(kernel, dim3(L.grid), dim3(kThreads), lds, stream, a, L, t, t, ks_wave);
+                                hipLaunchKernelGGL(kernel, dim3(L.grid), dim3(NW * kWave), lds, stream, a, L, t, t, ks_wave);
                                 hipError_t le = hipGetLastError();
                                 if (le != hipSuccess) return le;
                             }
@@ -2047,6 +2118,10 @@ hipError_t launch_rec_bwd(const RecLayout& L, const RecBwdArgs& a, hipStream_t s
     }
     const bool ds = L.persistent && !L.xcd_local;   // (as in launch_rec_fwd)
     if (!L.resident) return run_bwd<2, 1, false, 0, 2, false>(L, a, stream, graphs);
+    if (L.nt == 2 && L.nw == 8) {
+        if (L.mt == 1) return ds ? run_bwd<2, 16, true, 4, 1, true, 8>(L, a, stream, graphs) : run_bwd<2, 16, true, 4, 1, false, 8>(L, a, stream, graphs);
+        return ds ? run_bwd<2, 16, true, 4, 2, true, 8>(L, a, stream, graphs) : run_bwd<2, 16, true, 4, 2, false, 8>(L, a, stream, graphs);
+    }
     if (L.nt == 2) {
         if (L.mt == 1) return ds ? run_bwd<2, 32, true, 8, 1, true>(L, a, stream, graphs) : run_bwd<2, 32, true, 8, 1, false>(L, a, stream, graphs);
         return ds ? run_bwd<2, 32, true, 8, 2, true>(L, a, stream, graphs) : run_bwd<2, 32, true, 8, 2, false>(L, a, stream, graphs);
