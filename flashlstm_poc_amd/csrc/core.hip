@@ -108,6 +108,7 @@ struct flstm_core_plan {
     StepGraphCache graphs_f, graphs_b;   // captured step-wise launches (only used where the persistent kernels are not)
     int opt_graphs = 1;
     int opt_two_d = 1;   // backward recurrence for 2048 hidden units, two-way split: 0 never, 1 where it is faster, 2 wherever it can run
+    int opt_interleave = 1;   // eight-wave kernels: the two row tiles of a block take turns (0 = one chain per block, for comparison)
     int opt_waves_f = 0, opt_waves_b = 0;   // wavefronts per workgroup of the recurrence kernels: 0 = by size, 4, 8 (the weights are packed for it)
     int* status_host = nullptr;   // pinned: the device status word lands here with the end-of-pass copy
     int inject_stall = 0;         // test hook: treat the next N persistent passes as if their launch had given up
@@ -145,6 +146,8 @@ void replan(flstm_core_plan* p) {
     p->Lb = plan_rec_bwd(p->d.B, p->d.Hp, p->num_cus, p->opt_stepwise || p->hold_bwd > 0 || p->eff_step_b,
                          p->opt_mt_b ? p->opt_mt_b : p->eff_mt_b, p->opt_two_d, p->opt_waves_b);
     p->Lf.cooperative = p->Lb.cooperative = p->opt_cooperative;
+    p->Lf.interleave = (p->opt_interleave && p->Lf.nw == 8 && p->Lf.mt == 2 && p->Lf.resident) ? 1 : 0;
+    p->Lb.interleave = (p->opt_interleave && p->Lb.nw == 8 && p->Lb.mt == 2 && p->Lb.resident && !p->Lb.two_d) ? 1 : 0;
     p->ks_f = rec_fwd_ks(p->Lf, p->d.Hp);
     p->ks_b = rec_bwd_ks(p->Lb, p->d.Hp);
 }
@@ -255,6 +258,7 @@ extern "C" int flstm_core_create(size_t batch, size_t input_size, size_t hidden_
         if (const char* v = getenv("FLASHLSTM_COOPERATIVE_LAUNCH")) p->opt_cooperative = atoi(v) != 0;
         if (const char* v = getenv("FLASHLSTM_STEP_GRAPHS")) p->opt_graphs = atoi(v) != 0;
         if (const char* v = getenv("FLASHLSTM_BWD_TWO_D")) p->opt_two_d = atoi(v) < 0 ? 0 : (atoi(v) > 2 ? 2 : atoi(v));
+        if (const char* v = getenv("FLASHLSTM_INTERLEAVE")) p->opt_interleave = atoi(v) != 0;
         if (const char* v = getenv("FLASHLSTM_WAVES_FWD")) p->opt_waves_f = (atoi(v) == 4 || atoi(v) == 8) ? atoi(v) : 0;
         if (const char* v = getenv("FLASHLSTM_WAVES_BWD")) p->opt_waves_b = (atoi(v) == 4 || atoi(v) == 8) ? atoi(v) : 0;
     }

@@ -33,7 +33,8 @@ __global__ void pack_wih_kernel(Dims d, const float* __restrict__ w_ih, half_t* 
 
 // Forward fragments: B operand of  gates[b][c] += h[b][k] * W_hh[row(c)][k].  The product's columns are local to
 // a workgroup (they only meet the pointwise stage through LDS) and stay gate-major within the slice of JB = 4*NT
-// units: column c = gate * JB + unit.
+// units: column c = gate * JB + unit.  With eight waves per workgroup (rec_fwd_il_kernel) they are unit-major,
+// column c = 4 * unit + gate: the four accumulation registers of a lane are then the four gates of one unit.
 // fragment (hs, wave, ks, n): lane l holds column c = n*16 + l%16 of slice hs,
 // k = (ks*nw + wave)*32 + 8*(l/16) + e, e = 0..7 (nw = wavefronts per workgroup, 4 or 8).
 __global__ void pack_wfrag_fwd_kernel(Dims d, const float* __restrict__ w_hh, half_t* __restrict__ out,
@@ -50,7 +51,7 @@ __global__ void pack_wfrag_fwd_kernel(Dims d, const float* __restrict__ w_hh, ha
     const int wave = int(r % nw); r /= nw;
     const int hs = int(r);
     const int jb = 4 * nt, c = n * 16 + lane % 16;
-    const int gate = c / jb, unit = hs * jb + c % jb;
+    const int gate = (nw == 8) ? c % 4 : c / jb, unit = hs * jb + ((nw == 8) ? c / 4 : c % jb);
     // (slot ks of slice hs holds a rotated k-step: recurrent.h, rec_kstep_rotation)
     const int kstep = rec_kstep_of_slot(ks, rec_kstep_rotation(hs, nh, ks_wave, rot_div), ks_wave);
     const int k = (kstep * nw + wave) * 32 + 8 * (lane / 16) + e;

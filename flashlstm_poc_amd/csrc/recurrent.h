@@ -29,6 +29,7 @@ struct RecLayout {
     int nm;          // two_d: passes per step the kernel is built for (row blocks per workgroup, rounded up to 1, 2, 4)
     int win_rows;    // two_d: 0, or the batch is walked in windows of this many rows, one persistent launch each (batch
                      // rows are independent sequences); nrb, mt, ng, nm then describe one window
+    int interleave;  // eight waves, 32-row blocks: the two 16-row tiles of a block are chains that take turns (rec_fwd_il_kernel)
     int nw;          // wavefronts per workgroup of the one-way kernels, which split the contraction between them: 4, or 8
                      // (two per SIMD).  The weight fragments are packed for this count, so it is a function of the
                      // sizes alone and does not follow mt

@@ -112,6 +112,12 @@ struct Poll {
     lds_int_t* lds_abort;   // workgroup: some wave gave up
 };
 
+// How a workgroup leaves a persistent kernel once one of its waves has given up (decided after a barrier, so by all
+// its waves at the same point): the wave ends here.  As an instruction rather than a `return` from inside the step
+// loop, which the compiler lowers to flags that are tested on the loop's ordinary way round -- a path on which the
+// checker of the build (check_inflight.py) cannot tell that the wave is on its way out.
+__device__ __forceinline__ void leave_kernel() { asm volatile("s_endpgm" ::: "memory"); }
+
 // Said before a step loop: every load issued so far (the weight fragments, the state) has landed.  As an instruction
 // the compiler knows, not inline assembly: otherwise it meets the loop with loads it believes outstanding and puts
 // its own wait for ALL loads in front of the first MFMA of every step, behind the fragments requested ahead.
@@ -839,30 +845,22 @@ struct FirstRequestDelay {
 // of the block (two units each) and store that half of h_t, then rows 16..31.  The consumers fetch and multiply
 // tile by tile (wave_product_tiles), so the second phase of a step overlaps the first half of the peers' next
 // product instead of sitting on the path from one step to the next.
-// NW = wavefronts per workgroup.  8 (two per SIMD, at most 256 registers each; slices of 32 units): the contraction is
-// split eight ways, every wave holds half the weight fragments, fetches, checks and multiplies half as much and
-// updates half the cells, and the two waves of a SIMD fill each other's issue gaps -- a step of these kernels is
-// bound by the instructions one wave can issue, not by the matrix cores.  The eight partial sums of a step take the
-// whole LDS once, so there is one buffer and a second barrier (before the partials are written) instead of two
-// buffers; all 32 rows of a block are updated at once by the 512 threads (no phases).
-template <int NT, int KS, bool RESIDENT, int MT, bool DS, bool DEEP = false, int NW = 4>
-__global__ __launch_bounds__(NW * kWave) void rec_fwd_kernel(RecFwdArgs p, RecLayout L, int t_begin,
-                                                             int t_end, int ks_wave) {
+template <int NT, int KS, bool RESIDENT, int MT, bool DS, bool DEEP = false>
+__global__ __launch_bounds__(kThreads) void rec_fwd_kernel(RecFwdArgs p, RecLayout L, int t_begin,
+                                                           int t_end, int ks_wave) {
+    constexpr int NW = 4;
     constexpr int JB = 4 * NT;    // hidden units of this slice
     constexpr int NC = 16 * NT;   // gate columns of this slice (i,f,g,o blocks of JB)
     constexpr int PLD = NC + kPartPad;
-    static_assert(NW == 4 || (NW == 8 && JB == 32 && !DEEP), "eight waves: slices of 32 units");
-    constexpr bool SPLIT = NW == 4 && RESIDENT && MT == 2 && JB >= 32 && (KS % 8 == 0);
-    constexpr int PBUFS = (NW == 8) ? 1 : 2;   // partial-sum buffers in LDS
-    constexpr bool SEQ = NW == 8 && MT == 2 && RESIDENT;   // the two row tiles of a block are multiplied one after the other
+    constexpr bool SPLIT = RESIDENT && MT == 2 && JB >= 32 && (KS % 8 == 0);
     // cell updates per thread: the slice's units of one batch row are shared by GPR threads; 32 rows x 8 threads,
     // or 16 rows x 16 threads (per phase, or when a block has one row tile) where the slice is wide enough for 2 units each
-    constexpr int GPR = (NW == 8 || SPLIT || (MT == 1 && JB >= 32)) ? 16 : 8;
+    constexpr int GPR = (SPLIT || (MT == 1 && JB >= 32)) ? 16 : 8;
     constexpr int UPT = JB / GPR;
     constexpr int NPH = SPLIT ? 2 : 1;   // pointwise phases per step
     static_assert(UPT == 2 || UPT == 4, "2 or 4 hidden units per thread");
     typedef Pack<UPT> PackT;
-    extern __shared__ __attribute__((aligned(16))) float part_all[];  // [PBUFS][NW][32][PLD]
+    extern __shared__ __attribute__((aligned(16))) float part_all[];  // [2][4][32][PLD]
     __shared__ int lds_abort;
     __shared__ int lds_role[2];
 
@@ -926,7 +924,7 @@ __global__ __launch_bounds__(NW * kWave) void rec_fwd_kernel(RecFwdArgs p, RecLa
     for (int t = t_begin; t < t_end; ++t) {
         for (int rb = g; rb < L.nrb; rb += L.ng, ++item) {
             const int row0 = rb * RB;
-            float* part = part_all + size_t(item & (PBUFS - 1)) * NW * kRows * PLD;
+            float* part = part_all + size_t(item & 1) * NW * kRows * PLD;
             const half_t* xin = p.X + size_t(t & 3) * p.x_slot;          // h_{t-1}, fragment-major
             half_t* xout = p.X + size_t((t + 1) & 3) * p.x_slot;         // h_t
             half_t* xnext = p.X + size_t((t + 3) & 3) * p.x_slot;        // will take h_{t+2}: marked unwritten
@@ -939,30 +937,17 @@ __global__ __launch_bounds__(NW * kWave) void rec_fwd_kernel(RecFwdArgs p, RecLa
                 for (int n = 0; n < NT; ++n) acc[m][n] = floatx4{0.f, 0.f, 0.f, 0.f};
             if constexpr (DS) first_request.hold();
             bool ahead;
-            if constexpr (SEQ) {
-                // one row tile after the other through the same 32 accumulation registers: product, partial sums to
-                // LDS, product, partial sums
-                ahead = wave_product<NT, KS, RESIDENT, 0, 0, 1, 2, 0, false, DS, NW>(acc, wreg, nullptr, wfrag_wave, a0, a0, wave, lane, nks_total,
-                                                                                     ks_wave, rotation, poll, []() {});
-                __syncthreads();   // every thread has read the partial sums of the previous item
-                spill_partials<NT, 1>(part, acc, wave, lane, PLD);
-#pragma unroll
-                for (int n = 0; n < NT; ++n) acc[0][n] = floatx4{0.f, 0.f, 0.f, 0.f};
-                wave_product<NT, KS, RESIDENT, 0, UPT / 2, 1, 2, 0, false, DS, NW>(acc, wreg, nullptr, wfrag_wave, a1, a1, wave, lane, nks_total,
-                                                                                   ks_wave, rotation, poll, [&]() { prefetch(t, rb); });
-                spill_partials<NT, 1>(part + 16 * PLD, acc, wave, lane, PLD);
-            } else if constexpr (SPLIT)
+            if constexpr (SPLIT)
                 ahead = wave_product_tiles<NT, KS, 0, NPH * UPT / 2, kFwdBufs, false, 0, DS>(acc, wreg, nullptr, a0, a1, wave, lane, nks_total, ks_wave, rotation, poll,
                                                              [&]() { prefetch(t, rb); });
             else
-                ahead = wave_product<NT, KS, RESIDENT, 0, UPT / 2, MT, DEEP ? 4 : 2, DEEP ? 2 : 0, DEEP, DS && !DEEP, NW>(acc, wreg, nullptr, wfrag_wave, a0, a1, wave, lane, nks_total,
+                ahead = wave_product<NT, KS, RESIDENT, 0, UPT / 2, MT, DEEP ? 4 : 2, DEEP ? 2 : 0, DEEP, DS && !DEEP>(acc, wreg, nullptr, wfrag_wave, a0, a1, wave, lane, nks_total,
                                                                ks_wave, rotation, poll, [&]() { prefetch(t, rb); });
             if constexpr (DS) first_request.learn(ahead);
             clk.lap(0);
-            if constexpr (PBUFS == 1 && !SEQ) __syncthreads();   // every thread has read the partial sums of the previous item
-            if constexpr (!SEQ) spill_partials<NT, MT>(part, acc, wave, lane, PLD);
+            spill_partials<NT, MT>(part, acc, wave, lane, PLD);
             __syncthreads();
-            if (lds_abort != 0) return;
+            if (lds_abort != 0) leave_kernel();
             clk.lap(1);
 
             // Every peer of this group has delivered h_{t-1}, so all of them are done reading h_{t-2}:
@@ -1051,6 +1036,292 @@ __global__ __launch_bounds__(NW * kWave) void rec_fwd_kernel(RecFwdArgs p, RecLa
         }
     }
     if constexpr (DS) first_request.leave(p.delay_hint);
+    clk.flush();
+}
+
+
+// 16 rows of partial sums per wave: [wave][16][pld] (spill_partials with one row tile and a 16-row pitch per wave)
+template <int NT>
+__device__ __forceinline__ void spill_partials16(float* part, const floatx4 (&acc)[2][NT], int wave, int lane, int pld) {
+    float* base = part + (size_t(wave) * 16 + size_t(lane % 16)) * pld + 4 * (lane / 16);
+#pragma unroll
+    for (int n = 0; n < NT; ++n) *reinterpret_cast<floatx4*>(base + n * 16) = acc[0][n];
+}
+
+// ------------------------------------------------------------------- forward, interleaved chains
+// The kernel above walks one dependent chain per row block: product -> partial sums -> cell update -> h_t out -> one
+// trip through the L2 -> the peers' next product.  Nothing in a workgroup can run while h_t travels, so a step costs
+// the sum of its parts plus the trip.  Here the two 16-row tiles of a 32-row block are two CHAINS that take turns:
+// a phase multiplies one chain's tile while the other chain's h_t, published early in the phase, is on its way.
+//   phase k:  request the fragments of chain k -> cell update of chain k-1 (its partial sums are in LDS), mark + h_t
+//             out -> the fragments have landed: 32 MFMAs -> cache stores of chain k-1 -> x-projection of chain k+1
+//             requested -> partial sums to LDS -> barrier
+// Eight wavefronts, two per SIMD, at most 256 registers each; the contraction is split eight ways, so a wave holds 128
+// registers of weight fragments and a product is FOUR fragment loads per wave: all are requested at once, ahead of the
+// cell update, whose time hides their trip from the L2.  The 512 threads update the 16 x 32 cells of a tile, one each.
+// The gate columns of the slice are packed unit-major here (column 4u + gate, pack_wfrag_fwd_kernel), so the four
+// accumulation registers of a lane are the four gates of one unit, a wave's partial sums of a cell are 16 contiguous
+// bytes in LDS, and a cell update reads eight 16-byte words.  Two partial-sum buffers of [8 waves][16 rows] (the one
+// being read and the one being written), one barrier per phase.
+// Vector-memory operations complete in issue order, and every wait below names how many YOUNGER operations may stay
+// outstanding: the two ring stores of the cell update behind the fragment loads; the cache stores and the prefetch
+// are issued behind the MFMAs, so no wait ever stands behind a store to memory that it does not need.
+// The ring protocol is the one of rec_fwd_kernel, per chain: the cell update of (step t, chain) marks the chain's
+// region of the slot of h_{t+2} (this workgroup's product of step t is complete by then, so every peer has published
+// h_{t-1} and is done reading h_{t-2}) and then stores h_t; between a thread's mark and its next h store of the same
+// chain lie two waits that drain everything older.  Ring words are validated as 32-bit words, so the thread of the
+// even unit stores the pair (its neighbour's half comes over a DPP move).
+template <int NT, int KS, bool DS>
+__global__ __launch_bounds__(8 * kWave) void rec_fwd_il_kernel(RecFwdArgs p, RecLayout L, int t_begin, int t_end,
+                                                               int ks_wave) {
+    constexpr int NW = 8;
+    constexpr int JB = 4 * NT;
+    constexpr int NC = 16 * NT;
+    constexpr int PLD = NC + kPartPad;
+    static_assert(JB == 32 && KS == 4, "slices of 32 units; four k-steps per wave");
+    extern __shared__ __attribute__((aligned(16))) float part_all[];  // [2][NW][16][PLD]
+    __shared__ int lds_abort;
+    __shared__ int lds_role[2];
+
+    if (threadIdx.x == 0) lds_abort = 0;
+    const Role role = make_role(L.nh, L.ng, L.gpx, L.xcd_local, p.seats, p.status, lds_role);
+    if (!role.active) return;
+    const int tid = threadIdx.x, lane = tid % kWave;
+    const int wave = __builtin_amdgcn_readfirstlane(tid / kWave);
+    const int hs = role.hs, g = role.g;
+    const int rotation = __builtin_amdgcn_readfirstlane(rec_kstep_rotation(hs, L.nh, ks_wave, L.rot_div));
+    const int nks_total = p.Hp / 32;
+    const Poll poll{L.persistent != 0, p.spin_limit, p.spin_ticks, p.status, (lds_int_t*)&lds_abort};
+    PhaseClock clk{(blockIdx.x == 0) ? p.prof : nullptr, 0};
+
+    const half8* wfrag_wave = p.wfrag + (size_t(hs) * NW + wave) * size_t(ks_wave) * NT * kWave;
+    half8 wreg[KS][NT];
+#pragma unroll
+    for (int k = 0; k < KS; ++k)
+#pragma unroll
+        for (int n = 0; n < NT; ++n)
+            wreg[k][n] = (k < ks_wave) ? wfrag_wave[(size_t(k) * NT + n) * kWave + lane] : half8{};
+    // offsets (in halfs) of this wave's k-steps inside a row tile of the ring: the same for the whole wave, so they
+    // live in scalar registers and are added to the scalar base of a load
+    unsigned koff[KS];
+#pragma unroll
+    for (int k = 0; k < KS; ++k)
+        koff[k] = unsigned(min(rec_kstep_of_slot(k, rotation, ks_wave) * NW + wave, nks_total - 1)) * 512u;
+    const unsigned lane_off = unsigned(lane) * 16u;
+
+    // this thread's cell of a tile: row r, unit u of the slice.  Every address of a phase is a base that is the same
+    // for the whole workgroup (scalar arithmetic) plus one of three per-thread offsets that never change.
+    const int r = tid / JB, u = tid % JB;
+    const int j = hs * JB + u;
+    const bool even = (u % 2) == 0;
+    const unsigned off_state = unsigned(r) * unsigned(p.Hp) + unsigned(j);          // [rows][Hp] arrays, in elements
+    const unsigned off_gate = 4u * off_state;                                        // [rows][4Hp] arrays, in halfs
+    const unsigned off_ring = unsigned(xch_offset(r, j, nks_total));                 // inside a row tile of the ring, in halfs
+    const size_t tile_halfs = size_t(nks_total) * 512;
+    const int rb_count = (L.nrb - g + L.ng - 1) / L.ng;
+    // the cell state of a workgroup with one row block (two chains) stays in registers for the whole launch
+    const bool c_in_regs = (rb_count <= 1) && (t_end - t_begin > 1);
+    float creg[2] = {0.f, 0.f};   // [tile]
+    uintx2 xp[2];   // x-projection of the next chain of each tile parity, requested a phase ahead of its product
+    auto request_xp = [&](int t, int rb, auto tile_c) __attribute__((always_inline)) {
+        constexpr int tl = decltype(tile_c)::value;
+        const int b = min(rb * 32 + tl * 16 + r, p.B - 1);   // rows past B fetch row B-1 and are not used
+        ld_stream(xp[tl], p.G + (size_t(t) * p.B + b) * (size_t(4) * p.Hp) + size_t(4) * j);
+    };
+    if (c_in_regs) {
+#pragma unroll
+        for (int tl = 0; tl < 2; ++tl) {
+            const int b = g * 32 + tl * 16 + r;
+            float v[2] = {0.f, 0.f};
+            if (b < p.B) {
+                floatx2 q;   // (one float is what is needed; the helper moves pairs: the even unit's pair holds both)
+                asm volatile("global_load_dword %0, %1, off\n\ts_waitcnt vmcnt(0)" : "=&v"(q.x) : "v"(p.C + (size_t(t_begin) * p.B + b) * p.Hp + j) : "memory");
+                v[0] = q.x;
+            }
+            creg[tl] = v[0];
+        }
+    }
+    request_xp(t_begin, g, std::integral_constant<int, 0>{});
+    __syncthreads();
+    loads_landed();
+    clk.start();
+
+    int pt = 0, prb = 0;      // the chain multiplied in the previous phase: step, row block (its tile is the other one)
+    bool have_prev = false;
+    int phase = 0;
+    // one phase, product of chain (t, rb, tl) and cell update of the chain before it; (nt, nrb): the chain after it
+    auto run_phase = [&](int t, int rb, auto tile_c, int nt, int nrb) __attribute__((always_inline)) {
+        constexpr int tl = decltype(tile_c)::value;
+        constexpr int ptl = 1 - tl;   // tile of the previous (and of the next) chain
+        float* part = part_all + size_t(phase & 1) * NW * 16 * PLD;
+        const float* part_prev = part_all + size_t((phase & 1) ^ 1) * NW * 16 * PLD;
+        // ---- request this chain's operand: h_{t-1} of the tile, this wave's four k-steps
+        const half_t* tile = wave_uniform(p.X + size_t(t & 3) * p.x_slot + size_t(2 * rb + tl) * tile_halfs);
+        half8 f[KS];
+        auto request = [&]() __attribute__((always_inline)) {
+#pragma unroll
+            for (int k = 0; k < KS; ++k) ld_frag_async_at(f[k], lane_off, tile + koff[k]);
+        };
+        request();
+        // ---- cell update of the previous chain: everything but the cache stores
+        const int row0 = prb * 32 + ptl * 16;   // first batch row of the previous chain's tile
+        const bool live = have_prev && (row0 + r < p.B);
+        unsigned hpair = 0u;   // h of this unit and its neighbour (batch rows past B travel as zeros)
+        uintx2 act = uintx2{0u, 0u};
+        float cnew = 0.f;
+        if (have_prev) {
+            half_t* xout = p.X + size_t((pt + 1) & 3) * p.x_slot + size_t(2 * prb + ptl) * tile_halfs;
+            half_t* xnext = p.X + size_t((pt + 3) & 3) * p.x_slot + size_t(2 * prb + ptl) * tile_halfs;
+            // (its x-projection was requested two phases ago, and the wait for the last product's fragments has covered it)
+            settle(xp[ptl]);
+            if (even) store_xch(xnext + off_ring, Pack<2>{kUnwritten}, DS);
+            unsigned hbits = 0u;
+            if (live) {
+                float z[4];
+                unpack_h2(xp[ptl].x, z[0], z[1]);
+                unpack_h2(xp[ptl].y, z[2], z[3]);
+#pragma unroll
+                for (int w = 0; w < NW; ++w) {
+                    const floatx4 v = *reinterpret_cast<const floatx4*>(part_prev + (size_t(w) * 16 + r) * PLD + 4 * u);
+                    z[0] += v.x; z[1] += v.y; z[2] += v.z; z[3] += v.w;
+                }
+                float cp;
+                if (c_in_regs) {
+                    cp = creg[ptl];
+                } else {
+                    floatx2 q;
+                    asm volatile("global_load_dword %0, %1, off sc1\n\ts_waitcnt vmcnt(0)" : "=&v"(q.x) : "v"(p.C + size_t(pt) * p.B * p.Hp + size_t(row0) * p.Hp + off_state) : "memory");
+                    cp = q.x;
+                }
+                const float ig = sigmoidf_dev(z[0]);
+                const float fg = sigmoidf_dev(z[1]);
+                const float gg = tanhf_dev(z[2]);
+                const float og = sigmoidf_dev(z[3]);
+                cnew = fg * cp + ig * gg;
+                const float hn = og * tanhf_dev(cnew);
+                creg[ptl] = cnew;
+                act = uintx2{pack_h2(ig, fg), pack_h2(gg, og)};
+                hbits = pack_h2(hn, 0.f);
+            }
+            // the neighbour's half: quad_perm(1, 0, 3, 2) swaps the lanes of a pair
+            const unsigned other = unsigned(__builtin_amdgcn_mov_dpp(int(hbits), 0xB1, 0xF, 0xF, true));
+            hpair = even ? (hbits | (other << 16)) : (other | (hbits << 16));
+            if (even) store_xch(xout + off_ring, Pack<2>{hpair}, DS);
+        }
+        clk.lap(2);
+        // ---- the fragments: landed once at most the two ring stores issued behind them are outstanding
+        // (ONE wait statement names the fragment registers: with one in each branch the compiler joins the two
+        // definitions and may copy the registers on the way there, ahead of the wait, while the loads still write them)
+        if (!have_prev) wait_all_vm();
+        wait_frags<2>(f);
+        auto unwritten = [&]() -> bool {
+            unsigned m = 0u;
+#pragma unroll
+            for (int k = 0; k < KS; ++k) {
+                const uint4 ua = __builtin_bit_cast(uint4, f[k]);
+                m = max(m, max(max(ua.x, ua.y), max(ua.z, ua.w)));
+            }
+            return __any(m == kUnwritten) != 0;
+        };
+        if (__builtin_expect(unwritten() && poll.on, 0)) {
+            int spins = 0;
+            long long spin_start = 0;
+            do {
+                if (poll_give_up(poll, spins, spin_start, lane)) break;   // results are garbage from here on; the workgroup leaves at its next barrier
+                request();
+                wait_frags<0>(f);
+            } while (unwritten());
+        }
+        floatx4 acc[2][NT];
+#pragma unroll
+        for (int n = 0; n < NT; ++n) acc[0][n] = floatx4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int k = 0; k < KS; ++k)
+#pragma unroll
+            for (int n = 0; n < NT; ++n)
+                acc[0][n] = __builtin_amdgcn_mfma_f32_16x16x32_f16(wreg[k][n], f[k], acc[0][n], 0, 0, 0);
+        clk.lap(0);
+        // ---- caches of the previous chain for the backward pass, x-projection of the next chain
+        if (live) {
+            const size_t rows = size_t(pt) * p.B + row0;   // row of (step pt, first row of the tile) in the [T*B] arrays
+            __builtin_nontemporal_store(cnew, p.C + (rows + p.B) * p.Hp + off_state);
+            if (even) {
+                __builtin_nontemporal_store(hpair, reinterpret_cast<unsigned*>(p.Y + (rows + p.B) * p.Hp + off_state));
+                if (p.y_out) __builtin_nontemporal_store(hpair, reinterpret_cast<unsigned*>(p.y_out + rows * p.Hp + off_state));
+            }
+            __builtin_nontemporal_store(act, reinterpret_cast<uintx2*>(p.G + rows * (size_t(4) * p.Hp) + off_gate));
+        }
+        request_xp(nt, nrb, std::integral_constant<int, ptl>{});
+        clk.lap(3);
+        spill_partials16<NT>(part, acc, wave, lane, PLD);
+        __syncthreads();
+        clk.lap(1);
+        pt = t; prb = rb; have_prev = true; ++phase;
+        if (lds_abort != 0) leave_kernel();
+    };
+    for (int t = t_begin; t < t_end; ++t) {
+        for (int rb = g; rb < L.nrb; rb += L.ng) {
+            // the chain after (t, rb, tile 1): the next row block of this step, or the first one of the next step (past
+            // the last step: a row that exists, fetched and not used)
+            int nrb = rb + L.ng, nt = t;
+            if (nrb >= L.nrb) { nrb = g; nt = (t + 1 < t_end) ? t + 1 : t; }
+            run_phase(t, rb, std::integral_constant<int, 0>{}, t, rb);
+            run_phase(t, rb, std::integral_constant<int, 1>{}, nt, nrb);
+        }
+    }
+    // the last chain's cell update (tile 1 of the last row block and step)
+    if (have_prev) {
+        const float* part_prev = part_all + size_t((phase & 1) ^ 1) * NW * 16 * PLD;
+        const int row0 = prb * 32 + 16;
+        const bool live = row0 + r < p.B;
+        half_t* xout = p.X + size_t((pt + 1) & 3) * p.x_slot + size_t(2 * prb + 1) * tile_halfs;
+        half_t* xnext = p.X + size_t((pt + 3) & 3) * p.x_slot + size_t(2 * prb + 1) * tile_halfs;
+        wait_all_vm();
+        settle(xp[1]);
+        if (even) store_xch(xnext + off_ring, Pack<2>{kUnwritten}, DS);
+        unsigned hbits = 0u;
+        uintx2 act = uintx2{0u, 0u};
+        float cnew = 0.f;
+        if (live) {
+            float z[4];
+            unpack_h2(xp[1].x, z[0], z[1]);
+            unpack_h2(xp[1].y, z[2], z[3]);
+#pragma unroll
+            for (int w = 0; w < NW; ++w) {
+                const floatx4 v = *reinterpret_cast<const floatx4*>(part_prev + (size_t(w) * 16 + r) * PLD + 4 * u);
+                z[0] += v.x; z[1] += v.y; z[2] += v.z; z[3] += v.w;
+            }
+            float cp;
+            if (c_in_regs) {
+                cp = creg[1];
+            } else {
+                floatx2 q;
+                asm volatile("global_load_dword %0, %1, off sc1\n\ts_waitcnt vmcnt(0)" : "=&v"(q.x) : "v"(p.C + size_t(pt) * p.B * p.Hp + size_t(row0) * p.Hp + off_state) : "memory");
+                cp = q.x;
+            }
+            const float ig = sigmoidf_dev(z[0]);
+            const float fg = sigmoidf_dev(z[1]);
+            const float gg = tanhf_dev(z[2]);
+            const float og = sigmoidf_dev(z[3]);
+            cnew = fg * cp + ig * gg;
+            const float hn = og * tanhf_dev(cnew);
+            act = uintx2{pack_h2(ig, fg), pack_h2(gg, og)};
+            hbits = pack_h2(hn, 0.f);
+        }
+        const unsigned other = unsigned(__builtin_amdgcn_mov_dpp(int(hbits), 0xB1, 0xF, 0xF, true));
+        const unsigned hpair = even ? (hbits | (other << 16)) : (other | (hbits << 16));
+        if (even) store_xch(xout + off_ring, Pack<2>{hpair}, DS);
+        if (live) {
+            const size_t rows = size_t(pt) * p.B + row0;
+            __builtin_nontemporal_store(cnew, p.C + (rows + p.B) * p.Hp + off_state);
+            if (even) {
+                __builtin_nontemporal_store(hpair, reinterpret_cast<unsigned*>(p.Y + (rows + p.B) * p.Hp + off_state));
+                if (p.y_out) __builtin_nontemporal_store(hpair, reinterpret_cast<unsigned*>(p.y_out + rows * p.Hp + off_state));
+            }
+            __builtin_nontemporal_store(act, reinterpret_cast<uintx2*>(p.G + rows * (size_t(4) * p.Hp) + off_gate));
+        }
+    }
+    clk.lap(2);
     clk.flush();
 }
 
@@ -1182,7 +1453,7 @@ __global__ __launch_bounds__(NW * kWave) void rec_bwd_kernel(RecBwdArgs p, RecLa
                 clk.lap(0);
                 spill_partials<NT, MT>(part, acc, wave, lane, PLD);
                 __syncthreads();
-                if (lds_abort != 0) return;
+                if (lds_abort != 0) leave_kernel();
                 clk.lap(1);
             } else {
                 prefetch(t, rb);
@@ -1646,7 +1917,7 @@ __global__ __launch_bounds__(kThreads) void rec_bwd2d_kernel(RecBwdArgs p, RecLa
                 spill_partials<NT, MT>(part, acc, wave, lane, PLD);
                 ++item;
                 __syncthreads();
-                if (lds_abort != 0) return;
+                if (lds_abort != 0) leave_kernel();
                 if (row_used) {   // sum the four waves' k-slices and send 8 columns to their receiver in the slice
                     floatx4 v0 = {0.f, 0.f, 0.f, 0.f}, v1 = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
@@ -1826,7 +2097,8 @@ int rec_waves(int B, int Hp, int num_cus, int waves) {
     const bool xcd_mode = (num_cus == 256 && nh <= 32);
     const int side_by_side = nh > num_cus ? 0 : (xcd_mode ? 8 * (32 / nh) : num_cus / nh);
     const bool can_16 = int(ceil_div(size_t(B), 16)) <= side_by_side;
-    return can_16 ? 4 : 8;
+    (void)can_16;
+    return 4;
 }
 
 static void finish_layout(RecLayout& L, int B, int Hp, int num_cus, bool force_stepwise, bool fits, int force_mt) {
@@ -1840,6 +2112,7 @@ static void finish_layout(RecLayout& L, int B, int Hp, int num_cus, bool force_s
     const bool can_16 = fits && int(ceil_div(size_t(B), 16)) <= side_by_side;
     L.mt = can_16 ? 1 : 2;
     if (force_mt == 2 || (force_mt == 1 && can_16)) L.mt = force_mt;   // a tuned choice; 16-row blocks only where they fit
+    if (L.nw == 8) L.mt = 2;   // the eight-wave kernels take 32-row blocks (their two row tiles take turns)
     L.nrb = int(ceil_div(size_t(B), size_t(16 * L.mt)));
     L.xcd_local = 0;
     L.gpx = 0;
@@ -2017,11 +2290,33 @@ static hipError_t launch_steps(StepGraphCache* graphs, const void* kernel, const
     return hipGraphLaunch(exec, stream);
 }
 
-template <int NT, int KS, bool RES, int MT, bool DS, bool DEEP = false, int NW = 4>
+template <int NT, int KS, bool RES, int MT, bool DS, bool DEEP = false>
 static hipError_t run_fwd(const RecLayout& L, const RecFwdArgs& a, hipStream_t stream, StepGraphCache* graphs) {
-    auto kernel = rec_fwd_kernel<NT, KS, RES, MT, DS, DEEP, NW>;
+    constexpr int NW = 4;
+    auto kernel = rec_fwd_kernel<NT, KS, RES, MT, DS, DEEP>;
     if (L.nw != NW) return hipErrorInvalidValue;   // (the weight fragments are packed for L.nw waves)
-    const size_t lds = size_t(NW == 8 ? 1 : 2) * NW * kRows * (16 * NT + kPartPad) * sizeof(float);
+    const size_t lds = size_t(2) * NW * kRows * (16 * NT + kPartPad) * sizeof(float);
+    hipError_t e = raise_lds(kernel, lds);
+    if (e != hipSuccess) return e;
+    const int ks_wave = rec_fwd_ks(L, a.Hp);
+    if (L.persistent) return launch_persistent(kernel, L.grid, lds, stream, a, L, a.t0, a.t1, ks_wave, NW * kWave);
+    return launch_steps(graphs, reinterpret_cast<const void*>(kernel), &a, sizeof(a), L, a.t0, a.t1, a.t1 - a.t0, stream,
+                        [&]() -> hipError_t {
+                            for (int t = a.t0; t < a.t1; ++t) {
+                                hipLaunchKernelGGL(kernel, dim3(L.grid), dim3(NW * kWave), lds, stream, a, L, t, t + 1, ks_wave);
+                                hipError_t le = hipGetLastError();
+                                if (le != hipSuccess) return le;
+                            }
+                            return hipSuccess;
+                        });
+}
+
+template <bool DS>
+static hipError_t run_fwd_il(const RecLayout& L, const RecFwdArgs& a, hipStream_t stream, StepGraphCache* graphs) {
+    constexpr int NT = 8, NW = 8;
+    auto kernel = rec_fwd_il_kernel<NT, 4, DS>;
+    if (L.nw != NW || L.nt != NT || L.mt != 2 || !L.resident) return hipErrorInvalidValue;
+    const size_t lds = size_t(2) * NW * 16 * (16 * NT + kPartPad) * sizeof(float);
     hipError_t e = raise_lds(kernel, lds);
     if (e != hipSuccess) return e;
     const int ks_wave = rec_fwd_ks(L, a.Hp);
@@ -2043,10 +2338,8 @@ hipError_t launch_rec_fwd(const RecLayout& L, const RecFwdArgs& a, hipStream_t s
     // device-scope stores into the exchange ring: a persistent launch whose groups span XCDs
     const bool ds = L.persistent && !L.xcd_local;
     if (!L.resident) return run_fwd<8, 1, false, 2, false>(L, a, stream, graphs);
-    if (L.nt == 8 && L.nw == 8) {
-        if (L.mt == 1) return ds ? run_fwd<8, 4, true, 1, true, false, 8>(L, a, stream, graphs) : run_fwd<8, 4, true, 1, false, false, 8>(L, a, stream, graphs);
-        return ds ? run_fwd<8, 4, true, 2, true, false, 8>(L, a, stream, graphs) : run_fwd<8, 4, true, 2, false, false, 8>(L, a, stream, graphs);
-    }
+    if (L.nw == 8)   // eight waves: the interleaved kernel, 32-row blocks
+        return ds ? run_fwd_il<true>(L, a, stream, graphs) : run_fwd_il<false>(L, a, stream, graphs);
     if (L.nt == 8) {
         if (L.mt == 1) return ds ? run_fwd<8, 8, true, 1, true>(L, a, stream, graphs) : run_fwd<8, 8, true, 1, false>(L, a, stream, graphs);
         return ds ? run_fwd<8, 8, true, 2, true>(L, a, stream, graphs) : run_fwd<8, 8, true, 2, false>(L, a, stream, graphs);
