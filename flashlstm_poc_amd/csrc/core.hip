@@ -108,8 +108,7 @@ struct flstm_core_plan {
     StepGraphCache graphs_f, graphs_b;   // captured step-wise launches (only used where the persistent kernels are not)
     int opt_graphs = 1;
     int opt_two_d = 1;   // backward recurrence for 2048 hidden units, two-way split: 0 never, 1 where it is faster, 2 wherever it can run
-    int opt_interleave = 1;   // eight-wave kernels: the two row tiles of a block take turns (0 = one chain per block, for comparison)
-    int opt_waves_f = 0, opt_waves_b = 0;   // wavefronts per workgroup of the recurrence kernels: 0 = by size, 4, 8 (the weights are packed for it)
+    int opt_waves_f = 0;   // wavefronts per workgroup of the forward recurrence: 0 = by size, 4, 8 (the weights are packed for it)
     int* status_host = nullptr;   // pinned: the device status word lands here with the end-of-pass copy
     int inject_stall = 0;         // test hook: treat the next N persistent passes as if their launch had given up
     // weights
@@ -144,10 +143,8 @@ void replan(flstm_core_plan* p) {
     p->Lf = plan_rec_fwd(p->d.B, p->d.Hp, p->num_cus, p->opt_stepwise || p->hold_fwd > 0 || p->eff_step_f,
                          p->opt_mt_f ? p->opt_mt_f : p->eff_mt_f, p->opt_waves_f);
     p->Lb = plan_rec_bwd(p->d.B, p->d.Hp, p->num_cus, p->opt_stepwise || p->hold_bwd > 0 || p->eff_step_b,
-                         p->opt_mt_b ? p->opt_mt_b : p->eff_mt_b, p->opt_two_d, p->opt_waves_b);
+                         p->opt_mt_b ? p->opt_mt_b : p->eff_mt_b, p->opt_two_d);
     p->Lf.cooperative = p->Lb.cooperative = p->opt_cooperative;
-    p->Lf.interleave = (p->opt_interleave && p->Lf.nw == 8 && p->Lf.mt == 2 && p->Lf.resident) ? 1 : 0;
-    p->Lb.interleave = (p->opt_interleave && p->Lb.nw == 8 && p->Lb.mt == 2 && p->Lb.resident && !p->Lb.two_d) ? 1 : 0;
     p->ks_f = rec_fwd_ks(p->Lf, p->d.Hp);
     p->ks_b = rec_bwd_ks(p->Lb, p->d.Hp);
 }
@@ -258,9 +255,7 @@ extern "C" int flstm_core_create(size_t batch, size_t input_size, size_t hidden_
         if (const char* v = getenv("FLASHLSTM_COOPERATIVE_LAUNCH")) p->opt_cooperative = atoi(v) != 0;
         if (const char* v = getenv("FLASHLSTM_STEP_GRAPHS")) p->opt_graphs = atoi(v) != 0;
         if (const char* v = getenv("FLASHLSTM_BWD_TWO_D")) p->opt_two_d = atoi(v) < 0 ? 0 : (atoi(v) > 2 ? 2 : atoi(v));
-        if (const char* v = getenv("FLASHLSTM_INTERLEAVE")) p->opt_interleave = atoi(v) != 0;
         if (const char* v = getenv("FLASHLSTM_WAVES_FWD")) p->opt_waves_f = (atoi(v) == 4 || atoi(v) == 8) ? atoi(v) : 0;
-        if (const char* v = getenv("FLASHLSTM_WAVES_BWD")) p->opt_waves_b = (atoi(v) == 4 || atoi(v) == 8) ? atoi(v) : 0;
     }
     replan(p);
     e = p->status.reserve(64);
@@ -308,13 +303,14 @@ extern "C" int flstm_core_set_option(flstm_core_plan* p, const char* name, long 
     if (!strcmp(name, "cooperative")) { p->opt_cooperative = value != 0; replan(p); return 0; }
     if (!strcmp(name, "step_graphs")) { p->opt_graphs = value != 0; return 0; }
     if (!strcmp(name, "bwd_two_d")) { if (value < 0 || value > 2) return FLSTM_E_INVALID; p->opt_two_d = int(value); replan(p); return 0; }
-    if (!strcmp(name, "waves_fwd") || !strcmp(name, "waves_bwd")) {
-        // wavefronts per workgroup of a recurrence: the weight fragments are packed for it, so a change un-packs them
+    if (!strcmp(name, "waves_fwd")) {
+        // wavefronts per workgroup of the forward recurrence: the weight fragments are packed for it, so a change
+        // un-packs them
         if (value != 0 && value != 4 && value != 8) return FLSTM_E_INVALID;
-        const int before = name[6] == 'f' ? p->Lf.nw : p->Lb.nw;
-        (name[6] == 'f' ? p->opt_waves_f : p->opt_waves_b) = int(value);
+        const int before = p->Lf.nw;
+        p->opt_waves_f = int(value);
         replan(p);
-        if ((name[6] == 'f' ? p->Lf.nw : p->Lb.nw) != before) p->weights_packed = false;
+        if (p->Lf.nw != before) p->weights_packed = false;
         return 0;
     }
     if (!strcmp(name, "inject_stall")) { if (value < 0) return FLSTM_E_INVALID; p->inject_stall = int(value); return 0; }
@@ -337,7 +333,6 @@ extern "C" long flstm_core_get_info(const flstm_core_plan* p, const char* name) 
     if (!strcmp(name, "cooperative")) return p->opt_cooperative;
     if (!strcmp(name, "bwd_two_d")) return p->Lb.two_d;
     if (!strcmp(name, "waves_fwd")) return p->Lf.nw;
-    if (!strcmp(name, "waves_bwd")) return p->Lb.nw;
     if (!strcmp(name, "graph_captures")) return p->graphs_f.captures + p->graphs_b.captures;
     if (!strcmp(name, "graph_replays")) return p->graphs_f.replays + p->graphs_b.replays;
     if (!strcmp(name, "graphs_disabled")) return (p->graphs_f.disabled ? 1 : 0) + (p->graphs_b.disabled ? 2 : 0);

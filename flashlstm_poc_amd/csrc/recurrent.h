@@ -29,10 +29,10 @@ struct RecLayout {
     int nm;          // two_d: passes per step the kernel is built for (row blocks per workgroup, rounded up to 1, 2, 4)
     int win_rows;    // two_d: 0, or the batch is walked in windows of this many rows, one persistent launch each (batch
                      // rows are independent sequences); nrb, mt, ng, nm then describe one window
-    int interleave;  // eight waves, 32-row blocks: the two 16-row tiles of a block are chains that take turns (rec_fwd_il_kernel)
-    int nw;          // wavefronts per workgroup of the one-way kernels, which split the contraction between them: 4, or 8
-                     // (two per SIMD).  The weight fragments are packed for this count, so it is a function of the
-                     // sizes alone and does not follow mt
+    int nw;          // wavefronts per workgroup of the one-way kernels, which split the contraction between them: 4, or
+                     // (forward, slices of 32 units) 8, two per SIMD, with 32-row blocks whose two row tiles take turns
+                     // (rec_fwd_il_kernel).  The weight fragments are packed for this count, so it is a function of
+                     // the sizes alone and does not follow mt
 };
 
 struct RecFwdArgs {
@@ -143,11 +143,11 @@ constexpr size_t kGraphCacheEntries = 4;
 // Picks tile shapes and the group structure for a problem size on the current device.  force_mt: 0 = the rule of
 // thumb (16-row blocks whenever all of them can run side by side), 1 / 2 = that many 16-row tiles per row block
 // (1 only where it fits).  The choice does not change the weight-fragment layout.
-// waves: 0 = the rule of thumb (rec_waves), 4 or 8 = that many wavefronts per workgroup (8 only where it can run).
+// waves: 0 = the rule of thumb (rec_waves), 4 or 8 = that many wavefronts per workgroup (8 only up to 1024 units).
 RecLayout plan_rec_fwd(int B, int Hp, int num_cus, bool force_stepwise, int force_mt = 0, int waves = 0);
 // two_d: 0 = never the two-way split, 1 = where it is the faster layout, 2 = wherever it can run
-RecLayout plan_rec_bwd(int B, int Hp, int num_cus, bool force_stepwise, int force_mt = 0, int two_d = 1, int waves = 0);
-// Wavefronts per workgroup the one-way kernels run with for these sizes (a function of the sizes alone).
+RecLayout plan_rec_bwd(int B, int Hp, int num_cus, bool force_stepwise, int force_mt = 0, int two_d = 1);
+// Wavefronts per workgroup the forward kernel runs with for these sizes (a function of the sizes alone).
 int rec_waves(int B, int Hp, int num_cus, int waves);
 
 // The two-dimensional backward layout: whether a device/size can use it at all (decides whether its weight fragments

@@ -402,7 +402,7 @@ __device__ __forceinline__ bool wave_product_tiles(floatx4 (&acc)[2][NT], const 
 
 // `prefetch` issues exactly NPF vector loads (for every wave, whatever its lanes need) behind the last
 // fragment load.
-template <int NT, int KS, bool RESIDENT, int KL, int NPF, int MT, int NBUF = 2, int CKO = 0, bool LAZY = false, bool REASK = false, int NW = 4, typename Prefetch>
+template <int NT, int KS, bool RESIDENT, int KL, int NPF, int MT, int NBUF = 2, int CKO = 0, bool LAZY = false, bool REASK = false, int NW = 4, bool SADDR = (NW == 8), typename Prefetch>
 __device__ __forceinline__ bool wave_product(floatx4 (&acc)[2][NT], const half8 (&wreg)[KS - KL][NT],
                                              const half8* wlds, const half8* wfrag_wave, const half_t* a0,
                                              const half_t* a1, int wave, int lane, int nks_total,
@@ -425,8 +425,7 @@ __device__ __forceinline__ bool wave_product(floatx4 (&acc)[2][NT], const half8 
         for (;;) {
         const half_t *p0 = a0, *p1 = a1;   // (opaque copies, as in wave_product_tiles)
         if constexpr (LAZY) asm volatile("" : "+v"(p0), "+v"(p1));
-        // eight waves: scalar base + lane offset (ld_frag_async_at)
-        constexpr bool SADDR = (NW == 8);
+        // SADDR (kernels of two waves per SIMD): scalar base + lane offset (ld_frag_async_at)
         const unsigned lane_off = unsigned(lane) * 16u;
         const half_t *u0 = nullptr, *u1 = nullptr;
         int wv = wave;
@@ -775,6 +774,7 @@ __device__ __forceinline__ void to_floats(const F32<4>& r, float (&f)[4]) {
 struct PhaseClock {
     long long* out;
     long long last;
+
     __device__ __forceinline__ long long* acc() {
         __shared__ long long lds_acc[5];
         return lds_acc;
@@ -785,6 +785,7 @@ struct PhaseClock {
             last = wall_clock64();
         }
     }
+
     __device__ __forceinline__ void lap(int slot) {
         // (the pointer is the same for the whole workgroup: tested on its own and marked unlikely, a launch without
         // counters falls through one scalar branch instead of jumping over a masked block)
@@ -1328,11 +1329,10 @@ __global__ __launch_bounds__(8 * kWave) void rec_fwd_il_kernel(RecFwdArgs p, Rec
 // ----------------------------------------------------------------------------------- backward
 // Gate order and the pointwise derivative follow flashlstm_v2/src/lstm_backward.cu:199-211, except
 // that c_{t-1}, c_t come from the cell-state cache instead of being rebuilt through atanh.
-template <int NT, int KS, bool RESIDENT, int KL, int MT, bool DS, int NW = 4>
-__global__ __launch_bounds__(NW * kWave) void rec_bwd_kernel(RecBwdArgs p, RecLayout L, int t_first,
-                                                             int t_last, int ks_wave) {
-    static_assert(NW == 4 || (NW == 8 && NT == 2), "eight waves (see rec_fwd_kernel): slices of 32 units");
-    constexpr int THREADS = NW * kWave;
+template <int NT, int KS, bool RESIDENT, int KL, int MT, bool DS>
+__global__ __launch_bounds__(kThreads) void rec_bwd_kernel(RecBwdArgs p, RecLayout L, int t_first,
+                                                           int t_last, int ks_wave) {
+    constexpr int NW = 4, THREADS = kThreads;
     constexpr int JB = 16 * NT;  // hidden units (= output columns of dG*W_hh) of this slice
     constexpr int PLD = JB + kPartPad;
     constexpr int KR = KS - KL;  // k-steps whose weight fragments stay in registers
@@ -1340,8 +1340,8 @@ __global__ __launch_bounds__(NW * kWave) void rec_bwd_kernel(RecBwdArgs p, RecLa
     // dG_t, then rows 16..31, and fetch and multiply tile by tile, so the second half of a step's cell updates and its
     // cache stores run while the peers are already in the first half of their next product (measured at 1024 units
     // and 256 rows: 4.85 -> 4.5 us per step; without waiting for producers at all the step takes 4.2).
-    constexpr bool SPLIT = NW == 4 && RESIDENT && MT == 2 && JB >= 32 && (KS % 8 == 0);
-    constexpr int GPR = (NW == 8 || SPLIT || (MT == 1 && JB >= 32)) ? 16 : 8;   // threads per batch row (as in the forward kernel)
+    constexpr bool SPLIT = RESIDENT && MT == 2 && JB >= 32 && (KS % 8 == 0);
+    constexpr int GPR = (SPLIT || (MT == 1 && JB >= 32)) ? 16 : 8;   // threads per batch row (as in the forward kernel)
     constexpr int UPT = JB / GPR;
     constexpr int NPH = SPLIT ? 2 : 1;   // pointwise phases per step
     static_assert(UPT == 2 || UPT == 4, "2 or 4 hidden units per thread");
@@ -1447,7 +1447,7 @@ __global__ __launch_bounds__(NW * kWave) void rec_bwd_kernel(RecBwdArgs p, RecLa
                     ahead = wave_product_tiles<NT, KS, KL, NPF, 4, false, 4, DS>(acc, wreg, wlds, a0, a1, wave, lane, nks_total, ks_wave, rotation, poll,
                                                            [&]() { prefetch(t, rb); });
                 else
-                    ahead = wave_product<NT, KS, RESIDENT, KL, NPF, MT, (NW == 8) ? 3 : 2, (NW == 8) ? 2 : 0, false, DS, NW>(acc, wreg, wlds, wfrag_wave, a0, a1, wave, lane, nks_total,
+                    ahead = wave_product<NT, KS, RESIDENT, KL, NPF, MT, 2, 0, false, DS>(acc, wreg, wlds, wfrag_wave, a0, a1, wave, lane, nks_total,
                                                               ks_wave, rotation, poll, [&]() { prefetch(t, rb); });
                 if constexpr (DS) first_request.learn(ahead);
                 clk.lap(0);
@@ -2088,8 +2088,11 @@ size_t exchange_slot_halfs(int rows, int cols) { return round_up(size_t(rows), 3
 int rec_fwd_ks(const RecLayout& L, int Hp) { return int(ceil_div(size_t(Hp) / 32, size_t(L.nw))); }
 int rec_bwd_ks(const RecLayout& L, int Hp) { return int(ceil_div(size_t(Hp) / 8, size_t(L.nw))); }
 
-// Eight waves per workgroup where a slice has 32 units (up to 1024 hidden units) and the default split gives every
-// workgroup 32-row blocks: measured there (1024 units, 256 rows).
+// Wavefronts per workgroup of the forward recurrence: eight (rec_fwd_il_kernel: the two row tiles of a 32-row block
+// take turns) where a slice has 32 units -- up to 1024 hidden units -- and every workgroup gets exactly one 32-row
+// block: more rows than 16-row blocks can run side by side, no more than 32-row blocks can.  Measured, us per step,
+// four -> eight waves: 1024 units and 256 rows 3.45 -> 3.24, 768 units and 160 rows 3.06 -> 2.84, 512 units and 512
+// rows 3.19 -> 3.12; with two row blocks per workgroup (1024 units, 512 rows) 7.2 -> 8.6, so those stay with four.
 int rec_waves(int B, int Hp, int num_cus, int waves) {
     if (Hp > 1024) return 4;
     if (waves == 4 || waves == 8) return waves;
@@ -2097,8 +2100,8 @@ int rec_waves(int B, int Hp, int num_cus, int waves) {
     const bool xcd_mode = (num_cus == 256 && nh <= 32);
     const int side_by_side = nh > num_cus ? 0 : (xcd_mode ? 8 * (32 / nh) : num_cus / nh);
     const bool can_16 = int(ceil_div(size_t(B), 16)) <= side_by_side;
-    (void)can_16;
-    return 4;
+    const bool one_block_each = int(ceil_div(size_t(B), 32)) <= side_by_side;
+    return (!can_16 && one_block_each) ? 8 : 4;
 }
 
 static void finish_layout(RecLayout& L, int B, int Hp, int num_cus, bool force_stepwise, bool fits, int force_mt) {
@@ -2147,13 +2150,13 @@ RecLayout plan_rec_fwd(int B, int Hp, int num_cus, bool force_stepwise, int forc
     return L;
 }
 
-RecLayout plan_rec_bwd(int B, int Hp, int num_cus, bool force_stepwise, int force_mt, int two_d, int waves) {
+RecLayout plan_rec_bwd(int B, int Hp, int num_cus, bool force_stepwise, int force_mt, int two_d) {
     RecLayout L{};
     bool fits = true;
     if (Hp <= 1024) L.nt = 2;
     else if (Hp <= 2048) L.nt = 1;
     else { L.nt = 2; fits = false; }
-    L.nw = fits ? rec_waves(B, Hp, num_cus, waves) : 4;
+    L.nw = 4;
     L.jb = 16 * L.nt;
     finish_layout(L, B, Hp, num_cus, force_stepwise, fits, force_mt);
     // k-step rotation (recurrent.h): measured, it pays where a group spans the XCDs and a step fetches a lot -- the
@@ -2353,9 +2356,10 @@ hipError_t launch_rec_fwd(const RecLayout& L, const RecFwdArgs& a, hipStream_t s
     return hipErrorInvalidValue;
 }
 
-template <int NT, int KS, bool RES, int KL, int MT, bool DS, int NW = 4>
+template <int NT, int KS, bool RES, int KL, int MT, bool DS>
 static hipError_t run_bwd(const RecLayout& L, const RecBwdArgs& a, hipStream_t stream, StepGraphCache* graphs) {
-    auto kernel = rec_bwd_kernel<NT, KS, RES, KL, MT, DS, NW>;
+    constexpr int NW = 4;
+    auto kernel = rec_bwd_kernel<NT, KS, RES, KL, MT, DS>;
     if (L.nw != NW) return hipErrorInvalidValue;   // (the weight fragments are packed for L.nw waves)
     static_assert(size_t(2) * NW * kRows * (16 * NT + kPartPad) >= size_t(NW * kWave) * 8 * NT, "db reduction reuses the partial-sum area");
     const size_t lds = size_t(2) * NW * kRows * (16 * NT + kPartPad) * sizeof(float) + size_t(NW) * KL * NT * kWave * sizeof(half8);
@@ -2411,10 +2415,6 @@ hipError_t launch_rec_bwd(const RecLayout& L, const RecBwdArgs& a, hipStream_t s
     }
     const bool ds = L.persistent && !L.xcd_local;   // (as in launch_rec_fwd)
     if (!L.resident) return run_bwd<2, 1, false, 0, 2, false>(L, a, stream, graphs);
-    if (L.nt == 2 && L.nw == 8) {
-        if (L.mt == 1) return ds ? run_bwd<2, 16, true, 4, 1, true, 8>(L, a, stream, graphs) : run_bwd<2, 16, true, 4, 1, false, 8>(L, a, stream, graphs);
-        return ds ? run_bwd<2, 16, true, 4, 2, true, 8>(L, a, stream, graphs) : run_bwd<2, 16, true, 4, 2, false, 8>(L, a, stream, graphs);
-    }
     if (L.nt == 2) {
         if (L.mt == 1) return ds ? run_bwd<2, 32, true, 8, 1, true>(L, a, stream, graphs) : run_bwd<2, 32, true, 8, 1, false>(L, a, stream, graphs);
         return ds ? run_bwd<2, 32, true, 8, 2, true>(L, a, stream, graphs) : run_bwd<2, 32, true, 8, 2, false>(L, a, stream, graphs);
