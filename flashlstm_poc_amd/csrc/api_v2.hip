@@ -183,7 +183,7 @@ unsigned long long device_print(Entry& e, hipStream_t s, const float* w_ih, cons
                                 const float* b_hh, const __half* h0, const __half* c0) {
     using flstm_hip::checksum_add;
     const size_t G = 4 * e.H;
-    e.sum_dev.reserve(sizeof(unsigned long long));
+    e.sum_dev.reserve(sizeof(unsigned long long));   // (throws if the allocation fails)
     auto* acc = static_cast<flstm_hip::u64*>(e.sum_dev.p);
     check(flstm_hip::fill_zero(acc, sizeof(unsigned long long), s), "checksum");
     check(checksum_add(w_ih, G * e.I * sizeof(float), 0x1000000000ull, acc, s), "checksum");

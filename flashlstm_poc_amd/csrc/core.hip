@@ -96,6 +96,10 @@ struct flstm_core_plan {
     // tried again.  Every further give-up doubles the hold (at most kMaxHold passes).
     int hold_fwd = 0, hold_bwd = 0, backoff_fwd = kFirstHold, backoff_bwd = kFirstHold;
     long fallbacks = 0, demotions_fwd = 0, demotions_bwd = 0;
+    // A cooperative launch refused because the grid cannot be co-resident: that direction runs step-wise from then on.
+    bool refused_fwd = false, refused_bwd = false;
+    long coop_refusals = 0;
+    bool static_call = false;   // flstm_core_forward_static in force: nothing may allocate (no graph capture either)
     // Tuned launch choices per sequence length (flstm_core_tune): 16- or 32-row blocks and persistent or step-wise
     // launches per direction, split-K count of the weight-gradient GEMM.  eff_* hold the entry in force for the
     // sequence length of the current pass (0 = no tuned value: the rules of thumb decide); explicit options win.
@@ -110,7 +114,7 @@ struct flstm_core_plan {
     int opt_two_d = 1;   // backward recurrence for 2048 hidden units, two-way split: 0 never, 1 where it is faster, 2 wherever it can run
     int opt_waves_f = 0;   // wavefronts per workgroup of the forward recurrence: 0 = by size, 4, 8 (the weights are packed for it)
     int* status_host = nullptr;   // pinned: the device status word lands here with the end-of-pass copy
-    int inject_stall = 0;         // test hook: treat the next N persistent passes as if their launch had given up
+    int inject_stall = 0;         // test hook: treat the next N passes as if their launches had given up
     // weights
     DevBuf wih_p, wih_t, wfrag_f, wfrag_b, wfrag_b2, bias_p;
     bool weights_packed = false, bias_packed = false;
@@ -140,9 +144,9 @@ namespace {
     } while (0)
 
 void replan(flstm_core_plan* p) {
-    p->Lf = plan_rec_fwd(p->d.B, p->d.Hp, p->num_cus, p->opt_stepwise || p->hold_fwd > 0 || p->eff_step_f,
+    p->Lf = plan_rec_fwd(p->d.B, p->d.Hp, p->num_cus, p->opt_stepwise || p->hold_fwd > 0 || p->eff_step_f || p->refused_fwd,
                          p->opt_mt_f ? p->opt_mt_f : p->eff_mt_f, p->opt_waves_f);
-    p->Lb = plan_rec_bwd(p->d.B, p->d.Hp, p->num_cus, p->opt_stepwise || p->hold_bwd > 0 || p->eff_step_b,
+    p->Lb = plan_rec_bwd(p->d.B, p->d.Hp, p->num_cus, p->opt_stepwise || p->hold_bwd > 0 || p->eff_step_b || p->refused_bwd,
                          p->opt_mt_b ? p->opt_mt_b : p->eff_mt_b, p->opt_two_d);
     p->Lf.cooperative = p->Lb.cooperative = p->opt_cooperative;
     p->ks_f = rec_fwd_ks(p->Lf, p->d.Hp);
@@ -178,7 +182,8 @@ int enqueue_status_copy(flstm_core_plan* p, hipStream_t s) {
 int take_status(flstm_core_plan* p, bool fwd, hipStream_t s, int* out) {
     *out = *static_cast<volatile int*>(p->status_host);
     if (*out != 0) FL_TRY(fill_zero(p->status.p, sizeof(int), s));
-    if (*out == 0 && p->inject_stall > 0 && (fwd ? p->Lf.persistent : p->Lb.persistent)) {
+    (void)fwd;
+    if (*out == 0 && p->inject_stall > 0) {   // (2 in a row: the step-wise repeat of a pass fails too, i.e. the call does)
         p->inject_stall--;
         *out = 1;
     }
@@ -358,6 +363,7 @@ extern "C" long flstm_core_get_info(const flstm_core_plan* p, const char* name) 
     if (!strcmp(name, "fallbacks")) return p->fallbacks;
     if (!strcmp(name, "demotions_fwd")) return p->demotions_fwd;
     if (!strcmp(name, "demotions_bwd")) return p->demotions_bwd;
+    if (!strcmp(name, "cooperative_refusals")) return p->coop_refusals;
     if (!strcmp(name, "hold_fwd")) return p->hold_fwd;
     if (!strcmp(name, "hold_bwd")) return p->hold_bwd;
     if (!strcmp(name, "static_scratch_bytes")) return long(kStaticScratchBytes);
@@ -480,7 +486,18 @@ int forward_recur(flstm_core_plan* p, size_t t0, size_t n, hipStream_t s) {
     a.spin_limit = p->opt_spin_limit;
     a.spin_ticks = (long long)p->opt_spin_ms * p->wall_khz;
     a.prof = p->opt_profile ? p->prof.as<long long>() : nullptr;
-    FL_TRY(launch_rec_fwd(p->Lf, a, s, p->opt_graphs ? &p->graphs_f : nullptr));
+    // Step-wise launches are replayed from a captured graph only for whole passes: a sequence fed in ranges has a new
+    // range (a new graph) every call, each used once.  Never inside flstm_core_forward_static (a capture allocates).
+    const bool whole = (t0 == 0 && n == p->fw.T);
+    hipError_t e = launch_rec_fwd(p->Lf, a, s, (p->opt_graphs && whole && !p->static_call) ? &p->graphs_f : nullptr);
+    if (e == hipErrorCooperativeLaunchTooLarge && p->Lf.persistent) {
+        // the grid cannot be co-resident: this direction runs step-wise from now on, starting with these steps
+        p->refused_fwd = true;
+        p->coop_refusals++;
+        replan(p);
+        e = launch_rec_fwd(p->Lf, a, s, nullptr);
+    }
+    FL_TRY(e);
     return 0;
 }
 
@@ -552,6 +569,7 @@ extern "C" int flstm_core_forward(flstm_core_plan* p, size_t T, const void* x, f
     p->have_cache = false;
     int rc = forward_pass(p, T, x, x_dtype, h0, c0, state_dtype, y, y_dtype, hy, cy, out_state_dtype,
                           static_cast<hipStream_t>(stream));
+    p->fw.open = false;   // (also when the pass failed: no range of steps may follow it)
     if (rc) return rc;
     if (save_for_backward) { p->have_cache = true; p->T_cache = T; }
     return 0;
@@ -599,8 +617,11 @@ extern "C" int flstm_core_forward_static(flstm_core_plan* p, size_t T, const voi
     p->have_cache = false;   // (the plan's own caches are untouched, but no pass may use the borrowed ones later)
     // status word and seat counters start at zero; the array keeps whatever the last call left
     rc = int(fill_zero(p->status.p, 64, s));
+    p->static_call = true;   // (step-wise launches, if the pass comes to them, are plain launches: a graph capture allocates)
     if (rc == 0)
         rc = forward_pass(p, T, x, x_dtype, h0, c0, state_dtype, y, y_dtype, hy, cy, out_state_dtype, s);
+    p->static_call = false;
+    p->fw.open = false;   // (also when the pass failed: the next call must not find a pass in progress)
     for (int i = 0; i < 6; ++i) *slot[i] = saved[i];
     p->have_cache = had_cache;
     return rc;
@@ -694,7 +715,10 @@ int backward_recur(flstm_core_plan* p, long t_hi, long t_lo, hipStream_t s) {
             for (int k = 0; k < kRecBwdPartSlots; ++k)
                 FL_TRY(fill_words(static_cast<char*>(p->part_b.p) + size_t(k) * pslot, pslot, rec_bwd_part_fill(k, first_T), s));
         }
-        FL_TRY(launch_rec_bwd(p->Lb, a, s, p->opt_graphs ? &p->graphs_b : nullptr));
+        const bool whole = (t_hi == long(p->bw.T) - 1 && t_lo == -1);   // (graphs for whole passes only: see forward_recur)
+        hipError_t e = launch_rec_bwd(p->Lb, a, s, (p->opt_graphs && whole) ? &p->graphs_b : nullptr);
+        if (e == hipErrorCooperativeLaunchTooLarge && p->Lb.persistent) return int(e);   // (handled by the caller: the layout changes)
+        FL_TRY(e);
     }
     return 0;
 }
@@ -801,6 +825,13 @@ extern "C" int flstm_core_backward(flstm_core_plan* p, size_t T, const void* x, 
     // Only when the caller's gradients are added to (accumulate_grads) the status is checked first.
     for (int attempt = 0;; ++attempt) {
         int rc = backward_rec_once(p, T, dY, dy_dtype, d_hn, d_cn, dstate_dtype, S, dx, dx_dtype, s);
+        if (rc == int(hipErrorCooperativeLaunchTooLarge) && p->Lb.persistent && !p->refused_bwd) {
+            // the grid cannot be co-resident: nothing was launched; this direction runs step-wise from now on
+            p->refused_bwd = true;
+            p->coop_refusals++;
+            replan(p);
+            continue;
+        }
         if (rc) return rc;
         int st = 0;
         if (p->opt_accumulate) {
@@ -892,6 +923,15 @@ extern "C" int flstm_core_backward_steps(flstm_core_plan* p, size_t t_hi, size_t
     const long lo = long(t_hi) - long(nsteps) + 1;
     // the range that reaches step 0 also runs the closing product for dh0
     int rc = backward_recur(p, long(t_hi), lo == 0 ? -1 : lo, s);
+    if (rc == int(hipErrorCooperativeLaunchTooLarge) && p->Lb.persistent && !p->refused_bwd) {
+        // the grid cannot be co-resident: step-wise from now on; the rings of this pass were laid out for the persistent
+        // kernel, so the caller repeats the pass (as after a launch that gave up)
+        p->refused_bwd = true;
+        p->coop_refusals++;
+        p->bw.open = false;
+        replan(p);
+        return FLSTM_E_STALLED;
+    }
     if (rc) return rc;
     return backward_dx(p, long(t_hi), lo, s);
 }

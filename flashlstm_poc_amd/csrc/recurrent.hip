@@ -2067,6 +2067,10 @@ hipError_t launch_persistent(K kernel, int grid, size_t lds, hipStream_t stream,
                                                   unsigned(lds), stream);
         if (e == hipSuccess) return hipSuccess;
         (void)hipGetLastError();
+        // A grid the runtime says cannot be co-resident is exactly what a persistent launch must not be given: nothing
+        // is launched, and the caller runs the pass step-wise.  Any other refusal (no cooperative launch on this
+        // runtime) falls back to the plain launch, whose bounded waits cover a late workgroup.
+        if (e == hipErrorCooperativeLaunchTooLarge) return e;
     }
     hipLaunchKernelGGL(kernel, dim3(grid), dim3(threads), lds, stream, a, L, t_a, t_b, ks_wave);
     return hipGetLastError();

@@ -90,12 +90,15 @@ int flstm_core_forward(flstm_core_plan* plan, size_t seq_len,
                        void* hy, void* cy, flstm_dtype out_state_dtype,
                        int save_for_backward, void* stream);
 
-/* flstm_core_forward for callers that cannot allocate device memory (code under HIP graph capture, tight serving
- * loops, harnesses that forbid hipMalloc).  It has no counterpart in the reference.  Same arguments, results and
- * kernels as flstm_core_forward with save_for_backward = 0, but everything the kernels need beyond the caller's
+/* flstm_core_forward for callers that cannot allocate device memory (tight serving loops, harnesses that forbid
+ * hipMalloc, the host code around a HIP graph).  It has no counterpart in the reference.  Same arguments, results
+ * and kernels as flstm_core_forward with save_for_backward = 0, but everything the kernels need beyond the caller's
  * tensors and the plan's packed weights -- status word, converted x rows, x-projection / gate rows, state rows,
  * exchange ring -- lives in one fixed 64 MiB array in the library's device image instead of buffers grown by the
- * plan: the call allocates and frees nothing.  A pass that needs more (about T*B*(14*Hp + 2*Ip) bytes; the limit
+ * plan: the call allocates and frees nothing, also not when a persistent launch gives up and the pass is repeated
+ * with one launch per step (those are plain launches here, never a captured graph).  Like flstm_core_forward it is
+ * SYNCHRONOUS -- it waits for its stream and reads the status of the pass on the host -- so it cannot itself be
+ * recorded into a graph that is being captured.  A pass that needs more (about T*B*(14*Hp + 2*Ip) bytes; the limit
  * is flstm_core_get_info(plan, "static_scratch_bytes")) is rejected with FLSTM_E_TOO_LARGE before any work is
  * enqueued.  Nothing is kept for a backward pass, and a cache that an earlier flstm_core_forward left in the plan
  * stays valid.  Every call on a GPU uses that GPU's one array, whichever plan it comes from: calls that overlap

@@ -103,3 +103,55 @@ def test_static_forward_equals_the_allocating_forward_on_shrinking_calls():
     assert rc == 2004
     for h in (plan_a, plan_ref_a, plan_b, plan_ref_b):
         assert lib.flstm_core_destroy(h) == 0
+
+
+def test_static_forward_allocates_nothing_on_the_step_wise_path_and_after_a_give_up():
+    """The entry point's promise holds where the pass is one launch per step -- a plan with the `stepwise` option, and
+    the repeat after a persistent launch that gave up (forced from the host: `inject_stall`): plain launches, no graph
+    capture, device memory in use unchanged, results bit-identical to flstm_core_forward; and a call that failed
+    leaves the plan usable."""
+    from flashlstm_poc_amd import load_library
+    lib = load_library()
+    p = make_problem(20, 40, 64, 256, seed=43)
+    cvh = lambda t: t.cuda().half().contiguous()
+    x, h0, c0 = cvh(p["x"]), cvh(p["h0"]), cvh(p["c0"])
+    plan, keep = _plan(lib, p)
+    ref, keep_r = _plan(lib, p)
+    rc, want, _ = _call(lib, False, ref, x, h0, c0, F16, torch.float16)
+    assert rc == 0
+    # warm-up (code objects), then the measured calls
+    rc, _, _ = _call(lib, True, plan, x, h0, c0, F16, torch.float16)
+    assert rc == 0
+    # 1) a persistent launch that gives up: the pass is repeated with one launch per step inside the same call
+    assert lib.flstm_core_get_info(plan, b"persistent_fwd") == 1
+    assert lib.flstm_core_set_option(plan, b"inject_stall", 1) == 0
+    captures = lib.flstm_core_get_info(plan, b"graph_captures")
+    rc, got, grew = _call(lib, True, plan, x, h0, c0, F16, torch.float16)
+    assert rc == 0 and grew == 0, (rc, grew)
+    assert lib.flstm_core_get_info(plan, b"fallbacks") == 1 and lib.flstm_core_get_info(plan, b"persistent_fwd") == 0
+    assert lib.flstm_core_get_info(plan, b"graph_captures") == captures   # no graph was built
+    for g, w, what in zip(got, want, ("y", "hy", "cy")):
+        assert torch.equal(g, w), ("after a give-up", what)
+    # 2) the demoted plan (step-wise launches) and a plan with the option: the same, still without a graph
+    assert lib.flstm_core_set_option(plan, b"stepwise", 1) == 0
+    for _ in range(2):
+        rc, got, grew = _call(lib, True, plan, x, h0, c0, F16, torch.float16)
+        assert rc == 0 and grew == 0, (rc, grew)
+        for g, w, what in zip(got, want, ("y", "hy", "cy")):
+            assert torch.equal(g, w), ("step-wise", what)
+    assert lib.flstm_core_get_info(plan, b"graph_captures") == captures
+    # 3) a pass that fails (two give-ups in a row: the step-wise repeat is treated as failed too) returns "stalled" and
+    #    the next call works
+    assert lib.flstm_core_set_option(plan, b"stepwise", 0) == 0
+    assert lib.flstm_core_set_option(plan, b"clear_tuned", 0) == 0
+    plan2, keep2 = _plan(lib, p)
+    assert lib.flstm_core_set_option(plan2, b"inject_stall", 2) == 0
+    rc, _, _ = _call(lib, True, plan2, x, h0, c0, F16, torch.float16)
+    assert rc == 2003, rc   # FLSTM_E_STALLED
+    assert lib.flstm_core_set_option(plan2, b"inject_stall", 0) == 0
+    rc, got, _ = _call(lib, True, plan2, x, h0, c0, F16, torch.float16)
+    assert rc == 0
+    for g, w, what in zip(got, want, ("y", "hy", "cy")):
+        assert torch.equal(g, w), ("after a failed call", what)
+    for h in (plan, ref, plan2):
+        assert lib.flstm_core_destroy(h) == 0
