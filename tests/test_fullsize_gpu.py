@@ -139,3 +139,51 @@ def test_full_length_configs_against_fp32_torch_lstm(name, shape, backward):
     print(f"\n{name} T={T} B={B} I={I} H={H}: " + ", ".join(f"{k}={v:.2e}" for k, v in errs.items()))
     assert max(errs.values()) <= 1e-2, errs
     core.close()
+
+
+def _cpu_lstm_reference(p):
+    """fp32 torch.nn.LSTM on the host CPU -- the oracle the reference's own test uses (python/test_lstm.py:99-104) --
+    with the fp16-rounded weights and inputs the kernels see; forward and autograd for the loss sum(y * dY)."""
+    T, B, I = p["x"].shape
+    H = p["w_hh"].shape[1]
+    m = torch.nn.LSTM(I, H)
+    with torch.no_grad():
+        m.weight_ih_l0.copy_(p["w_ih"].half().float().cpu()); m.weight_hh_l0.copy_(p["w_hh"].half().float().cpu())
+        m.bias_ih_l0.copy_(p["b_ih"].cpu()); m.bias_hh_l0.copy_(p["b_hh"].cpu())
+    xr = p["x"].float().cpu().requires_grad_(True)
+    hr = p["h0"].float().cpu().requires_grad_(True); cr = p["c0"].float().cpu().requires_grad_(True)
+    yr, (hn, cn) = m(xr, (hr[None], cr[None]))
+    (yr * p["dy"].float().cpu()).sum().backward()
+    return dict(y=yr.detach(), h_T=hn[0].detach(), c_T=cn[0].detach(), dx=xr.grad, dW_ih=m.weight_ih_l0.grad,
+                dW_hh=m.weight_hh_l0.grad, db=m.bias_ih_l0.grad, db_hh=m.bias_hh_l0.grad, dh0=hr.grad, dc0=cr.grad)
+
+
+@pytest.mark.parametrize("name,shape", [("config3", (1024, 256, 1024, 1024)), ("config4", (2048, 16, 2048, 2048)),
+                                        ("config5_layer", (4096, 128, 2048, 2048))])
+def test_full_size_configs_against_cpu_fp32_torch_lstm(name, shape):
+    # The headline configurations and one full layer of the stack at FULL size against torch.nn.LSTM in fp32 on the
+    # CPU: all of y, h_T, c_T (max relative error <= 1e-2) and dx, dW_ih, dW_hh, db, dh0, dc0 (relative L2 <= 1e-2).
+    # The GPU library's nn.LSTM is not involved; the errors are printed.
+    import time
+    T, B, I, H = shape
+    p = problem(T, B, I, H, seed=17)
+    core = make_core(p)
+    y, hy, cy = core.forward(p["x"], p["h0"], p["c0"])
+    got = dict(zip(("dx", "dW_ih", "dW_hh", "db", "dh0", "dc0"), core.backward(p["x"], p["dy"])))
+    got.update(y=y, h_T=hy, c_T=cy)
+    assert core.info("persistent_fwd") == 1 and core.info("persistent_bwd") == 1 and core.info("fallbacks") == 0
+    got = {k: v.float().cpu() for k, v in got.items()}
+    core.close()
+    t0 = time.perf_counter()
+    ref = _cpu_lstm_reference(p)
+    cpu_s = time.perf_counter() - t0
+    errs = {}
+    for k in ("y", "h_T", "c_T"):
+        errs[k] = ((got[k] - ref[k]).abs().max() / ref[k].abs().max()).item()
+    errs["y_last_step"] = ((got["y"][-1] - ref["y"][-1]).abs().max() / ref["y"][-1].abs().max()).item()
+    for k in ("dx", "dW_ih", "dW_hh", "db", "dh0", "dc0"):
+        errs[k] = ((got[k].double() - ref[k].double()).norm() / ref[k].double().norm()).item()
+    errs["db_vs_db_hh"] = ((got["db"].double() - ref["db_hh"].double()).norm() / ref["db_hh"].double().norm()).item()
+    print(f"\n{name} T={T} B={B} I={I} H={H} vs CPU fp32 nn.LSTM ({cpu_s:.1f} s on {torch.get_num_threads()} threads): "
+          + ", ".join(f"{k}={v:.2e}" for k, v in errs.items()))
+    assert max(errs.values()) <= 1e-2, errs
