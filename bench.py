@@ -6,7 +6,11 @@ already resident in HBM (fp16 x / dY, packed fp16 weights); weight packing and p
 before the timed region.  Prints ONE JSON line.
 
   python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload config3|config2|config4|config5|config5_layer]
-                  [--no-cpu-baseline] [--no-parity]
+                  [--no-cpu-baseline] [--no-parity] [--no-others]
+
+Without --workload the line is the headline workload (config 3) and carries, under "other_workloads", short runs of
+the other BASELINE configurations (config 2, config 4, the config-5 stack: 1 warm-up + 3 timed steps each, with their
+parity check).
 """
 import argparse
 import json
@@ -113,6 +117,26 @@ def measured_traffic(workload, phase):
         return None, f"counter summary is from other kernel sources ({data.get('kernel_source_digest')})"
     try:
         return float(data["bytes_per_launch"][workload][phase]), data.get("taken", "")
+    except Exception:
+        return None, "phase not in the counter summary"
+
+
+def measured_counters(workload, phase):
+    """L2 request and LDS activity counters per launch of a phase's kernel from the same committed summary (rocprofv3
+    --pmc TCC_REQ_sum / SQ_LDS_IDX_ACTIVE / GRBM_GUI_ACTIVE and the kernel trace's duration, taken with plain launches:
+    a profiler tool and cooperative launches do not go together).  None unless the summary was taken from exactly
+    the kernel sources that are running now."""
+    import re
+    path = os.path.join(ROOT, "profiles", "hbm_traffic_per_kernel.md")
+    try:
+        text = open(path).read()
+        data = json.loads(re.search(r"```json traffic\n(.*?)```", text, flags=re.S).group(1))
+    except Exception:
+        return None, "no counter summary"
+    if data.get("kernel_source_digest") != kernel_source_digest():
+        return None, f"counter summary is from other kernel sources ({data.get('kernel_source_digest')})"
+    try:
+        return data["counters_per_launch"][workload][phase], data.get("taken", "")
     except Exception:
         return None, "phase not in the counter summary"
 
@@ -280,7 +304,8 @@ def bench_stack(args, device):
                         "peak": PEAK_FP16_TFLOPS, "unit": "TFLOP/s", "frac": round(tf / PEAK_FP16_TFLOPS, 4), "traffic": None},
            "us_per_timestep": {"fwd_rec": round(phases["fwd_rec"] * 1e3 / (T * L), 3),
                                "bwd_rec": round(phases["bwd_rec"] * 1e3 / (T * L), 3)},
-           "loss_scale": stack.last_loss_scale, "device": device, "cpu_baseline": None}
+           "loss_scale": stack.last_loss_scale, "device": device, "cpu_baseline": None,
+           "kernel_source_digest": kernel_source_digest()}
     stack.close()
     torch.cuda.empty_cache()
     if not args.no_parity:
@@ -293,10 +318,13 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=10)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--workload", default="config3", choices=sorted(WORKLOADS) + sorted(STACKS))
+    ap.add_argument("--workload", default=None, choices=sorted(WORKLOADS) + sorted(STACKS))
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-parity", action="store_true")
+    ap.add_argument("--no-others", action="store_true", help="the headline workload only (no other_workloads block)")
     args = ap.parse_args()
+    args.others = args.workload is None and not args.no_others
+    args.workload = args.workload or "config3"
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this build runs on ONE GPU (the recurrence shards over batch; no multi-GPU path is "
               "built) -- rerun with --gpus 1", file=sys.stderr)
@@ -321,6 +349,29 @@ def main():
     if args.workload in STACKS:
         print(json.dumps(bench_stack(args, device)))
         return
+    out = bench_single(args, device)
+    if args.others:
+        # the other BASELINE configurations, briefly: 1 warm-up + 3 timed steps each, parity on the timed tensors
+        others = {}
+        for wl in ("config2", "config4", "config5"):
+            sub = argparse.Namespace(**vars(args))
+            sub.workload, sub.steps, sub.warmup, sub.no_cpu_baseline = wl, 3, 1, True
+            torch.cuda.empty_cache()
+            r = bench_stack(sub, None) if wl in STACKS else bench_single(sub, None)
+            others[wl] = {"workload": r["config"]["workload"], "metric": r["metric"], "value": r["value"],
+                          "ms_per_step": r["ms_per_step"], "steps": 3, "warmup": 1, "mfu": r["mfu"],
+                          "us_per_timestep": r.get("us_per_timestep"),
+                          "phase_ms": r.get("phase_ms_all_layers") or {k["phase"]: k["ms"] for k in r.get("kernels", [])},
+                          "parity": ({"max_err": r["parity"]["max_err"], "ok": r["parity"]["ok"]} if "parity" in r else None)}
+        out["other_workloads"] = others
+    print(json.dumps(out))
+
+
+def bench_single(args, device):
+    """One single-layer workload: fwd (+ bwd) steps timed with hipEvents, per-phase times from the library's own
+    events on the launch stream, roofline of the dominant kernel, parity on the timed tensors."""
+    import torch
+    from flashlstm_poc_amd import LstmCore
     T, B, I, H, backward = WORKLOADS[args.workload]
     p = make_inputs(T, B, I, H)
     core = LstmCore(B, I, H)
@@ -395,24 +446,36 @@ def main():
         "us_per_timestep": {"fwd_rec": round(phase_ms["fwd_rec"] * 1e3 / T, 3),
                             **({"bwd_rec": round(phase_ms["bwd_rec"] * 1e3 / T, 3)} if backward else {})},
     }
-    # What the recurrence moves between workgroups each step: every workgroup (16 or 32 batch rows x one slice of hidden
-    # units) fetches the whole h_{t-1} (forward) or dG_{t+1} (backward) of its rows from the L2, and passes its
-    # fp32 partial sums (4 waves, written once and read once) through LDS.
+    # What the recurrence moves between workgroups each step.  Measured: requests to the L2 (TCC_REQ, each at most one
+    # 128-byte line) and the cycles the LDS address unit was busy (SQ_LDS_IDX_ACTIVE, summed over the CUs), from the
+    # committed counter summary -- taken with plain launches, 5 % slower than the cooperative launches timed here --
+    # divided by that profile's own kernel duration.  Beside them the byte model: every workgroup (16 or 32 batch rows x
+    # one slice of hidden units) fetches the whole h_{t-1} (forward) or dG_{t+1} (backward) of its rows from the L2.
     block = 16 * core.info("row_tiles")   # batch rows per workgroup
     Hp, rows = core.info("hidden_padded"), block * ((B + block - 1) // block)
     xch = {}
-    for d, k_cols, gate_cols in (("fwd", Hp, 4), ("bwd", 4 * Hp, 1)) if backward else (("fwd", Hp, 4),):
+    for d, k_cols in (("fwd", Hp), ("bwd", 4 * Hp)) if backward else (("fwd", Hp),):
         us = phase_ms[d + "_rec"] * 1e3 / T
         slices = Hp // core.info("slice_" + d)
         l2_bytes = rows * slices * k_cols * 2
-        lds_bytes = 2 * 4 * rows * slices * core.info("slice_" + d) * gate_cols * 4
         if d == "bwd" and core.info("bwd_two_d") == 1:
-            # 256 workgroups, each fetches an eighth of dG_{t+1} of every row; the fp32 partial products
-            # [rows][64 columns] of each go through LDS (4 waves) and, 7/8 of them, once through the L2 to the slice's peers
+            # 256 workgroups, each fetches an eighth of dG_{t+1} of every row and passes 7/8 of its fp32 partial
+            # products [rows][64 columns] once through the L2 to the slice's peers
             l2_bytes = rows * 256 * (k_cols // 8) * 2 + 2 * rows * 256 * 64 * 4
-            lds_bytes = 2 * 4 * rows * 256 * 64 * 4
-        xch[d] = {"l2_fetch_bytes_per_step": l2_bytes, "l2_fetch_gb_per_s": round(l2_bytes / us / 1e3, 1),
-                  "lds_bytes_per_step": lds_bytes, "lds_gb_per_s": round(lds_bytes / us / 1e3, 1)}
+        entry = {"model_l2_fetch_bytes_per_step": l2_bytes, "model_l2_fetch_gb_per_s": round(l2_bytes / us / 1e3, 1)}
+        c, note = measured_counters(args.workload, d + "_rec")
+        if c:
+            cus = device["compute_units"] if device else 256
+            entry.update({"measured": {
+                "l2_requests_per_step": round(c["TCC_REQ"] / T, 1),
+                "l2_gb_per_s_at_128B_per_request": round(c["TCC_REQ"] * 128 / (c["ms"] * 1e-3) / 1e9, 1),
+                "lds_busy_cycles_per_step_and_cu": round(c["SQ_LDS_IDX_ACTIVE"] / T / cus, 1),
+                "lds_busy_fraction": round(c["SQ_LDS_IDX_ACTIVE"] / cus / (c["GRBM_GUI_ACTIVE"] / 8), 4),
+                "profile_launch_ms": c["ms"], "launches": "plain (profiler attached)", "source": note}})
+        else:
+            entry["measured"] = None
+            entry["measured_note"] = note
+        xch[d] = entry
     out["exchange_per_step"] = xch
     core.close()
     out["kernel_source_digest"] = kernel_source_digest()
@@ -421,7 +484,7 @@ def main():
     last.clear()
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(B, I, H, backward)
-    print(json.dumps(out))
+    return out
 
 
 if __name__ == "__main__":

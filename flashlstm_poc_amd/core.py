@@ -58,8 +58,23 @@ def load_library() -> ctypes.CDLL:
     lib.flstm_core_tune.restype = i32
     lib.flstm_core_tuned_ms.argtypes = [vp, sz, c.c_char_p]
     lib.flstm_core_tuned_ms.restype = c.c_double
+    ip = c.POINTER(i32)
+    lib.flstm_core_get_tuned.argtypes = [vp, sz, c.POINTER(sz), ip, ip, ip, ip, ip, ip]
+    lib.flstm_core_get_tuned.restype = i32
+    lib.flstm_core_set_tuned.argtypes = [vp, sz, i32, i32, i32, i32, i32, i32]
+    lib.flstm_core_set_tuned.restype = i32
     lib.flstm_core_backward.argtypes = [vp, sz, vp, i32, vp, i32, vp, vp, i32, c.c_float, vp, i32,
                                         vp, vp, vp, vp, vp, vp, vp]
+    # the passes fed in ranges of steps
+    lib.flstm_core_forward_begin.argtypes = [vp, sz, vp, i32, vp, vp, i32, vp]
+    lib.flstm_core_forward_steps.argtypes = [vp, sz, sz, vp]
+    lib.flstm_core_forward_end.argtypes = [vp, vp, vp, i32, i32, vp]
+    lib.flstm_core_backward_begin.argtypes = [vp, sz, vp, i32, vp, vp, i32, c.c_float, vp, i32, vp]
+    lib.flstm_core_backward_steps.argtypes = [vp, sz, sz, vp]
+    lib.flstm_core_backward_end.argtypes = [vp, vp, i32, vp, vp, vp, vp, vp, vp, vp]
+    for name in ("flstm_core_forward_begin", "flstm_core_forward_steps", "flstm_core_forward_end",
+                 "flstm_core_backward_begin", "flstm_core_backward_steps", "flstm_core_backward_end"):
+        getattr(lib, name).restype = i32
     lib.flstm_core_cache_ptr.argtypes = [vp, i32, c.POINTER(vp), c.POINTER(sz)]
     lib.flstm_core_last_ms.argtypes = [vp, c.c_char_p]
     lib.flstm_core_last_ms.restype = c.c_double
@@ -129,10 +144,40 @@ class LstmCore:
         if rc != 0:
             raise RuntimeError(f"flstm_core_tune failed with status {rc}")
         out = {k: self.info("tuned_" + k) for k in ("T", "row_tiles_fwd", "row_tiles_bwd", "stepwise_fwd", "stepwise_bwd",
-                                                    "dw_splits")}
+                                                    "dw_splits", "bwd_two_d")}
         for ph in ("fwd_rec", "bwd_rec", "bwd_dw"):
             out[ph + "_ms"] = float(self.lib.flstm_core_tuned_ms(self._h, int(seq_len), ph.encode()))
         return out
+
+    _TUNED_KEYS = ("row_tiles_fwd", "row_tiles_bwd", "stepwise_fwd", "stepwise_bwd", "dw_splits", "bwd_two_d")
+
+    def tuned_table(self) -> list:
+        """The plan's tuned entries (flstm_core_get_tuned) as a list of dicts, JSON-serialisable: keep it between
+        processes and hand it to set_tuned_table of a plan of the same sizes."""
+        import ctypes as c
+        rows = []
+        for i in range(self.info("tuned_entries")):
+            T = c.c_size_t()
+            v = [c.c_int32() for _ in self._TUNED_KEYS]
+            rc = self.lib.flstm_core_get_tuned(self._h, i, c.byref(T), *[c.byref(x) for x in v])
+            if rc != 0:
+                raise RuntimeError(f"flstm_core_get_tuned failed with status {rc}")
+            rows.append({"T": int(T.value), "B": self.B, "I": self.I, "H": self.H,
+                         **{k: int(x.value) for k, x in zip(self._TUNED_KEYS, v)}})
+        return rows
+
+    def set_tuned_table(self, rows) -> int:
+        """Writes tuned entries (as tuned_table returns them) into the plan; rows of other sizes are skipped.  Returns
+        the number of entries taken."""
+        taken = 0
+        for r in rows:
+            if (r.get("B"), r.get("I"), r.get("H")) != (self.B, self.I, self.H):
+                continue
+            rc = self.lib.flstm_core_set_tuned(self._h, int(r["T"]), *[int(r[k]) for k in self._TUNED_KEYS])
+            if rc != 0:
+                raise RuntimeError(f"flstm_core_set_tuned failed with status {rc}")
+            taken += 1
+        return taken
 
     def pack(self, w_ih, w_hh, b_ih=None, b_hh=None) -> None:
         import torch

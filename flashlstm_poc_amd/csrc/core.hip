@@ -103,10 +103,11 @@ struct flstm_core_plan {
     // Tuned launch choices per sequence length (flstm_core_tune): 16- or 32-row blocks and persistent or step-wise
     // launches per direction, split-K count of the weight-gradient GEMM.  eff_* hold the entry in force for the
     // sequence length of the current pass (0 = no tuned value: the rules of thumb decide); explicit options win.
-    struct Tuned { size_t T; int mt_f, mt_b, step_f, step_b, dw_splits; float ms_f, ms_b, ms_dw; };
+    struct Tuned { size_t T; int mt_f, mt_b, step_f, step_b, dw_splits, two_d; float ms_f, ms_b, ms_dw; };   // two_d: -1 = not tuned, else the bwd_two_d option
     std::vector<Tuned> tuned;
     int opt_mt_f = 0, opt_mt_b = 0;
-    int eff_mt_f = 0, eff_mt_b = 0, eff_step_f = 0, eff_step_b = 0, eff_dw = 0;
+    int eff_mt_f = 0, eff_mt_b = 0, eff_step_f = 0, eff_step_b = 0, eff_dw = 0, eff_two_d = -1;
+    bool two_d_explicit = false;   // option "bwd_two_d" (or its environment variable) was given: a tuned value does not replace it
     size_t eff_T = 0;
     int opt_cooperative = 1;
     StepGraphCache graphs_f, graphs_b;   // captured step-wise launches (only used where the persistent kernels are not)
@@ -147,7 +148,8 @@ void replan(flstm_core_plan* p) {
     p->Lf = plan_rec_fwd(p->d.B, p->d.Hp, p->num_cus, p->opt_stepwise || p->hold_fwd > 0 || p->eff_step_f || p->refused_fwd,
                          p->opt_mt_f ? p->opt_mt_f : p->eff_mt_f, p->opt_waves_f);
     p->Lb = plan_rec_bwd(p->d.B, p->d.Hp, p->num_cus, p->opt_stepwise || p->hold_bwd > 0 || p->eff_step_b || p->refused_bwd,
-                         p->opt_mt_b ? p->opt_mt_b : p->eff_mt_b, p->opt_two_d);
+                         p->opt_mt_b ? p->opt_mt_b : p->eff_mt_b,
+                         (!p->two_d_explicit && p->eff_two_d >= 0) ? p->eff_two_d : p->opt_two_d);
     p->Lf.cooperative = p->Lb.cooperative = p->opt_cooperative;
     p->ks_f = rec_fwd_ks(p->Lf, p->d.Hp);
     p->ks_b = rec_bwd_ks(p->Lb, p->d.Hp);
@@ -163,11 +165,11 @@ void use_tuned(flstm_core_plan* p, size_t T) {
         if (dist <= best_d && (!best || dist < best_d)) { best = &t; best_d = dist; }
     }
     const int mt_f = best ? best->mt_f : 0, mt_b = best ? best->mt_b : 0, sf = best ? best->step_f : 0,
-              sb = best ? best->step_b : 0;
+              sb = best ? best->step_b : 0, td = best ? best->two_d : -1;
     p->eff_dw = best ? best->dw_splits : 0;
     p->eff_T = best ? best->T : 0;
-    if (mt_f != p->eff_mt_f || mt_b != p->eff_mt_b || sf != p->eff_step_f || sb != p->eff_step_b) {
-        p->eff_mt_f = mt_f; p->eff_mt_b = mt_b; p->eff_step_f = sf; p->eff_step_b = sb;
+    if (mt_f != p->eff_mt_f || mt_b != p->eff_mt_b || sf != p->eff_step_f || sb != p->eff_step_b || td != p->eff_two_d) {
+        p->eff_mt_f = mt_f; p->eff_mt_b = mt_b; p->eff_step_f = sf; p->eff_step_b = sb; p->eff_two_d = td;
         replan(p);
     }
 }
@@ -259,7 +261,7 @@ extern "C" int flstm_core_create(size_t batch, size_t input_size, size_t hidden_
         p->opt_cooperative = profiled ? 0 : 1;
         if (const char* v = getenv("FLASHLSTM_COOPERATIVE_LAUNCH")) p->opt_cooperative = atoi(v) != 0;
         if (const char* v = getenv("FLASHLSTM_STEP_GRAPHS")) p->opt_graphs = atoi(v) != 0;
-        if (const char* v = getenv("FLASHLSTM_BWD_TWO_D")) p->opt_two_d = atoi(v) < 0 ? 0 : (atoi(v) > 2 ? 2 : atoi(v));
+        if (const char* v = getenv("FLASHLSTM_BWD_TWO_D")) { p->opt_two_d = atoi(v) < 0 ? 0 : (atoi(v) > 2 ? 2 : atoi(v)); p->two_d_explicit = true; }
         if (const char* v = getenv("FLASHLSTM_WAVES_FWD")) p->opt_waves_f = (atoi(v) == 4 || atoi(v) == 8) ? atoi(v) : 0;
     }
     replan(p);
@@ -307,7 +309,7 @@ extern "C" int flstm_core_set_option(flstm_core_plan* p, const char* name, long 
     if (!strcmp(name, "clear_tuned")) { p->tuned.clear(); use_tuned(p, 1); return 0; }
     if (!strcmp(name, "cooperative")) { p->opt_cooperative = value != 0; replan(p); return 0; }
     if (!strcmp(name, "step_graphs")) { p->opt_graphs = value != 0; return 0; }
-    if (!strcmp(name, "bwd_two_d")) { if (value < 0 || value > 2) return FLSTM_E_INVALID; p->opt_two_d = int(value); replan(p); return 0; }
+    if (!strcmp(name, "bwd_two_d")) { if (value < 0 || value > 2) return FLSTM_E_INVALID; p->opt_two_d = int(value); p->two_d_explicit = true; replan(p); return 0; }
     if (!strcmp(name, "waves_fwd")) {
         // wavefronts per workgroup of the forward recurrence: the weight fragments are packed for it, so a change
         // un-packs them
@@ -348,6 +350,7 @@ extern "C" long flstm_core_get_info(const flstm_core_plan* p, const char* name) 
     if (!strcmp(name, "tuned_stepwise_fwd")) return p->eff_step_f;
     if (!strcmp(name, "tuned_stepwise_bwd")) return p->eff_step_b;
     if (!strcmp(name, "tuned_dw_splits")) return p->eff_dw;
+    if (!strcmp(name, "tuned_bwd_two_d")) return p->eff_two_d;
     if (!strcmp(name, "device_bytes")) {
         size_t sum = 0;
         for (const DevBuf* b : {&p->wih_p, &p->wih_t, &p->wfrag_f, &p->wfrag_b, &p->wfrag_b2, &p->part_b, &p->bias_p, &p->X16, &p->G, &p->Y, &p->C,
@@ -1045,7 +1048,8 @@ extern "C" int flstm_core_tune(flstm_core_plan* p, size_t T, int repeats, int tr
     hipStream_t s = static_cast<hipStream_t>(stream);
     const Dims& d = p->d;
     const size_t TB = T * size_t(d.B);
-    // synthetic inputs: zeros (the kernels' time does not depend on the values)
+    // synthetic inputs: varied values (the matrix cores draw more power on them than on constants, and the GEMMs run
+    // about a fifth slower: candidates are compared under the clock they will run at)
     DevBuf x, dy, dwi, dwh;
     int rc = 0;
     auto fail = [&](int code) { x.release(); dy.release(); dwi.release(); dwh.release(); return code; };
@@ -1053,18 +1057,20 @@ extern "C" int flstm_core_tune(flstm_core_plan* p, size_t T, int repeats, int tr
         dwi.reserve(size_t(4) * d.H * d.I * sizeof(float)) != hipSuccess ||
         dwh.reserve(size_t(4) * d.H * d.H * sizeof(float)) != hipSuccess)
         return fail(int(hipErrorOutOfMemory));
-    if (fill_zero(x.p, TB * d.I * sizeof(half_t), s) != hipSuccess || fill_zero(dy.p, TB * d.H * sizeof(half_t), s) != hipSuccess)
+    if (fill_noise(x.as<half_t>(), TB * d.I, 0x1234567u, 1.7f, s) != hipSuccess ||
+        fill_noise(dy.as<half_t>(), TB * d.H, 0x89ABCDEu, 1.7f, s) != hipSuccess)
         return fail(int(hipErrorUnknown));
     // the plan's explicit options and tuned state are set aside while candidates run
     const int keep_step = p->opt_stepwise, keep_mtf = p->opt_mt_f, keep_mtb = p->opt_mt_b, keep_dw = p->opt_dw_splits,
-              keep_acc = p->opt_accumulate;
+              keep_acc = p->opt_accumulate, keep_two_d = p->opt_two_d;
+    const bool keep_two_d_explicit = p->two_d_explicit;
     const bool keep_cache = p->have_cache;
     const std::vector<flstm_core_plan::Tuned> keep_tuned = p->tuned;
     p->tuned.clear();
     p->opt_accumulate = 0;
     auto restore = [&]() {
         p->opt_stepwise = keep_step; p->opt_mt_f = keep_mtf; p->opt_mt_b = keep_mtb; p->opt_dw_splits = keep_dw;
-        p->opt_accumulate = keep_acc;
+        p->opt_accumulate = keep_acc; p->opt_two_d = keep_two_d; p->two_d_explicit = keep_two_d_explicit;
         p->tuned = keep_tuned;
         p->have_cache = false;   // the caches now hold the synthetic sequence
         (void)keep_cache;
@@ -1072,7 +1078,7 @@ extern "C" int flstm_core_tune(flstm_core_plan* p, size_t T, int repeats, int tr
         replan(p);
     };
     flstm_core_plan::Tuned best{};
-    best.T = T; best.ms_f = best.ms_b = best.ms_dw = -1.f;
+    best.T = T; best.ms_f = best.ms_b = best.ms_dw = -1.f; best.two_d = -1;
     auto run = [&](float& f_ms, float& b_ms, float& dw_ms) -> int {
         f_ms = b_ms = dw_ms = 1e30f;
         for (int r = 0; r <= repeats; ++r) {   // first pass is a warm-up
@@ -1104,6 +1110,27 @@ extern "C" int flstm_core_tune(flstm_core_plan* p, size_t T, int repeats, int tr
             if (b_is && (best.ms_b < 0 || b_ms < best.ms_b)) { best.ms_b = b_ms; best.mt_b = mt; best.step_b = step; }
         }
     }
+    // 1b) the layout of the backward recurrence where the two-way split can run (2048 and 1024 hidden units): off /
+    // where the rule of thumb has it / wherever it fits, with the row-block height the rule picks for each
+    if (rec_bwd_two_d_possible(d.Hp, p->num_cus) && !keep_two_d_explicit) {
+        p->opt_stepwise = 0; p->opt_mt_f = best.mt_f; p->opt_mt_b = 0;
+        p->two_d_explicit = true;
+        float best_td_ms = -1.f;
+        for (int td = 0; td <= 2; ++td) {
+            p->opt_two_d = td;
+            replan(p);
+            if (!p->Lb.persistent) continue;
+            if (td == 2 && !p->Lb.two_d) continue;   // (nothing new: the split does not fit this batch)
+            float f_ms, b_ms, dw_ms;
+            rc = run(f_ms, b_ms, dw_ms);
+            if (rc) { restore(); return fail(rc); }
+            if (best_td_ms < 0 || b_ms < best_td_ms) { best_td_ms = b_ms; best.two_d = td; }
+        }
+        // (the entry keeps the better of: the best row-block height under the plan's own setting, the best setting)
+        if (best_td_ms >= 0 && best_td_ms < best.ms_b) { best.ms_b = best_td_ms; best.mt_b = 0; best.step_b = 0; }
+        else best.two_d = -1;
+        p->opt_two_d = keep_two_d; p->two_d_explicit = keep_two_d_explicit;
+    }
     // 2) split-K count of the weight-gradient GEMM around what the schedule model picks
     p->opt_stepwise = best.step_f && best.step_b; p->opt_mt_f = best.mt_f; p->opt_mt_b = best.mt_b;
     replan(p);
@@ -1127,6 +1154,36 @@ extern "C" int flstm_core_tune(flstm_core_plan* p, size_t T, int repeats, int tr
     p->tuned.push_back(best);
     use_tuned(p, T);
     return fail(0);
+}
+
+// A tuned entry written into / read out of a plan: what a tuning run found, kept by the caller between processes.
+extern "C" int flstm_core_set_tuned(flstm_core_plan* p, size_t T, int row_tiles_fwd, int row_tiles_bwd, int stepwise_fwd,
+                                    int stepwise_bwd, int dw_splits, int bwd_two_d) {
+    if (!p || T == 0 || T > (size_t(1) << 24) || row_tiles_fwd < 0 || row_tiles_fwd > 2 || row_tiles_bwd < 0 ||
+        row_tiles_bwd > 2 || dw_splits < 0 || dw_splits > 64 || bwd_two_d < -1 || bwd_two_d > 2)
+        return FLSTM_E_INVALID;
+    flstm_core_plan::Tuned t{};
+    t.T = T; t.mt_f = row_tiles_fwd; t.mt_b = row_tiles_bwd; t.step_f = stepwise_fwd != 0; t.step_b = stepwise_bwd != 0;
+    t.dw_splits = dw_splits; t.two_d = bwd_two_d; t.ms_f = t.ms_b = t.ms_dw = -1.f;
+    for (auto it = p->tuned.begin(); it != p->tuned.end();)
+        it = (it->T == T) ? p->tuned.erase(it) : it + 1;
+    p->tuned.push_back(t);
+    use_tuned(p, T);
+    return 0;
+}
+
+extern "C" int flstm_core_get_tuned(const flstm_core_plan* p, size_t index, size_t* T, int* row_tiles_fwd, int* row_tiles_bwd,
+                                    int* stepwise_fwd, int* stepwise_bwd, int* dw_splits, int* bwd_two_d) {
+    if (!p || index >= p->tuned.size()) return FLSTM_E_INVALID;
+    const auto& t = p->tuned[index];
+    if (T) *T = t.T;
+    if (row_tiles_fwd) *row_tiles_fwd = t.mt_f;
+    if (row_tiles_bwd) *row_tiles_bwd = t.mt_b;
+    if (stepwise_fwd) *stepwise_fwd = t.step_f;
+    if (stepwise_bwd) *stepwise_bwd = t.step_b;
+    if (dw_splits) *dw_splits = t.dw_splits;
+    if (bwd_two_d) *bwd_two_d = t.two_d;
+    return 0;
 }
 
 extern "C" double flstm_core_tuned_ms(const flstm_core_plan* p, size_t T, const char* phase) {

@@ -68,6 +68,8 @@ hipError_t reduce_partials(const float* partial, int splits, size_t per, int row
 hipError_t checksum_add(const void* p, size_t bytes, u64 salt, u64* out, hipStream_t s);
 
 hipError_t fill_zero(void* p, size_t bytes, hipStream_t s);
+// fp16 values spread over (-amp, amp) from a hash of the index (operands for timing runs)
+hipError_t fill_noise(half_t* p, size_t n, unsigned seed, float amp, hipStream_t s);
 // Fills a buffer (multiple of 4 bytes) with one 32-bit pattern; a kernel, so it may be captured in a graph.
 hipError_t fill_words(void* p, size_t bytes, unsigned value, hipStream_t s);
 

@@ -401,4 +401,23 @@ hipError_t fill_words(void* p, size_t bytes, unsigned value, hipStream_t s) {
 
 hipError_t fill_zero(void* p, size_t bytes, hipStream_t s) { return fill_words(p, bytes, 0u, s); }
 
+// n fp16 values spread over (-amp, amp) from a hash of the index: operands for timing runs (the matrix cores draw
+// more power, and run slower, on varied operands than on constant ones)
+__global__ void fill_noise_kernel(half_t* p, size_t n, unsigned seed, float amp) {
+    const size_t stride = size_t(gridDim.x) * kT;
+    for (size_t i = size_t(blockIdx.x) * kT + threadIdx.x; i < n; i += stride) {
+        unsigned h = unsigned(i) * 0x9E3779B1u + unsigned(i >> 32) * 0x85EBCA77u + seed;
+        h ^= h >> 15; h *= 0x2C1B3C6Du; h ^= h >> 12; h *= 0x297A2D39u; h ^= h >> 15;
+        p[i] = (half_t)(amp * (float(h >> 8) * (2.f / 16777216.f) - 1.f));
+    }
+}
+
+hipError_t fill_noise(half_t* p, size_t n, unsigned seed, float amp, hipStream_t s) {
+    if (n == 0) return hipSuccess;
+    int blocks = grid_for(n);
+    if (blocks > 4096) blocks = 4096;
+    hipLaunchKernelGGL(fill_noise_kernel, dim3(blocks), dim3(kT), 0, s, p, n, seed, amp);
+    return hipGetLastError();
+}
+
 }  // namespace flstm_hip

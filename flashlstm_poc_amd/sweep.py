@@ -13,6 +13,7 @@ plan.  Inputs are synthetic (seeded); every tensor is resident on the GPU before
 import argparse
 import csv
 import json
+import os
 import statistics
 import sys
 from typing import Dict, List, Optional, Sequence
@@ -78,7 +79,10 @@ def check_parity(core, p, I: int, H: int) -> Dict[str, float]:
 
 
 def sweep(B: int, I: int, H: int, seq_lens: Sequence[int], *, warmup: int = 3, repeats: int = 10, seed: int = 2025,
-          baseline: bool = True, check: bool = False, tune: bool = False, try_stepwise: bool = False) -> List[Dict]:
+          baseline: bool = True, check: bool = False, tune: bool = False, try_stepwise: bool = False,
+          tuned_table: Optional[List[Dict]] = None) -> List[Dict]:
+    """tuned_table: tuned entries (LstmCore.tuned_table) to start every plan from; with `tune` the entries found are
+    appended to it in place, so the caller can save the table for the next process."""
     import torch
     from . import LstmCore
     rows = []
@@ -87,9 +91,14 @@ def sweep(B: int, I: int, H: int, seq_lens: Sequence[int], *, warmup: int = 3, r
         core = LstmCore(B, I, H)
         core.pack(p["w_ih"], p["w_hh"], p["b_ih"], p["b_hh"])
         row: Dict = {"T": T, "B": B, "I": I, "H": H}
+        if tuned_table:
+            row["tuned_entries_loaded"] = core.set_tuned_table(tuned_table)
         if tune:
             row["untuned"] = {"row_tiles_fwd": core.info("row_tiles_fwd"), "row_tiles_bwd": core.info("row_tiles_bwd")}
             row["tuned"] = core.tune(T, repeats=3, try_stepwise=try_stepwise)
+            if tuned_table is not None:
+                tuned_table[:] = [r for r in tuned_table if (r["T"], r["B"], r["I"], r["H"]) != (T, B, I, H)]
+                tuned_table.extend(r for r in core.tuned_table() if r["T"] == T)
         if check:
             row["parity"] = check_parity(core, p, I, H)
             row["parity_ok"] = all(v <= 1e-2 for v in row["parity"].values())
@@ -190,6 +199,9 @@ def main(argv: Optional[Sequence[str]] = None) -> int:
     ap.add_argument("--tune", action="store_true", help="run the library's tuner for every length first (choices are "
                     "cached in the plan and printed)")
     ap.add_argument("--tune-stepwise", action="store_true", help="with --tune: also time one launch per step")
+    ap.add_argument("--tuned-table", type=str, default=None, help="JSON file of tuned entries: read (if it exists) "
+                    "before the sweep, so that a fresh process starts tuned, and with --tune written back with what "
+                    "the tuner found")
     ap.add_argument("--dw-splits-table", action="store_true", help="print the weight-gradient time for every "
                     "split-K count instead of sweeping")
     ap.add_argument("--side-stream", action="store_true", help="run on a stream of its own instead of the default "
@@ -216,9 +228,18 @@ def main(argv: Optional[Sequence[str]] = None) -> int:
             print(f"T={r['T']}: " + "  ".join(f"{k}:{v:.3f}ms" for k, v in r["dw_ms_by_splits"].items()) +
                   f"  best={r['best']}  automatic/best={r['automatic_over_best']:.3f}")
     else:
+        table = None
+        if args.tuned_table:
+            table = []
+            if os.path.exists(args.tuned_table):
+                with open(args.tuned_table) as f:
+                    table = json.load(f)
         results = sweep(args.batch, args.input_size, args.hidden_size, lens, warmup=args.warmup, repeats=args.repeats,
                         seed=args.seed, baseline=not args.no_baseline, check=args.check, tune=args.tune,
-                        try_stepwise=args.tune_stepwise)
+                        try_stepwise=args.tune_stepwise, tuned_table=table)
+        if args.tuned_table and args.tune:
+            with open(args.tuned_table, "w") as f:
+                json.dump(table, f, indent=1)
         if args.csv:
             keys = [k for k in results[0] if k not in ("parity", "tuned", "untuned")]
             with open(args.csv, "w", newline="") as f:

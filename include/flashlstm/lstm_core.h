@@ -156,17 +156,31 @@ double flstm_core_last_ms(const flstm_core_plan* plan, const char* phase);
 
 /* Tuner (the counterpart of the reference's projection-chunk tuner, src/tune_projchunksz.cu:56-226, and of the
  * autotune loop of python/benchmark_lstm.py:203-301, for the launch choices that matter in this library).  For
- * sequence length seq_len it times, on synthetic data in the plan's own buffers, `repeats` passes of every
- * candidate: 16- or 32-row blocks for each recurrence (where both fit), persistent or -- with try_stepwise -- one
- * launch per step, and the split-K count of the weight-gradient GEMM around the rule of thumb; the fastest choice
+ * sequence length seq_len it times, on synthetic data of varied values (the matrix cores run slower on those than
+ * on constants) in the plan's own buffers, `repeats` passes of every candidate: 16- or 32-row blocks for each
+ * recurrence (where both fit), persistent or -- with try_stepwise -- one launch per step, the layout of the
+ * backward recurrence where the two-way split can run (option "bwd_two_d" 0 / 1 / 2, unless that option was set
+ * explicitly), and the split-K count of the weight-gradient GEMM around the rule of thumb; the fastest choice
  * per phase is cached in the plan and used by every later pass whose length is within a factor of two of a tuned
  * one (explicit options "stepwise", "row_tiles_fwd", "row_tiles_bwd", "dw_splits" still win; option "clear_tuned"
  * forgets everything).  Read back with flstm_core_get_info: "tuned_entries", and for the entry in force for the
  * last pass "tuned_T", "tuned_row_tiles_fwd", "tuned_row_tiles_bwd", "tuned_stepwise_fwd", "tuned_stepwise_bwd",
- * "tuned_dw_splits" (0 = rule of thumb); flstm_core_tuned_ms gives the best time found per phase ("fwd_rec",
- * "bwd_rec", "bwd_dw").  The plan's forward cache is invalidated.  Allocates temporary device buffers. */
+ * "tuned_dw_splits" (0 = rule of thumb), "tuned_bwd_two_d" (-1 = not tuned); flstm_core_tuned_ms gives the best time
+ * found per phase ("fwd_rec", "bwd_rec", "bwd_dw").  The plan's forward cache is invalidated.  Allocates temporary
+ * device buffers. */
 int flstm_core_tune(flstm_core_plan* plan, size_t seq_len, int repeats, int try_stepwise, void* stream);
 double flstm_core_tuned_ms(const flstm_core_plan* plan, size_t seq_len, const char* phase);
+
+/* The tuned entries of a plan, read out and written back: what a tuning run found can be kept by the caller (the
+ * reference's tuner prints its table for exactly that reuse, src/tune_projchunksz.cu:200-226) and a fresh process
+ * starts tuned.  get: entry `index` of flstm_core_get_info(plan, "tuned_entries"); any output pointer may be null.
+ * set: replaces the entry of that sequence length; row_tiles 0 / 1 / 2 (0 = rule of thumb), dw_splits 0..64
+ * (0 = rule of thumb), bwd_two_d -1 (not tuned) / 0 / 1 / 2.  Values that do not fit the plan's sizes are ignored by
+ * the planner exactly as the corresponding options are. */
+int flstm_core_get_tuned(const flstm_core_plan* plan, size_t index, size_t* seq_len, int* row_tiles_fwd, int* row_tiles_bwd,
+                         int* stepwise_fwd, int* stepwise_bwd, int* dw_splits, int* bwd_two_d);
+int flstm_core_set_tuned(flstm_core_plan* plan, size_t seq_len, int row_tiles_fwd, int row_tiles_bwd, int stepwise_fwd,
+                         int stepwise_bwd, int dw_splits, int bwd_two_d);
 
 /* The fp16 x fp16 -> fp32-accumulate MFMA GEMMs the passes are built from, callable on their own (the counterpart
  * of flstm::GemmTN / GemmNN / GemmNT, reference flashlstm_v2/src/gemm.h:8-51; device pointers, work is enqueued on

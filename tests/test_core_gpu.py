@@ -444,3 +444,51 @@ def test_error_codes():
     with pytest.raises(ValueError):
         core.forward(torch.zeros(4, 3, 3, device="cuda", dtype=torch.float16))
     core.close()
+
+
+@pytest.mark.parametrize("shape", [(9, 40, 20, 96), (6, 33, 7, 9), (12, 300, 64, 256), (5, 70, 65, 1000), (8, 520, 32, 512)])
+def test_eight_wave_forward_kernel_on_ragged_shapes_ranges_and_single_steps(shape):
+    # The forward kernel with eight waves per workgroup and two interleaved row tiles (option "waves_fwd" = 8: the plan
+    # picks it by itself only where every workgroup has one 32-row block) on shapes it would not be chosen for --
+    # ragged batches and hidden sizes, batches of several row blocks per workgroup -- against the oracle, persistent,
+    # one launch per step, and fed in ranges of steps; its weights are packed for eight waves, so the option un-packs.
+    from flashlstm_poc_amd import LstmCore, load_library
+    p = make_problem(*shape, seed=77)
+    T, B, I, H = shape
+    ref, _ = oracle_reference(p)
+    core = LstmCore(B, I, H)
+    core.pack(*(p[k].cuda() for k in ("w_ih", "w_hh", "b_ih", "b_hh")))
+    core.set_option("waves_fwd", 8)
+    assert core.info("waves_fwd") == 8 and core.info("row_tiles_fwd") == 2
+    x, h0, c0 = p["x"].cuda().half(), p["h0"].cuda().half(), p["c0"].cuda().half()
+    with pytest.raises(RuntimeError):
+        core.forward(x, h0, c0)          # the weight fragments were packed for four waves
+    core.pack(*(p[k].cuda() for k in ("w_ih", "w_hh", "b_ih", "b_hh")))
+    got, info = run_core(p, core=core)
+    assert info["persistent_fwd"] == 1 and info["fallbacks"] == 0
+    check_against(ref, got, label=f"eight waves {shape}")
+    y_p = torch.from_numpy(got["y"])
+    got_s, info_s = run_core(p, core=core, stepwise=True)
+    assert info_s["persistent_fwd"] == 0
+    assert np.array_equal(got_s["y"], got["y"]) and np.array_equal(got_s["cn"], got["cn"])   # same kernel, one step per launch
+    core.set_option("stepwise", 0)
+    # ranges of steps through the C ABI: [0, a), [a, b), [b, T)
+    lib = load_library()
+    s = torch.cuda.current_stream().cuda_stream
+    hy = torch.empty(B, H, device="cuda", dtype=torch.float16); cy = torch.empty_like(hy)
+    assert lib.flstm_core_forward_begin(core._h, T, x.data_ptr(), 1, h0.data_ptr(), c0.data_ptr(), 1, s) == 0
+    cuts = sorted({0, max(1, T // 3), max(2, (2 * T) // 3), T})
+    for a, b in zip(cuts[:-1], cuts[1:]):
+        assert lib.flstm_core_forward_steps(core._h, a, b - a, s) == 0
+    assert lib.flstm_core_forward_end(core._h, hy.data_ptr(), cy.data_ptr(), 1, 1, s) == 0
+    torch.cuda.synchronize()
+    assert np.array_equal(to_np(hy), got["hn"]) and np.array_equal(to_np(cy), got["cn"])
+    core.close()
+
+
+def test_eight_wave_forward_kernel_is_the_rule_where_every_workgroup_has_one_32_row_block():
+    from flashlstm_poc_amd import LstmCore
+    for (B, H, want) in ((256, 1024, 8), (128, 1024, 4), (512, 1024, 4), (512, 512, 8), (256, 2048, 4), (160, 768, 8)):
+        core = LstmCore(B, 64, H)
+        assert core.info("waves_fwd") == want, (B, H, core.info("waves_fwd"))
+        core.close()

@@ -71,3 +71,57 @@ def test_sweep_with_tuning_prints_the_choices(capsys):
                      "--repeats", "2", "--tune", "--no-baseline"])
     assert rc == 0
     assert "tuned: rows/block" in capsys.readouterr().out
+
+
+def test_tuned_table_survives_the_process_through_a_file(tmp_path):
+    # What the tuner found is written to a JSON file and read into a FRESH plan (flstm_core_get_tuned /
+    # flstm_core_set_tuned): the new plan starts with the same choices in force, without tuning.
+    import json
+    from flashlstm_poc_amd import LstmCore, sweep
+    B, I, H, T = 16, 128, 256, 48
+    path = tmp_path / "tuned.json"
+    rc = sweep.main(["--batch", str(B), "--input-size", str(I), "--hidden-size", str(H), "--seq-lens", str(T), "--warmup", "1",
+                     "--repeats", "2", "--tune", "--no-baseline", "--tuned-table", str(path)])
+    assert rc == 0
+    table = json.loads(path.read_text())
+    assert len(table) == 1 and table[0]["T"] == T and (table[0]["B"], table[0]["I"], table[0]["H"]) == (B, I, H)
+    assert table[0]["row_tiles_fwd"] in (1, 2) and table[0]["dw_splits"] >= 1
+    p = sweep.make_problem(T, B, I, H, seed=5)
+    core = LstmCore(B, I, H)
+    core.pack(p["w_ih"], p["w_hh"], p["b_ih"], p["b_hh"])
+    assert core.info("tuned_entries") == 0
+    assert core.set_tuned_table(table + [dict(table[0], B=B + 1)]) == 1      # rows of other sizes are skipped
+    assert core.info("tuned_entries") == 1 and core.tuned_table()[0] == table[0]
+    core.forward(p["x"], p["h0"], p["c0"])
+    core.backward(p["x"], p["dy"])
+    assert core.info("tuned_T") == T and core.info("row_tiles_fwd") == table[0]["row_tiles_fwd"]
+    assert core.info("tuned_dw_splits") == table[0]["dw_splits"]
+    # values out of range are refused
+    assert core.lib.flstm_core_set_tuned(core._h, T, 3, 0, 0, 0, 0, -1) == 1
+    core.close()
+
+
+def test_tuner_tries_the_layouts_of_the_backward_recurrence_at_2048_units():
+    # 2048 hidden units: the two-way split of the backward recurrence is one of the tuner's candidates (bwd_two_d 0 / 1 /
+    # 2) unless the option was set explicitly; results do not depend on what it picks beyond summation order.
+    import torch
+    from flashlstm_poc_amd import LstmCore, sweep
+    B, I, H, T = 48, 64, 2048, 12
+    p = sweep.make_problem(T, B, I, H, seed=6)
+    core = LstmCore(B, I, H)
+    core.pack(p["w_ih"], p["w_hh"], p["b_ih"], p["b_hh"])
+    core.forward(p["x"], p["h0"], p["c0"])
+    g0 = core.backward(p["x"], p["dy"])
+    t = core.tune(T, repeats=1)
+    assert t["bwd_two_d"] in (-1, 0, 1, 2) and t["bwd_rec_ms"] > 0
+    core.forward(p["x"], p["h0"], p["c0"])
+    g1 = core.backward(p["x"], p["dy"])
+    assert core.info("tuned_bwd_two_d") == t["bwd_two_d"]
+    if t["bwd_two_d"] >= 0:
+        assert core.info("bwd_two_d") == (1 if t["bwd_two_d"] > 0 and core.info("bwd_two_d") else core.info("bwd_two_d"))
+    for a, b in zip(g0, g1):
+        assert ((a.float() - b.float()).norm() / b.float().norm()).item() <= 2e-3
+    core.set_option("bwd_two_d", 0)          # an explicit option wins over the tuned entry
+    core.forward(p["x"], p["h0"], p["c0"]); core.backward(p["x"], p["dy"])
+    assert core.info("bwd_two_d") == 0
+    core.close()
