@@ -131,11 +131,14 @@ __device__ __forceinline__ void store_tile(const GemmNT& g, floatx16 (&acc)[4][k
 // ------------------------------------------------------------------------------------- NT kernel
 // C[M][N] = alpha * A[M][K] * B[N][K]^T (+ bias[n]).  Operand slabs go from global memory straight into
 // LDS (global_load_lds_dwordx4: no staging registers, no LDS store instructions), double buffered in
-// slabs of 64 k.  Every wave copies 8 KiB of the next slab, one 1 KiB copy after every second MFMA of the
-// first half of the current slab: a copy instruction holds its wave until the texture-address unit takes
-// it (16+ clocks each, 64 per slab and workgroup), so they are spread out rather than issued in a burst.
+// slabs of 64 k.  Every wave copies 8 KiB of a slab with eight 1 KiB copies, each addressed as a scalar base
+// plus a per-lane offset that is fixed for the tile, and issues them behind the MFMAs of the last k-step
+// of the slab before, right after the barrier that frees the buffer: a slab is requested one slab ahead and
+// a slab boundary costs no wave a wait with nothing to multiply.  (The copies used to carry 64-bit address
+// arithmetic per lane: ~15 instructions each in the shadow of two MFMAs, which made instruction issue,
+// not the matrix cores, the limit while they ran.)
 // The kernel is persistent: each workgroup walks its list of work items and the copies keep running
-// across item boundaries, so the first slab of the next tile arrives during the last MFMAs and the
+// across item boundaries, so the first slabs of the next tile arrive during the last MFMAs and the
 // output stores of this one.
 //
 // LDS rows are 128 bytes (8 chunks of 16).  The LDS has 64 banks of 4 bytes and serves a 16-byte read
@@ -220,32 +223,41 @@ __global__ __launch_bounds__(kThreads) void gemm_nt_stream(GemmNT g, TileOrder o
     // ---- copier state: the slab copied next is slab ld_k of item ordinal ld_n.  Copy c of a slab
     // (operand c % 2, row block i = c / 2) fills rows [64q + 8i, +8) of the tile, q = wave % 4; lane l
     // lands at row l / 8, chunk position l % 8 and therefore fetches chunk (l % 8) ^ swizzle(row).
-    int ld_n = 0, ld_k = 0, ld_nk = 0, ld_m0 = 0, ld_n0 = 0, ld_kb = 0;
-    bool ld_valid = false;
-    auto loader_open = [&]() {
-        int z;
-        ld_valid = false;
-        while (ld_n < rounds && !(ld_valid = decode(ld_n, ld_m0, ld_n0, z, ld_kb, ld_nk))) ++ld_n;
-        ld_k = 0;
-    };
+    // A copy is addressed as a wave-uniform base (the slab's first row and column, kept in scalar
+    // registers and advanced by 128 bytes per slab) plus a 32-bit byte offset per lane that is fixed for
+    // the whole tile: one instruction per copy, no address arithmetic in the shadow of the MFMAs.
+    int ld_n = 0, ld_k = 0, ld_nk = 0;
+    const char* ld_a = reinterpret_cast<const char*>(g.A);
+    const char* ld_b = reinterpret_cast<const char*>(g.B);
+    unsigned voff_a[4], voff_b[4];
     const int cp_row = wave * 32 + lane / 8;
-    auto issue_copy = [&](int slot, int c) {
-        if (!ld_valid) return;
-        const int i = c / 2;
-        const int rt = cp_row + 8 * i;
-        const int chunk = (lane % 8) ^ ((rt >> 1) & 7);
-        const int koff = ld_kb + ld_k * BK + chunk * 8;
-        char* dst = lds + slot * kSlabBytes + wave * 4096 + i * 1024;
-        if (c % 2 == 0) {
-            const int row = min(ld_m0 + rt, g.M - 1);
-            copy_1k_to_lds(reinterpret_cast<const char*>(g.A + size_t(row) * g.lda + koff), dst);
-        } else {
-            const int row = min(ld_n0 + rt, g.N - 1);
-            copy_1k_to_lds(reinterpret_cast<const char*>(g.B + size_t(row) * g.ldb + koff), dst + BM * BK * 2);
+    auto loader_open = [&]() {
+        int z, m0 = 0, n0 = 0, kb = 0;
+        bool valid = false;
+        while (ld_n < rounds && !(valid = decode(ld_n, m0, n0, z, kb, ld_nk))) ++ld_n;
+        // past the last item the copies go on, from the first rows of the operands into a buffer nobody
+        // reads any more: cheaper than a branch around every copy
+        if (!valid) m0 = n0 = kb = 0, ld_nk = 1 << 30;
+        ld_k = 0;
+        ld_a = reinterpret_cast<const char*>(g.A + size_t(m0) * g.lda + kb);
+        ld_b = reinterpret_cast<const char*>(g.B + size_t(n0) * g.ldb + kb);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int rt = cp_row + 8 * i;
+            const unsigned chunk = unsigned((lane % 8) ^ ((rt >> 1) & 7)) * 16u;
+            voff_a[i] = unsigned(min(m0 + rt, g.M - 1) - m0) * unsigned(g.lda * 2) + chunk;
+            voff_b[i] = unsigned(min(n0 + rt, g.N - 1) - n0) * unsigned(g.ldb * 2) + chunk;
         }
     };
+    auto issue_copy = [&](int slot, int c) {
+        const int i = c / 2;
+        char* dst = lds + slot * kSlabBytes + wave * 4096 + i * 1024;
+        if (c % 2 == 0) copy_1k_to_lds(ld_a + voff_a[i], dst);
+        else copy_1k_to_lds(ld_b + voff_b[i], dst + BM * BK * 2);
+    };
     auto loader_advance = [&]() {
-        if (!ld_valid) return;
+        ld_a += BK * 2;
+        ld_b += BK * 2;
         if (++ld_k == ld_nk) {
             ++ld_n;
             loader_open();
@@ -260,14 +272,33 @@ __global__ __launch_bounds__(kThreads) void gemm_nt_stream(GemmNT g, TileOrder o
 #pragma unroll
     for (int kk = 0; kk < BK / 16; ++kk) pos[kk] = ((2 * kk + lane / 32) ^ ((lane % 32) >> 1 & 7)) * 16;
 
-    bool copied = false;   // this wave has copies in flight for the slab consumed next
+    constexpr int KK = BK / 16;
+    constexpr int kPerStep = 4 * kTN;   // MFMAs per k-step
+    static_assert(kPerStep == kCopiesPerWave, "one copy behind every MFMA of a slab's last k-step");
+    half8 af[2][4], bf[2][kTN];
+    auto read_frags = [&](const char* st, int kk, int set) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+            af[set][i] = *reinterpret_cast<const half8*>(st + a_frag + i * 32 * BK * 2 + pos[kk]);
+#pragma unroll
+        for (int j = 0; j < kTN; ++j)
+            bf[set][j] = *reinterpret_cast<const half8*>(st + b_frag + j * 32 * BK * 2 + pos[kk]);
+    };
+
+    // Prologue: the first two slabs are requested, the first one awaited (copies complete in the order
+    // they were issued, so at most the second slab's 8 may be outstanding) and its first fragments read.
     loader_open();
-    copied = ld_valid;
 #pragma unroll
     for (int c = 0; c < kCopiesPerWave; ++c) issue_copy(0, c);
     loader_advance();
+#pragma unroll
+    for (int c = 0; c < kCopiesPerWave; ++c) issue_copy(1, c);
+    loader_advance();
+    wait_vm<kCopiesPerWave>();
+    __builtin_amdgcn_s_barrier();
+    read_frags(lds, 0, 0);
 
-    int slot = 0;            // LDS buffer of the slab consumed next
+    int slot = 0;            // LDS buffer of the slab being multiplied
     for (int n = 0; n < rounds; ++n) {
         int m0, n0, z, kb, nk;
         if (!decode(n, m0, n0, z, kb, nk)) continue;
@@ -280,52 +311,47 @@ __global__ __launch_bounds__(kThreads) void gemm_nt_stream(GemmNT g, TileOrder o
                 for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
 
         for (int ks = 0; ks < nk; ++ks) {
-            // Loads complete in issue order among themselves, but stores may be acknowledged out of order
-            // with them, so a count that discounts the output stores issued after the copies would not be
-            // safe: wait for everything.  (Store acknowledgements come from the L2 and take no longer than
-            // the copies that are in flight with them.)
-            if (copied) wait_vm<0>();
-            // a bare barrier: every copier has waited for its own copies above, and a fence here would
-            // make the compiler drain memory operations that are meant to stay in flight
-            __builtin_amdgcn_s_barrier();   // slab complete in LDS; the other buffer is no longer read
-            const int fill = slot ^ 1;
             const char* st = lds + slot * kSlabBytes;
-            slot ^= 1;
-            // Source order below is the schedule (pinned by sched_barrier): fragments of the next 16-wide
-            // k-step are read while this one is multiplied; a copier issues one copy after each of its
-            // first 16 MFMAs.
-            constexpr int KK = BK / 16;
-            constexpr int kPerStep = 4 * kTN;   // MFMAs per k-step
-            half8 af[2][4], bf[2][kTN];
-            auto read_frags = [&](int kk, int set) {
-#pragma unroll
-                for (int i = 0; i < 4; ++i)
-                    af[set][i] = *reinterpret_cast<const half8*>(st + a_frag + i * 32 * BK * 2 + pos[kk]);
-#pragma unroll
-                for (int j = 0; j < kTN; ++j)
-                    bf[set][j] = *reinterpret_cast<const half8*>(st + b_frag + j * 32 * BK * 2 + pos[kk]);
-            };
-            read_frags(0, 0);
-            __builtin_amdgcn_sched_barrier(0);
+            const char* st_next = lds + (slot ^ 1) * kSlabBytes;
+            // Source order below is the schedule (pinned by sched_barrier): the fragments of the next
+            // 16-wide k-step are read while this one is multiplied.
 #pragma unroll
             for (int kk = 0; kk < KK; ++kk) {
                 const int cur = kk & 1;
-                if (kk + 1 < KK) read_frags(kk + 1, cur ^ 1);
-                __builtin_amdgcn_sched_barrier(0);
+                if (kk + 1 < KK) {
+                    read_frags(st, kk + 1, cur ^ 1);
+                    __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-                for (int m = 0; m < kPerStep; ++m) {
-                    const int i = m / kTN, j = m % kTN;
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(bf[cur][j], af[cur][i], acc[i][j], 0, 0, 0);
-                    const int done = kk * kPerStep + m;
-                    if (done < 2 * kCopiesPerWave && done % 2 == 1) {
+                    for (int m = 0; m < kPerStep; ++m) {
+                        const int i = m / kTN, j = m % kTN;
+                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(bf[cur][j], af[cur][i], acc[i][j], 0, 0, 0);
+                    }
+                    __builtin_amdgcn_sched_barrier(0);
+                } else {
+                    // The slab's last fragments have been requested.  Once they are in registers nothing of
+                    // this wave reads the buffer again, and the copies this wave made of the next slab, issued
+                    // one slab ago, are awaited here too: behind the barrier the next slab is complete and
+                    // this buffer is free.  The next slab's first fragments are then read, and the slab after
+                    // it requested, under the MFMAs of this last k-step, so no wave ever waits at a slab
+                    // boundary with nothing to multiply.  (The wait is for everything: loads complete in issue
+                    // order among themselves, but the output stores of the previous tile may be acknowledged
+                    // out of order with them and would spoil a count.)
+                    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+                    __builtin_amdgcn_s_barrier();
+                    if (ks + 1 < nk) read_frags(st_next, 0, cur ^ 1);   // (a tile's last slab: after its epilogue)
+                    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                    for (int m = 0; m < kPerStep; ++m) {
+                        const int i = m / kTN, j = m % kTN;
+                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(bf[cur][j], af[cur][i], acc[i][j], 0, 0, 0);
                         __builtin_amdgcn_sched_barrier(0);
-                        issue_copy(fill, done / 2);
+                        issue_copy(slot, m);
                         __builtin_amdgcn_sched_barrier(0);
                     }
                 }
             }
-            copied = ld_valid;
             loader_advance();
+            slot ^= 1;
         }
         const bool full = (m0 + BM <= g.M) && (n0 + BN <= g.N) && vector_output(g);
         if (full && g.C16 && g.ldc % 8 == 0 && reinterpret_cast<uintptr_t>(g.C16) % 16 == 0) {
@@ -333,6 +359,7 @@ __global__ __launch_bounds__(kThreads) void gemm_nt_stream(GemmNT g, TileOrder o
         } else {
             store_tile(g, acc, m0, n0, wm, wn, lane, z);
         }
+        read_frags(lds + slot * kSlabBytes, 0, 0);
     }
     wait_vm<0>();   // no copy may still be heading for LDS when the workgroup retires
 }
@@ -533,6 +560,8 @@ static TileOrder make_order(int tiles_m, int tiles_n, int splits) {
 hipError_t launch_gemm_nt(const GemmNT& g, hipStream_t stream) {
     if (g.M <= 0 || g.N <= 0 || g.K <= 0) return hipSuccess;
     if (g.K % BK != 0 || g.lda % 8 != 0 || g.ldb % 8 != 0) return hipErrorInvalidValue;
+    // (a copy addresses a tile's 256 rows with 32-bit byte offsets from the tile's first row)
+    if (g.lda >= (size_t(1) << 22) || g.ldb >= (size_t(1) << 22)) return hipErrorInvalidValue;
     if ((g.C16 == nullptr) == (g.C32 == nullptr)) return hipErrorInvalidValue;
     if (g.bias && (reinterpret_cast<uintptr_t>(g.bias) % 16 != 0 || g.splits > 1)) return hipErrorInvalidValue;
     int splits = g.splits < 1 ? 1 : g.splits;
