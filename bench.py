@@ -411,7 +411,7 @@ def bench_single(args, device):
     kname = {"fwd_proj": "gemm_nt_stream (X*W_ih^T + bias)", "fwd_rec": "rec_fwd_kernel (persistent recurrence)",
              "bwd_rec": ("rec_bwd2d_kernel (persistent BPTT, product split over columns and contraction)"
                          if core.info("bwd_two_d") == 1 else "rec_bwd_kernel (persistent BPTT)"), "bwd_dx": "gemm_nt_stream (dG*W_ih)",
-             "bwd_dw": "gemm_tn_256x256 split-K x2 (dG^T*X, dG^T*H) + reduce_dw"}
+             "bwd_dw": "gemm_tn_stream split-K x2 (dG^T*X, dG^T*H) + reduce_dw"}
     kernels = []
     for k in phases:
         tf = kflops[k] / (phase_ms[k] * 1e-3) / 1e12 if phase_ms[k] > 0 else 0.0

@@ -21,7 +21,6 @@ constexpr int BM = 256, BN = 256, BK = 64;
 constexpr int kWavesN = 4;                 // wavefronts along N (2 along M): wave tile 128 x (256 / kWavesN)
 constexpr int kThreads = 128 * kWavesN;
 constexpr int kTN = 8 / kWavesN;            // 32-wide MFMA tiles per wave along N
-constexpr int kLd = 2048 / kThreads;        // 16-byte chunks per thread, operand and slab
 
 // Work order.  The hardware deals workgroups round-robin over the 8 XCDs in dispatch order, so the 32
 // workgroups with the same (dispatch index mod 8) that run together share one XCD and its 4 MiB L2.  They
@@ -227,6 +226,7 @@ __global__ __launch_bounds__(kThreads) void gemm_nt_stream(GemmNT g, TileOrder o
     // registers and advanced by 128 bytes per slab) plus a 32-bit byte offset per lane that is fixed for
     // the whole tile: one instruction per copy, no address arithmetic in the shadow of the MFMAs.
     int ld_n = 0, ld_k = 0, ld_nk = 0;
+    bool ld_live = false;
     const char* ld_a = reinterpret_cast<const char*>(g.A);
     const char* ld_b = reinterpret_cast<const char*>(g.B);
     unsigned voff_a[4], voff_b[4];
@@ -235,9 +235,10 @@ __global__ __launch_bounds__(kThreads) void gemm_nt_stream(GemmNT g, TileOrder o
         int z, m0 = 0, n0 = 0, kb = 0;
         bool valid = false;
         while (ld_n < rounds && !(valid = decode(ld_n, m0, n0, z, kb, ld_nk))) ++ld_n;
-        // past the last item the copies go on, from the first rows of the operands into a buffer nobody
-        // reads any more: cheaper than a branch around every copy
-        if (!valid) m0 = n0 = kb = 0, ld_nk = 1 << 30;
+        // past the last item the copies go on, of the first slab of the operands (the copier no longer
+        // advances) into a buffer nobody reads any more: cheaper than a branch around every copy
+        if (!valid) m0 = n0 = kb = 0;
+        ld_live = valid;
         ld_k = 0;
         ld_a = reinterpret_cast<const char*>(g.A + size_t(m0) * g.lda + kb);
         ld_b = reinterpret_cast<const char*>(g.B + size_t(n0) * g.ldb + kb);
@@ -256,6 +257,7 @@ __global__ __launch_bounds__(kThreads) void gemm_nt_stream(GemmNT g, TileOrder o
         else copy_1k_to_lds(ld_b + voff_b[i], dst + BM * BK * 2);
     };
     auto loader_advance = [&]() {
+        if (!ld_live) return;
         ld_a += BK * 2;
         ld_b += BK * 2;
         if (++ld_k == ld_nk) {
@@ -366,22 +368,26 @@ __global__ __launch_bounds__(kThreads) void gemm_nt_stream(GemmNT g, TileOrder o
 
 // TN form: C[M][N] = alpha * sum_k A[k][m] * B[k][n] with both operands stored k-major ([K][M] and
 // [K][N], m / n contiguous) -- the shape of the weight gradients dW = dG^T * X, whose operands come out
-// of the recurrence as [time*batch][features].  Slabs are staged in LDS exactly as they sit in memory
-// (coalesced 16-byte rows along m / n) and the MFMA fragments, which need 8 consecutive k per lane,
-// are read with the gfx950 transposing LDS load ds_read_b64_tr_b16: in every group of 16 lanes, lane j
-// supplies 4 halfs of row j/4 and receives the k-column for its own m, so no transposed copy of the
-// operands ever exists in HBM.  Rows k >= K read as zero.
-constexpr int kPitchT = 256 + 32;   // halfs per LDS row: 576 bytes = 64 mod 256, so the four k rows that 32 lanes
-                                    // read together (64 bytes each) cover the 64 banks exactly once
-constexpr size_t kLdsBytesTN = size_t(2) * 2 * BK * kPitchT * sizeof(half_t);
+// of the recurrence as [time*batch][features].  Slabs sit in LDS as they sit in memory (64 k-rows of
+// 256 halfs per operand) and the MFMA fragments, which need 8 consecutive k per lane, are read with the
+// gfx950 transposing LDS load ds_read_b64_tr_b16: in every group of 16 lanes, lane j supplies 4 halfs of
+// row j/4 and receives the k-column for its own m, so no transposed copy of the operands ever exists in
+// HBM.  Rows k >= K read as zero.
+//
+// The kernel has the structure of gemm_nt_stream: persistent, slabs copied from global memory straight
+// into LDS one slab ahead (a copy instruction fills two 512-byte k-rows), the barrier of a slab boundary
+// taken under the last k-step's MFMAs.  LDS rows are 512 bytes without padding; the four k-rows that 32
+// lanes read together (64 bytes each) are kept in different quarters of the 256-byte bank row by
+// exchanging the 64-byte chunks of a row: chunk c of k-row r sits at position c ^ (r % 4).
 
 typedef short short4v __attribute__((ext_vector_type(4)));
 typedef __attribute__((address_space(3))) short4v lds_short4;
 
-__device__ __forceinline__ half8 read_frag_tr(const half_t* lds_lane) {
+// one MFMA operand fragment: 8 consecutive k for this lane's column, as two transposing reads 4 k-rows apart
+__device__ __forceinline__ half8 read_frag_tr(const char* lds_lane) {
     union { short4v s[2]; half8 h; } u;
     u.s[0] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_short4*)(lds_lane));
-    u.s[1] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_short4*)(lds_lane + 4 * kPitchT));
+    u.s[1] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_short4*)(lds_lane + 4 * 512));
     return u.h;
 }
 
@@ -417,126 +423,209 @@ __device__ __forceinline__ void store_tile_lines_f32(const GemmNT& g, floatx16 (
     }
 }
 
-__global__ __launch_bounds__(kThreads) void gemm_tn_256x256(GemmNT g, TileOrder order, int slabs_per_split) {
-    extern __shared__ __attribute__((aligned(16))) half_t smem[];
-    half_t* As = smem;                        // [2][BK][kPitchT]
-    half_t* Bs = smem + 2 * BK * kPitchT;     // [2][BK][kPitchT]
+__global__ __launch_bounds__(kThreads) void gemm_tn_stream(GemmNT g, TileOrder order, int slabs_per_split) {
+    extern __shared__ __attribute__((aligned(1024))) char lds[];
 
-    int tm, tn, z;
-    if (!work_item(order, blockIdx.x, tm, tn, z)) return;
-    // two B operands side by side: each side has its own tiles, so a tile reads one operand only
-    if (g.B2) {
-        const int tiles_n1 = (g.N1 + BN - 1) / BN;
-        if (tn >= tiles_n1) {
-            tn -= tiles_n1;
-            g.B = g.B2; g.ldb = g.ldb2;
-            g.C32 += g.N1;
-            g.N -= g.N1;
-        } else {
-            g.N = g.N1;
-        }
-    }
-    const int m0 = tm * BM, n0 = tn * BN;
-    const int nslab_total = (g.K + BK - 1) / BK;
-    const int slab_begin = z * slabs_per_split;
-    const int nslab = min(nslab_total - slab_begin, slabs_per_split);
-    const int k_begin = slab_begin * BK;
-
-    const int tid = threadIdx.x, wave = tid / 64, lane = tid % 64;
+    const int tid = threadIdx.x, lane = tid % 64;
+    const int wave = __builtin_amdgcn_readfirstlane(tid / 64);
     const int wm = wave / kWavesN, wn = wave % kWavesN;
+    const int rounds = order.per_xcd;
+    const int nslab_total = (g.K + BK - 1) / BK;
+    const int tiles_n1 = g.B2 ? (g.N1 + BN - 1) / BN : (1 << 30);
 
-    // Global->LDS staging: 16-byte chunk c = tid + kThreads*i is k-row c/32, columns [8*(c%32), +8).
-    const int ld_k = tid / 32, ld_c = (tid % 32) * 8;
-    constexpr int kRowStep = kThreads / 32;
-    const bool a_ok = (m0 + ld_c) < g.M, b_ok = (n0 + ld_c) < g.N;
-    const half_t* a_src = g.A + min(m0 + ld_c, g.M - 8);
-    const half_t* b_src = g.B + min(n0 + ld_c, g.N - 8);
-    const int st_off = ld_k * kPitchT + ld_c;
-    half8 ra[kLd], rb[kLd];
-    // per-thread row pointers advance by one slab per fetch; only the slab that crosses K (always the
-    // last one of the matrix) needs per-row masking
-    const half_t* a_ptr = a_src + size_t(k_begin + ld_k) * g.lda;
-    const half_t* b_ptr = b_src + size_t(k_begin + ld_k) * g.ldb;
-    const size_t a_step = size_t(kRowStep) * g.lda, b_step = size_t(kRowStep) * g.ldb;
-    auto fetch = [&](int slab) {
-        const int k0 = k_begin + slab * BK;
-        if (a_ok && b_ok && k0 + BK <= g.K) {
+    // ordinal n of this workgroup -> (tile, split).  With two B operands side by side each side has its
+    // own tiles, so a tile reads one operand only: side 1 is B2 and columns [N1, N) of C.
+    struct Item { int m0, n0, side, z, slab0, nk; };
+    auto decode = [&](int n, Item& it) -> bool {
+        int tm, tn;
+        if (!work_item(order, n * int(gridDim.x) + blockIdx.x, tm, tn, it.z)) return false;
+        it.side = tn >= tiles_n1 ? 1 : 0;
+        it.m0 = tm * BM;
+        it.n0 = (tn - (it.side ? tiles_n1 : 0)) * BN;
+        it.slab0 = it.z * slabs_per_split;
+        it.nk = min(nslab_total - it.slab0, slabs_per_split);
+        return it.nk > 0;
+    };
+
+    // ---- copier.  Copy c of a slab (operand c % 2, row pair i = c / 2) fills k-rows 8*wave + 2i, +1; lane l
+    // lands in row l / 32 of the pair at 16-byte position l % 32, i.e. in 64-byte position p = (l % 32) / 4,
+    // and therefore fetches chunk p ^ (row % 4).  Addressing as in gemm_nt_stream: scalar base (the slab's
+    // first k-row) + a per-lane byte offset fixed for the item; only a slab that crosses K computes clamped
+    // row addresses (rows >= K are then cleared in LDS by the wave that copied them).
+    int ld_n = 0, ld_k = 0, ld_nk = 0, ld_rows = BK, ld_slab = 0;
+    bool ld_live = false;
+    const char* ld_a = reinterpret_cast<const char*>(g.A);
+    const char* ld_b = reinterpret_cast<const char*>(g.B);
+    unsigned ld_pa = 0, ld_pb = 0;          // bytes per k-row of the operands of the item being copied
+    unsigned col_a[2], col_b[2], voff_a[2], voff_b[2];   // [row pair % 2]: the chunk exchange depends on row % 4
+    const int cp_row = 8 * wave + lane / 32;
+    auto loader_open = [&]() {
+        Item it{0, 0, 0, 0, 0, 0};
+        bool valid = false;
+        while (ld_n < rounds && !(valid = decode(ld_n, it))) ++ld_n;
+        if (!valid) it = Item{0, 0, 0, 0, 0, 0};   // past the last item: harmless copies of the first slab, no advance
+        ld_live = valid;
+        ld_k = 0;
+        ld_nk = it.nk;
+        ld_slab = it.slab0;
+        const half_t* bsrc = it.side ? g.B2 : g.B;
+        const int nside = g.B2 ? (it.side ? g.N - g.N1 : g.N1) : g.N;
+        ld_pa = unsigned(g.lda * 2);
+        ld_pb = unsigned((it.side ? g.ldb2 : g.ldb) * 2);
+        ld_a = reinterpret_cast<const char*>(g.A) + size_t(ld_slab) * BK * ld_pa;
+        ld_b = reinterpret_cast<const char*>(bsrc) + size_t(ld_slab) * BK * ld_pb;
 #pragma unroll
-            for (int i = 0; i < kLd; ++i) {
-                ra[i] = ld_half8(a_ptr + i * a_step);
-                rb[i] = ld_half8(b_ptr + i * b_step);
-            }
+        for (int e = 0; e < 2; ++e) {
+            const int sw = (2 * e + lane / 32) % 4;
+            const int c = (((lane % 32) / 4) ^ sw) * 32 + (lane % 4) * 8;   // column (halfs) inside the tile
+            col_a[e] = unsigned(min(it.m0 + c, g.M - 8)) * 2u;
+            col_b[e] = unsigned(min(it.n0 + c, nside - 8)) * 2u;
+        }
+#pragma unroll
+        for (int e = 0; e < 2; ++e) {
+            voff_a[e] = unsigned(cp_row) * ld_pa + col_a[e];
+            voff_b[e] = unsigned(cp_row) * ld_pb + col_b[e];
+        }
+        ld_rows = min(BK, g.K - ld_slab * BK);
+    };
+    auto issue_copy = [&](int slot, int c) {
+        const int i = c / 2;
+        char* dst = lds + slot * kSlabBytes + (c % 2) * (BM * BK * 2) + (8 * wave + 2 * i) * 512;
+        const unsigned pitch = c % 2 == 0 ? ld_pa : ld_pb;
+        const char* base = c % 2 == 0 ? ld_a : ld_b;
+        if (ld_rows < BK) {
+            const unsigned row = unsigned(min(cp_row + 2 * i, ld_rows - 1));
+            copy_1k_to_lds(base + (row * pitch + (c % 2 == 0 ? col_a[i % 2] : col_b[i % 2])), dst);
         } else {
+            copy_1k_to_lds(base + size_t(2 * i) * pitch + (c % 2 == 0 ? voff_a[i % 2] : voff_b[i % 2]), dst);
+        }
+    };
+    auto loader_advance = [&]() {
+        if (!ld_live) return;
+        ld_a += size_t(BK) * ld_pa;
+        ld_b += size_t(BK) * ld_pb;
+        ++ld_slab;
+        if (++ld_k == ld_nk) {
+            ++ld_n;
+            loader_open();
+        } else {
+            ld_rows = min(BK, g.K - ld_slab * BK);
+        }
+    };
+    // rows >= `rows` of the slab in `st`, as far as this wave copied them, are cleared
+    auto clear_tail = [&](char* st, int rows) {
+        if (rows >= BK) return;
 #pragma unroll
-            for (int i = 0; i < kLd; ++i) {
-                const int k = k0 + ld_k + kRowStep * i;
-                const int kc = min(k, g.K - 1);
-                ra[i] = ld_half8(a_src + size_t(kc) * g.lda);
-                rb[i] = ld_half8(b_src + size_t(kc) * g.ldb);
-                if (!(a_ok && k < g.K)) ra[i] = half8{};
-                if (!(b_ok && k < g.K)) rb[i] = half8{};
+        for (int r = 0; r < 8; ++r) {
+            const int row = 8 * wave + r;
+            if (row >= rows) {
+                *reinterpret_cast<unsigned long long*>(st + row * 512 + lane * 8) = 0ull;
+                *reinterpret_cast<unsigned long long*>(st + BM * BK * 2 + row * 512 + lane * 8) = 0ull;
             }
         }
-        a_ptr += size_t(BK) * g.lda;
-        b_ptr += size_t(BK) * g.ldb;
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
     };
-    auto stage = [&](int buf) {
-#pragma unroll
-        for (int i = 0; i < kLd; ++i) {
-            st_half8(As + buf * BK * kPitchT + st_off + kRowStep * i * kPitchT, ra[i]);
-            st_half8(Bs + buf * BK * kPitchT + st_off + kRowStep * i * kPitchT, rb[i]);
-        }
-    };
-    // transposing fragment read: lane (group gq = lane/16, j = lane%16) addresses k-row 8*(gq/2) + j/4,
-    // column 16*(gq%2) + 4*(j%4) of a 32-wide tile; it receives k = 8*(lane/32) .. +7 for column lane%32.
+
+    // ---- consumer.  Transposing fragment read: lane (group gq = lane / 16, j = lane % 16) addresses k-row
+    // 8*(gq/2) + j/4 and halfs 16*(gq%2) + 4*(j%4) of a 32-wide tile; it receives k = 8*(lane/32) .. +7 for
+    // column lane % 32.  k-row % 4 = j / 4 for every read of a lane, so the chunk exchange is a per-lane
+    // constant: 32-column tile t of the operand (64 bytes per k-row = one chunk) sits at chunk t ^ (j / 4).
     const int gq = lane / 16, jq = lane % 16;
-    const int frag_off = (8 * (gq / 2) + jq / 4) * kPitchT + 16 * (gq % 2) + 4 * (jq % 4);
-    const int a_frag_off = frag_off + wm * 128;
-    const int b_frag_off = frag_off + wn * 32 * kTN;
+    const int frag_lane = (8 * (gq / 2) + jq / 4) * 512 + 32 * (gq % 2) + 8 * (jq % 4);
+    int a_frag[4], b_frag[kTN];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) a_frag[i] = frag_lane + ((wm * 4 + i) ^ (jq / 4)) * 64;
+#pragma unroll
+    for (int j = 0; j < kTN; ++j) b_frag[j] = BM * BK * 2 + frag_lane + ((wn * kTN + j) ^ (jq / 4)) * 64;
 
-    floatx16 acc[4][kTN];
+    constexpr int KK = BK / 16;
+    constexpr int kPerStep = 4 * kTN;
+    static_assert(kPerStep == kCopiesPerWave, "one copy behind every MFMA of a slab's last k-step");
+    half8 af[2][4], bf[2][kTN];
+    auto read_frags = [&](const char* st, int kk, int set) {
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
+        for (int i = 0; i < 4; ++i) af[set][i] = read_frag_tr(st + a_frag[i] + kk * 16 * 512);
 #pragma unroll
-        for (int j = 0; j < kTN; ++j)
-#pragma unroll
-            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
+        for (int j = 0; j < kTN; ++j) bf[set][j] = read_frag_tr(st + b_frag[j] + kk * 16 * 512);
+    };
 
-    if (nslab > 0) {
-        fetch(0);
-        stage(0);
-    }
-    __syncthreads();
+    loader_open();
+    const int rows_first = ld_rows;
+#pragma unroll
+    for (int c = 0; c < kCopiesPerWave; ++c) issue_copy(0, c);
+    loader_advance();
+    int rows_next = ld_rows;   // valid k-rows of the slab that the next barrier completes
+#pragma unroll
+    for (int c = 0; c < kCopiesPerWave; ++c) issue_copy(1, c);
+    loader_advance();
+    wait_vm<kCopiesPerWave>();
+    clear_tail(lds, rows_first);
+    __builtin_amdgcn_s_barrier();
+    read_frags(lds, 0, 0);
 
-    for (int s = 0; s < nslab; ++s) {
-        const int cur = s & 1;
-        const bool more = (s + 1 < nslab);
-        if (more) fetch(s + 1);
-        const half_t* Ac = As + cur * BK * kPitchT + a_frag_off;
-        const half_t* Bc = Bs + cur * BK * kPitchT + b_frag_off;
+    int slot = 0;
+    for (int n = 0; n < rounds; ++n) {
+        Item it;
+        if (!decode(n, it)) continue;
+        floatx16 acc[4][kTN];
 #pragma unroll
-        for (int kk = 0; kk < BK / 16; ++kk) {
-            half8 af[4], bf[kTN];
+        for (int i = 0; i < 4; ++i)
 #pragma unroll
-            for (int i = 0; i < 4; ++i) af[i] = read_frag_tr(Ac + kk * 16 * kPitchT + i * 32);
+            for (int j = 0; j < kTN; ++j)
 #pragma unroll
-            for (int j = 0; j < kTN; ++j) bf[j] = read_frag_tr(Bc + kk * 16 * kPitchT + j * 32);
+                for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
+
+        for (int ks = 0; ks < it.nk; ++ks) {
+            char* st = lds + slot * kSlabBytes;
+            char* st_next = lds + (slot ^ 1) * kSlabBytes;
 #pragma unroll
-            for (int i = 0; i < 4; ++i)
+            for (int kk = 0; kk < KK; ++kk) {
+                const int cur = kk & 1;
+                if (kk + 1 < KK) {
+                    read_frags(st, kk + 1, cur ^ 1);
+                    __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-                for (int j = 0; j < kTN; ++j)
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(bf[j], af[i], acc[i][j], 0, 0, 0);
+                    for (int m = 0; m < kPerStep; ++m) {
+                        const int i = m / kTN, j = m % kTN;
+                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(bf[cur][j], af[cur][i], acc[i][j], 0, 0, 0);
+                    }
+                    __builtin_amdgcn_sched_barrier(0);
+                } else {
+                    // (see gemm_nt_stream: this slab's reads and this wave's copies of the next slab are
+                    // complete; behind the barrier the next slab is whole and this buffer is free)
+                    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+                    clear_tail(st_next, rows_next);
+                    __builtin_amdgcn_s_barrier();
+                    if (ks + 1 < it.nk) read_frags(st_next, 0, cur ^ 1);
+                    __builtin_amdgcn_sched_barrier(0);
+                    rows_next = ld_rows;
+#pragma unroll
+                    for (int m = 0; m < kPerStep; ++m) {
+                        const int i = m / kTN, j = m % kTN;
+                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(bf[cur][j], af[cur][i], acc[i][j], 0, 0, 0);
+                        __builtin_amdgcn_sched_barrier(0);
+                        issue_copy(slot, m);
+                        __builtin_amdgcn_sched_barrier(0);
+                    }
+                }
+            }
+            loader_advance();
+            slot ^= 1;
         }
-        if (more) stage(cur ^ 1);
-        __syncthreads();
+        GemmNT gi = g;
+        if (g.B2) {
+            if (it.side) { gi.C32 += g.N1; gi.N = g.N - g.N1; }
+            else gi.N = g.N1;
+        }
+        const bool full = (it.m0 + BM <= gi.M) && (it.n0 + BN <= gi.N) && vector_output(gi);
+        if (full && gi.C32) {
+            store_tile_lines_f32(gi, acc, it.m0, it.n0, wm, wn, lane, it.z, lds + 2 * kSlabBytes + wave * kEpiBytesPerWave);
+        } else {
+            store_tile(gi, acc, it.m0, it.n0, wm, wn, lane, it.z);
+        }
+        read_frags(lds + slot * kSlabBytes, 0, 0);
     }
-    const bool full = (m0 + BM <= g.M) && (n0 + BN <= g.N) && vector_output(g);
-    if (full && g.C32) {
-        // the slab buffers are free once every wave has left the main loop (the barrier that ends it)
-        store_tile_lines_f32(g, acc, m0, n0, wm, wn, lane, z, reinterpret_cast<char*>(smem) + wave * 4096);
-        return;
-    }
-    store_tile(g, acc, m0, n0, wm, wn, lane, z);
+    wait_vm<0>();   // no copy may still be heading for LDS when the workgroup retires
 }
 
 }  // namespace
@@ -595,8 +684,14 @@ hipError_t launch_gemm_tn(const GemmNT& g, hipStream_t stream) {
     const int splits = g.splits < 1 ? 1 : g.splits;
     if (splits > 1 && g.C32 == nullptr) return hipErrorInvalidValue;
     if (gemm_effective_splits(g.K, splits) != splits) return hipErrorInvalidValue;
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_tn_256x256),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, int(kLdsBytesTN));
+    if (reinterpret_cast<uintptr_t>(g.A) % 16 != 0 || reinterpret_cast<uintptr_t>(g.B) % 16 != 0 ||
+        (g.B2 && reinterpret_cast<uintptr_t>(g.B2) % 16 != 0))
+        return hipErrorInvalidValue;
+    // (a copy addresses a slab's 64 k-rows with 32-bit byte offsets from the slab's first row)
+    if (g.lda >= (size_t(1) << 22) || g.ldb >= (size_t(1) << 22) || (g.B2 && g.ldb2 >= (size_t(1) << 22)))
+        return hipErrorInvalidValue;
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_tn_stream),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, int(kLdsBytesStream));
     if (e != hipSuccess) return e;
     const int nslab = (g.K + BK - 1) / BK;
     const int slabs_per_split = (nslab + splits - 1) / splits;
@@ -604,7 +699,7 @@ hipError_t launch_gemm_tn(const GemmNT& g, hipStream_t stream) {
     const int tiles_m = (g.M + BM - 1) / BM;
     const int tiles_n = g.B2 ? (g.N1 + BN - 1) / BN + (g.N - g.N1 + BN - 1) / BN : (g.N + BN - 1) / BN;
     const TileOrder order = make_order(tiles_m, tiles_n, splits);
-    hipLaunchKernelGGL(gemm_tn_256x256, dim3(order.per_xcd * 256), dim3(kThreads), kLdsBytesTN, stream, g, order,
+    hipLaunchKernelGGL(gemm_tn_stream, dim3(256), dim3(kThreads), kLdsBytesStream, stream, g, order,
                        slabs_per_split);
     return hipGetLastError();
 }
