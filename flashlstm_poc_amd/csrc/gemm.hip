@@ -155,6 +155,19 @@ __device__ __forceinline__ void copy_1k_to_lds(const char* src_lane, char* lds_b
     __builtin_amdgcn_global_load_lds((global_void*)(src_lane), (lds_void*)(lds_block), 16, 0, 0);
 }
 
+// The same copy issued by hand: scalar base + 32-bit offset per lane, LDS destination in M0.  The compiler
+// does not know that it writes LDS, so it places no wait for it in front of LDS reads (it cannot tell that
+// the transposing reads of gemm_tn_stream never touch the buffer being filled, and would wait for every
+// copy right after it was issued); the kernel's own s_waitcnt vmcnt(0) + barrier order copies and reads.
+// Counted waits that the compiler places for its own loads and stores only become stricter by the extra
+// operations in flight.
+typedef __attribute__((address_space(3))) char lds_char;
+__device__ __forceinline__ void copy_1k_to_lds_unseen(const char* base, unsigned lane_off, char* lds_block) {
+    const unsigned m = unsigned(reinterpret_cast<unsigned long>((lds_char*)(lds_block)));
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
+                 :: "v"(lane_off), "s"(base), "s"(m) : "m0", "memory");
+}
+
 template <int N>
 __device__ __forceinline__ void wait_vm() {
     asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
@@ -495,9 +508,9 @@ __global__ __launch_bounds__(kThreads) void gemm_tn_stream(GemmNT g, TileOrder o
         const char* base = c % 2 == 0 ? ld_a : ld_b;
         if (ld_rows < BK) {
             const unsigned row = unsigned(min(cp_row + 2 * i, ld_rows - 1));
-            copy_1k_to_lds(base + (row * pitch + (c % 2 == 0 ? col_a[i % 2] : col_b[i % 2])), dst);
+            copy_1k_to_lds_unseen(base, row * pitch + (c % 2 == 0 ? col_a[i % 2] : col_b[i % 2]), dst);
         } else {
-            copy_1k_to_lds(base + size_t(2 * i) * pitch + (c % 2 == 0 ? voff_a[i % 2] : voff_b[i % 2]), dst);
+            copy_1k_to_lds_unseen(base + size_t(2 * i) * pitch, c % 2 == 0 ? voff_a[i % 2] : voff_b[i % 2], dst);
         }
     };
     auto loader_advance = [&]() {
