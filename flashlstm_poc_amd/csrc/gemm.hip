@@ -291,13 +291,14 @@ __global__ __launch_bounds__(kThreads) void gemm_nt_stream(GemmNT g, TileOrder o
     constexpr int kPerStep = 4 * kTN;   // MFMAs per k-step
     static_assert(kPerStep == kCopiesPerWave, "one copy behind every MFMA of a slab's last k-step");
     half8 af[2][4], bf[2][kTN];
+    // fragment f of a k-step: 0..3 the A rows, 4.. the B rows
+    auto read_frag = [&](const char* st, int kk, int set, int f) {
+        if (f < 4) af[set][f] = *reinterpret_cast<const half8*>(st + a_frag + f * 32 * BK * 2 + pos[kk]);
+        else bf[set][f - 4] = *reinterpret_cast<const half8*>(st + b_frag + (f - 4) * 32 * BK * 2 + pos[kk]);
+    };
     auto read_frags = [&](const char* st, int kk, int set) {
 #pragma unroll
-        for (int i = 0; i < 4; ++i)
-            af[set][i] = *reinterpret_cast<const half8*>(st + a_frag + i * 32 * BK * 2 + pos[kk]);
-#pragma unroll
-        for (int j = 0; j < kTN; ++j)
-            bf[set][j] = *reinterpret_cast<const half8*>(st + b_frag + j * 32 * BK * 2 + pos[kk]);
+        for (int f = 0; f < 4 + kTN; ++f) read_frag(st, kk, set, f);
     };
 
     // Prologue: the first two slabs are requested, the first one awaited (copies complete in the order
@@ -329,19 +330,20 @@ __global__ __launch_bounds__(kThreads) void gemm_nt_stream(GemmNT g, TileOrder o
             const char* st = lds + slot * kSlabBytes;
             const char* st_next = lds + (slot ^ 1) * kSlabBytes;
             // Source order below is the schedule (pinned by sched_barrier): the fragments of the next
-            // 16-wide k-step are read while this one is multiplied.
+            // 16-wide k-step are read one by one behind the first MFMAs of this one, so that a wave never
+            // stands at a wait for fragments it has only just asked for.
 #pragma unroll
             for (int kk = 0; kk < KK; ++kk) {
                 const int cur = kk & 1;
                 if (kk + 1 < KK) {
-                    read_frags(st, kk + 1, cur ^ 1);
-                    __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
                     for (int m = 0; m < kPerStep; ++m) {
                         const int i = m / kTN, j = m % kTN;
                         acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(bf[cur][j], af[cur][i], acc[i][j], 0, 0, 0);
+                        __builtin_amdgcn_sched_barrier(0);
+                        if (m < 4 + kTN) read_frag(st, kk + 1, cur ^ 1, m);
+                        __builtin_amdgcn_sched_barrier(0);
                     }
-                    __builtin_amdgcn_sched_barrier(0);
                 } else {
                     // The slab's last fragments have been requested.  Once they are in registers nothing of
                     // this wave reads the buffer again, and the copies this wave made of the next slab, issued
@@ -353,13 +355,14 @@ __global__ __launch_bounds__(kThreads) void gemm_nt_stream(GemmNT g, TileOrder o
                     // out of order with them and would spoil a count.)
                     asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
                     __builtin_amdgcn_s_barrier();
-                    if (ks + 1 < nk) read_frags(st_next, 0, cur ^ 1);   // (a tile's last slab: after its epilogue)
+                    const bool more = ks + 1 < nk;   // (a tile's last slab: fragments after its epilogue)
                     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
                     for (int m = 0; m < kPerStep; ++m) {
                         const int i = m / kTN, j = m % kTN;
                         acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(bf[cur][j], af[cur][i], acc[i][j], 0, 0, 0);
                         __builtin_amdgcn_sched_barrier(0);
+                        if (more && m < 4 + kTN) read_frag(st_next, 0, cur ^ 1, m);
                         issue_copy(slot, m);
                         __builtin_amdgcn_sched_barrier(0);
                     }
@@ -555,11 +558,13 @@ __global__ __launch_bounds__(kThreads) void gemm_tn_stream(GemmNT g, TileOrder o
     constexpr int kPerStep = 4 * kTN;
     static_assert(kPerStep == kCopiesPerWave, "one copy behind every MFMA of a slab's last k-step");
     half8 af[2][4], bf[2][kTN];
+    auto read_frag = [&](const char* st, int kk, int set, int f) {
+        if (f < 4) af[set][f] = read_frag_tr(st + a_frag[f] + kk * 16 * 512);
+        else bf[set][f - 4] = read_frag_tr(st + b_frag[f - 4] + kk * 16 * 512);
+    };
     auto read_frags = [&](const char* st, int kk, int set) {
 #pragma unroll
-        for (int i = 0; i < 4; ++i) af[set][i] = read_frag_tr(st + a_frag[i] + kk * 16 * 512);
-#pragma unroll
-        for (int j = 0; j < kTN; ++j) bf[set][j] = read_frag_tr(st + b_frag[j] + kk * 16 * 512);
+        for (int f = 0; f < 4 + kTN; ++f) read_frag(st, kk, set, f);
     };
 
     loader_open();
@@ -595,21 +600,21 @@ __global__ __launch_bounds__(kThreads) void gemm_tn_stream(GemmNT g, TileOrder o
             for (int kk = 0; kk < KK; ++kk) {
                 const int cur = kk & 1;
                 if (kk + 1 < KK) {
-                    read_frags(st, kk + 1, cur ^ 1);
-                    __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
                     for (int m = 0; m < kPerStep; ++m) {
                         const int i = m / kTN, j = m % kTN;
                         acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(bf[cur][j], af[cur][i], acc[i][j], 0, 0, 0);
+                        __builtin_amdgcn_sched_barrier(0);
+                        if (m < 4 + kTN) read_frag(st, kk + 1, cur ^ 1, m);
+                        __builtin_amdgcn_sched_barrier(0);
                     }
-                    __builtin_amdgcn_sched_barrier(0);
                 } else {
                     // (see gemm_nt_stream: this slab's reads and this wave's copies of the next slab are
                     // complete; behind the barrier the next slab is whole and this buffer is free)
                     asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
                     clear_tail(st_next, rows_next);
                     __builtin_amdgcn_s_barrier();
-                    if (ks + 1 < it.nk) read_frags(st_next, 0, cur ^ 1);
+                    const bool more = ks + 1 < it.nk;
                     __builtin_amdgcn_sched_barrier(0);
                     rows_next = ld_rows;
 #pragma unroll
@@ -617,6 +622,7 @@ __global__ __launch_bounds__(kThreads) void gemm_tn_stream(GemmNT g, TileOrder o
                         const int i = m / kTN, j = m % kTN;
                         acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(bf[cur][j], af[cur][i], acc[i][j], 0, 0, 0);
                         __builtin_amdgcn_sched_barrier(0);
+                        if (more && m < 4 + kTN) read_frag(st_next, 0, cur ^ 1, m);
                         issue_copy(slot, m);
                         __builtin_amdgcn_sched_barrier(0);
                     }
