@@ -401,6 +401,19 @@ def bench_single(args, device):
     wall_ms = (time.perf_counter() - t0) * 1e3 / args.steps
     ms = e0.elapsed_time(e1) / args.steps
     phase_ms = {k: v / args.steps for k, v in acc.items()}
+    # Engine clock inside the recurrence kernels, from two untimed passes with the kernels' own counters on: workgroup 0
+    # reads the shader clock counter and the constant 100 MHz counter at its first and last step.  (The part lowers its
+    # clock under the GEMMs and raises it again only slowly, so the recurrences that follow them run below 2.4 GHz.)
+    core.set_option("profile", 1)
+    engine_mhz = {}
+    for _ in range(2):
+        step()
+    torch.cuda.synchronize()
+    for d in ("fwd", "bwd") if backward else ("fwd",):
+        ticks = core.last_ms(f"{d}_clk6")
+        if ticks > 0:
+            engine_mhz[f"{d}_rec"] = round(core.last_ms(f"{d}_clk5") / ticks * 100.0, 1)
+    core.set_option("profile", 0)
 
     flops_fwd = 8.0 * T * B * H * (I + H)
     flops = flops_fwd * (3.0 if backward else 1.0)
@@ -445,6 +458,7 @@ def bench_single(args, device):
         "roofline": roofline, "kernels": kernels, "device": device,
         "us_per_timestep": {"fwd_rec": round(phase_ms["fwd_rec"] * 1e3 / T, 3),
                             **({"bwd_rec": round(phase_ms["bwd_rec"] * 1e3 / T, 3)} if backward else {})},
+        "engine_mhz_in_recurrence": engine_mhz,
     }
     # What the recurrence moves between workgroups each step.  Measured: requests to the L2 (TCC_REQ, each at most one
     # 128-byte line) and the cycles the LDS address unit was busy (SQ_LDS_IDX_ACTIVE, summed over the CUs), from the

@@ -979,7 +979,9 @@ extern "C" double flstm_core_last_ms(const flstm_core_plan* p, const char* phase
     if (!strcmp(phase, "bwd_dx")) return p->ms_bwd[1];
     if (!strcmp(phase, "bwd_dw")) return p->ms_bwd[2];
     if (!strcmp(phase, "bwd_total")) return p->ms_bwd[3];
-    // cycle counters of workgroup 0 (option "profile"): wait, product, partials, pointwise, publish
+    // counters of workgroup 0 (option "profile"), in milliseconds of the constant-rate clock: 0..4 wait, product, partials,
+    // pointwise, publish; 6 the whole launch; 5 the launch in shader-engine clocks / the constant clock's rate, so that
+    // clk5 / clk6 x that rate is the engine clock the kernel ran at
     if (!strncmp(phase, "fwd_clk", 7) && phase[7] >= '0' && phase[7] <= '7')
         return double(p->prof_f[phase[7] - '0']) / p->wall_khz;
     if (!strncmp(phase, "bwd_clk", 7) && phase[7] >= '0' && phase[7] <= '7')

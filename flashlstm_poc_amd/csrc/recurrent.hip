@@ -774,6 +774,7 @@ __device__ __forceinline__ void to_floats(const F32<4>& r, float (&f)[4]) {
 struct PhaseClock {
     long long* out;
     long long last;
+    long long core_start = 0, wall_start = 0;   // slots 5 and 6: engine clocks and 100 MHz ticks of the whole launch
 
     __device__ __forceinline__ long long* acc() {
         __shared__ long long lds_acc[5];
@@ -783,6 +784,8 @@ struct PhaseClock {
         if (out && threadIdx.x == 0) {
             for (int i = 0; i < 5; ++i) acc()[i] = 0;
             last = wall_clock64();
+            wall_start = last;
+            core_start = clock64();
         }
     }
 
@@ -798,8 +801,11 @@ struct PhaseClock {
         }
     }
     __device__ __forceinline__ void flush() {
-        if (out && threadIdx.x == 0)
+        if (out && threadIdx.x == 0) {
             for (int i = 0; i < 5; ++i) out[i] += acc()[i];
+            out[5] += clock64() - core_start;
+            out[6] += wall_clock64() - wall_start;
+        }
     }
 };
 
