@@ -6,7 +6,7 @@ already resident in HBM (fp16 x / dY, packed fp16 weights); weight packing and p
 before the timed region.  Prints ONE JSON line.
 
   python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload config3|config2|config4|config5|config5_layer]
-                  [--no-cpu-baseline] [--no-parity] [--no-others]
+                  [--no-cpu-baseline] [--no-parity] [--no-engine-clock] [--no-others]
 
 Without --workload the line is the headline workload (config 3) and carries, under "other_workloads", short runs of
 the other BASELINE configurations (config 2, config 4, the config-5 stack: 1 warm-up + 3 timed steps each, with their
@@ -321,6 +321,8 @@ def main():
     ap.add_argument("--workload", default=None, choices=sorted(WORKLOADS) + sorted(STACKS))
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-parity", action="store_true")
+    ap.add_argument("--no-engine-clock", action="store_true",
+                    help="skip the two extra passes that read the engine clock inside the recurrence kernels (profiler runs)")
     ap.add_argument("--no-others", action="store_true", help="the headline workload only (no other_workloads block)")
     args = ap.parse_args()
     args.others = args.workload is None and not args.no_others
@@ -404,16 +406,17 @@ def bench_single(args, device):
     # Engine clock inside the recurrence kernels, from two untimed passes with the kernels' own counters on: workgroup 0
     # reads the shader clock counter and the constant 100 MHz counter at its first and last step.  (The part lowers its
     # clock under the GEMMs and raises it again only slowly, so the recurrences that follow them run below 2.4 GHz.)
-    core.set_option("profile", 1)
     engine_mhz = {}
-    for _ in range(2):
-        step()
-    torch.cuda.synchronize()
-    for d in ("fwd", "bwd") if backward else ("fwd",):
-        ticks = core.last_ms(f"{d}_clk6")
-        if ticks > 0:
-            engine_mhz[f"{d}_rec"] = round(core.last_ms(f"{d}_clk5") / ticks * 100.0, 1)
-    core.set_option("profile", 0)
+    if not args.no_engine_clock:
+        core.set_option("profile", 1)
+        for _ in range(2):
+            step()
+        torch.cuda.synchronize()
+        for d in ("fwd", "bwd") if backward else ("fwd",):
+            ticks = core.last_ms(f"{d}_clk6")
+            if ticks > 0:
+                engine_mhz[f"{d}_rec"] = round(core.last_ms(f"{d}_clk5") / ticks * 100.0, 1)
+        core.set_option("profile", 0)
 
     flops_fwd = 8.0 * T * B * H * (I + H)
     flops = flops_fwd * (3.0 if backward else 1.0)
