@@ -123,3 +123,14 @@ def test_gemm_argument_checks():
     assert L.flstm_gemm_tn(t.data_ptr(), 64, t.data_ptr(), 64, 64, 64, 64, c.data_ptr(), 64, 1.0, 4, None, s) in (0, 1)  # 1 slab -> no split
     assert L.flstm_gemm_tn(t.data_ptr(), 64, t.data_ptr(), 64, 64, 64, 256, c.data_ptr(), 64, 1.0, 4, None, s) == 1    # split without workspace
     torch.cuda.synchronize()
+
+
+def test_the_comparison_tool_runs_both_libraries_on_the_same_operands_and_they_agree():
+    """python -m flashlstm_poc_amd.gemm_compare at a small size: the three products through this library's C ABI and
+    through torch.matmul (the vendor GEMM library), outputs within fp16 rounding of each other."""
+    from flashlstm_poc_amd.gemm_compare import compare
+    rows = compare(rows=4096, hidden=256, inputs=320, reps=1)
+    assert [r["product"].split()[0] for r in rows] == ["projection", "dX", "dW"]
+    for r in rows:
+        assert r["own_ms"] > 0 and r["vendor_ms"] > 0
+        assert r["max_rel_diff"] < 2e-3, r
