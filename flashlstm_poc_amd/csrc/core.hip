@@ -125,9 +125,11 @@ struct flstm_core_plan {
     bool have_cache = false;
     // pass in progress (begin / steps / end)
     struct { size_t T = 0; const void* x = nullptr; flstm_dtype x_dtype = FLSTM_F16; bool open = false;
-             half_t* y_direct = nullptr; } fw;   // y_direct: the recurrence writes the caller's y itself
+             half_t* y_direct = nullptr; bool seats_clean = false; } fw;   // y_direct: the recurrence writes the caller's y itself
+    // (seats_clean: the pass's setup has zeroed the seat counters for the first recurrence launch that follows it)
     struct { size_t T = 0; const half_t* dYk = nullptr; const void* dY = nullptr; flstm_dtype dy_dtype = FLSTM_F16;
-             float S = 1.f, dy_scale = 1.f; void* dx = nullptr; flstm_dtype dx_dtype = FLSTM_F16; bool open = false; } bw;
+             float S = 1.f, dy_scale = 1.f; void* dx = nullptr; flstm_dtype dx_dtype = FLSTM_F16; bool open = false;
+             bool seats_clean = false; } bw;
     // backward scratch
     DevBuf dYp, dG, dHn, dC, dH0, db_part, dw_part, prof, part_b;
     int opt_profile = 0, wall_khz = 100000;
@@ -427,18 +429,20 @@ int forward_setup(flstm_core_plan* p, size_t T, const void* x, flstm_dtype x_dty
     FL_TRY(p->G.reserve(TB * 4 * d.Hp * sizeof(half_t)));
     FL_TRY(p->Y.reserve((TB + d.B) * d.Hp * sizeof(half_t)));
     FL_TRY(p->C.reserve((TB + d.B) * d.Hp * sizeof(float)));
-    // initial state rows
-    if (h0) FL_TRY(convert_pad(h0, state_dtype == FLSTM_F32, size_t(d.B), d.H, size_t(d.H), 1.f, p->Y.as<half_t>(),
-                               size_t(d.B), size_t(d.Hp), s));
-    else FL_TRY(fill_zero(p->Y.p, size_t(d.B) * d.Hp * sizeof(half_t), s));
-    FL_TRY(convert_pad_f32(c0, state_dtype == FLSTM_F32, size_t(d.B), d.H, 1.f, p->C.as<float>(), size_t(d.Hp), s));
     const size_t xslot = exchange_slot_halfs(d.B, d.Hp);
-    // exchange ring: slot 0 = h0 (rows past B zero), slots 1 to 3 = the 'unwritten' pattern
     FL_TRY(p->xch_f.reserve(4 * xslot * sizeof(half_t)));
-    FL_TRY(fill_zero(p->xch_f.p, xslot * sizeof(half_t), s));
-    FL_TRY(fill_words(p->xch_f.as<half_t>() + xslot, 3 * xslot * sizeof(half_t), 0xFFFFFFFFu, s));
+    // One launch: the initial state rows (a null h0 / c0 reads as zeros), the exchange ring -- slot 0 zero (h0 goes in
+    // below; rows past B stay zero), slots 1 to 3 the 'unwritten' pattern --, the seat counters and the phase counters.
+    PrepList prep;
+    prep.to_half(h0, state_dtype == FLSTM_F32, size_t(d.B), d.H, size_t(d.H), 1.f, p->Y.as<half_t>(), size_t(d.B), size_t(d.Hp));
+    prep.to_float(c0, state_dtype == FLSTM_F32, size_t(d.B), d.H, 1.f, p->C.as<float>(), size_t(d.Hp));
+    prep.fill(p->xch_f.p, xslot * sizeof(half_t), 0u);
+    prep.fill(p->xch_f.as<half_t>() + xslot, 3 * xslot * sizeof(half_t), 0xFFFFFFFFu);
+    prep.fill(p->status.as<unsigned>() + 8, 8 * sizeof(unsigned), 0u);
+    if (p->opt_profile) prep.fill(p->prof.p, 8 * sizeof(long long), 0u);
+    FL_TRY(run_prep(prep, s));
+    p->fw.seats_clean = true;
     FL_TRY(to_exchange_layout(p->Y.as<half_t>(), d.B, d.Hp, size_t(d.Hp), p->xch_f.as<half_t>(), s));
-    if (p->opt_profile) FL_TRY(fill_zero(p->prof.p, 8 * sizeof(long long), s));
     return 0;
 }
 
@@ -484,7 +488,8 @@ int forward_recur(flstm_core_plan* p, size_t t0, size_t n, hipStream_t s) {
     a.status = p->status.as<int>();
     a.seats = p->status.as<unsigned>() + 8;
     a.delay_hint = p->status.as<int>() + 1;   // (the status block: word 0 status, 1 / 2 delay hints, 8..15 seats)
-    FL_TRY(fill_zero(a.seats, 8 * sizeof(unsigned), s));
+    if (!p->fw.seats_clean) FL_TRY(fill_zero(a.seats, 8 * sizeof(unsigned), s));
+    p->fw.seats_clean = false;
     a.B = d.B; a.Hp = d.Hp; a.T = int(p->fw.T); a.t0 = int(t0); a.t1 = int(t0 + n);
     a.spin_limit = p->opt_spin_limit;
     a.spin_ticks = (long long)p->opt_spin_ms * p->wall_khz;
@@ -539,10 +544,10 @@ int forward_pass(flstm_core_plan* p, size_t T, const void* x, flstm_dtype x_dtyp
         if (rc) return rc;
         if (!y_direct)
             FL_TRY(unpad_from_half(p->Y.as<half_t>() + size_t(d.B) * d.Hp, size_t(d.Hp), TB, d.H, y, y_dtype == FLSTM_F32, s));
-        FL_TRY(unpad_from_half(p->Y.as<half_t>() + TB * d.Hp, size_t(d.Hp), size_t(d.B), d.H, hy,
-                               out_state_dtype == FLSTM_F32, s));
-        FL_TRY(unpad_from_float(p->C.as<float>() + TB * d.Hp, size_t(d.Hp), size_t(d.B), d.H, 1.f, cy,
-                                out_state_dtype == FLSTM_F32, s));
+        PrepList out;   // final states, one launch
+        out.unpad(p->Y.as<half_t>() + TB * d.Hp, 0, size_t(d.Hp), size_t(d.B), d.H, 1.f, hy, out_state_dtype == FLSTM_F32);
+        out.unpad(p->C.as<float>() + TB * d.Hp, 1, size_t(d.Hp), size_t(d.B), d.H, 1.f, cy, out_state_dtype == FLSTM_F32);
+        FL_TRY(run_prep(out, s));
         int st = 0;
         rc = wait_status(p, true, s, &st);
         if (rc) return rc;
@@ -659,17 +664,24 @@ int backward_setup(flstm_core_plan* p, size_t T, const void* dY, flstm_dtype dy_
     const size_t xslot = exchange_slot_halfs(rec_bwd_ring_rows(p->Lb, d.B), 4 * d.Hp);
     const size_t dg_slots = size_t(rec_bwd_dg_slots(p->Lb));
     FL_TRY(p->xch_b.reserve(dg_slots * xslot * sizeof(half_t)));
-    FL_TRY(fill_words(p->xch_b.p, dg_slots * xslot * sizeof(half_t), 0xFFFFFFFFu, s));
+    // One launch (see forward_setup): the dG ring 'unwritten', the ring of partial sums in its starting parities, the
+    // scaled state gradients, the bias-gradient partials, the seat counters, the phase counters.
+    static_assert(kRecBwdPartSlots + 6 <= 10, "PrepList holds ten operations");
+    PrepList prep;
+    prep.fill(p->xch_b.p, dg_slots * xslot * sizeof(half_t), 0xFFFFFFFFu);
     if (p->Lb.two_d) {
         const size_t pslot = rec_bwd_part_slot_floats(p->Lb) * sizeof(float);
         FL_TRY(p->part_b.reserve(kRecBwdPartSlots * pslot));
         for (int k = 0; k < kRecBwdPartSlots; ++k)
-            FL_TRY(fill_words(static_cast<char*>(p->part_b.p) + size_t(k) * pslot, pslot, rec_bwd_part_fill(k, int(T)), s));
+            prep.fill(static_cast<char*>(p->part_b.p) + size_t(k) * pslot, pslot, rec_bwd_part_fill(k, int(T)));
     }
-    FL_TRY(convert_pad_f32(d_hn, dstate_dtype == FLSTM_F32, size_t(d.B), d.H, S, p->dHn.as<float>(), size_t(d.Hp), s));
-    FL_TRY(convert_pad_f32(d_cn, dstate_dtype == FLSTM_F32, size_t(d.B), d.H, S, p->dC.as<float>(), size_t(d.Hp), s));
-    FL_TRY(fill_zero(p->db_part.p, size_t(p->Lb.ng) * 4 * d.Hp * sizeof(float), s));
-    if (p->opt_profile) FL_TRY(fill_zero(p->prof.as<long long>() + 8, 8 * sizeof(long long), s));
+    prep.to_float(d_hn, dstate_dtype == FLSTM_F32, size_t(d.B), d.H, S, p->dHn.as<float>(), size_t(d.Hp));
+    prep.to_float(d_cn, dstate_dtype == FLSTM_F32, size_t(d.B), d.H, S, p->dC.as<float>(), size_t(d.Hp));
+    prep.fill(p->db_part.p, size_t(p->Lb.ng) * 4 * d.Hp * sizeof(float), 0u);
+    prep.fill(p->status.as<unsigned>() + 8, 8 * sizeof(unsigned), 0u);
+    if (p->opt_profile) prep.fill(p->prof.as<long long>() + 8, 8 * sizeof(long long), 0u);
+    FL_TRY(run_prep(prep, s));
+    p->bw.seats_clean = true;
     return 0;
 }
 
@@ -711,7 +723,8 @@ int backward_recur(flstm_core_plan* p, long t_hi, long t_lo, hipStream_t s) {
     for (int b_lo = 0; b_lo < d.B; b_lo += win) {
         a.b_lo = b_lo;
         a.b_hi = b_lo + win < d.B ? b_lo + win : d.B;
-        FL_TRY(fill_zero(a.seats, 8 * sizeof(unsigned), s));
+        if (!p->bw.seats_clean) FL_TRY(fill_zero(a.seats, 8 * sizeof(unsigned), s));
+        p->bw.seats_clean = false;
         if (win < d.B) {
             const size_t pslot = a.p_slot * sizeof(float);
             const int first_T = t_hi >= long(p->bw.T) - 1 ? int(p->bw.T) : int(t_hi) + 2;   // (its first product step is first_T - 2)
@@ -797,8 +810,10 @@ int backward_finish(flstm_core_plan* p, const void* x, flstm_dtype x_dtype, floa
     FL_TRY(hipEventRecord(p->tm.ev[6], s));
     if (db_ih || db_hh)
         FL_TRY(reduce_db(d, p->db_part.as<float>(), p->Lb.ng, invS, p->opt_accumulate != 0, db_ih, db_hh, s));
-    FL_TRY(unpad_from_float(p->dH0.as<float>(), size_t(d.Hp), size_t(d.B), d.H, invS, dh0, 1, s));
-    FL_TRY(unpad_from_float(p->dC.as<float>(), size_t(d.Hp), size_t(d.B), d.H, invS, dc0, 1, s));
+    PrepList out;   // state gradients, one launch
+    out.unpad(p->dH0.as<float>(), 1, size_t(d.Hp), size_t(d.B), d.H, invS, dh0, 1);
+    out.unpad(p->dC.as<float>(), 1, size_t(d.Hp), size_t(d.B), d.H, invS, dc0, 1);
+    FL_TRY(run_prep(out, s));
     FL_TRY(hipEventRecord(p->tm.ev[7], s));
     int rc = enqueue_status_copy(p, s);
     if (rc) return rc;

@@ -68,6 +68,51 @@ hipError_t reduce_partials(const float* partial, int splits, size_t per, int row
 hipError_t checksum_add(const void* p, size_t bytes, u64 salt, u64* out, hipStream_t s);
 
 hipError_t fill_zero(void* p, size_t bytes, hipStream_t s);
+
+// Up to ten of the small operations above in ONE launch: a pass starts with half a dozen of them (state rows, rings,
+// counters), each a few microseconds of kernel plus a launch gap of its own when issued one by one.
+struct PrepOp {
+    enum Kind : int { kNone = 0, kFill = 1, kToHalf = 2, kToFloat = 3, kUnpad = 4 };
+    int kind = kNone;
+    int in_f32 = 0, out_f32 = 0;
+    void* dst = nullptr;
+    const void* src = nullptr;   // kToHalf / kToFloat: null reads as zeros
+    size_t n = 0;                // kFill: 32-bit words; kToHalf / kToFloat: rows_out * ld_out elements; kUnpad: rows * cols
+    unsigned word = 0;           // kFill
+    size_t rows = 0, ld_in = 0, ld_out = 1;
+    int cols = 0;
+    float scale = 1.f;
+};
+struct PrepList {
+    int count = 0;
+    PrepOp op[10];
+    void fill(void* p, size_t bytes, unsigned word) {
+        if (bytes == 0) return;
+        PrepOp& o = op[count++];
+        o.kind = PrepOp::kFill; o.dst = p; o.n = bytes / 4; o.word = word;
+    }
+    // the operations of convert_pad() and convert_pad_f32()
+    void to_half(const void* in, int in_f32, size_t rows, int cols, size_t ld_in, float scale, half_t* out, size_t rows_out, size_t ld_out) {
+        if (rows_out * ld_out == 0) return;
+        PrepOp& o = op[count++];
+        o.kind = PrepOp::kToHalf; o.in_f32 = in_f32; o.dst = out; o.src = in; o.n = rows_out * ld_out;
+        o.rows = rows; o.cols = cols; o.ld_in = ld_in; o.ld_out = ld_out; o.scale = scale;
+    }
+    void to_float(const void* in, int in_f32, size_t rows, int cols, float scale, float* out, size_t ld_out) {
+        if (rows * ld_out == 0) return;
+        PrepOp& o = op[count++];
+        o.kind = PrepOp::kToFloat; o.in_f32 = in_f32; o.dst = out; o.src = in; o.n = rows * ld_out;
+        o.rows = rows; o.cols = cols; o.ld_in = size_t(cols); o.ld_out = ld_out; o.scale = scale;
+    }
+    // the operation of unpad_from_half() / unpad_from_float(): out[r][c] = scale * in[r][c], c < cols; a null `out` adds nothing
+    void unpad(const void* in, int in_f32, size_t ld_in, size_t rows, int cols, float scale, void* out, int out_f32) {
+        if (out == nullptr || rows * size_t(cols) == 0) return;
+        PrepOp& o = op[count++];
+        o.kind = PrepOp::kUnpad; o.in_f32 = in_f32; o.out_f32 = out_f32; o.dst = out; o.src = in; o.n = rows * size_t(cols);
+        o.rows = rows; o.cols = cols; o.ld_in = ld_in; o.ld_out = size_t(cols); o.scale = scale;
+    }
+};
+hipError_t run_prep(const PrepList& list, hipStream_t s);
 // fp16 values spread over (-amp, amp) from a hash of the index (operands for timing runs)
 hipError_t fill_noise(half_t* p, size_t n, unsigned seed, float amp, hipStream_t s);
 // Fills a buffer (multiple of 4 bytes) with one 32-bit pattern; a kernel, so it may be captured in a graph.

@@ -220,6 +220,36 @@ __global__ void fill_words_kernel(unsigned* p, size_t words, unsigned value) {
     for (size_t i = size_t(blockIdx.x) * kT + threadIdx.x; i < words; i += stride) p[i] = value;
 }
 
+// blockIdx.y selects the operation, the blocks of a row walk it with a grid stride
+__global__ void prep_kernel(PrepList list) {
+    const PrepOp& o = list.op[blockIdx.y];
+    const size_t stride = size_t(gridDim.x) * kT;
+    const size_t first = size_t(blockIdx.x) * kT + threadIdx.x;
+    if (o.kind == PrepOp::kFill) {
+        unsigned* p = static_cast<unsigned*>(o.dst);
+        for (size_t i = first; i < o.n; i += stride) p[i] = o.word;
+    } else if (o.kind == PrepOp::kToHalf || o.kind == PrepOp::kToFloat) {
+        for (size_t i = first; i < o.n; i += stride) {
+            const size_t r = i / o.ld_out;
+            const int c = int(i % o.ld_out);
+            float v = 0.f;
+            if (o.src != nullptr && r < o.rows && c < o.cols) {
+                const size_t at = r * o.ld_in + c;
+                v = o.scale * (o.in_f32 ? static_cast<const float*>(o.src)[at] : (float)static_cast<const half_t*>(o.src)[at]);
+            }
+            if (o.kind == PrepOp::kToHalf) static_cast<half_t*>(o.dst)[i] = (half_t)v;
+            else static_cast<float*>(o.dst)[i] = v;
+        }
+    } else if (o.kind == PrepOp::kUnpad) {
+        for (size_t i = first; i < o.n; i += stride) {
+            const size_t at = (i / o.cols) * o.ld_in + i % o.cols;
+            const float v = o.scale * (o.in_f32 ? static_cast<const float*>(o.src)[at] : (float)static_cast<const half_t*>(o.src)[at]);
+            if (o.out_f32) static_cast<float*>(o.dst)[i] = v;
+            else static_cast<half_t*>(o.dst)[i] = (half_t)v;
+        }
+    }
+}
+
 }  // namespace
 
 hipError_t pack_weights(const Dims& d, const float* w_ih, const float* w_hh, half_t* wih_p, half_t* wih_t,
@@ -396,6 +426,17 @@ hipError_t fill_words(void* p, size_t bytes, unsigned value, hipStream_t s) {
     int blocks = grid_for(words);
     if (blocks > 4096) blocks = 4096;
     hipLaunchKernelGGL(fill_words_kernel, dim3(blocks), dim3(kT), 0, s, static_cast<unsigned*>(p), words, value);
+    return hipGetLastError();
+}
+
+hipError_t run_prep(const PrepList& list, hipStream_t s) {
+    if (list.count <= 0) return hipSuccess;
+    size_t most = 0;
+    for (int i = 0; i < list.count; ++i) most = list.op[i].n > most ? list.op[i].n : most;
+    size_t blocks = (most + kT - 1) / kT;
+    if (blocks > 256) blocks = 256;
+    if (blocks < 1) blocks = 1;
+    hipLaunchKernelGGL(prep_kernel, dim3(unsigned(blocks), unsigned(list.count)), dim3(kT), 0, s, list);
     return hipGetLastError();
 }
 
