@@ -134,3 +134,39 @@ def test_the_comparison_tool_runs_both_libraries_on_the_same_operands_and_they_a
     for r in rows:
         assert r["own_ms"] > 0 and r["vendor_ms"] > 0
         assert r["max_rel_diff"] < 2e-3, r
+
+
+def test_gemm_kernels_on_seeded_random_shapes():
+    """Twenty-four seeded random shapes per kernel -- tile counts from one to a few dozen (several rounds of the
+    persistent kernels' work lists, workgroups with and without work), K tails, split-K -- against the fp64 product."""
+    L = lib()
+    rng = np.random.default_rng(20240607)
+    s = torch.cuda.current_stream().cuda_stream
+    for case in range(24):
+        g = torch.Generator(device="cuda").manual_seed(1000 + case)
+        # NT: any M, N; K a multiple of 64
+        M, N, K = int(rng.integers(1, 1500)), int(rng.integers(1, 1100)), 64 * int(rng.integers(1, 9))
+        lda, ldb = K + 8 * int(rng.integers(0, 3)), K + 8 * int(rng.integers(0, 3))
+        ldc = N + 4 * int(rng.integers(0, 3))
+        A = rand16(g, M, lda); Bm = rand16(g, N, ldb)
+        f16 = bool(rng.integers(0, 2))
+        bias = torch.randn(N, generator=g, device="cuda") if rng.integers(0, 2) else None
+        C = torch.full((M, ldc), 7.0, device="cuda", dtype=torch.float16 if f16 else torch.float32)
+        rc = L.flstm_gemm_nt(A.data_ptr(), lda, Bm.data_ptr(), ldb, M, N, K, C.data_ptr(), F16 if f16 else F32, ldc, 1.0,
+                             bias.data_ptr() if bias is not None else None, s)
+        assert rc == 0, (case, M, N, K)
+        torch.cuda.synchronize()
+        check(C[:, :N], A[:, :K].double(), Bm[:, :K].double().T, 1.0, bias, f16)
+        assert (C[:, N:] == 7.0).all()
+        # TN: M, N multiples of 8; any K
+        M, N, K = 8 * int(rng.integers(1, 160)), 8 * int(rng.integers(1, 130)), int(rng.integers(1, 1200))
+        splits = int(rng.integers(1, 6))
+        lda, ldb, ldc = M + 8 * int(rng.integers(0, 3)), N + 8 * int(rng.integers(0, 3)), N + 4 * int(rng.integers(0, 2))
+        A = rand16(g, K, lda); Bm = rand16(g, K, ldb)
+        C = torch.full((M, ldc), -3.0, device="cuda")
+        ws = torch.empty(max(L.flstm_gemm_tn_workspace_bytes(M, N, K, splits), 16) // 4, device="cuda")
+        rc = L.flstm_gemm_tn(A.data_ptr(), lda, Bm.data_ptr(), ldb, M, N, K, C.data_ptr(), ldc, 1.0, splits, ws.data_ptr(), s)
+        assert rc == 0, (case, M, N, K, splits)
+        torch.cuda.synchronize()
+        check(C[:, :N], A[:, :M].double().T, Bm[:, :N].double(), 1.0, None, False)
+        assert (C[:, N:] == -3.0).all()
