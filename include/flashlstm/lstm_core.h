@@ -188,9 +188,11 @@ int flstm_core_set_tuned(flstm_core_plan* plan, size_t seq_len, int row_tiles_fw
  *
  * flstm_gemm_nt:  C[M][N] = alpha * A[M][K] * B[N][K]^T (+ bias[n]); A, B fp16 row-major with K contiguous (this
  *   is the input projection X * W_ih^T and, with the transposed weights, dX = dG * W_ih).  K must be a multiple
- *   of 64, lda and ldb multiples of 8; C is fp16 or fp32 with any ldc >= N; bias (fp32, 16-byte aligned) may be null.
+ *   of 64, lda and ldb multiples of 8 and below 2^22; C is fp16 or fp32 with any ldc >= N; bias (fp32, 16-byte aligned)
+ *   may be null.
  * flstm_gemm_tn:  C[M][N] = alpha * sum_k A[k][m] * B[k][n]; A is [K][lda], B is [K][ldb] fp16 (the weight gradients
- *   dG^T * X).  M and N must be multiples of 8, K is arbitrary; C is fp32, 16-byte aligned.  splits > 1 cuts K
+ *   dG^T * X).  M and N must be multiples of 8, K is arbitrary; A and B are 16-byte aligned, lda and ldb multiples of 8
+ *   and below 2^22; C is fp32, 16-byte aligned.  splits > 1 cuts K
  *   into that many slices (at most: every slice gets whole 64-row slabs) whose partial products go to `workspace`
  *   (flstm_gemm_tn_workspace_bytes() bytes of device memory, 16-byte aligned) and are then summed into C.
  * flstm_gemm_tn_auto_splits:  the split count flstm_gemm_tn runs fastest with on a 256-CU part, at most max_splits
